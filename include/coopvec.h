@@ -1,0 +1,261 @@
+/*
+ * coopvec.h -- C-ABI of the MI355X (gfx950) cooperative-vector library.
+ *
+ * The library serves the operator surface Slang declares for CoopVec<T,N>
+ * (source/slang/hlsl.meta.slang:32540-33841) and the two host calls the example
+ * examples/mlp-training-coopvec/mlp-training-coopvec.cpp makes on slang-rhi
+ * (getCooperativeVectorMatrixSize :305, convertCooperativeVectorMatrix :227).
+ *
+ * Slang maps one logical vector to one shader thread; here one call processes a whole
+ * batch of vectors ("samples"): sample s of a batch lives at `base + s * stride` bytes.
+ * Arguments that are `constexpr` in Slang (interpretations, k, layout, transpose, stride)
+ * select a kernel specialisation; everything else is a device pointer or byte offset.
+ *
+ * Conventions
+ *   - every pointer named *device* memory is a plain HIP device address owned by the caller;
+ *     the library never allocates or frees device memory (scratch comes in as `workspace`);
+ *   - every call is asynchronous on the given stream (a `hipStream_t` passed as void*;
+ *     NULL = the default stream) and returns a SlangResult-compatible code
+ *     (include/slang.h:1377-1464): 0 = OK, negative = failure; nothing throws;
+ *   - calls are thread-compatible: no mutable global state besides a per-thread error string;
+ *   - vectors must start at 16-byte-aligned addresses (hlsl.meta.slang:30761-30764,
+ *     30874-30878); matrices and biases at 64-byte-aligned addresses like the example's
+ *     sub-allocations (mlp-training-coopvec.cpp:273-279).
+ */
+#ifndef COOPVEC_H
+#define COOPVEC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(_WIN32)
+#define CV_API __declspec(dllexport)
+#else
+#define CV_API __attribute__((visibility("default")))
+#endif
+
+/* ---- result codes: numerically equal to SLANG_OK / SLANG_E_* (include/slang.h:1400-1464) */
+typedef int32_t CvResult;
+#define CV_OK                  ((CvResult)0)
+#define CV_FAIL                ((CvResult)0x80004005)
+#define CV_E_NOT_IMPLEMENTED   ((CvResult)0x80004001)
+#define CV_E_INVALID_ARG       ((CvResult)0x80070057)
+#define CV_E_BUFFER_TOO_SMALL  ((CvResult)0x82000001)
+#define CV_E_INTERNAL_FAIL     ((CvResult)0x82000006)
+#define CV_E_NOT_AVAILABLE     ((CvResult)0x82000007)
+#define CV_FAILED(r)           ((r) < 0)
+
+/* ---- CoopVecMatrixLayout (hlsl.meta.slang:32547-32553, include/slang.h:948-955) */
+typedef enum CvMatrixLayout {
+    CV_LAYOUT_ROW_MAJOR = 0,
+    CV_LAYOUT_COLUMN_MAJOR = 1,
+    CV_LAYOUT_INFERENCING_OPTIMAL = 2,
+    CV_LAYOUT_TRAINING_OPTIMAL = 3
+} CvMatrixLayout;
+
+/* ---- CoopVecComponentType (hlsl.meta.slang:32558-32575), same numeric values.  Used both
+ *      for interpretations and for the element type of a vector in memory. */
+typedef enum CvComponentType {
+    CV_FLOAT_E4M3 = 0, CV_FLOAT_E5M2 = 1, CV_FLOAT16 = 2, CV_FLOAT32 = 3, CV_FLOAT64 = 4,
+    CV_SINT8 = 5, CV_SINT16 = 6, CV_SINT32 = 7, CV_SINT64 = 8, CV_SINT8_PACKED = 9,
+    CV_UINT8 = 10, CV_UINT16 = 11, CV_UINT32 = 12, CV_UINT64 = 13, CV_UINT8_PACKED = 14,
+    CV_COMPONENT_NONE = -1
+} CvComponentType;
+
+/* Activation fused behind a matMulAdd.  RELU is max(z, 0) as the neural module defines it
+ * (source/standard-modules/neural/activations.slang:25-42); LEAKY_RELU is the example's
+ * max(z, z * slope) evaluated in half (examples/mlp-training-coopvec/fflayer.slang:64-65). */
+typedef enum CvActivation { CV_ACT_NONE = 0, CV_ACT_RELU = 1, CV_ACT_LEAKY_RELU = 2 } CvActivation;
+
+/* Mirrors the fields the example fills in rhi::CooperativeVectorMatrixDesc
+ * (mlp-training-coopvec.cpp:204-225).  `offset` is in bytes from the buffer handed to
+ * cvConvertMatrices; rowColumnStride is bytes between rows (RowMajor) or columns
+ * (ColumnMajor), 0 = tightly packed, ignored for the Optimal layouts. */
+typedef struct CvMatrixDesc {
+    uint32_t rowCount;
+    uint32_t colCount;
+    int32_t  componentType;   /* CvComponentType */
+    int32_t  layout;          /* CvMatrixLayout */
+    size_t   size;
+    size_t   offset;
+    size_t   rowColumnStride;
+} CvMatrixDesc;
+
+/* Shape of include/slang.h:5215-5229 CooperativeVectorCombination, with component types. */
+typedef struct CvCombination {
+    int32_t  inputType;
+    int32_t  inputInterpretation;
+    uint32_t inputPackingFactor;
+    int32_t  matrixInterpretation;
+    int32_t  biasInterpretation;   /* CV_COMPONENT_NONE: no bias operand */
+    int32_t  resultType;
+    int32_t  transpose;
+} CvCombination;
+
+/* ------------------------------------------------------------------------------------ */
+/* library                                                                              */
+/* ------------------------------------------------------------------------------------ */
+
+/* Version of this ABI (major<<16 | minor). */
+CV_API uint32_t cvGetVersion(void);
+/* Message describing the last failure on the calling thread ("" if none). */
+CV_API const char* cvGetLastErrorMessage(void);
+/* Helpers replacing hlsl.meta.slang:32578-32593 / :32596-32633 / :32636-32670. */
+CV_API int32_t cvComponentPackingFactor(int32_t componentType);
+CV_API int32_t cvComponentScalarType(int32_t componentType);      /* SLANG_SCALAR_TYPE_* or -1 */
+CV_API int32_t cvComponentTypeStride(int32_t componentType);      /* bytes, -1 if unknown */
+/* The (type, interpretation) combinations cvMatMul accepts, in the shape a host compares
+ * against ICooperativeTypesMetadata (include/slang.h:5231-5273).  Returns the total count;
+ * fills at most `capacity` entries. */
+CV_API uint32_t cvQuerySupportedCombinations(CvCombination* out, uint32_t capacity);
+
+/* ------------------------------------------------------------------------------------ */
+/* host surface: size query and layout conversion                                       */
+/* ------------------------------------------------------------------------------------ */
+
+/* Replaces rhi::IDevice::getCooperativeVectorMatrixSize (call site
+ * mlp-training-coopvec.cpp:305-311).  Size in bytes (multiple of 64 for Optimal layouts). */
+CV_API CvResult cvGetMatrixSize(uint32_t rowCount, uint32_t colCount, int32_t componentType,
+                                int32_t layout, size_t rowColumnStride, size_t* outSize);
+
+/* Replaces rhi::ICommandEncoder::convertCooperativeVectorMatrix (call site
+ * mlp-training-coopvec.cpp:227-232): converts `count` matrices from srcDescs[i] inside
+ * srcBuffer to dstDescs[i] inside dstBuffer in one launch.  Row/column counts must match;
+ * component types must match or be a FLOAT16/FLOAT32 pair (round to nearest even).
+ * Padding of Optimal destinations is written as zero.  Source and destination ranges must
+ * not overlap.  At most 64 matrices per call. */
+CV_API CvResult cvConvertMatrices(void* stream, void* dstBuffer, const CvMatrixDesc* dstDescs,
+                                  const void* srcBuffer, const CvMatrixDesc* srcDescs,
+                                  uint32_t count);
+
+/* ------------------------------------------------------------------------------------ */
+/* operator surface                                                                     */
+/* ------------------------------------------------------------------------------------ */
+
+/* coopVecMatMul / coopVecMatMulAdd / coopVecMatMul[Add]Packed over a batch
+ * (hlsl.meta.slang:32786-33190; IR operand order slang-ir-insts.lua:1694-1718):
+ *
+ *   output[s][i] = act( cast<resultType>( sum_{j<k} W[i][j] * input[s][j]  + bias[i] ) )
+ *
+ * W is M x k unless `transpose`, in which case memory holds k x M and is used transposed.
+ * Float types accumulate in fp32, integer types in int32 (exact).
+ * accumulate != 0 gives the member forms matMulAccum / matMulAddAccum
+ * (hlsl.meta.slang:31476-31650): output += result (activation must be NONE).
+ */
+typedef struct CvMatMulDesc {
+    /* vectors */
+    const void* input;          /* device; sample s at input + s*inputStride */
+    size_t      inputStride;    /* bytes */
+    int32_t     inputType;      /* element type of CoopVec<U,PackedK> in memory */
+    int32_t     inputInterpretation;
+    int32_t     k;              /* logical input length; == 4*PackedK for *_PACKED */
+    void*       output;         /* device; sample s at output + s*outputStride */
+    size_t      outputStride;
+    int32_t     resultType;     /* element type T of CoopVec<T,M> */
+    int32_t     m;
+    /* matrix */
+    const void* matrix;         /* device */
+    size_t      matrixOffset;   /* bytes */
+    int32_t     matrixInterpretation;
+    int32_t     layout;         /* CvMatrixLayout */
+    int32_t     transpose;
+    uint32_t    matrixStride;   /* bytes; ignored for Optimal layouts */
+    /* bias (optional) */
+    const void* bias;           /* device or NULL (coopVecMatMul) */
+    size_t      biasOffset;
+    int32_t     biasInterpretation;
+    /* extras */
+    int32_t     activation;     /* CvActivation */
+    float       leakySlope;
+    int32_t     accumulate;
+    uint32_t    batch;          /* number of samples */
+} CvMatMulDesc;
+
+CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* desc);
+
+/* coopVecOuterProductAccumulate over a batch (hlsl.meta.slang:33227-33316):
+ *   Mat[i][j] += sum_s a[s][i] * b[s][j]
+ * The per-sample atomics of the reference are replaced by an MFMA contraction over the batch,
+ * per-workgroup fp32 partials in `workspace` and one fixed-order reduction, so the result is
+ * bitwise reproducible.  a and b are FLOAT16 vectors; the matrix interpretation is FLOAT16
+ * or FLOAT32; all four layouts are accepted for the destination. */
+CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t m, int32_t n, uint32_t batch,
+                                                      size_t* outBytes);
+CV_API CvResult cvOuterProductAccumulate(void* stream,
+                                         const void* a, size_t aStride, int32_t m,
+                                         const void* b, size_t bStride, int32_t n,
+                                         int32_t elementType, uint32_t batch,
+                                         void* matrix, size_t matrixOffset, uint32_t matrixStride,
+                                         int32_t layout, int32_t matrixInterpretation,
+                                         void* workspace, size_t workspaceBytes);
+
+/* coopVecReduceSumAccumulate over a batch (hlsl.meta.slang:33330-33353):
+ *   buffer[i] += sum_s v[s][i]
+ * v is FLOAT16; `bufferType` is FLOAT16 (the reference's rule: destination type = vector
+ * type) or FLOAT32 (what "bias gradients into fp32 buffers" needs). Deterministic. */
+CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t n, uint32_t batch, size_t* outBytes);
+CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStride, int32_t n,
+                                      int32_t elementType, uint32_t batch,
+                                      void* buffer, size_t offset, int32_t bufferType,
+                                      void* workspace, size_t workspaceBytes);
+
+/* ------------------------------------------------------------------------------------ */
+/* fused MLP: the example's FeedForwardLayer chain                                       */
+/* ------------------------------------------------------------------------------------ */
+
+/* One layer; pointers are arranged like the example's per-layer 4 x u64 block
+ * {weights, weightsGrad, biases, biasesGrad} (mlp-training-coopvec.cpp:146-158,
+ * fflayer.slang:9-12). */
+typedef struct CvMlpLayer {
+    const void* weights;        /* device */
+    void*       weightsGrad;    /* device or NULL (forward only) */
+    const void* biases;         /* device or NULL */
+    void*       biasesGrad;     /* device or NULL */
+    int32_t     inputSize;
+    int32_t     outputSize;
+    int32_t     weightLayout;   /* layout of `weights` */
+    uint32_t    weightStride;   /* bytes, Row/ColumnMajor only */
+    int32_t     gradLayout;     /* layout of `weightsGrad` */
+    uint32_t    gradStride;
+    int32_t     activation;     /* CvActivation applied to this layer's output */
+    float       leakySlope;
+} CvMlpLayer;
+
+typedef struct CvMlpDesc {
+    const CvMlpLayer* layers;   /* host array */
+    int32_t  numLayers;
+    int32_t  inputType;         /* element type of the input vectors in memory */
+    int32_t  weightType;        /* matrix interpretation of every layer: FLOAT16 or FLOAT_E4M3 */
+    int32_t  biasType;          /* FLOAT16 */
+    int32_t  outputType;        /* FLOAT16 */
+    int32_t  gradType;          /* FLOAT16 or FLOAT32: element type of weightsGrad/biasesGrad */
+} CvMlpDesc;
+
+/* y = layer_{n-1}( ... layer_0(x) ): every layer is coopVecMatMulAdd + activation with
+ * CoopVec<half> as the carrier between layers; with weightType FLOAT_E4M3 the carrier is
+ * re-quantised to OCP e4m3 (saturating) in front of every layer.  Activations stay in
+ * registers between layers. */
+CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp,
+                             const void* input, size_t inputStride,
+                             void* output, size_t outputStride, uint32_t batch);
+
+/* Forward + reverse pass of loss_s = sum_i (y[s][i] - target[s][i])^2 with seed `lossScale`
+ * (the example: bwd_diff(loss)(network, x, y, 1.0h), kernels.slang:20): accumulates
+ * sum_s dY (x) X into every layer's weightsGrad and sum_s dY into biasesGrad ("+=").
+ * targets == NULL selects target = sin(sum of the sample's inputs) for every output.
+ * lossSum (device, optional, one float) is overwritten with sum_s loss_s. */
+CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes);
+CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp,
+                               const void* input, size_t inputStride,
+                               const void* targets, size_t targetStride,
+                               float lossScale, uint32_t batch, float* lossSum,
+                               void* workspace, size_t workspaceBytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COOPVEC_H */

@@ -1,0 +1,118 @@
+"""Loader for the gfx950 shared library.  There is no CPU fallback: if the library is
+missing or cannot be loaded every operator raises."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG_DIR, "libcoopvec_mi355x.so")
+
+_lib = None
+
+
+class CoopVecLibraryMissing(ImportError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Return the loaded library, loading it on first use."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise CoopVecLibraryMissing(
+            "%s is not built; run `python -m slang_amd.build` (needs hipcc). "
+            "There is no CPU fallback for the cooperative-vector operators." % LIB_PATH)
+    # torch ships the HIP runtime this process uses for device memory and streams; importing it
+    # first makes the library bind to that same runtime instance (same SONAME).
+    import torch  # noqa: F401
+    _lib = ctypes.CDLL(LIB_PATH)
+    _declare(_lib)
+    return _lib
+
+
+class CvMatrixDesc(ctypes.Structure):
+    _fields_ = [("rowCount", ctypes.c_uint32), ("colCount", ctypes.c_uint32),
+                ("componentType", ctypes.c_int32), ("layout", ctypes.c_int32),
+                ("size", ctypes.c_size_t), ("offset", ctypes.c_size_t),
+                ("rowColumnStride", ctypes.c_size_t)]
+
+
+class CvCombination(ctypes.Structure):
+    _fields_ = [("inputType", ctypes.c_int32), ("inputInterpretation", ctypes.c_int32),
+                ("inputPackingFactor", ctypes.c_uint32), ("matrixInterpretation", ctypes.c_int32),
+                ("biasInterpretation", ctypes.c_int32), ("resultType", ctypes.c_int32),
+                ("transpose", ctypes.c_int32)]
+
+
+class CvMatMulDesc(ctypes.Structure):
+    _fields_ = [("input", ctypes.c_void_p), ("inputStride", ctypes.c_size_t),
+                ("inputType", ctypes.c_int32), ("inputInterpretation", ctypes.c_int32),
+                ("k", ctypes.c_int32),
+                ("output", ctypes.c_void_p), ("outputStride", ctypes.c_size_t),
+                ("resultType", ctypes.c_int32), ("m", ctypes.c_int32),
+                ("matrix", ctypes.c_void_p), ("matrixOffset", ctypes.c_size_t),
+                ("matrixInterpretation", ctypes.c_int32), ("layout", ctypes.c_int32),
+                ("transpose", ctypes.c_int32), ("matrixStride", ctypes.c_uint32),
+                ("bias", ctypes.c_void_p), ("biasOffset", ctypes.c_size_t),
+                ("biasInterpretation", ctypes.c_int32),
+                ("activation", ctypes.c_int32), ("leakySlope", ctypes.c_float),
+                ("accumulate", ctypes.c_int32), ("batch", ctypes.c_uint32)]
+
+
+class CvMlpLayer(ctypes.Structure):
+    _fields_ = [("weights", ctypes.c_void_p), ("weightsGrad", ctypes.c_void_p),
+                ("biases", ctypes.c_void_p), ("biasesGrad", ctypes.c_void_p),
+                ("inputSize", ctypes.c_int32), ("outputSize", ctypes.c_int32),
+                ("weightLayout", ctypes.c_int32), ("weightStride", ctypes.c_uint32),
+                ("gradLayout", ctypes.c_int32), ("gradStride", ctypes.c_uint32),
+                ("activation", ctypes.c_int32), ("leakySlope", ctypes.c_float)]
+
+
+class CvMlpDesc(ctypes.Structure):
+    _fields_ = [("layers", ctypes.POINTER(CvMlpLayer)), ("numLayers", ctypes.c_int32),
+                ("inputType", ctypes.c_int32), ("weightType", ctypes.c_int32),
+                ("biasType", ctypes.c_int32), ("outputType", ctypes.c_int32),
+                ("gradType", ctypes.c_int32)]
+
+
+# name -> (restype, argtypes); every function include/coopvec.h declares
+SIGNATURES = {
+    "cvGetVersion": (ctypes.c_uint32, []),
+    "cvGetLastErrorMessage": (ctypes.c_char_p, []),
+    "cvComponentPackingFactor": (ctypes.c_int32, [ctypes.c_int32]),
+    "cvComponentScalarType": (ctypes.c_int32, [ctypes.c_int32]),
+    "cvComponentTypeStride": (ctypes.c_int32, [ctypes.c_int32]),
+    "cvQuerySupportedCombinations": (ctypes.c_uint32, [ctypes.POINTER(CvCombination), ctypes.c_uint32]),
+    "cvGetMatrixSize": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int32, ctypes.c_int32,
+                                         ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]),
+    "cvConvertMatrices": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(CvMatrixDesc),
+                                           ctypes.c_void_p, ctypes.POINTER(CvMatrixDesc), ctypes.c_uint32]),
+    "cvMatMul": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMatMulDesc)]),
+    "cvOuterProductAccumulateWorkspaceSize": (ctypes.c_int32, [ctypes.c_int32, ctypes.c_int32, ctypes.c_uint32,
+                                                               ctypes.POINTER(ctypes.c_size_t)]),
+    "cvOuterProductAccumulate": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32,
+                                                  ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32, ctypes.c_int32,
+                                                  ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32,
+                                                  ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t]),
+    "cvReduceSumAccumulateWorkspaceSize": (ctypes.c_int32, [ctypes.c_int32, ctypes.c_uint32,
+                                                            ctypes.POINTER(ctypes.c_size_t)]),
+    "cvReduceSumAccumulate": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32,
+                                               ctypes.c_int32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t,
+                                               ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t]),
+    "cvMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                      ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
+    "cvMlpTrainStepWorkspaceSize": (ctypes.c_int32, [ctypes.POINTER(CvMlpDesc), ctypes.c_uint32,
+                                                     ctypes.POINTER(ctypes.c_size_t)]),
+    "cvMlpTrainStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                        ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32,
+                                        ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+}
+
+
+def _declare(lib: ctypes.CDLL) -> None:
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)   # AttributeError if the library lacks a declared symbol
+        fn.restype = restype
+        fn.argtypes = argtypes

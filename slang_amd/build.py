@@ -1,0 +1,92 @@
+"""Build recipe for the gfx950 library and (optionally) the CPU oracle.
+
+    python -m slang_amd.build            # compile slang_amd/libcoopvec_mi355x.so
+    python -m slang_amd.build --oracle   # also oracle/libcoopvec_oracle.so
+
+hipcc cross-compiles for gfx950 without a GPU.  Objects go to build/ (git-ignored), the
+shared library next to this file so that it travels with the source tree.
+"""
+from __future__ import annotations
+
+import argparse
+import concurrent.futures as cf
+import os
+import shutil
+import subprocess
+import sys
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_DIR = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+LIB_NAME = "libcoopvec_mi355x.so"
+LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
+ORACLE_DIR = os.path.join(REPO_DIR, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "libcoopvec_oracle.so")
+
+HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul.hip", "cv_mlp.hip", "cv_train.hip"]
+
+# packed-fp32 instructions are switched off on purpose (see the flag below): hipcc would
+# otherwise form v_pk_*_f32 from ordinary float code.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+
+
+def build_library(jobs: int = 4, verbose: bool = False) -> str:
+    """Compile every HIP source for gfx950 and link the shared library.  Always recompiles."""
+    hipcc = _hipcc()
+    obj_dir = os.path.join(REPO_DIR, "build", "obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = []
+    cmds = []
+    for src in sources:
+        obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmds.append([hipcc, *HIPCC_FLAGS, "-I", os.path.join(REPO_DIR, "include"), "-c",
+                     os.path.join(CSRC, src), "-o", obj])
+    with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
+        for cmd, _ in zip(cmds, pool.map(_run, cmds)):
+            if verbose:
+                print(" ".join(cmd))
+    tmp = LIB_PATH + ".tmp"
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs])
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+def build_oracle() -> str:
+    """Compile the CPU oracle (test infrastructure) with the host C compiler."""
+    _run(["make", "-C", ORACLE_DIR, "-B", "libcoopvec_oracle.so"])
+    return ORACLE_LIB
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--oracle", action="store_true", help="also build the CPU oracle")
+    ap.add_argument("-j", "--jobs", type=int, default=4)
+    ap.add_argument("-v", "--verbose", action="store_true")
+    args = ap.parse_args(argv)
+    print(build_library(args.jobs, args.verbose))
+    if args.oracle:
+        print(build_oracle())
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

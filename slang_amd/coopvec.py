@@ -1,0 +1,299 @@
+"""Host-side mirror of Slang's cooperative-vector operator surface, served by the gfx950 library.
+
+Names, argument order and argument meaning follow the Slang declarations
+(source/slang/hlsl.meta.slang:32954 coopVecMatMul, :32786 coopVecMatMulPacked,
+:33160 coopVecMatMulAdd, :32983 coopVecMatMulAddPacked, :33227 coopVecOuterProductAccumulate,
+:33330 coopVecReduceSumAccumulate) and the two slang-rhi calls the example makes
+(examples/mlp-training-coopvec/mlp-training-coopvec.cpp:305 getCooperativeVectorMatrixSize,
+:227 convertCooperativeVectorMatrix).
+
+Where Slang has one CoopVec<T,N> per shader thread, these functions take a batch: a 2-D torch
+tensor [batch, N] on the GPU, one row per thread.  Buffers (ByteAddressBuffer in Slang) are 1-D
+torch tensors used as raw bytes.  torch only supplies device memory and the stream; all
+arithmetic happens in the HIP library, and every function raises if that library is missing.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+from dataclasses import dataclass
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+
+
+class CoopVecMatrixLayout(enum.IntEnum):
+    """hlsl.meta.slang:32547-32553"""
+    RowMajor = 0
+    ColumnMajor = 1
+    InferencingOptimal = 2
+    TrainingOptimal = 3
+
+
+class CoopVecComponentType(enum.IntEnum):
+    """hlsl.meta.slang:32558-32575"""
+    FloatE4M3 = 0
+    FloatE5M2 = 1
+    Float16 = 2
+    Float32 = 3
+    Float64 = 4
+    SignedInt8 = 5
+    SignedInt16 = 6
+    SignedInt32 = 7
+    SignedInt64 = 8
+    SignedInt8Packed = 9
+    UnsignedInt8 = 10
+    UnsignedInt16 = 11
+    UnsignedInt32 = 12
+    UnsignedInt64 = 13
+    UnsignedInt8Packed = 14
+
+
+class Activation(enum.IntEnum):
+    NoActivation = 0
+    ReLU = 1
+    LeakyReLU = 2
+
+
+# SlangResult values (include/slang.h:1400-1464)
+SLANG_OK = 0
+SLANG_FAIL = -2147467259            # 0x80004005
+SLANG_E_NOT_IMPLEMENTED = -2147467263   # 0x80004001
+SLANG_E_INVALID_ARG = -2147024809   # 0x80070057
+SLANG_E_BUFFER_TOO_SMALL = -2113929215  # 0x82000001
+SLANG_E_INTERNAL_FAIL = -2113929210     # 0x82000006
+SLANG_E_NOT_AVAILABLE = -2113929209     # 0x82000007
+
+
+class CoopVecError(RuntimeError):
+    """A failed library call; `.result` is the SlangResult-compatible code."""
+
+    def __init__(self, result: int, message: str):
+        super().__init__("%s (SlangResult 0x%08x)" % (message, result & 0xFFFFFFFF))
+        self.result = result
+
+
+def _check(rc: int) -> None:
+    if rc < 0:
+        raise CoopVecError(rc, _lib.load().cvGetLastErrorMessage().decode("utf-8", "replace"))
+
+
+def _stream_handle(stream) -> ctypes.c_void_p:
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    if isinstance(stream, torch.cuda.Stream):
+        return ctypes.c_void_p(stream.cuda_stream)
+    return ctypes.c_void_p(int(stream))
+
+
+_TORCH_TO_CT = {
+    torch.float16: CoopVecComponentType.Float16,
+    torch.float32: CoopVecComponentType.Float32,
+    torch.int8: CoopVecComponentType.SignedInt8,
+    torch.uint8: CoopVecComponentType.UnsignedInt8,
+    torch.int32: CoopVecComponentType.SignedInt32,
+}
+if hasattr(torch, "uint32"):
+    _TORCH_TO_CT[torch.uint32] = CoopVecComponentType.UnsignedInt32
+if hasattr(torch, "float8_e4m3fn"):
+    _TORCH_TO_CT[torch.float8_e4m3fn] = CoopVecComponentType.FloatE4M3
+
+_CT_TO_TORCH = {
+    CoopVecComponentType.Float16: torch.float16,
+    CoopVecComponentType.Float32: torch.float32,
+    CoopVecComponentType.SignedInt32: torch.int32,
+}
+
+
+def componentPackingFactor(componentType: int) -> int:
+    """hlsl.meta.slang:32578-32587"""
+    return _lib.load().cvComponentPackingFactor(int(componentType))
+
+
+def componentTypeStride(componentType: int) -> int:
+    return _lib.load().cvComponentTypeStride(int(componentType))
+
+
+def querySupportedCombinations():
+    lib = _lib.load()
+    n = lib.cvQuerySupportedCombinations(None, 0)
+    arr = (_lib.CvCombination * n)()
+    lib.cvQuerySupportedCombinations(arr, n)
+    return [dict(inputType=CoopVecComponentType(c.inputType),
+                 inputInterpretation=CoopVecComponentType(c.inputInterpretation),
+                 inputPackingFactor=c.inputPackingFactor,
+                 matrixInterpretation=CoopVecComponentType(c.matrixInterpretation),
+                 biasInterpretation=CoopVecComponentType(c.biasInterpretation),
+                 resultType=CoopVecComponentType(c.resultType),
+                 transpose=bool(c.transpose)) for c in arr]
+
+
+# ---------------------------------------------------------------------------------------------
+# host surface
+# ---------------------------------------------------------------------------------------------
+
+def getCooperativeVectorMatrixSize(rowCount: int, colCount: int, componentType: int, layout: int,
+                                   rowColumnStride: int = 0) -> int:
+    """Bytes needed for a matrix (rhi::IDevice::getCooperativeVectorMatrixSize,
+    mlp-training-coopvec.cpp:305-311)."""
+    out = ctypes.c_size_t(0)
+    _check(_lib.load().cvGetMatrixSize(rowCount, colCount, int(componentType), int(layout),
+                                       rowColumnStride, ctypes.byref(out)))
+    return out.value
+
+
+@dataclass
+class CooperativeVectorMatrixDesc:
+    """Fields of rhi::CooperativeVectorMatrixDesc as the example fills them
+    (mlp-training-coopvec.cpp:204-225)."""
+    rowCount: int = 0
+    colCount: int = 0
+    componentType: int = CoopVecComponentType.Float16
+    layout: int = CoopVecMatrixLayout.RowMajor
+    size: int = 0
+    offset: int = 0
+    rowColumnStride: int = 0
+
+    def _c(self) -> "_lib.CvMatrixDesc":
+        return _lib.CvMatrixDesc(self.rowCount, self.colCount, int(self.componentType), int(self.layout),
+                                 self.size, self.offset, self.rowColumnStride)
+
+
+def _buffer_ptr(buf: torch.Tensor, what: str) -> int:
+    if not isinstance(buf, torch.Tensor) or not buf.is_cuda:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "%s must be a GPU tensor" % what)
+    if not buf.is_contiguous():
+        raise CoopVecError(SLANG_E_INVALID_ARG, "%s must be contiguous" % what)
+    return buf.data_ptr()
+
+
+def convertCooperativeVectorMatrix(dstBuffer: torch.Tensor, dstDescs: Sequence[CooperativeVectorMatrixDesc],
+                                   srcBuffer: torch.Tensor, srcDescs: Sequence[CooperativeVectorMatrixDesc],
+                                   matrixCount: Optional[int] = None, stream=None) -> None:
+    """rhi::ICommandEncoder::convertCooperativeVectorMatrix (mlp-training-coopvec.cpp:227-232)."""
+    n = len(srcDescs) if matrixCount is None else matrixCount
+    if len(dstDescs) < n or len(srcDescs) < n:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "fewer descs than matrixCount")
+    d = (_lib.CvMatrixDesc * max(n, 1))(*[x._c() for x in dstDescs[:n]])
+    s = (_lib.CvMatrixDesc * max(n, 1))(*[x._c() for x in srcDescs[:n]])
+    for descs, buf, what in ((dstDescs[:n], dstBuffer, "dst"), (srcDescs[:n], srcBuffer, "src")):
+        nbytes = buf.numel() * buf.element_size()
+        for i, x in enumerate(descs):
+            if x.offset + x.size > nbytes:
+                raise CoopVecError(SLANG_E_BUFFER_TOO_SMALL,
+                                   "%s desc %d: offset+size %d exceeds the buffer (%d bytes)"
+                                   % (what, i, x.offset + x.size, nbytes))
+    _check(_lib.load().cvConvertMatrices(_stream_handle(stream), _buffer_ptr(dstBuffer, "dstBuffer"), d,
+                                         _buffer_ptr(srcBuffer, "srcBuffer"), s, n))
+
+
+# ---------------------------------------------------------------------------------------------
+# operator surface
+# ---------------------------------------------------------------------------------------------
+
+def _vector_info(v: torch.Tensor, interpretation: int, what: str):
+    if not isinstance(v, torch.Tensor) or not v.is_cuda or v.dim() != 2:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "%s must be a 2-D GPU tensor [batch, N]" % what)
+    if v.stride(1) != 1:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "%s: elements of one vector must be contiguous" % what)
+    ct = _TORCH_TO_CT.get(v.dtype)
+    if ct is None:
+        raise CoopVecError(SLANG_E_NOT_AVAILABLE, "%s: unsupported element dtype %s" % (what, v.dtype))
+    # a byte tensor interpreted as e4m3 carries e4m3 elements
+    if ct == CoopVecComponentType.UnsignedInt8 and interpretation == CoopVecComponentType.FloatE4M3:
+        ct = CoopVecComponentType.FloatE4M3
+    return ct, v.stride(0) * v.element_size()
+
+
+def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, bias, biasOffset,
+            biasInterpretation, memoryLayout, transpose, matrixStride, M, resultType, activation, leakySlope,
+            accumulate, out, stream):
+    lib = _lib.load()
+    inCt, inStride = _vector_info(input, inputInterpretation, "input")
+    batch = input.shape[0]
+    if resultType is None:
+        resultType = (CoopVecComponentType.SignedInt32 if inCt in (
+            CoopVecComponentType.SignedInt8, CoopVecComponentType.SignedInt32,
+            CoopVecComponentType.UnsignedInt32) else CoopVecComponentType.Float16)
+    if out is None:
+        if accumulate:
+            raise CoopVecError(SLANG_E_INVALID_ARG, "the accumulate forms need `out` (the vector added to)")
+        dt = _CT_TO_TORCH.get(CoopVecComponentType(resultType))
+        if dt is None:
+            raise CoopVecError(SLANG_E_NOT_AVAILABLE, "unsupported result type %s" % resultType)
+        out = torch.empty((batch, M), dtype=dt, device=input.device)
+    outCt, outStride = _vector_info(out, resultType, "out")
+    if out.shape[0] != batch or out.shape[1] != M or outCt != resultType:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "out must be [batch, M] of the result type")
+    d = _lib.CvMatMulDesc()
+    d.input = input.data_ptr(); d.inputStride = inStride
+    d.inputType = int(inCt); d.inputInterpretation = int(inputInterpretation); d.k = int(k)
+    d.output = out.data_ptr(); d.outputStride = outStride
+    d.resultType = int(resultType); d.m = int(M)
+    d.matrix = _buffer_ptr(matrix, "matrix"); d.matrixOffset = int(matrixOffset)
+    d.matrixInterpretation = int(matrixInterpretation); d.layout = int(memoryLayout)
+    d.transpose = 1 if transpose else 0; d.matrixStride = int(matrixStride)
+    if bias is not None:
+        d.bias = _buffer_ptr(bias, "bias"); d.biasOffset = int(biasOffset)
+        d.biasInterpretation = int(biasInterpretation)
+    else:
+        d.bias = None; d.biasOffset = 0; d.biasInterpretation = -1
+    d.activation = int(activation); d.leakySlope = float(leakySlope)
+    d.accumulate = 1 if accumulate else 0; d.batch = batch
+    _check(lib.cvMatMul(_stream_handle(stream), ctypes.byref(d)))
+    return out
+
+
+def coopVecMatMulPacked(input: torch.Tensor, inputInterpretation: int, k: int, matrix: torch.Tensor,
+                        matrixOffset: int, matrixInterpretation: int, memoryLayout: int, transpose: bool,
+                        matrixStride: int, *, M: int, resultType: Optional[int] = None,
+                        out: Optional[torch.Tensor] = None, accumulate: bool = False, stream=None):
+    """coopVecMatMulPacked<T,M,PackedK,U> (hlsl.meta.slang:32786-32796); accumulate=True is the
+    member form matMulAccumPacked (:31476)."""
+    return _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, None, 0, -1,
+                   memoryLayout, transpose, matrixStride, M, resultType, Activation.NoActivation, 0.0,
+                   accumulate, out, stream)
+
+
+def coopVecMatMul(input: torch.Tensor, inputInterpretation: int, matrix: torch.Tensor, matrixOffset: int,
+                  matrixInterpretation: int, memoryLayout: int, transpose: bool, matrixStride: int, *,
+                  M: int, resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                  accumulate: bool = False, stream=None):
+    """coopVecMatMul<T,M,K,U> (hlsl.meta.slang:32954-32963)."""
+    if componentPackingFactor(inputInterpretation) != 1:   # static_assert :32965
+        raise CoopVecError(SLANG_E_INVALID_ARG,
+                           "for packed inputInterpretation values please use coopVecMatMulPacked and specify k manually")
+    return coopVecMatMulPacked(input, inputInterpretation, input.shape[1], matrix, matrixOffset,
+                               matrixInterpretation, memoryLayout, transpose, matrixStride, M=M,
+                               resultType=resultType, out=out, accumulate=accumulate, stream=stream)
+
+
+def coopVecMatMulAddPacked(input: torch.Tensor, inputInterpretation: int, k: int, matrix: torch.Tensor,
+                           matrixOffset: int, matrixInterpretation: int, bias: torch.Tensor, biasOffset: int,
+                           biasInterpretation: int, memoryLayout: int, transpose: bool, matrixStride: int, *,
+                           M: int, resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                           accumulate: bool = False, activation: int = Activation.NoActivation,
+                           leakySlope: float = 0.0, stream=None):
+    """coopVecMatMulAddPacked<T,M,PackedK,U> (hlsl.meta.slang:32983-32996)."""
+    return _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, bias, biasOffset,
+                   biasInterpretation, memoryLayout, transpose, matrixStride, M, resultType, activation,
+                   leakySlope, accumulate, out, stream)
+
+
+def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torch.Tensor, matrixOffset: int,
+                     matrixInterpretation: int, bias: torch.Tensor, biasOffset: int, biasInterpretation: int,
+                     memoryLayout: int, transpose: bool, matrixStride: int, *, M: int,
+                     resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                     accumulate: bool = False, activation: int = Activation.NoActivation,
+                     leakySlope: float = 0.0, stream=None):
+    """coopVecMatMulAdd<T,M,K,U> (hlsl.meta.slang:33160-33173)."""
+    if componentPackingFactor(inputInterpretation) != 1:
+        raise CoopVecError(SLANG_E_INVALID_ARG,
+                           "for packed inputInterpretation values please use coopVecMatMulAddPacked and specify k manually")
+    return coopVecMatMulAddPacked(input, inputInterpretation, input.shape[1], matrix, matrixOffset,
+                                  matrixInterpretation, bias, biasOffset, biasInterpretation, memoryLayout,
+                                  transpose, matrixStride, M=M, resultType=resultType, out=out,
+                                  accumulate=accumulate, activation=activation, leakySlope=leakySlope,
+                                  stream=stream)

@@ -1,0 +1,319 @@
+// cv_abi.hip -- the extern "C" entry points declared in include/coopvec.h: argument
+// validation, specialisation lookup and kernel launches.  No device memory is allocated here.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+
+#include "../../include/coopvec.h"
+#include "cv_kernels.h"
+
+namespace {
+
+thread_local char tlsError[512] = "";
+
+CvResult fail(CvResult code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(tlsError, sizeof(tlsError), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+CvResult fromHip(hipError_t e, const char* what)
+{
+    if (e == hipSuccess) return CV_OK;
+    return fail(CV_E_INTERNAL_FAIL, "%s: %s", what, hipGetErrorString(e));
+}
+
+// number of compute units of the current device (cached; immutable once read)
+int currentDeviceCUs(CvResult* rc)
+{
+    static int cus[64];
+    static std::once_flag once[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) {
+        *rc = fail(CV_E_NOT_AVAILABLE, "no usable HIP device: %s", hipGetErrorString(e));
+        return 0;
+    }
+    std::call_once(once[dev], [dev] {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev] = n;
+    });
+    *rc = CV_OK;
+    return cus[dev];
+}
+
+uint32_t alignOf(const void* p, size_t stride)
+{
+    uintptr_t v = (uintptr_t)p | (uintptr_t)stride | 16u;
+    return (uint32_t)(v & (~v + 1));
+}
+
+bool isOptimal(int layout) { return layout == CV_LAYOUT_INFERENCING_OPTIMAL || layout == CV_LAYOUT_TRAINING_OPTIMAL; }
+
+struct Combo {
+    int32_t inputType, inputInterp; uint32_t packing; int32_t matrixInterp, biasInterp, resultType;
+    cv::MmaKind kind;
+};
+
+// What the kernels implement.  Rows with a bias also cover the bias-less coopVecMatMul.
+const Combo kCombos[] = {
+    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT16, CV_FLOAT16, cv::MmaKind::F16},
+    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT16, CV_FLOAT32, cv::MmaKind::F16},
+    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT16, cv::MmaKind::F16},
+    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT32, cv::MmaKind::F16},
+    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT16, cv::MmaKind::Fp8},
+    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT32, cv::MmaKind::Fp8},
+    {CV_SINT8,      CV_SINT8,        1, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
+    {CV_UINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
+    {CV_SINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
+};
+constexpr uint32_t kNumCombos = sizeof(kCombos) / sizeof(kCombos[0]);
+
+} // namespace
+
+extern "C" {
+
+CV_API uint32_t cvGetVersion(void) { return (1u << 16) | 0u; }
+
+CV_API const char* cvGetLastErrorMessage(void) { return tlsError; }
+
+CV_API int32_t cvComponentPackingFactor(int32_t ct)
+{
+    return (ct == CV_SINT8_PACKED || ct == CV_UINT8_PACKED) ? 4 : 1;
+}
+
+CV_API int32_t cvComponentScalarType(int32_t ct)
+{
+    switch (ct) {   // SLANG_SCALAR_TYPE_* values, include/slang.h:2139-2157
+    case CV_FLOAT_E4M3: return 17;
+    case CV_FLOAT_E5M2: return 18;
+    case CV_FLOAT16: return 7;
+    case CV_FLOAT32: return 8;
+    case CV_FLOAT64: return 9;
+    case CV_SINT8: case CV_SINT8_PACKED: return 10;
+    case CV_SINT16: return 12;
+    case CV_SINT32: return 3;
+    case CV_SINT64: return 5;
+    case CV_UINT8: case CV_UINT8_PACKED: return 11;
+    case CV_UINT16: return 13;
+    case CV_UINT32: return 4;
+    case CV_UINT64: return 6;
+    }
+    return -1;
+}
+
+CV_API int32_t cvComponentTypeStride(int32_t ct)
+{
+    const uint32_t s = cv::elemSize(ct);
+    return s ? (int32_t)s : -1;
+}
+
+CV_API uint32_t cvQuerySupportedCombinations(CvCombination* out, uint32_t capacity)
+{
+    for (uint32_t i = 0; i < kNumCombos && out && i < capacity; ++i) {
+        out[i].inputType = kCombos[i].inputType;
+        out[i].inputInterpretation = kCombos[i].inputInterp;
+        out[i].inputPackingFactor = kCombos[i].packing;
+        out[i].matrixInterpretation = kCombos[i].matrixInterp;
+        out[i].biasInterpretation = kCombos[i].biasInterp;
+        out[i].resultType = kCombos[i].resultType;
+        out[i].transpose = 0;
+    }
+    return kNumCombos;
+}
+
+CV_API CvResult cvGetMatrixSize(uint32_t rowCount, uint32_t colCount, int32_t componentType,
+                                int32_t layout, size_t rowColumnStride, size_t* outSize)
+{
+    if (!outSize) return fail(CV_E_INVALID_ARG, "cvGetMatrixSize: outSize is null");
+    *outSize = 0;
+    if (rowCount == 0 || colCount == 0) return fail(CV_E_INVALID_ARG, "cvGetMatrixSize: empty matrix %ux%u", rowCount, colCount);
+    if (layout < 0 || layout > 3) return fail(CV_E_INVALID_ARG, "cvGetMatrixSize: unknown layout %d", layout);
+    if (!cv::layoutSupports(componentType, layout))
+        return fail(CV_E_NOT_AVAILABLE, "cvGetMatrixSize: component type %d has no layout %d", componentType, layout);
+    const cv::MatrixShape s{rowCount, colCount, componentType, layout, isOptimal(layout) ? 0 : rowColumnStride};
+    const size_t n = cv::matrixSize(s);
+    if (!n) return fail(CV_E_INVALID_ARG, "cvGetMatrixSize: stride %zu is smaller than one row/column", rowColumnStride);
+    *outSize = n;
+    return CV_OK;
+}
+
+CV_API CvResult cvConvertMatrices(void* stream, void* dstBuffer, const CvMatrixDesc* dstDescs,
+                                  const void* srcBuffer, const CvMatrixDesc* srcDescs, uint32_t count)
+{
+    if (count == 0) return CV_OK;
+    if (!dstBuffer || !srcBuffer || !dstDescs || !srcDescs) return fail(CV_E_INVALID_ARG, "cvConvertMatrices: null argument");
+    if (count > 64) return fail(CV_E_INVALID_ARG, "cvConvertMatrices: %u matrices in one call (limit 64)", count);
+    for (uint32_t base = 0; base < count; base += cv::kMaxConvertItems) {
+        cv::ConvertArgs args;
+        args.count = (count - base < (uint32_t)cv::kMaxConvertItems) ? count - base : (uint32_t)cv::kMaxConvertItems;
+        for (uint32_t i = 0; i < args.count; ++i) {
+            const CvMatrixDesc& s = srcDescs[base + i];
+            const CvMatrixDesc& d = dstDescs[base + i];
+            if (s.rowCount != d.rowCount || s.colCount != d.colCount || s.rowCount == 0 || s.colCount == 0)
+                return fail(CV_E_INVALID_ARG, "cvConvertMatrices[%u]: shapes differ or are empty (%ux%u -> %ux%u)",
+                            base + i, s.rowCount, s.colCount, d.rowCount, d.colCount);
+            if (!cv::layoutSupports(s.componentType, s.layout) || !cv::layoutSupports(d.componentType, d.layout))
+                return fail(CV_E_NOT_AVAILABLE, "cvConvertMatrices[%u]: unsupported type/layout (%d,%d) -> (%d,%d)",
+                            base + i, s.componentType, s.layout, d.componentType, d.layout);
+            const bool f16f32 = (s.componentType == CV_FLOAT16 || s.componentType == CV_FLOAT32) &&
+                                (d.componentType == CV_FLOAT16 || d.componentType == CV_FLOAT32);
+            if (s.componentType != d.componentType && !f16f32)
+                return fail(CV_E_NOT_AVAILABLE, "cvConvertMatrices[%u]: no conversion from component type %d to %d",
+                            base + i, s.componentType, d.componentType);
+            cv::ConvertItem& it = args.items[i];
+            it.srcShape = cv::MatrixShape{s.rowCount, s.colCount, s.componentType, s.layout, isOptimal(s.layout) ? 0 : s.rowColumnStride};
+            it.dstShape = cv::MatrixShape{d.rowCount, d.colCount, d.componentType, d.layout, isOptimal(d.layout) ? 0 : d.rowColumnStride};
+            const size_t sNeed = cv::matrixSize(it.srcShape), dNeed = cv::matrixSize(it.dstShape);
+            if (!sNeed || !dNeed) return fail(CV_E_INVALID_ARG, "cvConvertMatrices[%u]: stride smaller than a row/column", base + i);
+            if (s.size < sNeed || d.size < dNeed)
+                return fail(CV_E_BUFFER_TOO_SMALL, "cvConvertMatrices[%u]: desc.size too small (src %zu < %zu or dst %zu < %zu)",
+                            base + i, s.size, sNeed, d.size, dNeed);
+            const uint32_t esS = cv::elemSize(s.componentType), esD = cv::elemSize(d.componentType);
+            if (s.offset % esS || d.offset % esD || s.rowColumnStride % esS || d.rowColumnStride % esD)
+                return fail(CV_E_INVALID_ARG, "cvConvertMatrices[%u]: offset/stride not a multiple of the element size", base + i);
+            if (dNeed > 0xffffffffull) return fail(CV_E_INVALID_ARG, "cvConvertMatrices[%u]: matrix too large", base + i);
+            it.src = (const uint8_t*)srcBuffer + s.offset;
+            it.dst = (uint8_t*)dstBuffer + d.offset;
+            it.dstBytes = (uint32_t)dNeed;
+            const uint8_t *s0 = it.src, *s1 = it.src + sNeed, *d0 = it.dst, *d1 = it.dst + dNeed;
+            if (s0 < d1 && d0 < s1) return fail(CV_E_INVALID_ARG, "cvConvertMatrices[%u]: source and destination overlap", base + i);
+        }
+        CvResult rc = fromHip(cv::launchConvert((hipStream_t)stream, args), "cvConvertMatrices launch");
+        if (CV_FAILED(rc)) return rc;
+    }
+    return CV_OK;
+}
+
+CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
+{
+    if (!d) return fail(CV_E_INVALID_ARG, "cvMatMul: desc is null");
+    if (d->batch == 0) return CV_OK;
+    if (!d->input || !d->output || !d->matrix) return fail(CV_E_INVALID_ARG, "cvMatMul: null input/output/matrix");
+    if (d->m <= 0 || d->k <= 0) return fail(CV_E_INVALID_ARG, "cvMatMul: m=%d k=%d", d->m, d->k);
+    if (d->layout < 0 || d->layout > 3) return fail(CV_E_INVALID_ARG, "cvMatMul: unknown layout %d", d->layout);
+    // static_asserts of the Slang signatures (hlsl.meta.slang:32798-32803, 33004)
+    if (cvComponentPackingFactor(d->matrixInterpretation) != 1)
+        return fail(CV_E_INVALID_ARG, "cvMatMul: can't use packed component type in matrixInterpretation");
+    if (d->bias && cvComponentPackingFactor(d->biasInterpretation) != 1)
+        return fail(CV_E_INVALID_ARG, "cvMatMul: can't use packed component type in biasInterpretation");
+    if (d->transpose && !isOptimal(d->layout))   // hlsl.meta.slang:32947
+        return fail(CV_E_INVALID_ARG, "cvMatMul: transpose must be false for RowMajor/ColumnMajor");
+    if (d->accumulate && d->activation != CV_ACT_NONE)
+        return fail(CV_E_INVALID_ARG, "cvMatMul: accumulate forms take no activation");
+    if (d->activation < CV_ACT_NONE || d->activation > CV_ACT_LEAKY_RELU)
+        return fail(CV_E_INVALID_ARG, "cvMatMul: unknown activation %d", d->activation);
+    const uint32_t packing = (uint32_t)cvComponentPackingFactor(d->inputInterpretation);
+    if (packing != 1 && d->k % 4 != 0)   // fallback rule k == 4*PackedK (hlsl.meta.slang:32846)
+        return fail(CV_E_NOT_AVAILABLE, "cvMatMul: packed input needs k to be a multiple of 4 (k=%d)", d->k);
+
+    const Combo* combo = nullptr;
+    for (uint32_t i = 0; i < kNumCombos; ++i) {
+        const Combo& c = kCombos[i];
+        if (c.inputType == d->inputType && c.inputInterp == d->inputInterpretation &&
+            c.matrixInterp == d->matrixInterpretation && c.resultType == d->resultType &&
+            (!d->bias || c.biasInterp == d->biasInterpretation)) { combo = &c; break; }
+    }
+    if (!combo)
+        return fail(CV_E_NOT_AVAILABLE,
+                    "cvMatMul: unsupported combination input %d as %d, matrix %d, bias %d, result %d",
+                    d->inputType, d->inputInterpretation, d->matrixInterpretation,
+                    d->bias ? d->biasInterpretation : -1, d->resultType);
+    if (!cv::layoutSupports(d->matrixInterpretation, d->layout))
+        return fail(CV_E_NOT_AVAILABLE, "cvMatMul: component type %d has no layout %d", d->matrixInterpretation, d->layout);
+
+    cv::MatMulArgs a;
+    memset(&a, 0, sizeof(a));
+    const uint32_t inEsz = combo->kind == cv::MmaKind::F16 ? 2u : 1u;
+    const uint32_t outEsz = d->resultType == CV_FLOAT16 ? 2u : 4u;
+    if ((uintptr_t)d->input % inEsz || d->inputStride % inEsz || (uintptr_t)d->output % outEsz || d->outputStride % outEsz)
+        return fail(CV_E_INVALID_ARG, "cvMatMul: vector address/stride not aligned to the element size");
+    if (d->batch > 1 && (d->inputStride < (size_t)d->k * inEsz || d->outputStride < (size_t)d->m * outEsz))
+        return fail(CV_E_INVALID_ARG, "cvMatMul: vector stride smaller than the vector");
+    a.in = (const uint8_t*)d->input;
+    a.out = (uint8_t*)d->output;
+    a.inStride = d->inputStride;
+    a.outStride = d->outputStride;
+    a.mat = (const uint8_t*)d->matrix + d->matrixOffset;
+    const uint32_t rows = d->transpose ? (uint32_t)d->k : (uint32_t)d->m;
+    const uint32_t cols = d->transpose ? (uint32_t)d->m : (uint32_t)d->k;
+    a.shape = cv::MatrixShape{rows, cols, d->matrixInterpretation, d->layout, isOptimal(d->layout) ? 0 : (size_t)d->matrixStride};
+    if (cv::matrixSize(a.shape) == 0) return fail(CV_E_INVALID_ARG, "cvMatMul: matrixStride %u smaller than a row/column", d->matrixStride);
+    const uint32_t wEsz = cv::elemSize(d->matrixInterpretation);
+    if ((uintptr_t)a.mat % (isOptimal(d->layout) ? 16u : wEsz) || (!isOptimal(d->layout) && d->matrixStride % wEsz))
+        return fail(CV_E_INVALID_ARG, "cvMatMul: matrix address/stride misaligned");
+    a.transpose = d->transpose ? 1 : 0;
+    a.m = d->m;
+    a.k = d->k;
+    a.inCt = d->inputType;
+    if (d->bias) {
+        a.bias = (const uint8_t*)d->bias + d->biasOffset;
+        a.biasCt = d->biasInterpretation;
+        if ((uintptr_t)a.bias % cv::elemSize(a.biasCt)) return fail(CV_E_INVALID_ARG, "cvMatMul: bias misaligned");
+    }
+    a.outCt = d->resultType;
+    a.act = d->activation;
+    a.slope = d->leakySlope;
+    a.accumulate = d->accumulate ? 1 : 0;
+    a.batch = d->batch;
+    a.inAlign = alignOf(d->input, d->inputStride);
+    a.outAlign = alignOf(d->output, d->outputStride);
+
+    CvResult rc;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const hipError_t e = cv::launchMatMul((hipStream_t)stream, combo->kind, a, cus);
+    if (e == hipErrorInvalidValue)
+        return fail(CV_E_NOT_AVAILABLE, "cvMatMul: no kernel specialisation for m=%d k=%d (limits: m<=128; k<=128 fp16/fp8, k<=256 int8)", d->m, d->k);
+    return fromHip(e, "cvMatMul launch");
+}
+
+CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t, int32_t, uint32_t, size_t* outBytes)
+{
+    if (outBytes) *outBytes = 0;
+    return fail(CV_E_NOT_IMPLEMENTED, "cvOuterProductAccumulate: not implemented yet");
+}
+
+CV_API CvResult cvOuterProductAccumulate(void*, const void*, size_t, int32_t, const void*, size_t, int32_t,
+                                         int32_t, uint32_t, void*, size_t, uint32_t, int32_t, int32_t, void*, size_t)
+{
+    return fail(CV_E_NOT_IMPLEMENTED, "cvOuterProductAccumulate: not implemented yet");
+}
+
+CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t, uint32_t, size_t* outBytes)
+{
+    if (outBytes) *outBytes = 0;
+    return fail(CV_E_NOT_IMPLEMENTED, "cvReduceSumAccumulate: not implemented yet");
+}
+
+CV_API CvResult cvReduceSumAccumulate(void*, const void*, size_t, int32_t, int32_t, uint32_t, void*, size_t,
+                                      int32_t, void*, size_t)
+{
+    return fail(CV_E_NOT_IMPLEMENTED, "cvReduceSumAccumulate: not implemented yet");
+}
+
+CV_API CvResult cvMlpForward(void*, const CvMlpDesc*, const void*, size_t, void*, size_t, uint32_t)
+{
+    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpForward: not implemented yet");
+}
+
+CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc*, uint32_t, size_t* outBytes)
+{
+    if (outBytes) *outBytes = 0;
+    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpTrainStep: not implemented yet");
+}
+
+CV_API CvResult cvMlpTrainStep(void*, const CvMlpDesc*, const void*, size_t, const void*, size_t, float,
+                               uint32_t, float*, void*, size_t)
+{
+    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpTrainStep: not implemented yet");
+}
+
+} // extern "C"

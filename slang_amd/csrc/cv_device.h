@@ -1,0 +1,103 @@
+// cv_device.h -- device-side building blocks shared by the gfx950 kernels.
+//
+// Mapping used by every kernel here: one 64-lane wavefront works on tiles of 16 samples.
+// Lane l = 16*g + n belongs to sample n of the tile and to lane group g.  A vector of P
+// (padded) features is spread over the wave so that group g owns the contiguous quarter
+// [g*P/4, (g+1)*P/4) of it -- which is at once the B-operand register layout of
+// v_mfma_*_16x16x{32,64} (k-slots of group g) and, for the result D = W . X^T, the
+// accumulator layout (rows 4g..4g+3 of every 16-row tile) under the row order of
+// cv_layout.h.  A layer's accumulators therefore feed the next layer's MFMA without any
+// cross-lane movement.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cv_layout.h"
+
+namespace cv {
+
+typedef _Float16 half_t;
+typedef _Float16 halfx2 __attribute__((ext_vector_type(2)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+enum : int { kActNone = 0, kActRelu = 1, kActLeakyRelu = 2 };
+
+// ---- MFMA flavours ---------------------------------------------------------------------
+// Each flavour: element size, k-slots per lane per fragment (EPL), dwords per fragment (FD),
+// accumulator type, and D += A.B with A/B given as dword arrays.
+
+struct F16Mma {
+    static constexpr int kEsz = 2, kEpl = 8, kFD = 4;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, av),
+                                                      __builtin_bit_cast(halfx8, bv), c, 0, 0, 0);
+    }
+};
+
+struct Fp8Mma {  // OCP e4m3 x e4m3 -> fp32
+    static constexpr int kEsz = 1, kEpl = 8, kFD = 2;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        u32x2 av = {a[0], a[1]}, bv = {b[0], b[1]};
+        return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(__builtin_bit_cast(long, av),
+                                                          __builtin_bit_cast(long, bv), c, 0, 0, 0);
+    }
+};
+
+struct I8Mma {   // int8 x int8 -> int32
+    static constexpr int kEsz = 1, kEpl = 16, kFD = 4;
+    static constexpr bool kIsFloat = false;
+    typedef intx4 Acc;
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        intx4 av = {(int)a[0], (int)a[1], (int)a[2], (int)a[3]};
+        intx4 bv = {(int)b[0], (int)b[1], (int)b[2], (int)b[3]};
+        return __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, c, 0, 0, 0);
+    }
+};
+
+// ---- scalar helpers ---------------------------------------------------------------------
+
+__device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct)
+{
+    switch (ct) {
+    case kF16: return (float)*(const half_t*)p;
+    case kF32: return *(const float*)p;
+    }
+    return 0.f;
+}
+
+// fp32 -> OCP e4m3, saturating, round to nearest even; two values per call (bytes 0,1)
+__device__ __forceinline__ uint32_t packE4M3Sat(float a, float b)
+{
+    // v_cvt_pk_fp8_f32 rounds to nearest even and produces NaN above the finite range:
+    // clamp to +-448 first (v_med3 keeps NaN as NaN on the min/max path is not guaranteed,
+    // so NaN inputs are not supported by the fused paths).
+    a = __builtin_fminf(__builtin_fmaxf(a, -448.f), 448.f);
+    b = __builtin_fminf(__builtin_fmaxf(b, -448.f), 448.f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+
+// activation on a value already rounded to fp16 (the carrier type is CoopVec<half>)
+__device__ __forceinline__ half_t activateHalf(half_t z, int act, float slope)
+{
+    if (act == kActRelu) return z > (half_t)0 ? z : (half_t)0;
+    if (act == kActLeakyRelu) {
+        const half_t zs = (half_t)((float)z * slope);   // exact product, one rounding
+        return z >= zs ? z : zs;
+    }
+    return z;
+}
+
+} // namespace cv

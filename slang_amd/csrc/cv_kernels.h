@@ -1,0 +1,49 @@
+// cv_kernels.h -- host-callable launchers of the gfx950 kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "cv_layout.h"
+
+namespace cv {
+
+// ---- batched matMul[Add] ------------------------------------------------------------------
+struct MatMulArgs {
+    const uint8_t* in;      // sample s at in + s*inStride
+    uint8_t* out;           // sample s at out + s*outStride
+    const uint8_t* mat;     // matrix base (offset already applied)
+    const uint8_t* bias;    // bias base (offset already applied) or nullptr
+    uint64_t inStride, outStride;
+    MatrixShape shape;      // the matrix as it lies in memory
+    int32_t transpose;      // memory holds k x m and is used transposed
+    int32_t m, k;
+    int32_t inCt;           // element type of the input vectors in memory
+    int32_t biasCt;
+    int32_t outCt;          // kF16, kF32 or kS32
+    int32_t act;
+    float slope;
+    int32_t accumulate;
+    uint32_t batch;
+    uint32_t inAlign, outAlign;   // largest power of two (<= 16) dividing base address and stride
+};
+
+enum class MmaKind : int { F16 = 0, Fp8 = 1, I8 = 2 };
+
+// Returns hipSuccess, or hipErrorInvalidValue when no specialisation covers (m,k).
+hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& args, int numCUs);
+
+// ---- layout conversion --------------------------------------------------------------------
+struct ConvertItem {
+    const uint8_t* src;
+    uint8_t* dst;
+    MatrixShape srcShape, dstShape;
+    uint32_t dstBytes;      // bytes of the destination to cover (padding is zero-filled)
+};
+constexpr int kMaxConvertItems = 32;   // keeps ConvertArgs under the 4 KB kernel-argument limit
+struct ConvertArgs {
+    ConvertItem items[kMaxConvertItems];
+    uint32_t count;
+};
+hipError_t launchConvert(hipStream_t stream, const ConvertArgs& args);
+
+} // namespace cv
