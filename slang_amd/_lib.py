@@ -58,7 +58,7 @@ class CvMatMulDesc(ctypes.Structure):
                 ("bias", ctypes.c_void_p), ("biasOffset", ctypes.c_size_t),
                 ("biasInterpretation", ctypes.c_int32),
                 ("activation", ctypes.c_int32), ("leakySlope", ctypes.c_float),
-                ("accumulate", ctypes.c_int32), ("batch", ctypes.c_uint32)]
+                ("accumulate", ctypes.c_int32), ("batch", ctypes.c_uint32), ("flags", ctypes.c_uint32)]
 
 
 class CvMlpLayer(ctypes.Structure):
@@ -74,7 +74,7 @@ class CvMlpDesc(ctypes.Structure):
     _fields_ = [("layers", ctypes.POINTER(CvMlpLayer)), ("numLayers", ctypes.c_int32),
                 ("inputType", ctypes.c_int32), ("weightType", ctypes.c_int32),
                 ("biasType", ctypes.c_int32), ("outputType", ctypes.c_int32),
-                ("gradType", ctypes.c_int32)]
+                ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32)]
 
 
 # name -> (restype, argtypes); every function include/coopvec.h declares

@@ -51,6 +51,9 @@ class CoopVecComponentType(enum.IntEnum):
     UnsignedInt8Packed = 14
 
 
+FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.h
+
+
 class Activation(enum.IntEnum):
     NoActivation = 0
     ReLU = 1
@@ -209,7 +212,7 @@ def _vector_info(v: torch.Tensor, interpretation: int, what: str):
 
 def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, bias, biasOffset,
             biasInterpretation, memoryLayout, transpose, matrixStride, M, resultType, activation, leakySlope,
-            accumulate, out, stream):
+            accumulate, out, stream, flags=0):
     lib = _lib.load()
     inCt, inStride = _vector_info(input, inputInterpretation, "input")
     batch = input.shape[0]
@@ -241,7 +244,7 @@ def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpret
     else:
         d.bias = None; d.biasOffset = 0; d.biasInterpretation = -1
     d.activation = int(activation); d.leakySlope = float(leakySlope)
-    d.accumulate = 1 if accumulate else 0; d.batch = batch
+    d.accumulate = 1 if accumulate else 0; d.batch = batch; d.flags = int(flags)
     _check(lib.cvMatMul(_stream_handle(stream), ctypes.byref(d)))
     return out
 
@@ -249,25 +252,27 @@ def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpret
 def coopVecMatMulPacked(input: torch.Tensor, inputInterpretation: int, k: int, matrix: torch.Tensor,
                         matrixOffset: int, matrixInterpretation: int, memoryLayout: int, transpose: bool,
                         matrixStride: int, *, M: int, resultType: Optional[int] = None,
-                        out: Optional[torch.Tensor] = None, accumulate: bool = False, stream=None):
+                        out: Optional[torch.Tensor] = None, accumulate: bool = False, stream=None,
+                        flags: int = 0):
     """coopVecMatMulPacked<T,M,PackedK,U> (hlsl.meta.slang:32786-32796); accumulate=True is the
     member form matMulAccumPacked (:31476)."""
     return _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, None, 0, -1,
                    memoryLayout, transpose, matrixStride, M, resultType, Activation.NoActivation, 0.0,
-                   accumulate, out, stream)
+                   accumulate, out, stream, flags)
 
 
 def coopVecMatMul(input: torch.Tensor, inputInterpretation: int, matrix: torch.Tensor, matrixOffset: int,
                   matrixInterpretation: int, memoryLayout: int, transpose: bool, matrixStride: int, *,
                   M: int, resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
-                  accumulate: bool = False, stream=None):
+                  accumulate: bool = False, stream=None, flags: int = 0):
     """coopVecMatMul<T,M,K,U> (hlsl.meta.slang:32954-32963)."""
     if componentPackingFactor(inputInterpretation) != 1:   # static_assert :32965
         raise CoopVecError(SLANG_E_INVALID_ARG,
                            "for packed inputInterpretation values please use coopVecMatMulPacked and specify k manually")
     return coopVecMatMulPacked(input, inputInterpretation, input.shape[1], matrix, matrixOffset,
                                matrixInterpretation, memoryLayout, transpose, matrixStride, M=M,
-                               resultType=resultType, out=out, accumulate=accumulate, stream=stream)
+                               resultType=resultType, out=out, accumulate=accumulate, stream=stream,
+                               flags=flags)
 
 
 def coopVecMatMulAddPacked(input: torch.Tensor, inputInterpretation: int, k: int, matrix: torch.Tensor,
@@ -275,11 +280,11 @@ def coopVecMatMulAddPacked(input: torch.Tensor, inputInterpretation: int, k: int
                            biasInterpretation: int, memoryLayout: int, transpose: bool, matrixStride: int, *,
                            M: int, resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
                            accumulate: bool = False, activation: int = Activation.NoActivation,
-                           leakySlope: float = 0.0, stream=None):
+                           leakySlope: float = 0.0, stream=None, flags: int = 0):
     """coopVecMatMulAddPacked<T,M,PackedK,U> (hlsl.meta.slang:32983-32996)."""
     return _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpretation, bias, biasOffset,
                    biasInterpretation, memoryLayout, transpose, matrixStride, M, resultType, activation,
-                   leakySlope, accumulate, out, stream)
+                   leakySlope, accumulate, out, stream, flags)
 
 
 def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torch.Tensor, matrixOffset: int,
@@ -287,7 +292,7 @@ def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torc
                      memoryLayout: int, transpose: bool, matrixStride: int, *, M: int,
                      resultType: Optional[int] = None, out: Optional[torch.Tensor] = None,
                      accumulate: bool = False, activation: int = Activation.NoActivation,
-                     leakySlope: float = 0.0, stream=None):
+                     leakySlope: float = 0.0, stream=None, flags: int = 0):
     """coopVecMatMulAdd<T,M,K,U> (hlsl.meta.slang:33160-33173)."""
     if componentPackingFactor(inputInterpretation) != 1:
         raise CoopVecError(SLANG_E_INVALID_ARG,
@@ -296,4 +301,4 @@ def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torc
                                   matrixInterpretation, bias, biasOffset, biasInterpretation, memoryLayout,
                                   transpose, matrixStride, M=M, resultType=resultType, out=out,
                                   accumulate=accumulate, activation=activation, leakySlope=leakySlope,
-                                  stream=stream)
+                                  stream=stream, flags=flags)

@@ -68,8 +68,8 @@ const Combo kCombos[] = {
     {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT16, CV_FLOAT32, cv::MmaKind::F16},
     {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT16, cv::MmaKind::F16},
     {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT32, cv::MmaKind::F16},
-    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT16, cv::MmaKind::Fp8},
-    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT32, cv::MmaKind::Fp8},
+    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT16, cv::MmaKind::Fp8AsF16},
+    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT32, cv::MmaKind::Fp8AsF16},
     {CV_SINT8,      CV_SINT8,        1, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
     {CV_UINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
     {CV_SINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
@@ -269,7 +269,9 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     CvResult rc;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    const hipError_t e = cv::launchMatMul((hipStream_t)stream, combo->kind, a, cus);
+    cv::MmaKind kind = combo->kind;
+    if (kind == cv::MmaKind::Fp8AsF16 && (d->flags & CV_FLAG_FP8_MATRIX_PIPELINE)) kind = cv::MmaKind::Fp8Native;
+    const hipError_t e = cv::launchMatMul((hipStream_t)stream, kind, a, cus);
     if (e == hipErrorInvalidValue)
         return fail(CV_E_NOT_AVAILABLE, "cvMatMul: no kernel specialisation for m=%d k=%d (limits: m<=128; k<=128 fp16/fp8, k<=256 int8)", d->m, d->k);
     return fromHip(e, "cvMatMul launch");

@@ -28,13 +28,18 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 enum : int { kActNone = 0, kActRelu = 1, kActLeakyRelu = 2 };
 
 // ---- MFMA flavours ---------------------------------------------------------------------
-// Each flavour: element size, k-slots per lane per fragment (EPL), dwords per fragment (FD),
-// accumulator type, and D += A.B with A/B given as dword arrays.
+// Each flavour describes how elements lie in memory (kEsz bytes each; kEpl k-slots per lane
+// per fragment = kRawDW dwords as loaded) and in the MFMA operand registers (kFD dwords per
+// fragment after decode()), the accumulator type, and D += A.B.
 
 struct F16Mma {
-    static constexpr int kEsz = 2, kEpl = 8, kFD = 4;
+    static constexpr int kEsz = 2, kEpl = 8, kRawDW = 4, kFD = 4;
     static constexpr bool kIsFloat = true;
     typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        frag[0] = raw[0]; frag[1] = raw[1]; frag[2] = raw[2]; frag[3] = raw[3];
+    }
     static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
     {
         u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
@@ -43,10 +48,17 @@ struct F16Mma {
     }
 };
 
-struct Fp8Mma {  // OCP e4m3 x e4m3 -> fp32
-    static constexpr int kEsz = 1, kEpl = 8, kFD = 2;
+// OCP e4m3 operands on the fp8 matrix pipeline.  Measured on gfx950: this pipeline aligns the
+// products of one instruction to the largest of them and keeps about 11 bits below it, so sums
+// that cancel carry an absolute error of up to ~2^-12 * sum|terms|.
+struct Fp8NativeMma {
+    static constexpr int kEsz = 1, kEpl = 8, kRawDW = 2, kFD = 2;
     static constexpr bool kIsFloat = true;
     typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        frag[0] = raw[0]; frag[1] = raw[1];
+    }
     static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
     {
         u32x2 av = {a[0], a[1]}, bv = {b[0], b[1]};
@@ -55,10 +67,34 @@ struct Fp8Mma {  // OCP e4m3 x e4m3 -> fp32
     }
 };
 
+// OCP e4m3 in memory, decoded (exactly: e4m3 is a subset of fp16) to fp16 operands of the
+// fp16 matrix pipeline, whose accumulation is fp32-grade.  This is the flavour that meets the
+// fp32-accumulated parity bar for e4m3 matrices.
+struct Fp8AsF16Mma {
+    static constexpr int kEsz = 1, kEpl = 8, kRawDW = 2, kFD = 4;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        frag[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[0], 1.0f, false));
+        frag[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[0], 1.0f, true));
+        frag[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[1], 1.0f, false));
+        frag[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[1], 1.0f, true));
+    }
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        return F16Mma::mma(a, b, c);
+    }
+};
+
 struct I8Mma {   // int8 x int8 -> int32
-    static constexpr int kEsz = 1, kEpl = 16, kFD = 4;
+    static constexpr int kEsz = 1, kEpl = 16, kRawDW = 4, kFD = 4;
     static constexpr bool kIsFloat = false;
     typedef intx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        frag[0] = raw[0]; frag[1] = raw[1]; frag[2] = raw[2]; frag[3] = raw[3];
+    }
     static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
     {
         intx4 av = {(int)a[0], (int)a[1], (int)a[2], (int)a[3]};

@@ -27,7 +27,7 @@ struct MatMulArgs {
     uint32_t inAlign, outAlign;   // largest power of two (<= 16) dividing base address and stride
 };
 
-enum class MmaKind : int { F16 = 0, Fp8 = 1, I8 = 2 };
+enum class MmaKind : int { F16 = 0, Fp8AsF16 = 1, Fp8Native = 2, I8 = 3 };
 
 // Returns hipSuccess, or hipErrorInvalidValue when no specialisation covers (m,k).
 hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& args, int numCUs);

@@ -3,7 +3,9 @@
 // Replaces the per-thread operator of source/slang/hlsl.meta.slang:32786-33190 (whose only
 // in-tree executable form is the scalar fallback :32835-32912 / :33043-33103) by a dense
 // contraction: the 16 samples of a tile are the N dimension of D = W . X^T, computed with
-// v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x32_fp8_fp8 / v_mfma_i32_16x16x64_i8.
+// v_mfma_f32_16x16x32_f16 / v_mfma_f32_16x16x32_fp8_fp8 / v_mfma_i32_16x16x64_i8.  e4m3
+// matrices run on the fp16 pipeline by default (exact decode, fp32-grade accumulation) and on
+// the fp8 pipeline on request (see cv_device.h for the measured difference).
 //
 //  - the workgroup stages the matrix once into LDS in fragment order (any source layout is
 //    gathered through cv::elemOffset; an InferencingOptimal source of matching shape is a
@@ -56,12 +58,12 @@ __device__ __forceinline__ void loadSlots(uint32_t (&s)[DW], const uint8_t* p, i
 template <class Mma, int MT, int KT, int NT, typename OutT>
 __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 {
-    constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz;
-    constexpr int SLOT_DW = FD * KT;          // B-operand dwords per lane per 16-sample tile
+    constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
+    constexpr int SLOT_DW = RAW * KT;         // input dwords per lane per 16-sample tile
     constexpr int ROWS = 4 * MT;              // output rows per lane
     typedef typename Mma::Acc Acc;
 
-    __shared__ __attribute__((aligned(16))) uint32_t ldsW[MT * KT * 64 * FD];
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[MT * KT * 64 * RAW];
 
     const uint32_t gs = optGS((uint32_t)a.k);   // k-slots owned by one lane group
 
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
         if (direct) {
             const u32x4* src = (const u32x4*)a.mat;
             u32x4* dst = (u32x4*)ldsW;
-            for (int i = threadIdx.x; i < MT * KT * 64 * FD / 4; i += 256) dst[i] = src[i];
+            for (int i = threadIdx.x; i < MT * KT * 64 * RAW / 4; i += 256) dst[i] = src[i];
         } else {
             uint8_t* dst = (uint8_t*)ldsW;
             for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
@@ -99,8 +101,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int d = 0; d < FD; ++d) afrag[t][kt][d] = ldsW[((t * KT + kt) * 64 + lane) * FD + d];
+            Mma::decode(&ldsW[((t * KT + kt) * 64 + lane) * RAW], afrag[t][kt]);
 
     // ---- per-lane constants -------------------------------------------------------------
     const int rowBase = g * ROWS;
@@ -156,10 +157,12 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 #pragma unroll
             for (int t = 0; t < MT; ++t) acc[t] = biasv[t];
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+            for (int kt = 0; kt < KT; ++kt) {
+                uint32_t bfrag[FD];
+                Mma::decode(&cur[j][kt * RAW], bfrag);
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    acc[t] = Mma::mma(afrag[t][kt], &cur[j][kt * FD], acc[t]);
+                for (int t = 0; t < MT; ++t) acc[t] = Mma::mma(afrag[t][kt], bfrag, acc[t]);
+            }
 
             const uint32_t sample = tile * TILE + 16 * j + n;
             if (sample < a.batch && validRows > 0) {
@@ -273,9 +276,12 @@ hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& a, i
     case MmaKind::F16:
         return a.outCt == kF32 ? dispatchShape<F16Mma, float>(stream, a, numCUs)
                                : dispatchShape<F16Mma, half_t>(stream, a, numCUs);
-    case MmaKind::Fp8:
-        return a.outCt == kF32 ? dispatchShape<Fp8Mma, float>(stream, a, numCUs)
-                               : dispatchShape<Fp8Mma, half_t>(stream, a, numCUs);
+    case MmaKind::Fp8AsF16:
+        return a.outCt == kF32 ? dispatchShape<Fp8AsF16Mma, float>(stream, a, numCUs)
+                               : dispatchShape<Fp8AsF16Mma, half_t>(stream, a, numCUs);
+    case MmaKind::Fp8Native:
+        return a.outCt == kF32 ? dispatchShape<Fp8NativeMma, float>(stream, a, numCUs)
+                               : dispatchShape<Fp8NativeMma, half_t>(stream, a, numCUs);
     case MmaKind::I8:
         return dispatchShape<I8Mma, int32_t>(stream, a, numCUs);
     }

@@ -1,0 +1,205 @@
+"""ctypes binding of the CPU oracle (oracle/libcoopvec_oracle.so) for the tests.
+
+The oracle is the checker; nothing under slang_amd/ imports this module."""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(REPO, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "libcoopvec_oracle.so")
+
+# CoopVecComponentType / layout values (hlsl.meta.slang:32547-32575)
+E4M3, E5M2, F16, F32, F64, S8, S16, S32, S64, S8P, U8, U16, U32, U64, U8P = range(15)
+ROW, COL, INF_OPT, TRAIN_OPT = range(4)
+HALF_RNE, HALF_SLANG = 0, 1
+ACT_NONE, ACT_RELU, ACT_LEAKY = 0, 1, 2
+
+_c = ctypes
+_vp, _sz, _i32, _u32, _f32 = _c.c_void_p, _c.c_size_t, _c.c_int32, _c.c_uint32, _c.c_float
+
+
+class CvoLayer(_c.Structure):
+    _fields_ = [("inDim", _c.c_int), ("outDim", _c.c_int), ("weightType", _c.c_int),
+                ("weights", _vp), ("weightStride", _u32), ("bias", _vp),
+                ("activation", _c.c_int), ("leakySlope", _f32)]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(ORACLE_LIB):
+        subprocess.check_call(["make", "-C", ORACLE_DIR, "libcoopvec_oracle.so"])
+    L = ctypes.CDLL(ORACLE_LIB)
+    L.cvo_f32_to_f16_rne.argtypes = [_f32]; L.cvo_f32_to_f16_rne.restype = _c.c_uint16
+    L.cvo_f32_to_f16_slang.argtypes = [_f32]; L.cvo_f32_to_f16_slang.restype = _c.c_uint16
+    L.cvo_f16_to_f32.argtypes = [_c.c_uint16]; L.cvo_f16_to_f32.restype = _f32
+    L.cvo_f32_to_e4m3_sat.argtypes = [_f32]; L.cvo_f32_to_e4m3_sat.restype = _c.c_uint8
+    L.cvo_e4m3_to_f32.argtypes = [_c.c_uint8]; L.cvo_e4m3_to_f32.restype = _f32
+    for n in ("cvo_component_packing_factor", "cvo_component_scalar_type", "cvo_component_type_stride"):
+        getattr(L, n).argtypes = [_c.c_int]; getattr(L, n).restype = _c.c_int
+    L.cvo_slang_matmul.argtypes = [_vp, _c.c_int, _c.c_int, _c.c_int, _c.c_int, _vp, _c.c_int, _c.c_int,
+                                   _vp, _i32, _c.c_int, _c.c_int, _c.c_int, _u32, _vp, _i32, _c.c_int,
+                                   _c.c_int, _c.c_int]
+    L.cvo_slang_matmul.restype = _c.c_int
+    L.cvo_slang_outer_product_accumulate.argtypes = [_vp, _c.c_int, _vp, _c.c_int, _c.c_int, _vp, _i32, _u32,
+                                                     _c.c_int, _c.c_int, _c.c_int]
+    L.cvo_slang_outer_product_accumulate.restype = _c.c_int
+    L.cvo_slang_reduce_sum_accumulate.argtypes = [_vp, _c.c_int, _c.c_int, _vp, _i32, _c.c_int]
+    L.cvo_slang_reduce_sum_accumulate.restype = _c.c_int
+    L.cvo_slang_dispatch_matmul_add.argtypes = [_u32, _u32, _u32, _vp, _sz, _c.c_int, _c.c_int, _c.c_int, _c.c_int,
+                                                _vp, _sz, _c.c_int, _c.c_int, _vp, _i32, _c.c_int, _c.c_int,
+                                                _c.c_int, _u32, _vp, _i32, _c.c_int, _c.c_int]
+    L.cvo_slang_dispatch_matmul_add.restype = _c.c_int
+    L.cvo_ref_matmul_f32.argtypes = [_vp, _sz, _c.c_int, _c.c_int, _vp, _sz, _c.c_int, _c.c_int, _c.c_int, _u32,
+                                     _c.c_int, _vp, _sz, _c.c_int, _u32, _vp, _vp]
+    L.cvo_ref_matmul_f32.restype = _c.c_int
+    L.cvo_ref_matmul_i32.argtypes = [_vp, _sz, _c.c_int, _c.c_int, _vp, _sz, _c.c_int, _c.c_int, _c.c_int, _u32,
+                                     _c.c_int, _vp, _sz, _c.c_int, _u32, _vp]
+    L.cvo_ref_matmul_i32.restype = _c.c_int
+    L.cvo_ref_mlp_forward.argtypes = [_c.POINTER(CvoLayer), _c.c_int, _vp, _sz, _c.c_int, _u32, _vp, _vp]
+    L.cvo_ref_mlp_forward.restype = _c.c_int
+    L.cvo_ref_mlp_train.argtypes = [_c.POINTER(CvoLayer), _c.c_int, _vp, _sz, _vp, _f32, _u32,
+                                    _c.POINTER(_vp), _c.POINTER(_vp), _c.POINTER(_c.c_double), _c.c_int]
+    L.cvo_ref_mlp_train.restype = _c.c_int
+    L.cvo_layout_matrix_size.argtypes = [_u32, _u32, _c.c_int, _c.c_int, _sz]
+    L.cvo_layout_matrix_size.restype = _sz
+    L.cvo_layout_elem_offset.argtypes = [_u32, _u32, _c.c_int, _c.c_int, _sz, _u32, _u32]
+    L.cvo_layout_elem_offset.restype = _c.c_int64
+    L.cvo_layout_convert.argtypes = [_vp, _u32, _u32, _c.c_int, _c.c_int, _sz, _vp, _c.c_int, _c.c_int, _sz]
+    L.cvo_layout_convert.restype = _c.c_int
+    _lib = L
+    return L
+
+
+def ptr(a: np.ndarray):
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(_vp)
+
+
+# ---- numpy-level helpers ------------------------------------------------------------------
+
+def ref_matmul_f32(x: np.ndarray, x_ct: int, W_bytes: np.ndarray, w_ct: int, layout: int, stride: int,
+                   M: int, K: int, bias: np.ndarray | None = None, bias_ct: int = -1, transpose: bool = False,
+                   matrix_offset: int = 0):
+    """Returns (fp32 unrounded result [B,M], sum of |terms| [B,M])."""
+    B = x.shape[0]
+    out = np.empty((B, M), np.float32)
+    ab = np.empty((B, M), np.float32)
+    rc = lib().cvo_ref_matmul_f32(ptr(x), x.strides[0], x_ct, K, ptr(W_bytes), matrix_offset, w_ct, layout,
+                                  int(transpose), stride, M, ptr(bias) if bias is not None else None, 0,
+                                  bias_ct if bias is not None else -1, B, ptr(out), ptr(ab))
+    assert rc == 0
+    return out, ab
+
+
+def ref_matmul_i32(x: np.ndarray, W_bytes: np.ndarray, layout: int, stride: int, M: int, K: int,
+                   bias: np.ndarray | None = None, transpose: bool = False):
+    B = x.shape[0]
+    out = np.empty((B, M), np.int32)
+    rc = lib().cvo_ref_matmul_i32(ptr(x), x.strides[0], S8, K, ptr(W_bytes), 0, S8, layout, int(transpose),
+                                  stride, M, ptr(bias) if bias is not None else None, 0,
+                                  S32 if bias is not None else -1, B, ptr(out))
+    assert rc == 0
+    return out
+
+
+def make_layers(specs):
+    """specs: list of dict(W=np.ndarray [out,in] (float16 or uint8 e4m3), b=np.float16|None, act, slope).
+    Returns (ctypes array, keepalive list)."""
+    arr = (CvoLayer * len(specs))()
+    keep = []
+    for i, s in enumerate(specs):
+        W = np.ascontiguousarray(s["W"])
+        keep.append(W)
+        arr[i].inDim = W.shape[1]; arr[i].outDim = W.shape[0]
+        arr[i].weightType = F16 if W.dtype == np.float16 else E4M3
+        arr[i].weights = W.ctypes.data; arr[i].weightStride = W.strides[0]
+        b = s.get("b")
+        if b is not None:
+            b = np.ascontiguousarray(b, dtype=np.float16); keep.append(b)
+            arr[i].bias = b.ctypes.data
+        else:
+            arr[i].bias = None
+        arr[i].activation = s.get("act", ACT_NONE)
+        arr[i].leakySlope = float(s.get("slope", 0.0))
+    return arr, keep
+
+
+def ref_mlp_forward(specs, x: np.ndarray, x_ct: int, want_acts: bool = False):
+    arr, keep = make_layers(specs)
+    B = x.shape[0]
+    out = np.empty((B, specs[-1]["W"].shape[0]), np.uint16)
+    acts = None
+    if want_acts:
+        acts = np.empty(sum(B * s["W"].shape[0] for s in specs), np.uint16)
+    rc = lib().cvo_ref_mlp_forward(arr, len(specs), ptr(x), x.strides[0], x_ct, B, ptr(out),
+                                   ptr(acts) if acts is not None else None)
+    assert rc == 0
+    out = out.view(np.float16)
+    if not want_acts:
+        return out
+    res, off = [], 0
+    for s in specs:
+        n = B * s["W"].shape[0]
+        res.append(acts[off:off + n].view(np.float16).reshape(B, -1)); off += n
+    return out, res
+
+
+def ref_mlp_train(specs, x: np.ndarray, targets: np.ndarray | None, loss_scale: float = 1.0, tie_rule: bool = True):
+    arr, keep = make_layers(specs)
+    B = x.shape[0]
+    dW = [np.zeros(s["W"].shape, np.float64) for s in specs]
+    dB = [np.zeros(s["W"].shape[0], np.float64) for s in specs]
+    pW = (_vp * len(specs))(*[a.ctypes.data for a in dW])
+    pB = (_vp * len(specs))(*[a.ctypes.data for a in dB])
+    loss = _c.c_double(0)
+    rc = lib().cvo_ref_mlp_train(arr, len(specs), ptr(x), x.strides[0],
+                                 ptr(targets) if targets is not None else None, loss_scale, B, pW, pB,
+                                 _c.byref(loss), int(tie_rule))
+    assert rc == 0
+    return dW, dB, loss.value
+
+
+def encode_e4m3(a: np.ndarray) -> np.ndarray:
+    L = lib()
+    flat = np.asarray(a, np.float32).ravel()
+    return np.array([L.cvo_f32_to_e4m3_sat(float(v)) for v in flat], np.uint8).reshape(np.shape(a))
+
+
+_E4M3_TABLE = None
+
+
+def decode_e4m3(b: np.ndarray) -> np.ndarray:
+    global _E4M3_TABLE
+    if _E4M3_TABLE is None:
+        L = lib()
+        _E4M3_TABLE = np.array([L.cvo_e4m3_to_f32(i) for i in range(256)], np.float32)
+    return _E4M3_TABLE[np.asarray(b, np.uint8)]
+
+
+def f16_ulp(ref: np.ndarray) -> np.ndarray:
+    """Spacing of fp16 at |ref| (fp32 array in, fp32 out); 2^-24 in the subnormal range."""
+    a = np.abs(ref.astype(np.float32))
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -14)))
+    return np.exp2(e - 10).astype(np.float32)
+
+
+def float_parity_violations(got_f16: np.ndarray, ref_f32: np.ndarray, abs_terms: np.ndarray | None = None):
+    """The float parity bar: |got - fp16(ref)| <= max(2 ulp_fp16(ref), 1e-3*|ref|, 2^-18*sum|terms|).
+    The third term is the fp32 summation-order floor (k*eps32 for k <= 64 terms) and only matters
+    where the result cancels to (almost) zero.  Returns the boolean violation mask."""
+    ref16 = ref_f32.astype(np.float16).astype(np.float32)
+    err = np.abs(got_f16.astype(np.float32) - ref16)
+    tol = np.maximum(2.0 * f16_ulp(ref16), 1e-3 * np.abs(ref16))
+    if abs_terms is not None:
+        tol = np.maximum(tol, abs_terms * np.float32(2.0 ** -18))
+    return err > tol
