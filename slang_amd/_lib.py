@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG_DIR, "libcoopvec_mi355x.so")
+# COOPVEC_MI355X_LIB points at another build of the same library (e.g. a tuning variant)
+LIB_PATH = os.environ.get("COOPVEC_MI355X_LIB") or os.path.join(_PKG_DIR, "libcoopvec_mi355x.so")
 
 _lib = None
 

@@ -23,7 +23,8 @@ LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
 ORACLE_DIR = os.path.join(REPO_DIR, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libcoopvec_oracle.so")
 
-HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul.hip", "cv_mlp.hip", "cv_train.hip"]
+HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul_f16.hip", "cv_matmul_fp8.hip",
+               "cv_matmul_i8.hip", "cv_mlp.hip", "cv_train.hip"]
 
 # packed-fp32 instructions are switched off on purpose (see the flag below): hipcc would
 # otherwise form v_pk_*_f32 from ordinary float code.
@@ -47,7 +48,7 @@ def _run(cmd: list[str]) -> None:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
 
 
-def build_library(jobs: int = 4, verbose: bool = False) -> str:
+def build_library(jobs: int = 8, verbose: bool = False) -> str:
     """Compile every HIP source for gfx950 and link the shared library.  Always recompiles."""
     hipcc = _hipcc()
     obj_dir = os.path.join(REPO_DIR, "build", "obj")
@@ -79,7 +80,7 @@ def build_oracle() -> str:
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--oracle", action="store_true", help="also build the CPU oracle")
-    ap.add_argument("-j", "--jobs", type=int, default=4)
+    ap.add_argument("-j", "--jobs", type=int, default=8)
     ap.add_argument("-v", "--verbose", action="store_true")
     args = ap.parse_args(argv)
     print(build_library(args.jobs, args.verbose))

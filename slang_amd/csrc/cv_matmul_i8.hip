@@ -1,0 +1,11 @@
+// cv_matmul_i8.hip -- int8 -> int32 instantiations of the batched matMul kernel (bit-exact).
+#include "cv_matmul_impl.h"
+
+namespace cv {
+
+hipError_t launchMatMulI8(hipStream_t stream, const MatMulArgs& a, int numCUs)
+{
+    return dispatchShape<I8Mma, int32_t>(stream, a, numCUs);
+}
+
+} // namespace cv

@@ -1,4 +1,4 @@
-// cv_matmul.hip -- batched coopVecMatMul / coopVecMatMulAdd for gfx950.
+// cv_matmul_impl.h -- batched coopVecMatMul / coopVecMatMulAdd kernel template for gfx950.
 //
 // Replaces the per-thread operator of source/slang/hlsl.meta.slang:32786-33190 (whose only
 // in-tree executable form is the scalar fallback :32835-32912 / :33043-33103) by a dense
@@ -16,30 +16,41 @@
 //    contiguous quarter g of its output vector (see cv_device.h), so a K=64 fp16 sample row
 //    of 128 B is read by four lanes with two 16-byte loads each and written the same way;
 //  - bias seeds the accumulators; activation and the cast to the result type are fused.
+//
+// Two instantiations per shape: FAST (full-width aligned vectors, m a multiple of 16, no
+// leaky ReLU, no accumulate form: a branch-free streaming loop) and the general one (ragged
+// shapes, unaligned vectors, `this += ...`, every activation).
+#pragma once
 #include "cv_device.h"
 #include "cv_kernels.h"
 
 namespace cv {
-
 namespace {
 
+template <int DW>
+__device__ __forceinline__ void loadSlotsVec(uint32_t (&s)[DW], const uint8_t* p)
+{
+    if constexpr (DW % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < DW / 4; ++i) {
+            const u32x4 v = *(const u32x4*)(p + 16 * i);
+            s[4 * i] = v.x; s[4 * i + 1] = v.y; s[4 * i + 2] = v.z; s[4 * i + 3] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < DW / 2; ++i) {
+            const u32x2 v = *(const u32x2*)(p + 8 * i);
+            s[2 * i] = v.x; s[2 * i + 1] = v.y;
+        }
+    }
+}
+
+// mode 0: full-width vector loads, 1: masked dwords, 2: masked bytes
 template <int DW>
 __device__ __forceinline__ void loadSlots(uint32_t (&s)[DW], const uint8_t* p, int validBytes, int mode)
 {
     if (mode == 0) {
-        if constexpr (DW % 4 == 0) {
-#pragma unroll
-            for (int i = 0; i < DW / 4; ++i) {
-                const u32x4 v = *(const u32x4*)(p + 16 * i);
-                s[4 * i] = v.x; s[4 * i + 1] = v.y; s[4 * i + 2] = v.z; s[4 * i + 3] = v.w;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < DW / 2; ++i) {
-                const u32x2 v = *(const u32x2*)(p + 8 * i);
-                s[2 * i] = v.x; s[2 * i + 1] = v.y;
-            }
-        }
+        loadSlotsVec<DW>(s, p);
     } else if (mode == 1) {
 #pragma unroll
         for (int i = 0; i < DW; ++i) s[i] = (4 * i < validBytes) ? *(const uint32_t*)(p + 4 * i) : 0u;
@@ -55,12 +66,31 @@ __device__ __forceinline__ void loadSlots(uint32_t (&s)[DW], const uint8_t* p, i
     }
 }
 
-template <class Mma, int MT, int KT, int NT, typename OutT>
+template <int DW>
+__device__ __forceinline__ void storeVec(uint8_t* o, const uint32_t (&pk)[DW])
+{
+    if constexpr (DW % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < DW / 4; ++i) {
+            const u32x4 v = {pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]};
+            ((u32x4*)o)[i] = v;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < DW / 2; ++i) {
+            const u32x2 v = {pk[2 * i], pk[2 * i + 1]};
+            ((u32x2*)o)[i] = v;
+        }
+    }
+}
+
+template <class Mma, int MT, int KT, int NT, typename OutT, bool FAST>
 __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 {
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     constexpr int SLOT_DW = RAW * KT;         // input dwords per lane per 16-sample tile
     constexpr int ROWS = 4 * MT;              // output rows per lane
+    constexpr int OUT_DW = ROWS * (int)sizeof(OutT) / 4;
     typedef typename Mma::Acc Acc;
 
     __shared__ __attribute__((aligned(16))) uint32_t ldsW[MT * KT * 64 * RAW];
@@ -108,7 +138,6 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     const int validRows = min(max(a.m - rowBase, 0), ROWS);
     const int colBase = (int)(g * gs);
     const int validBytes = min((int)gs, max(a.k - colBase, 0)) * ESZ;
-    // 0: full-width vector loads, 1: masked dwords, 2: masked bytes
     const int loadMode = (validBytes == SLOT_DW * 4 && a.inAlign >= (SLOT_DW % 4 == 0 ? 16u : 8u)) ? 0
                        : ((validBytes & 3) == 0 && a.inAlign >= 4u) ? 1 : 2;
 
@@ -123,9 +152,16 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
             else
                 biasv[t][r] = (a.bias && row < a.m) ? ((const int32_t*)a.bias)[row] : 0;
         }
+    // ReLU as a lower bound: max(z, 0) when on, max(z, -inf) = z when off (FAST path)
+    const float reluFloor = a.act == kActRelu ? 0.f : -__builtin_inff();
+    const int reluFloorI = a.act == kActRelu ? 0 : (int)0x80000000;
 
     constexpr uint32_t TILE = 16 * NT;
-    const uint32_t numTiles = (a.batch + TILE - 1) / TILE;
+    // FAST handles whole tiles only (the launcher sends the ragged tail to the general kernel),
+    // so its loop has no per-lane predicates and the prefetch below is unconditional: with a
+    // fixed number of loads and stores per iteration the compiler can wait for exactly the
+    // current tile's loads while the next tile's stay in flight.
+    const uint32_t numTiles = FAST ? a.batch / TILE : (a.batch + TILE - 1) / TILE;
     const uint32_t tileStride = gridDim.x * 4;
     uint32_t tile = blockIdx.x * 4 + wave;
     if (tile >= numTiles) return;
@@ -134,23 +170,21 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     uint8_t* outLane = a.out + (size_t)rowBase * sizeof(OutT);
     const uint32_t lastSample = a.batch - 1;
 
-    uint32_t cur[NT][SLOT_DW], nxt[NT][SLOT_DW];
+    // One tile's input registers are loaded a whole tile ahead.  The two buffers swap roles
+    // (no register copies: a copy would have to wait for the prefetch it is meant to hide).
+    auto loadTile = [&](uint32_t (&buf)[NT][SLOT_DW], uint32_t t) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
-        const uint32_t s = min(tile * TILE + 16 * j + n, lastSample);
-        loadSlots<SLOT_DW>(cur[j], inLane + (size_t)s * a.inStride, validBytes, loadMode);
-    }
-
-    for (; tile < numTiles; tile += tileStride) {
-        const uint32_t nextTile = tile + tileStride;
-        if (nextTile < numTiles) {
-#pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const uint32_t s = min(nextTile * TILE + 16 * j + n, lastSample);
-                loadSlots<SLOT_DW>(nxt[j], inLane + (size_t)s * a.inStride, validBytes, loadMode);
+        for (int j = 0; j < NT; ++j) {
+            if constexpr (FAST) {
+                loadSlotsVec<SLOT_DW>(buf[j], inLane + (size_t)(t * TILE + 16 * j + n) * a.inStride);
+            } else {
+                const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
+                loadSlots<SLOT_DW>(buf[j], inLane + (size_t)s * a.inStride, validBytes, loadMode);
             }
         }
+    };
 
+    auto computeStore = [&](const uint32_t (&buf)[NT][SLOT_DW], uint32_t t0) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
             Acc acc[MT];
@@ -159,16 +193,36 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt) {
                 uint32_t bfrag[FD];
-                Mma::decode(&cur[j][kt * RAW], bfrag);
+                Mma::decode(&buf[j][kt * RAW], bfrag);
 #pragma unroll
                 for (int t = 0; t < MT; ++t) acc[t] = Mma::mma(afrag[t][kt], bfrag, acc[t]);
             }
 
-            const uint32_t sample = tile * TILE + 16 * j + n;
-            if (sample < a.batch && validRows > 0) {
-                OutT* o = (OutT*)(outLane + (size_t)sample * a.outStride);
-                constexpr int OUT_DW = ROWS * (int)sizeof(OutT) / 4;
-                uint32_t pk[OUT_DW];
+            const uint32_t sample = t0 * TILE + 16 * j + n;
+            uint8_t* o = outLane + (size_t)sample * a.outStride;
+            uint32_t pk[OUT_DW];
+            if constexpr (FAST) {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    if constexpr (sizeof(OutT) == 2) {
+                        // max on the fp32 accumulator commutes with the rounding to fp16
+                        halfx2 lo, hi;
+                        lo.x = (half_t)fmaxf(acc[t][0], reluFloor); lo.y = (half_t)fmaxf(acc[t][1], reluFloor);
+                        hi.x = (half_t)fmaxf(acc[t][2], reluFloor); hi.y = (half_t)fmaxf(acc[t][3], reluFloor);
+                        pk[2 * t] = __builtin_bit_cast(uint32_t, lo);
+                        pk[2 * t + 1] = __builtin_bit_cast(uint32_t, hi);
+                    } else if constexpr (Mma::kIsFloat) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            pk[4 * t + r] = __builtin_bit_cast(uint32_t, fmaxf(acc[t][r], reluFloor));
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) pk[4 * t + r] = (uint32_t)max(acc[t][r], reluFloorI);
+                    }
+                }
+                storeVec<OUT_DW>(o, pk);
+            } else {
+                if (sample >= a.batch || validRows <= 0) continue;
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
                     if constexpr (sizeof(OutT) == 2) {
@@ -197,57 +251,102 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                     }
                 }
                 if (a.accumulate || validRows != ROWS || a.outAlign < (OUT_DW % 4 == 0 ? 16u : 8u)) {
-                    // element-wise tail: the member forms `this += ...` and ragged m
+                    // element-wise tail: the member forms `this += ...`, ragged m, unaligned rows
+                    OutT* oe = (OutT*)o;
 #pragma unroll
                     for (int e = 0; e < ROWS; ++e) {
                         if (e < validRows) {
                             if constexpr (sizeof(OutT) == 2) {
                                 const uint16_t bits = (uint16_t)(pk[e / 2] >> (16 * (e & 1)));
                                 half_t v = __builtin_bit_cast(half_t, bits);
-                                if (a.accumulate) v = (half_t)((float)o[e] + (float)v);
-                                o[e] = v;
+                                if (a.accumulate) v = (half_t)((float)oe[e] + (float)v);
+                                oe[e] = v;
                             } else {
                                 OutT v = __builtin_bit_cast(OutT, pk[e]);
-                                if (a.accumulate) v = o[e] + v;
-                                o[e] = v;
+                                if (a.accumulate) v = oe[e] + v;
+                                oe[e] = v;
                             }
                         }
                     }
-                } else if constexpr (OUT_DW % 4 == 0) {
-#pragma unroll
-                    for (int i = 0; i < OUT_DW / 4; ++i) {
-                        const u32x4 v = {pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]};
-                        ((u32x4*)o)[i] = v;
-                    }
                 } else {
-#pragma unroll
-                    for (int i = 0; i < OUT_DW / 2; ++i) {
-                        const u32x2 v = {pk[2 * i], pk[2 * i + 1]};
-                        ((u32x2*)o)[i] = v;
-                    }
+                    storeVec<OUT_DW>(o, pk);
                 }
             }
         }
+    };
 
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int d = 0; d < SLOT_DW; ++d) cur[j][d] = nxt[j][d];
+    uint32_t bufA[NT][SLOT_DW], bufB[NT][SLOT_DW];
+    loadTile(bufA, tile);
+    while (true) {
+        // a prefetch past the end re-reads a valid tile instead of branching around the loads
+        const uint32_t t1 = tile + tileStride;
+        loadTile(bufB, t1 < numTiles ? t1 : tile);
+        computeStore(bufA, tile);
+        if (t1 >= numTiles) break;
+        const uint32_t t2 = t1 + tileStride;
+        loadTile(bufA, t2 < numTiles ? t2 : t1);
+        computeStore(bufB, t1);
+        if (t2 >= numTiles) break;
+        tile = t2;
     }
 }
 
-template <class Mma, int MT, int KT, typename OutT>
+#ifndef CV_MATMUL_NT_SMALL
+#define CV_MATMUL_NT_SMALL 2
+#endif
+
+template <int MT, int KT>
+struct TileShape {
+    // samples per wave-iteration: as many 16-sample tiles as the register budget allows
+    static constexpr int NT = (MT * KT <= 8) ? CV_MATMUL_NT_SMALL : (MT * KT <= 16 ? 2 : 1);
+};
+
+template <class Mma, int MT, int KT, typename OutT, bool FAST>
 hipError_t launchOne(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
-    // samples per wave-iteration: as many 16-sample tiles as the register budget allows
-    constexpr int NT = (MT * KT <= 8) ? 4 : (MT * KT <= 16 ? 2 : 1);
+    constexpr int NT = TileShape<MT, KT>::NT;
+    // Persistent grid: exactly as many workgroups as are resident at once, so that every wave
+    // strides over the same number of tiles (a partial second round would run at a fraction of
+    // the occupancy).  The residency of a kernel is fixed, so it is queried once.
+    static int blocksPerCU = 0;
+    if (blocksPerCU == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, matmulKernel<Mma, MT, KT, NT, OutT, FAST>, 256, 0) != hipSuccess || n < 1) n = 1;
+        blocksPerCU = n;
+    }
     const uint32_t tile = 16 * NT;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
-    const uint32_t blocksMax = (uint32_t)numCUs * 4u;
+    const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
-    hipLaunchKernelGGL((matmulKernel<Mma, MT, KT, NT, OutT>), dim3(blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((matmulKernel<Mma, MT, KT, NT, OutT, FAST>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
+}
+
+template <class Mma, int MT, int KT, typename OutT>
+hipError_t launchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
+{
+    constexpr uint32_t slotBytes = Mma::kRawDW * 4 * KT;
+    constexpr uint32_t tile = 16 * TileShape<MT, KT>::NT;
+    const bool fast = (uint32_t)a.k == 4u * Mma::kEpl * KT && a.m == 16 * MT &&
+                      a.inAlign >= (slotBytes % 16 == 0 ? 16u : 8u) &&
+                      a.outAlign >= ((4 * MT * sizeof(OutT)) % 16 == 0 ? 16u : 8u) &&
+                      !a.accumulate && a.act != kActLeakyRelu;
+    if (!fast) return launchOne<Mma, MT, KT, OutT, false>(stream, a, numCUs);
+    // whole tiles on the streaming kernel, the ragged tail (< one tile) on the general one
+    const uint32_t whole = a.batch / tile * tile;
+    if (whole) {
+        MatMulArgs b = a;
+        b.batch = whole;
+        const hipError_t e = launchOne<Mma, MT, KT, OutT, true>(stream, b, numCUs);
+        if (e != hipSuccess) return e;
+    }
+    if (whole == a.batch) return hipSuccess;
+    MatMulArgs t = a;
+    t.in += (size_t)whole * a.inStride;
+    t.out += (size_t)whole * a.outStride;
+    t.batch = a.batch - whole;
+    return launchOne<Mma, MT, KT, OutT, false>(stream, t, numCUs);
 }
 
 template <class Mma, typename OutT>
@@ -258,7 +357,7 @@ hipError_t dispatchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
     const int KTs = kt <= 1 ? 1 : kt <= 2 ? 2 : kt <= 4 ? 4 : 0;
     if (!MTs || !KTs) return hipErrorInvalidValue;
 #define CV_CASE(M_, K_) \
-    if (MTs == M_ && KTs == K_) return launchOne<Mma, M_, K_, OutT>(stream, a, numCUs);
+    if (MTs == M_ && KTs == K_) return launchShape<Mma, M_, K_, OutT>(stream, a, numCUs);
     CV_CASE(1, 1) CV_CASE(1, 2) CV_CASE(1, 4)
     CV_CASE(2, 1) CV_CASE(2, 2) CV_CASE(2, 4)
     CV_CASE(4, 1) CV_CASE(4, 2) CV_CASE(4, 4)
@@ -268,24 +367,4 @@ hipError_t dispatchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
 }
 
 } // namespace
-
-hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& a, int numCUs)
-{
-    if (a.batch == 0) return hipSuccess;
-    switch (kind) {
-    case MmaKind::F16:
-        return a.outCt == kF32 ? dispatchShape<F16Mma, float>(stream, a, numCUs)
-                               : dispatchShape<F16Mma, half_t>(stream, a, numCUs);
-    case MmaKind::Fp8AsF16:
-        return a.outCt == kF32 ? dispatchShape<Fp8AsF16Mma, float>(stream, a, numCUs)
-                               : dispatchShape<Fp8AsF16Mma, half_t>(stream, a, numCUs);
-    case MmaKind::Fp8Native:
-        return a.outCt == kF32 ? dispatchShape<Fp8NativeMma, float>(stream, a, numCUs)
-                               : dispatchShape<Fp8NativeMma, half_t>(stream, a, numCUs);
-    case MmaKind::I8:
-        return dispatchShape<I8Mma, int32_t>(stream, a, numCUs);
-    }
-    return hipErrorInvalidValue;
-}
-
 } // namespace cv
