@@ -302,3 +302,61 @@ def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torc
                                   transpose, matrixStride, M=M, resultType=resultType, out=out,
                                   accumulate=accumulate, activation=activation, leakySlope=leakySlope,
                                   stream=stream, flags=flags)
+
+
+# ---------------------------------------------------------------------------------------------
+# fused MLP: the example's FeedForwardLayer chain
+# ---------------------------------------------------------------------------------------------
+
+@dataclass
+class FeedForwardLayer:
+    """One layer of the example's network (examples/mlp-training-coopvec/fflayer.slang:7-67):
+    device buffers for weights / weightsGrad / biases / biasesGrad plus what is constexpr in Slang."""
+    inputSize: int
+    outputSize: int
+    weights: torch.Tensor                  # raw bytes (any dtype), layout `weightLayout`
+    biases: Optional[torch.Tensor] = None  # fp16 [outputSize]
+    weightLayout: int = CoopVecMatrixLayout.RowMajor
+    weightStride: int = 0
+    activation: int = Activation.NoActivation
+    leakySlope: float = 0.0
+    weightsGrad: Optional[torch.Tensor] = None
+    biasesGrad: Optional[torch.Tensor] = None
+    gradLayout: int = CoopVecMatrixLayout.TrainingOptimal
+    gradStride: int = 0
+
+
+def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int, flags: int):
+    arr = (_lib.CvMlpLayer * len(layers))()
+    for i, L in enumerate(layers):
+        arr[i].weights = _buffer_ptr(L.weights, "weights")
+        arr[i].weightsGrad = _buffer_ptr(L.weightsGrad, "weightsGrad") if L.weightsGrad is not None else None
+        arr[i].biases = _buffer_ptr(L.biases, "biases") if L.biases is not None else None
+        arr[i].biasesGrad = _buffer_ptr(L.biasesGrad, "biasesGrad") if L.biasesGrad is not None else None
+        arr[i].inputSize = L.inputSize; arr[i].outputSize = L.outputSize
+        arr[i].weightLayout = int(L.weightLayout); arr[i].weightStride = int(L.weightStride)
+        arr[i].gradLayout = int(L.gradLayout); arr[i].gradStride = int(L.gradStride)
+        arr[i].activation = int(L.activation); arr[i].leakySlope = float(L.leakySlope)
+    d = _lib.CvMlpDesc()
+    d.layers = arr; d.numLayers = len(layers)
+    d.inputType = int(weightType); d.weightType = int(weightType)
+    d.biasType = int(CoopVecComponentType.Float16); d.outputType = int(CoopVecComponentType.Float16)
+    d.gradType = int(gradType); d.flags = int(flags)
+    return d, arr
+
+
+def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
+               weightType: int = CoopVecComponentType.Float16, out: Optional[torch.Tensor] = None,
+               flags: int = 0, stream=None) -> torch.Tensor:
+    """network.eval over a batch: every layer is coopVecMatMulAdd + activation with CoopVec<half>
+    between layers (network.slang:41-47), fused into one kernel."""
+    inCt, inStride = _vector_info(input, weightType, "input")
+    batch = input.shape[0]
+    if out is None:
+        out = torch.empty((batch, layers[-1].outputSize), dtype=torch.float16, device=input.device)
+    _, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
+    d, keep = _mlp_desc(layers, weightType, CoopVecComponentType.Float32, flags)
+    d.inputType = int(inCt)
+    _check(_lib.load().cvMlpForward(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride,
+                                    out.data_ptr(), outStride, batch))
+    return out

@@ -301,9 +301,84 @@ CV_API CvResult cvReduceSumAccumulate(void*, const void*, size_t, int32_t, int32
     return fail(CV_E_NOT_IMPLEMENTED, "cvReduceSumAccumulate: not implemented yet");
 }
 
-CV_API CvResult cvMlpForward(void*, const CvMlpDesc*, const void*, size_t, void*, size_t, uint32_t)
+// Validates the parts of a CvMlpDesc that forward and training share and fills the per-layer
+// kernel arguments.
+static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLayerArgs* out)
 {
-    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpForward: not implemented yet");
+    if (!mlp || !mlp->layers) return fail(CV_E_INVALID_ARG, "%s: mlp/layers is null", who);
+    if (mlp->numLayers < 1 || mlp->numLayers > cv::kMaxMlpLayers)
+        return fail(CV_E_INVALID_ARG, "%s: numLayers=%d (supported: 1..%d)", who, mlp->numLayers, cv::kMaxMlpLayers);
+    if (mlp->weightType != CV_FLOAT16 && mlp->weightType != CV_FLOAT_E4M3)
+        return fail(CV_E_NOT_AVAILABLE, "%s: weightType %d (supported: FLOAT16, FLOAT_E4M3)", who, mlp->weightType);
+    if (mlp->biasType != CV_FLOAT16 || mlp->outputType != CV_FLOAT16)
+        return fail(CV_E_NOT_AVAILABLE, "%s: biasType/outputType must be FLOAT16", who);
+    if (mlp->inputType != mlp->weightType)
+        return fail(CV_E_NOT_AVAILABLE, "%s: inputType %d must equal weightType %d", who, mlp->inputType, mlp->weightType);
+    const uint32_t wEsz = cv::elemSize(mlp->weightType);
+    for (int l = 0; l < mlp->numLayers; ++l) {
+        const CvMlpLayer& L = mlp->layers[l];
+        if (!L.weights) return fail(CV_E_INVALID_ARG, "%s: layer %d has no weights", who, l);
+        if (L.inputSize <= 0 || L.outputSize <= 0) return fail(CV_E_INVALID_ARG, "%s: layer %d is %dx%d", who, l, L.outputSize, L.inputSize);
+        if (l > 0 && L.inputSize != mlp->layers[l - 1].outputSize)
+            return fail(CV_E_INVALID_ARG, "%s: layer %d takes %d inputs but layer %d produces %d", who, l, L.inputSize, l - 1, mlp->layers[l - 1].outputSize);
+        if (L.weightLayout < 0 || L.weightLayout > 3 || !cv::layoutSupports(mlp->weightType, L.weightLayout))
+            return fail(CV_E_NOT_AVAILABLE, "%s: layer %d: component type %d has no layout %d", who, l, mlp->weightType, L.weightLayout);
+        if (L.activation < CV_ACT_NONE || L.activation > CV_ACT_LEAKY_RELU)
+            return fail(CV_E_INVALID_ARG, "%s: layer %d: unknown activation %d", who, l, L.activation);
+        cv::MlpLayerArgs& o = out[l];
+        o.w = (const uint8_t*)L.weights;
+        o.bias = (const uint8_t*)L.biases;
+        o.shape = cv::MatrixShape{(uint32_t)L.outputSize, (uint32_t)L.inputSize, mlp->weightType, L.weightLayout,
+                                  isOptimal(L.weightLayout) ? 0 : (size_t)L.weightStride};
+        if (cv::matrixSize(o.shape) == 0) return fail(CV_E_INVALID_ARG, "%s: layer %d: weightStride %u smaller than a row/column", who, l, L.weightStride);
+        if ((uintptr_t)o.w % (isOptimal(L.weightLayout) ? 16u : wEsz) || (!isOptimal(L.weightLayout) && L.weightStride % wEsz) ||
+            (uintptr_t)o.bias % 2)
+            return fail(CV_E_INVALID_ARG, "%s: layer %d: weights/bias misaligned", who, l);
+        o.in = L.inputSize; o.out = L.outputSize; o.act = L.activation; o.slope = L.leakySlope;
+    }
+    return CV_OK;
+}
+
+CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
+                             void* output, size_t outputStride, uint32_t batch)
+{
+    cv::MlpArgs a;
+    memset(&a, 0, sizeof(a));
+    CvResult rc = fillMlpLayers("cvMlpForward", mlp, a.layers);
+    if (CV_FAILED(rc)) return rc;
+    if (batch == 0) return CV_OK;
+    if (!input || !output) return fail(CV_E_INVALID_ARG, "cvMlpForward: null input/output");
+    const uint32_t inEsz = cv::elemSize(mlp->inputType);
+    const int L = mlp->numLayers;
+    if ((uintptr_t)input % inEsz || inputStride % inEsz || (uintptr_t)output % 2 || outputStride % 2)
+        return fail(CV_E_INVALID_ARG, "cvMlpForward: vector address/stride not aligned to the element size");
+    if (batch > 1 && (inputStride < (size_t)mlp->layers[0].inputSize * inEsz || outputStride < (size_t)mlp->layers[L - 1].outputSize * 2))
+        return fail(CV_E_INVALID_ARG, "cvMlpForward: vector stride smaller than the vector");
+    if (L == 1) {   // a single layer is the plain operator
+        const CvMlpLayer& l0 = mlp->layers[0];
+        CvMatMulDesc d;
+        memset(&d, 0, sizeof(d));
+        d.input = input; d.inputStride = inputStride; d.inputType = mlp->inputType; d.inputInterpretation = mlp->weightType;
+        d.k = l0.inputSize; d.output = output; d.outputStride = outputStride; d.resultType = CV_FLOAT16; d.m = l0.outputSize;
+        d.matrix = l0.weights; d.matrixInterpretation = mlp->weightType; d.layout = l0.weightLayout; d.matrixStride = l0.weightStride;
+        d.bias = l0.biases; d.biasInterpretation = CV_FLOAT16; d.activation = l0.activation; d.leakySlope = l0.leakySlope;
+        d.batch = batch; d.flags = mlp->flags;
+        return cvMatMul(stream, &d);
+    }
+    a.numLayers = L;
+    a.in = (const uint8_t*)input; a.out = (uint8_t*)output;
+    a.inStride = inputStride; a.outStride = outputStride; a.batch = batch;
+    a.inAlign = alignOf(input, inputStride); a.outAlign = alignOf(output, outputStride);
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16
+                     : (mlp->flags & CV_FLAG_FP8_MATRIX_PIPELINE) ? cv::MmaKind::Fp8Native : cv::MmaKind::Fp8AsF16;
+    const hipError_t e = cv::launchMlpForward((hipStream_t)stream, kind, a, cus);
+    if (e == hipErrorInvalidValue)
+        return fail(CV_E_NOT_AVAILABLE, "cvMlpForward: no fused specialisation for these layer sizes "
+                    "(needs equal-width hidden layers of at most 64 and one of the built-in tile shapes); "
+                    "chain cvMatMul calls instead");
+    return fromHip(e, "cvMlpForward launch");
 }
 
 CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc*, uint32_t, size_t* outBytes)

@@ -32,6 +32,28 @@ enum class MmaKind : int { F16 = 0, Fp8AsF16 = 1, Fp8Native = 2, I8 = 3 };
 // Returns hipSuccess, or hipErrorInvalidValue when no specialisation covers (m,k).
 hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& args, int numCUs);
 
+// ---- fused forward MLP --------------------------------------------------------------------
+constexpr int kMaxMlpLayers = 8;
+struct MlpLayerArgs {
+    const uint8_t* w;       // weights base
+    const uint8_t* bias;    // fp16 biases or nullptr
+    MatrixShape shape;      // out x in as it lies in memory
+    int32_t in, out;
+    int32_t act;
+    float slope;
+};
+struct MlpArgs {
+    MlpLayerArgs layers[kMaxMlpLayers];
+    int32_t numLayers;
+    const uint8_t* in;
+    uint8_t* out;           // fp16 [batch][lastOut]
+    uint64_t inStride, outStride;
+    uint32_t batch;
+    uint32_t inAlign, outAlign;
+};
+// hipErrorInvalidValue when no built-in specialisation covers the layer shapes
+hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
+
 // ---- layout conversion --------------------------------------------------------------------
 struct ConvertItem {
     const uint8_t* src;

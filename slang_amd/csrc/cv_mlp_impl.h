@@ -1,0 +1,344 @@
+// cv_mlp_impl.h -- fused forward MLP kernel template for gfx950.
+//
+// Runs the chain the example builds from FeedForwardLayer.eval
+// (examples/mlp-training-coopvec/fflayer.slang:60-66: coopVecMatMulAdd + activation, with
+// CoopVec<half> as the carrier between layers; network.slang:41-47) for a whole batch:
+//
+//   - every layer is D = W . X^T on the matrix cores with the 16 samples of a tile as N;
+//   - under the row order of cv_layout.h the fp32 accumulators of layer l are, register for
+//     register, the B operand of layer l+1 once rounded to fp16 (and, for e4m3 networks,
+//     re-quantised): activations never leave the VGPRs and never cross lanes;
+//   - the workgroup stages all weights into LDS once (any source layout), then every wave
+//     keeps all A fragments and the biases (packed fp16) in VGPRs while it strides over
+//     tiles of NT*16 samples with the next tile's inputs prefetched.
+//
+// The kernel is specialised on tile counts (input k-tiles, hidden width in 16-row tiles,
+// number of hidden layers, output tiles); actual dimensions are runtime values padded with
+// zero weights.
+#pragma once
+#include <type_traits>
+
+#include "cv_device.h"
+#include "cv_kernels.h"
+
+namespace cv {
+namespace {
+
+template <int B, int E, class F>
+__device__ __forceinline__ void staticFor(F&& f)
+{
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        staticFor<B + 1, E>(f);
+    }
+}
+
+// hidden layers all 16*HT wide: layer 0 is in->hidden, layers 1..NHID-1 hidden->hidden,
+// layer NHID hidden->out
+template <int KT0_, int HT_, int NHID_, int MTL_>
+struct UniformNet {
+    static constexpr int KT0 = KT0_, HT = HT_, NHID = NHID_, MTL = MTL_;
+    static constexpr int L = NHID_ + 1;
+    static constexpr int KTH = (HT_ + 1) / 2;
+    static constexpr int MTMAX = HT_ > MTL_ ? HT_ : MTL_;
+    static constexpr int KTMAX = KT0_ > KTH ? KT0_ : KTH;
+    static constexpr int mt(int l) { return l < NHID_ ? HT_ : MTL_; }
+    static constexpr int kt(int l) { return l == 0 ? KT0_ : KTH; }
+    static constexpr int fragBase(int l)   // index of layer l's first fragment in LDS
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += mt(i) * kt(i);
+        return b;
+    }
+    static constexpr int totalFrags = fragBase(L);
+    static constexpr int biasBase(int l)   // in 16-row tiles
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += mt(i);
+        return b;
+    }
+    static constexpr int totalBiasTiles = biasBase(L);
+};
+
+// accumulators (one 16-row tile, 4 values per lane) -> the carrier: fp16, activation
+__device__ __forceinline__ void carrierFromAcc(const floatx4& acc, int act, float slope, half_t (&h)[4])
+{
+#pragma unroll
+    for (int r = 0; r < 4; ++r) h[r] = activateHalf((half_t)acc[r], act, slope);
+}
+
+// Two accumulator tiles -> one B fragment of the next layer (8 k-slots per lane).
+template <class Mma>
+__device__ __forceinline__ void fragFromCarrier(const half_t (&lo)[4], const half_t (&hi)[4], uint32_t* frag)
+{
+    if constexpr (std::is_same<Mma, F16Mma>::value) {
+        halfx2 a = {lo[0], lo[1]}, b = {lo[2], lo[3]}, c = {hi[0], hi[1]}, d = {hi[2], hi[3]};
+        frag[0] = __builtin_bit_cast(uint32_t, a); frag[1] = __builtin_bit_cast(uint32_t, b);
+        frag[2] = __builtin_bit_cast(uint32_t, c); frag[3] = __builtin_bit_cast(uint32_t, d);
+    } else {
+        // re-quantise the fp16 carrier to OCP e4m3 (saturating, nearest even)
+        const uint32_t q0 = packE4M3Sat((float)lo[0], (float)lo[1]) | (packE4M3Sat((float)lo[2], (float)lo[3]) << 16);
+        const uint32_t q1 = packE4M3Sat((float)hi[0], (float)hi[1]) | (packE4M3Sat((float)hi[2], (float)hi[3]) << 16);
+        const uint32_t raw[2] = {q0, q1};
+        Mma::decode(raw, frag);      // e4m3 bytes as they are, or decoded back to fp16 operands
+    }
+}
+
+template <class Mma, class Net, int NT>
+__global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
+{
+    constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
+    constexpr int L = Net::L;
+    constexpr int IN_DW = RAW * Net::KT0;
+    static_assert(EPL == 8, "the layer chain needs 8 k-slots per lane per fragment");
+
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[Net::totalFrags * 64 * RAW];
+    __shared__ __attribute__((aligned(16))) uint16_t ldsB[Net::totalBiasTiles * 16];
+
+    // ---- stage weights (fragment order) and biases (fp16, kernel row order) into LDS -------
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
+        const MlpLayerArgs& ly = a.layers[l];
+        const uint32_t gs = optGS((uint32_t)ly.in);
+        uint32_t* base = ldsW + Net::fragBase(l) * 64 * RAW;
+        const bool direct = ly.shape.layout == kInferencingOptimal &&
+                            optMT(ly.shape.rows) == (uint32_t)MT && optKT(ly.shape.cols, EPL) == (uint32_t)KT;
+        if (direct) {
+            const u32x2* src = (const u32x2*)ly.w;
+            u32x2* dst = (u32x2*)base;
+            for (int i = threadIdx.x; i < MT * KT * 64 * RAW / 2; i += 256) dst[i] = src[i];
+        } else {
+            uint8_t* dst = (uint8_t*)base;
+            for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
+                const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
+                const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
+                const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
+                const uint32_t q = (uint32_t)(kt * EPL + s), col = g * gs + q;
+                const bool valid = row < (uint32_t)ly.out && q < gs && col < (uint32_t)ly.in;
+                const size_t off = valid ? elemOffset(ly.shape, row, col) : 0;
+                if constexpr (ESZ == 2) ((uint16_t*)dst)[e] = valid ? *(const uint16_t*)(ly.w + off) : (uint16_t)0;
+                else                    dst[e] = valid ? ly.w[off] : (uint8_t)0;
+            }
+        }
+        // bias of tile t, lane group g, r: row g*ROWS + 4t + r  ->  ldsB[(biasBase + t)*16 + 4g + r]
+        for (int e = threadIdx.x; e < MT * 16; e += 256) {
+            const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
+            const int row = g * ROWS + 4 * t + r;
+            uint16_t v = 0;
+            if (ly.bias && row < ly.out) v = ((const uint16_t*)ly.bias)[row];
+            ldsB[(Net::biasBase(l) + t) * 16 + 4 * g + r] = v;
+        }
+    });
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, n = lane & 15;
+
+    // ---- weights and biases to registers ---------------------------------------------------
+    uint32_t W[L][Net::MTMAX][Net::KTMAX][FD];
+    uint32_t Bs[L][Net::MTMAX][2];          // 4 fp16 biases per tile, packed
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+#pragma unroll
+        for (int t = 0; t < Net::mt(l); ++t) {
+#pragma unroll
+            for (int kt = 0; kt < Net::kt(l); ++kt)
+                Mma::decode(&ldsW[((Net::fragBase(l) + t * Net::kt(l) + kt) * 64 + lane) * RAW], W[l][t][kt]);
+            const u32x2 b = *(const u32x2*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+            Bs[l][t][0] = b.x; Bs[l][t][1] = b.y;
+        }
+    });
+
+    // ---- per-lane constants ----------------------------------------------------------------
+    const uint32_t gs0 = optGS((uint32_t)a.layers[0].in);
+    const int colBase = (int)(g * gs0);
+    const int validBytes = min((int)gs0, max(a.layers[0].in - colBase, 0)) * ESZ;
+    const int loadMode = (validBytes == IN_DW * 4 && a.inAlign >= (IN_DW % 4 == 0 ? 16u : 8u)) ? 0
+                       : ((validBytes & 3) == 0 && a.inAlign >= 4u) ? 1 : 2;
+    constexpr int OROWS = 4 * Net::MTL;
+    const int outDim = a.layers[L - 1].out;
+    const int rowBase = g * OROWS;
+    const int validRows = min(max(outDim - rowBase, 0), OROWS);
+    const bool vecStore = validRows == OROWS && a.outAlign >= 8u;
+
+    constexpr uint32_t TILE = 16 * NT;
+    const uint32_t numTiles = (a.batch + TILE - 1) / TILE;
+    const uint32_t tileStride = gridDim.x * 4;
+    uint32_t tile = blockIdx.x * 4 + wave;
+    if (tile >= numTiles) return;
+    const uint8_t* inLane = a.in + (size_t)colBase * ESZ;
+    uint8_t* outLane = a.out + (size_t)rowBase * 2;
+    const uint32_t lastSample = a.batch - 1;
+
+    auto loadTile = [&](uint32_t (&buf)[NT][IN_DW], uint32_t t) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
+            const uint8_t* p = inLane + (size_t)s * a.inStride;
+            if (loadMode == 0) {
+                if constexpr (IN_DW % 4 == 0) {
+#pragma unroll
+                    for (int i = 0; i < IN_DW / 4; ++i) {
+                        const u32x4 v = *(const u32x4*)(p + 16 * i);
+                        buf[j][4 * i] = v.x; buf[j][4 * i + 1] = v.y; buf[j][4 * i + 2] = v.z; buf[j][4 * i + 3] = v.w;
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < IN_DW / 2; ++i) {
+                        const u32x2 v = *(const u32x2*)(p + 8 * i);
+                        buf[j][2 * i] = v.x; buf[j][2 * i + 1] = v.y;
+                    }
+                }
+            } else if (loadMode == 1) {
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) buf[j][i] = (4 * i < validBytes) ? *(const uint32_t*)(p + 4 * i) : 0u;
+            } else {
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) {
+                    uint32_t v = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; ++b)
+                        if (4 * i + b < validBytes) v |= (uint32_t)p[4 * i + b] << (8 * b);
+                    buf[j][i] = v;
+                }
+            }
+        }
+    };
+
+    auto computeStore = [&](const uint32_t (&buf)[NT][IN_DW], uint32_t t0) {
+        uint32_t act[NT][Net::KTMAX][FD];    // B fragments of the current layer's input
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&buf[j][kt * RAW], act[j][kt]);
+
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int MT = Net::mt(l), KT = Net::kt(l);
+            const int actv = a.layers[l].act;
+            const float slope = a.layers[l].slope;
+            floatx4 acc[NT][MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const halfx2 b01 = __builtin_bit_cast(halfx2, Bs[l][t][0]);
+                const halfx2 b23 = __builtin_bit_cast(halfx2, Bs[l][t][1]);
+                const floatx4 bv = {(float)b01.x, (float)b01.y, (float)b23.x, (float)b23.y};
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[j][t] = bv;
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+#pragma unroll
+                    for (int j = 0; j < NT; ++j) acc[j][t] = Mma::mma(W[l][t][kt], act[j][kt], acc[j][t]);
+
+            if constexpr (l + 1 < L) {
+                // this layer's output becomes the next layer's B operand, in place
+                constexpr int KTN = Net::kt(l + 1);
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+#pragma unroll
+                    for (int kt = 0; kt < KTN; ++kt) {
+                        half_t lo[4], hi[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+                        carrierFromAcc(acc[j][2 * kt], actv, slope, lo);
+                        if (2 * kt + 1 < MT) carrierFromAcc(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], actv, slope, hi);
+                        fragFromCarrier<Mma>(lo, hi, act[j][kt]);
+                    }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) {
+                    const uint32_t sample = t0 * TILE + 16 * j + n;
+                    if (sample >= a.batch || validRows <= 0) continue;
+                    half_t* o = (half_t*)(outLane + (size_t)sample * a.outStride);
+                    uint32_t pk[2 * MT];
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) {
+                        half_t h[4];
+                        carrierFromAcc(acc[j][t], actv, slope, h);
+                        halfx2 p0 = {h[0], h[1]}, p1 = {h[2], h[3]};
+                        pk[2 * t] = __builtin_bit_cast(uint32_t, p0);
+                        pk[2 * t + 1] = __builtin_bit_cast(uint32_t, p1);
+                    }
+                    if (vecStore) {
+#pragma unroll
+                        for (int t = 0; t < MT; ++t) {
+                            const u32x2 v = {pk[2 * t], pk[2 * t + 1]};
+                            ((u32x2*)o)[t] = v;
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < OROWS; ++e)
+                            if (e < validRows) {
+                                const uint16_t bits = (uint16_t)(pk[e / 2] >> (16 * (e & 1)));
+                                o[e] = __builtin_bit_cast(half_t, bits);
+                            }
+                    }
+                }
+            }
+        });
+    };
+
+    uint32_t bufA[NT][IN_DW], bufB[NT][IN_DW];
+    loadTile(bufA, tile);
+    while (true) {
+        const uint32_t t1 = tile + tileStride;
+        loadTile(bufB, t1 < numTiles ? t1 : tile);
+        computeStore(bufA, tile);
+        if (t1 >= numTiles) break;
+        const uint32_t t2 = t1 + tileStride;
+        loadTile(bufA, t2 < numTiles ? t2 : t1);
+        computeStore(bufB, t1);
+        if (t2 >= numTiles) break;
+        tile = t2;
+    }
+}
+
+template <class Mma, class Net>
+hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
+{
+    constexpr int NT = (Net::totalFrags * Mma::kFD <= 64) ? 4 : 2;
+    static int blocksPerCU = 0;
+    if (blocksPerCU == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mlpForwardKernel<Mma, Net, NT>, 256, 0) != hipSuccess || n < 1) n = 1;
+        blocksPerCU = n;
+    }
+    const uint32_t tile = 16 * NT;
+    const uint32_t numTiles = (a.batch + tile - 1) / tile;
+    const uint32_t blocksNeeded = (numTiles + 3) / 4;
+    const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
+    const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
+    hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT>), dim3(blocks), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+// The specialisations built into the library: (input k-tiles, hidden tiles, hidden layers,
+// output tiles).  Dimensions smaller than a tile are padded with zeros at run time.
+#define CV_MLP_SHAPES(X) \
+    X(1, 1, 1, 1) X(1, 1, 2, 1) X(1, 1, 3, 1) \
+    X(1, 2, 1, 1) X(1, 2, 2, 1) X(1, 2, 3, 1) X(1, 2, 1, 2) X(1, 2, 2, 2) X(1, 2, 3, 2) \
+    X(1, 4, 1, 1) X(1, 4, 2, 1) X(1, 4, 3, 1) X(1, 4, 4, 1) X(1, 4, 2, 4) X(1, 4, 3, 4) \
+    X(2, 4, 1, 4) X(2, 4, 2, 4) X(2, 4, 3, 4) X(2, 4, 2, 1)
+
+template <class Mma>
+hipError_t dispatchMlp(hipStream_t stream, const MlpArgs& a, int numCUs)
+{
+    const int L = a.numLayers;
+    if (L < 2) return hipErrorInvalidValue;
+    const int kt0 = (int)optKT((uint32_t)a.layers[0].in, Mma::kEpl);
+    const int ht = (int)optMT((uint32_t)a.layers[0].out);
+    for (int l = 1; l + 1 < L; ++l)
+        if ((int)optMT((uint32_t)a.layers[l].out) != ht) return hipErrorInvalidValue;
+    const int mtl = (int)optMT((uint32_t)a.layers[L - 1].out);
+#define CV_X(K0, HT, NH, ML) \
+    if (kt0 <= K0 && (K0 == 1 || kt0 == K0) && ht == HT && L - 1 == NH && mtl == ML) \
+        return launchMlpNet<Mma, UniformNet<K0, HT, NH, ML>>(stream, a, numCUs);
+    CV_MLP_SHAPES(CV_X)
+#undef CV_X
+    return hipErrorInvalidValue;
+}
+
+} // namespace
+} // namespace cv

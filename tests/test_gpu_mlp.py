@@ -1,0 +1,177 @@
+"""GPU parity of the fused forward MLP against the CPU oracle, through the C-ABI.
+
+Two checks per network:
+  (1) chain rule of parity: the fused kernel equals, bit for bit, the chain of single-layer GPU
+      operators (each of which is held to the float bar against the oracle in test_gpu_matmul.py);
+  (2) end to end against the oracle that applies the same rounding points (fp32 accumulate ->
+      fp16 -> activation -> [e4m3 re-quantisation]): max(2 ulp-fp16, 1e-3 relative) on the final
+      fp16, with the propagated summation-order floor 2^-18 * sum|terms| of the last layer, on at
+      least 99.9 % of the outputs; the remainder are samples where an fp32 sum of a hidden unit
+      fell within one rounding of an fp16 (or e4m3) boundary and rounded the other way.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle_binding as ob
+from gpu_util import DEV, as_bytes, matrix_in_layout, to_dev
+from slang_amd import coopvec as cv
+from slang_amd.coopvec import Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML, FeedForwardLayer
+
+pytestmark = pytest.mark.gpu
+
+
+def make_net(rng, dims, wtype, act=Activation.ReLU, slope=0.0, bias="zero", init="fan_in"):
+    specs = []
+    for i in range(len(dims) - 1):
+        fan_in, out = dims[i], dims[i + 1]
+        std = np.sqrt(2.0 / fan_in) if init == "he" else (0.5 if init == "half" else np.sqrt(1.0 / fan_in))
+        Wf = rng.standard_normal((out, fan_in)) * std
+        W = Wf.astype(np.float16) if wtype == CT.Float16 else ob.encode_e4m3(Wf)
+        if bias == "zero":
+            b = np.zeros(out, np.float16)
+        elif bias == "none":
+            b = None
+        else:
+            b = rng.uniform(-0.1, 0.1, out).astype(np.float16)
+        last = i == len(dims) - 2
+        specs.append(dict(W=W, b=b, act=int(Activation.NoActivation if last else act), slope=slope))
+    return specs
+
+
+def gpu_layers(specs, wtype, layout):
+    layers = []
+    for s in specs:
+        out, fan_in = s["W"].shape
+        wb = to_dev(matrix_in_layout(s["W"], wtype, layout))
+        esz = s["W"].dtype.itemsize
+        layers.append(FeedForwardLayer(fan_in, out, wb, as_bytes(to_dev(s["b"])) if s["b"] is not None else None,
+                                       layout, fan_in * esz if layout == ML.RowMajor else 0,
+                                       s["act"], s["slope"]))
+    return layers
+
+
+def chain_of_single_layers(specs, x_dev, wtype, flags=0):
+    """The same network as separate coopVecMatMulAdd launches; fp16 between layers, re-quantised
+    to e4m3 on the host side of each launch for e4m3 networks."""
+    h = x_dev
+    for s in specs:
+        out, fan_in = s["W"].shape
+        wb = as_bytes(to_dev(s["W"]))
+        esz = s["W"].dtype.itemsize
+        if wtype == CT.FloatE4M3 and h.dtype == torch.float16:
+            h = h.float().clamp(-448, 448).to(torch.float8_e4m3fn)
+        args = (h, wtype, wb, 0, wtype)
+        kw = dict(M=out, activation=s["act"], leakySlope=s["slope"], flags=flags)
+        if s["b"] is not None:
+            h = cv.coopVecMatMulAdd(*args, as_bytes(to_dev(s["b"])), 0, CT.Float16, ML.RowMajor, False, fan_in * esz, **kw)
+        else:
+            bz = torch.zeros(out, dtype=torch.float16, device=DEV).view(torch.uint8)
+            h = cv.coopVecMatMulAdd(*args, bz, 0, CT.Float16, ML.RowMajor, False, fan_in * esz, **kw)
+    return h
+
+
+def end_to_end_ok(y, specs, x, x_ct, min_frac=0.999):
+    ref, acts = ob.ref_mlp_forward(specs, x, x_ct, want_acts=True)
+    # floor from the last layer's terms: |W| . |a_prev|
+    prev = acts[-2].astype(np.float32) if len(acts) > 1 else None
+    Wl = specs[-1]["W"]
+    Wl = np.abs(Wl.astype(np.float32)) if Wl.dtype == np.float16 else np.abs(ob.decode_e4m3(Wl))
+    ab = np.abs(prev) @ Wl.T
+    bad = ob.float_parity_violations(y, ref.astype(np.float32), ab)
+    return 1.0 - bad.mean(), bad
+
+
+@pytest.mark.parametrize("layout", [ML.RowMajor, ML.InferencingOptimal])
+def test_small_fp16_mlp_config(layout):
+    # 2 -> 16 -> 16 -> 16 -> 1, ReLU on hidden layers, batch 65536, inputs U[0,1)^2,
+    # weights N(0, 1/fan_in) as fp16, zero biases
+    rng = np.random.default_rng(2024)
+    dims = [2, 16, 16, 16, 1]
+    B = 65536
+    specs = make_net(rng, dims, CT.Float16)
+    x = rng.uniform(0, 1, (B, 2)).astype(np.float16)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, layout), xd)
+    assert y.shape == (B, 1)
+    yc = chain_of_single_layers(specs, xd, CT.Float16)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    frac, bad = end_to_end_ok(y.cpu().numpy(), specs, x, ob.F16)
+    assert frac >= 0.999, "only %.5f within tolerance" % frac
+
+
+def test_example_network_leaky_relu():
+    # the example's 4 -> 16 -> 4 with max(z, 0.001 z) after *every* layer (fflayer.slang:60-66),
+    # parameters U[-1,1], inputs (x, y, x^2, y^2) (network.slang:35-38)
+    rng = np.random.default_rng(1072)
+    slope = float(np.float16(0.001))
+    specs = []
+    for fan_in, out in ((4, 16), (16, 4)):
+        specs.append(dict(W=rng.uniform(-1, 1, (out, fan_in)).astype(np.float16),
+                          b=rng.uniform(-1, 1, out).astype(np.float16), act=int(Activation.LeakyReLU), slope=slope))
+    B = 1000
+    xy = rng.uniform(0, 1, (B, 2)).astype(np.float16)
+    x = np.concatenate([xy, (xy.astype(np.float32) ** 2).astype(np.float16)], axis=1)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), xd)
+    yc = chain_of_single_layers(specs, xd, CT.Float16)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, ob.F16)
+    assert frac >= 0.999
+
+
+@pytest.mark.parametrize("dims", [[8, 64, 64, 64, 64, 1], [32, 64, 64, 8], [64, 64, 64, 64], [5, 30, 30, 3],
+                                  [40, 64, 64, 64], [16, 32, 32, 32, 20], [3, 60, 7]])
+def test_fp16_mlp_shapes(dims):
+    rng = np.random.default_rng(sum(dims))
+    B = 2000 + 13
+    specs = make_net(rng, dims, CT.Float16, bias="rand", init="he")
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.InferencingOptimal), xd)
+    yc = chain_of_single_layers(specs, xd, CT.Float16)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, ob.F16)
+    assert frac >= 0.999
+
+
+@pytest.mark.parametrize("flags", [0, cv.FLAG_FP8_MATRIX_PIPELINE])
+def test_e4m3_decoder_config(flags):
+    # 32 -> 64 -> 64 -> 8, weights and inputs 0.5*N(0,1) saturate-cast to e4m3, activations
+    # fp16 -> ReLU -> e4m3, fp16 output (a 2^16 slice of the 2^24 batch)
+    rng = np.random.default_rng(4096)
+    dims = [32, 64, 64, 8]
+    B = 1 << 16
+    specs = make_net(rng, dims, CT.FloatE4M3, bias="none", init="half")
+    x = ob.encode_e4m3(rng.standard_normal((B, 32)) * 0.5)
+    xd = to_dev(x)
+    for layout in (ML.RowMajor, ML.InferencingOptimal):
+        y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, layout), xd, weightType=CT.FloatE4M3, flags=flags)
+        yc = chain_of_single_layers(specs, xd, CT.FloatE4M3, flags)
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    frac, bad = end_to_end_ok(y.cpu().numpy(), specs, x, ob.E4M3)
+    if flags == 0:
+        # fp32-grade accumulation: the oracle's bar
+        assert frac >= 0.999, "only %.5f within tolerance" % frac
+    else:
+        # fp8 matrix pipeline: products far below the largest one of an instruction are truncated,
+        # which moves some hidden units across an e4m3 rounding boundary; report, and require the
+        # bulk to agree
+        assert frac >= 0.80, "only %.5f within tolerance" % frac
+
+
+def test_mlp_argument_validation():
+    rng = np.random.default_rng(0)
+    specs = make_net(rng, [8, 16, 4], CT.Float16)
+    layers = gpu_layers(specs, CT.Float16, ML.RowMajor)
+    x = torch.zeros(10, 8, dtype=torch.float16, device=DEV)
+    assert cv.mlpForward(layers, x[:0]).shape == (0, 4)
+    layers[1].inputSize = 15
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.mlpForward(layers, x)
+    assert e.value.result == cv.SLANG_E_INVALID_ARG
+    # hidden layers of different tile widths have no fused specialisation
+    specs = make_net(rng, [8, 16, 64, 4], CT.Float16)
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), x)
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
