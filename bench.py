@@ -112,7 +112,156 @@ def workload_c2(torch, cv, steps, warmup):
                 extra={"layout_conversion_us": conv_us}, cpu_baseline=cpu_baseline, key="c2")
 
 
-WORKLOADS = {"c2": workload_c2}
+def _time_cpu(fn, per_item, n):
+    t0 = time.perf_counter(); fn(); t1 = time.perf_counter()
+    return n / (t1 - t0)
+
+
+def workload_c3(torch, cv, steps, warmup):
+    """int8 128x128 -> int32 + int32 bias, batch 2^22, InferencingOptimal weights (bit-exact path)."""
+    import numpy as np
+    from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML, CooperativeVectorMatrixDesc as D
+    dev = "cuda"
+    B, M, K = 1 << 22, 128, 128
+    g = torch.Generator(device=dev); g.manual_seed(20253)
+    x = torch.randint(-128, 128, (B, K), device=dev, dtype=torch.int8, generator=g)
+    W = torch.randint(-127, 128, (M, K), device=dev, dtype=torch.int8, generator=g)
+    b = torch.randint(-65536, 65537, (M,), device=dev, dtype=torch.int32, generator=g)
+    wcol = W.t().contiguous().view(torch.uint8).flatten()          # ColumnMajor storage of the M x K matrix
+    size = cv.getCooperativeVectorMatrixSize(M, K, CT.SignedInt8, ML.InferencingOptimal)
+    wopt = torch.empty(size, dtype=torch.uint8, device=dev)
+    cv.convertCooperativeVectorMatrix(wopt, [D(M, K, CT.SignedInt8, ML.InferencingOptimal, size, 0, 0)],
+                                      wcol, [D(M, K, CT.SignedInt8, ML.ColumnMajor, M * K, 0, M)])
+    bb = b.view(torch.uint8)
+    out = torch.empty(B, M, dtype=torch.int32, device=dev)
+
+    def step():
+        cv.coopVecMatMulAdd(x, CT.SignedInt8, wopt, 0, CT.SignedInt8, bb, 0, CT.SignedInt32, ML.InferencingOptimal,
+                            False, 0, M=M, out=out)
+
+    def cpu_baseline():
+        import concurrent.futures as cf
+        import oracle_binding as ob
+        L = ob.lib()
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")), 16)
+        per_core = 1 << 12
+        n = per_core * cores
+        xs = x[:n].cpu().numpy().view(np.uint32); Wn = wcol.cpu().numpy(); bn = b.cpu().numpy()
+        outn = np.zeros((n, M), np.int32)
+
+        def run(g0, g1):
+            rc = L.cvo_slang_dispatch_matmul_add(g0, g1, n, ob.ptr(xs), K, ob.U32, K // 4, ob.S8P, K, ob.ptr(outn),
+                                                 M * 4, ob.S32, M, ob.ptr(Wn), 0, ob.S8, ob.COL, 0, M,
+                                                 ob.ptr(bn), 0, ob.S32, ob.HALF_RNE)
+            assert rc == 0
+        t0 = time.perf_counter(); run(0, per_core // 256); t1 = time.perf_counter()
+        one_core = per_core / (t1 - t0)
+        chunk = (n // 256) // cores
+        t0 = time.perf_counter()
+        with cf.ThreadPoolExecutor(cores) as pool:
+            list(pool.map(lambda c: run(c * chunk, (c + 1) * chunk), range(cores)))
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": cores, "kind": "port", "value_1core": one_core,
+                "sample": "first %d of the 2^22 vectors; C restatement of the Slang CPU-target fallback "
+                          "(packed int8, ColumnMajor, int32 accumulate), -O2" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * (K + M * 4), alg_flops=B * 2 * M * K, bound="hbm", dtype="int8",
+                kernel="matmulKernel<I8Mma,8,2,2,int,fast>",
+                config={"workload": "c3: int8 coopVecMatMulAdd 128x128 -> int32 + int32 bias, batch 2^22, "
+                                    "InferencingOptimal weights", "batch": B, "m": M, "k": K},
+                cpu_baseline=cpu_baseline, key="c3")
+
+
+def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std):
+    import numpy as np
+    from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
+                                   CooperativeVectorMatrixDesc as D, FeedForwardLayer)
+    dev = "cuda"
+    g = torch.Generator(device=dev); g.manual_seed(20250 + len(dims))
+    wtype = CT.Float16 if wtype_name == "f16" else CT.FloatE4M3
+    layers, host = [], []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        Wf = torch.randn(fo, fi, device=dev, generator=g) * init_std(fi)
+        Wt = Wf.half() if wtype == CT.Float16 else Wf.clamp(-448, 448).to(torch.float8_e4m3fn)
+        esz = Wt.element_size()
+        wrow = Wt.contiguous().view(torch.uint8).flatten()
+        size = cv.getCooperativeVectorMatrixSize(fo, fi, wtype, ML.InferencingOptimal)
+        wopt = torch.empty(size, dtype=torch.uint8, device=dev)
+        cv.convertCooperativeVectorMatrix(wopt, [D(fo, fi, wtype, ML.InferencingOptimal, size, 0, 0)],
+                                          wrow, [D(fo, fi, wtype, ML.RowMajor, fo * fi * esz, 0, fi * esz)])
+        bias = torch.zeros(fo, dtype=torch.float16, device=dev)
+        last = i == len(dims) - 2
+        layers.append(FeedForwardLayer(fi, fo, wopt, bias.view(torch.uint8), ML.InferencingOptimal, 0,
+                                       Activation.NoActivation if last else Activation.ReLU, 0.0))
+        host.append((Wt, bias))
+    x = x_maker(torch, g, B, dims[0], dev)
+    out = torch.empty(B, dims[-1], dtype=torch.float16, device=dev)
+
+    def step():
+        cv.mlpForward(layers, x, weightType=wtype, out=out, flags=flags)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+    in_bytes = dims[0] * x.element_size()
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        if wtype != CT.Float16:
+            # the reference's CPU target cannot compile e4m3 CoopVec (no case in
+            # __coopVecComponentTypeStride, hlsl.meta.slang:32636-32668): time the fp32 oracle instead
+            n = 1 << 14
+            specs = [dict(W=W.view(torch.uint8).cpu().numpy(), b=None, act=1 if i < len(host) - 1 else 0)
+                     for i, (W, _) in enumerate(host)]
+            xs = x[:n].view(torch.uint8).cpu().numpy()
+            t0 = time.perf_counter(); ob.ref_mlp_forward(specs, xs, ob.E4M3); t1 = time.perf_counter()
+            return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                    "sample": "first %d vectors; fp32-accumulate parity oracle (the Slang CPU target has no "
+                              "e4m3 CoopVec, so there is no reference CPU build of this configuration)" % n}
+        L = ob.lib()
+        n = 1 << 13
+        cur = x[:n].cpu().numpy()
+        t0 = time.perf_counter()
+        for i, (W, bias) in enumerate(host):
+            fo, fi = W.shape
+            Wn = W.cpu().numpy(); bn = bias.cpu().numpy()
+            nxt = np.zeros((n, fo), np.float16)
+            rc = L.cvo_slang_dispatch_matmul_add(0, (n + 255) // 256, n, ob.ptr(cur), fi * 2, ob.F16, fi, ob.F16, fi,
+                                                 ob.ptr(nxt), fo * 2, ob.F16, fo, ob.ptr(Wn), 0, ob.F16, ob.ROW, 0,
+                                                 fi * 2, ob.ptr(bn), 0, ob.F16, ob.HALF_SLANG)
+            assert rc == 0
+            cur = np.maximum(nxt, np.float16(0)) if i < len(host) - 1 else nxt
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vectors, one core; C restatement of the Slang CPU-target fallback layer by "
+                          "layer (fp16 accumulate, software half), -O2" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * (in_bytes + dims[-1] * 2), alg_flops=B * 2 * macs,
+                bound="hbm", dtype=wtype_name, kernel="mlpForwardKernel",
+                config={"workload": desc, "batch": B, "layers": dims}, cpu_baseline=cpu_baseline, key=key)
+
+
+def workload_c1(torch, cv, steps, warmup):
+    """fp16 2->16->16->16->1 ReLU MLP, batch 65536 (the CPU-runnable configuration)."""
+    return _mlp_workload(torch, cv, [2, 16, 16, 16, 1], 65536, "f16", 0, "c1",
+                         "c1: fp16 MLP 2->16->16->16->1, ReLU, batch 65536, fused forward",
+                         lambda torch, g, B, k, dev: torch.rand(B, k, device=dev, generator=g).half(),
+                         lambda fi: (1.0 / fi) ** 0.5)
+
+
+def workload_c4(torch, cv, steps, warmup, flags=0):
+    """e4m3 32->64->64->8 decoder MLP, batch 2^24."""
+    return _mlp_workload(torch, cv, [32, 64, 64, 8], 1 << 24, "fp8", flags, "c4" if not flags else "c4n",
+                         "c4: e4m3 MLP 32->64->64->8, ReLU, fp16 out, batch 2^24, fused forward, "
+                         + ("fp8 matrix pipeline" if flags else "e4m3 decoded to the fp16 matrix pipeline"),
+                         lambda torch, g, B, k, dev: (torch.randn(B, k, device=dev, generator=g) * 0.5).to(torch.float8_e4m3fn),
+                         lambda fi: 0.5)
+
+
+def workload_c4n(torch, cv, steps, warmup):
+    return workload_c4(torch, cv, steps, warmup, flags=1)
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n}
 
 
 def main(argv=None) -> int:

@@ -94,6 +94,14 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     typedef typename Mma::Acc Acc;
 
     __shared__ __attribute__((aligned(16))) uint32_t ldsW[MT * KT * 64 * RAW];
+    // Output rows of 128 bytes or more leave through a per-wave LDS transpose so that every
+    // store instruction writes whole 128-byte lines (lane l -> 16 consecutive bytes of the
+    // tile's output block) instead of 16-byte pieces of many lines.  Rows are padded by 16
+    // bytes in LDS, which makes both the scattered writes and the linear reads conflict-free.
+    constexpr int ROW_DW = 4 * OUT_DW;                      // dwords of one sample's output row
+    constexpr bool LDS_STORE = FAST && ROW_DW >= 32;
+    constexpr int STAGE_DW = LDS_STORE ? 16 * (ROW_DW + 4) : 4;
+    __shared__ __attribute__((aligned(16))) uint32_t ldsStage[4 * STAGE_DW];
 
     const uint32_t gs = optGS((uint32_t)a.k);   // k-slots owned by one lane group
 
@@ -220,7 +228,31 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                         for (int r = 0; r < 4; ++r) pk[4 * t + r] = (uint32_t)max(acc[t][r], reluFloorI);
                     }
                 }
-                storeVec<OUT_DW>(o, pk);
+                if constexpr (LDS_STORE) {
+                    uint32_t* st = ldsStage + wave * STAGE_DW;
+                    u32x4* w = (u32x4*)(st + n * (ROW_DW + 4) + g * OUT_DW);
+#pragma unroll
+                    for (int i = 0; i < OUT_DW / 4; ++i) {
+                        const u32x4 v = {pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]};
+                        w[i] = v;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    constexpr int CPR = ROW_DW / 4;            // 16-byte chunks per row (power of two)
+                    uint8_t* tileOut = a.out + (size_t)(t0 * TILE + 16 * j) * a.outStride;
+#pragma unroll
+                    for (int i = 0; i < ROW_DW / 16; ++i) {
+                        const int c = i * 64 + lane, srow = c / CPR, ch = c % CPR;
+                        const u32x4 v = *(const u32x4*)(st + srow * (ROW_DW + 4) + ch * 4);
+                        *(u32x4*)(tileOut + (size_t)srow * a.outStride + ch * 16) = v;
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                } else {
+                    storeVec<OUT_DW>(o, pk);
+                }
             } else {
                 if (sample >= a.batch || validRows <= 0) continue;
 #pragma unroll
