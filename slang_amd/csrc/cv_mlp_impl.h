@@ -60,32 +60,73 @@ struct UniformNet {
     static constexpr int totalBiasTiles = biasBase(L);
 };
 
-// accumulators (one 16-row tile, 4 values per lane) -> the carrier: fp16, activation
-__device__ __forceinline__ void carrierFromAcc(const floatx4& acc, int act, float slope, half_t (&h)[4])
+// Per-layer constants of the carrier conversion.  ReLU is a lower bound on the packed fp16
+// pair (max(z, 0), or max(z, -inf) = z when off); e4m3 networks also clamp to +-448 so that
+// the conversion saturates (the instruction itself yields NaN beyond the finite range).
+struct CarrierCfg {
+    halfx2 floor2, ceil2;
+    int act;
+    float slope;
+};
+
+template <class Mma>
+__device__ __forceinline__ CarrierCfg makeCarrierCfg(int act, float slope)
 {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) h[r] = activateHalf((half_t)acc[r], act, slope);
+    constexpr bool quant = !std::is_same<Mma, F16Mma>::value;
+    const half_t lo = act == kActRelu ? (half_t)0.f : (quant ? (half_t)-448.f : (half_t)-__builtin_inff());
+    CarrierCfg c;
+    c.floor2 = halfx2{lo, lo};
+    c.ceil2 = halfx2{(half_t)448.f, (half_t)448.f};
+    c.act = act; c.slope = slope;
+    return c;
 }
 
-// Two accumulator tiles -> one B fragment of the next layer (8 k-slots per lane).
+// accumulators (one 16-row tile, 4 values per lane) -> the carrier CoopVec<half>: round to
+// fp16 (v_cvt_pk_f16_f32, nearest even), then the activation, on packed pairs
+__device__ __forceinline__ void carrierFromAcc(const floatx4& acc, const CarrierCfg& c, halfx2& h01, halfx2& h23)
+{
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    const floatx2 a01 = {acc[0], acc[1]}, a23 = {acc[2], acc[3]};
+    h01 = __builtin_convertvector(a01, halfx2);
+    h23 = __builtin_convertvector(a23, halfx2);
+    if (c.act == kActLeakyRelu) {      // max(z, z*slope) in half, fflayer.slang:64-65
+        h01 = halfx2{activateHalf(h01.x, kActLeakyRelu, c.slope), activateHalf(h01.y, kActLeakyRelu, c.slope)};
+        h23 = halfx2{activateHalf(h23.x, kActLeakyRelu, c.slope), activateHalf(h23.y, kActLeakyRelu, c.slope)};
+    }
+    h01 = __builtin_elementwise_max(h01, c.floor2);
+    h23 = __builtin_elementwise_max(h23, c.floor2);
+}
+
+// fp16 pair x2 -> one dword of four e4m3 bytes (saturating, nearest even: v_cvt_scalef32_pk_fp8_f16
+// rounds like the fp32 route for every fp16 input within +-448)
+__device__ __forceinline__ uint32_t quantE4M3x4(halfx2 h01, halfx2 h23, const CarrierCfg& c)
+{
+    typedef short shortx2 __attribute__((ext_vector_type(2)));
+    h01 = __builtin_elementwise_min(h01, c.ceil2);
+    h23 = __builtin_elementwise_min(h23, c.ceil2);
+    shortx2 r = {0, 0};
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h01, 1.0f, false);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h23, 1.0f, true);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// Two accumulator tiles (already carriers) -> one B fragment of the next layer (8 k-slots per lane).
 template <class Mma>
-__device__ __forceinline__ void fragFromCarrier(const half_t (&lo)[4], const half_t (&hi)[4], uint32_t* frag)
+__device__ __forceinline__ void fragFromCarrier(halfx2 lo01, halfx2 lo23, halfx2 hi01, halfx2 hi23,
+                                                const CarrierCfg& c, uint32_t* frag)
 {
     if constexpr (std::is_same<Mma, F16Mma>::value) {
-        halfx2 a = {lo[0], lo[1]}, b = {lo[2], lo[3]}, c = {hi[0], hi[1]}, d = {hi[2], hi[3]};
-        frag[0] = __builtin_bit_cast(uint32_t, a); frag[1] = __builtin_bit_cast(uint32_t, b);
-        frag[2] = __builtin_bit_cast(uint32_t, c); frag[3] = __builtin_bit_cast(uint32_t, d);
+        frag[0] = __builtin_bit_cast(uint32_t, lo01); frag[1] = __builtin_bit_cast(uint32_t, lo23);
+        frag[2] = __builtin_bit_cast(uint32_t, hi01); frag[3] = __builtin_bit_cast(uint32_t, hi23);
     } else {
-        // re-quantise the fp16 carrier to OCP e4m3 (saturating, nearest even)
-        const uint32_t q0 = packE4M3Sat((float)lo[0], (float)lo[1]) | (packE4M3Sat((float)lo[2], (float)lo[3]) << 16);
-        const uint32_t q1 = packE4M3Sat((float)hi[0], (float)hi[1]) | (packE4M3Sat((float)hi[2], (float)hi[3]) << 16);
-        const uint32_t raw[2] = {q0, q1};
+        // re-quantise the fp16 carrier to OCP e4m3
+        const uint32_t raw[2] = {quantE4M3x4(lo01, lo23, c), quantE4M3x4(hi01, hi23, c)};
         Mma::decode(raw, frag);      // e4m3 bytes as they are, or decoded back to fp16 operands
     }
 }
 
-template <class Mma, class Net, int NT>
-__global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
+template <class Mma, class Net, int NT, int S>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void mlpForwardKernel(const MlpArgs a)
 {
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     constexpr int L = Net::L;
@@ -162,7 +203,10 @@ __global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
     const int validRows = min(max(outDim - rowBase, 0), OROWS);
     const bool vecStore = validRows == OROWS && a.outAlign >= 8u;
 
-    constexpr uint32_t TILE = 16 * NT;
+    // One wave-iteration covers a super-tile of S tiles (16*S samples): all of its inputs are
+    // loaded at once, a whole iteration ahead (narrow inputs need many samples in flight to keep
+    // HBM busy), and then pushed through the layers NT tiles at a time.
+    constexpr uint32_t TILE = 16 * S;
     const uint32_t numTiles = (a.batch + TILE - 1) / TILE;
     const uint32_t tileStride = gridDim.x * 4;
     uint32_t tile = blockIdx.x * 4 + wave;
@@ -171,9 +215,19 @@ __global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
     uint8_t* outLane = a.out + (size_t)rowBase * 2;
     const uint32_t lastSample = a.batch - 1;
 
-    auto loadTile = [&](uint32_t (&buf)[NT][IN_DW], uint32_t t) {
+    CarrierCfg cc[L];
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        cc[l] = makeCarrierCfg<Mma>(a.layers[l].act, a.layers[l].slope);
+        if constexpr (l + 1 == L) {   // the last layer's output is not re-quantised: plain ReLU floor
+            const half_t lo = a.layers[l].act == kActRelu ? (half_t)0.f : (half_t)-__builtin_inff();
+            cc[l].floor2 = halfx2{lo, lo};
+        }
+    });
+
+    auto loadTile = [&](uint32_t (&buf)[S][IN_DW], uint32_t t) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
+        for (int j = 0; j < S; ++j) {
             const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
             const uint8_t* p = inLane + (size_t)s * a.inStride;
             if (loadMode == 0) {
@@ -206,81 +260,81 @@ __global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
         }
     };
 
-    auto computeStore = [&](const uint32_t (&buf)[NT][IN_DW], uint32_t t0) {
-        uint32_t act[NT][Net::KTMAX][FD];    // B fragments of the current layer's input
+    auto computeStore = [&](const uint32_t (&buf)[S][IN_DW], uint32_t t0) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
+        for (int r0 = 0; r0 < S; r0 += NT) {
+            uint32_t act[NT][Net::KTMAX][FD];    // B fragments of the current layer's input
 #pragma unroll
-            for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&buf[j][kt * RAW], act[j][kt]);
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&buf[r0 + j][kt * RAW], act[j][kt]);
 
-        staticFor<0, L>([&](auto lc) {
-            constexpr int l = decltype(lc)::value;
-            constexpr int MT = Net::mt(l), KT = Net::kt(l);
-            const int actv = a.layers[l].act;
-            const float slope = a.layers[l].slope;
-            floatx4 acc[NT][MT];
+            staticFor<0, L>([&](auto lc) {
+                constexpr int l = decltype(lc)::value;
+                constexpr int MT = Net::mt(l), KT = Net::kt(l);
+                floatx4 acc[NT][MT];
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                const halfx2 b01 = __builtin_bit_cast(halfx2, Bs[l][t][0]);
-                const halfx2 b23 = __builtin_bit_cast(halfx2, Bs[l][t][1]);
-                const floatx4 bv = {(float)b01.x, (float)b01.y, (float)b23.x, (float)b23.y};
+                for (int t = 0; t < MT; ++t) {
+                    const halfx2 b01 = __builtin_bit_cast(halfx2, Bs[l][t][0]);
+                    const halfx2 b23 = __builtin_bit_cast(halfx2, Bs[l][t][1]);
+                    const floatx4 bv = {(float)b01.x, (float)b01.y, (float)b23.x, (float)b23.y};
 #pragma unroll
-                for (int j = 0; j < NT; ++j) acc[j][t] = bv;
-            }
+                    for (int j = 0; j < NT; ++j) acc[j][t] = bv;
+                }
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
+                for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
+                    for (int t = 0; t < MT; ++t)
 #pragma unroll
-                    for (int j = 0; j < NT; ++j) acc[j][t] = Mma::mma(W[l][t][kt], act[j][kt], acc[j][t]);
+                        for (int j = 0; j < NT; ++j) acc[j][t] = Mma::mma(W[l][t][kt], act[j][kt], acc[j][t]);
 
-            if constexpr (l + 1 < L) {
-                // this layer's output becomes the next layer's B operand, in place
-                constexpr int KTN = Net::kt(l + 1);
+                if constexpr (l + 1 < L) {
+                    // this layer's output becomes the next layer's B operand, in place
+                    constexpr int KTN = Net::kt(l + 1);
 #pragma unroll
-                for (int j = 0; j < NT; ++j)
+                    for (int j = 0; j < NT; ++j)
 #pragma unroll
-                    for (int kt = 0; kt < KTN; ++kt) {
-                        half_t lo[4], hi[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-                        carrierFromAcc(acc[j][2 * kt], actv, slope, lo);
-                        if (2 * kt + 1 < MT) carrierFromAcc(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], actv, slope, hi);
-                        fragFromCarrier<Mma>(lo, hi, act[j][kt]);
-                    }
-            } else {
+                        for (int kt = 0; kt < KTN; ++kt) {
+                            halfx2 lo01, lo23, hi01 = {(half_t)0, (half_t)0}, hi23 = {(half_t)0, (half_t)0};
+                            carrierFromAcc(acc[j][2 * kt], cc[l], lo01, lo23);
+                            if (2 * kt + 1 < MT) carrierFromAcc(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], cc[l], hi01, hi23);
+                            fragFromCarrier<Mma>(lo01, lo23, hi01, hi23, cc[l], act[j][kt]);
+                        }
+                } else {
 #pragma unroll
-                for (int j = 0; j < NT; ++j) {
-                    const uint32_t sample = t0 * TILE + 16 * j + n;
-                    if (sample >= a.batch || validRows <= 0) continue;
-                    half_t* o = (half_t*)(outLane + (size_t)sample * a.outStride);
-                    uint32_t pk[2 * MT];
-#pragma unroll
-                    for (int t = 0; t < MT; ++t) {
-                        half_t h[4];
-                        carrierFromAcc(acc[j][t], actv, slope, h);
-                        halfx2 p0 = {h[0], h[1]}, p1 = {h[2], h[3]};
-                        pk[2 * t] = __builtin_bit_cast(uint32_t, p0);
-                        pk[2 * t + 1] = __builtin_bit_cast(uint32_t, p1);
-                    }
-                    if (vecStore) {
+                    for (int j = 0; j < NT; ++j) {
+                        const uint32_t sample = t0 * TILE + 16 * (r0 + j) + n;
+                        if (sample >= a.batch || validRows <= 0) continue;
+                        half_t* o = (half_t*)(outLane + (size_t)sample * a.outStride);
+                        uint32_t pk[2 * MT];
 #pragma unroll
                         for (int t = 0; t < MT; ++t) {
-                            const u32x2 v = {pk[2 * t], pk[2 * t + 1]};
-                            ((u32x2*)o)[t] = v;
+                            halfx2 p0, p1;
+                            carrierFromAcc(acc[j][t], cc[l], p0, p1);
+                            pk[2 * t] = __builtin_bit_cast(uint32_t, p0);
+                            pk[2 * t + 1] = __builtin_bit_cast(uint32_t, p1);
                         }
-                    } else {
+                        if (vecStore) {
 #pragma unroll
-                        for (int e = 0; e < OROWS; ++e)
-                            if (e < validRows) {
-                                const uint16_t bits = (uint16_t)(pk[e / 2] >> (16 * (e & 1)));
-                                o[e] = __builtin_bit_cast(half_t, bits);
+                            for (int t = 0; t < MT; ++t) {
+                                const u32x2 v = {pk[2 * t], pk[2 * t + 1]};
+                                ((u32x2*)o)[t] = v;
                             }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < OROWS; ++e)
+                                if (e < validRows) {
+                                    const uint16_t bits = (uint16_t)(pk[e / 2] >> (16 * (e & 1)));
+                                    o[e] = __builtin_bit_cast(half_t, bits);
+                                }
+                        }
                     }
                 }
-            }
-        });
+            });
+        }
     };
 
-    uint32_t bufA[NT][IN_DW], bufB[NT][IN_DW];
+    uint32_t bufA[S][IN_DW], bufB[S][IN_DW];
     loadTile(bufA, tile);
     while (true) {
         const uint32_t t1 = tile + tileStride;
@@ -295,22 +349,30 @@ __global__ __launch_bounds__(256) void mlpForwardKernel(const MlpArgs a)
     }
 }
 
+#ifndef CV_MLP_PREFETCH_DW
+#define CV_MLP_PREFETCH_DW 16     // input dwords per lane held in flight per buffer
+#endif
+
 template <class Mma, class Net>
 hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
-    constexpr int NT = (Net::totalFrags * Mma::kFD <= 64) ? 4 : 2;
+    // tiles pushed through the layers together (independent MFMA chains), limited by registers
+    constexpr int NT = (Net::totalFrags * Mma::kFD <= 32) ? 4 : 2;
+    constexpr int IN_DW = Mma::kRawDW * Net::KT0;
+    constexpr int S0 = CV_MLP_PREFETCH_DW / IN_DW;
+    constexpr int S = S0 < NT ? NT : (S0 > 16 ? 16 : S0 / NT * NT);
     static int blocksPerCU = 0;
     if (blocksPerCU == 0) {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mlpForwardKernel<Mma, Net, NT>, 256, 0) != hipSuccess || n < 1) n = 1;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mlpForwardKernel<Mma, Net, NT, S>, 256, 0) != hipSuccess || n < 1) n = 1;
         blocksPerCU = n;
     }
-    const uint32_t tile = 16 * NT;
+    const uint32_t tile = 16 * S;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
-    hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT>), dim3(blocks), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
