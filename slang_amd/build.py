@@ -29,7 +29,7 @@ HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul_f16.hip", "cv_matmul_f
 # packed-fp32 instructions are switched off on purpose (see the flag below): hipcc would
 # otherwise form v_pk_*_f32 from ordinary float code.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden",
+    "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-fno-strict-aliasing",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]

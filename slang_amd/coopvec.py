@@ -360,3 +360,38 @@ def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
     _check(_lib.load().cvMlpForward(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride,
                                     out.data_ptr(), outStride, batch))
     return out
+
+
+def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
+                              gradType: int = CoopVecComponentType.Float32) -> int:
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+    out = ctypes.c_size_t(0)
+    _check(_lib.load().cvMlpTrainStepWorkspaceSize(ctypes.byref(d), batch, ctypes.byref(out)))
+    return out.value
+
+
+def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor] = None, *,
+                 lossScale: float = 1.0, gradType: int = CoopVecComponentType.Float32,
+                 workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None, stream=None):
+    """learnGradient over a batch (kernels.slang:9-27): forward, bwd_diff of the squared-error loss,
+    weight gradients accumulated into every layer's weightsGrad (coopVecOuterProductAccumulate,
+    fflayer.slang:35-41) and bias gradients into biasesGrad (coopVecReduceSumAccumulate, :44),
+    deterministically.  Returns (workspace, lossSum) so that both can be reused."""
+    _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+    batch = input.shape[0]
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+    lib = _lib.load()
+    if workspace is None:
+        need = ctypes.c_size_t(0)
+        _check(lib.cvMlpTrainStepWorkspaceSize(ctypes.byref(d), batch, ctypes.byref(need)))
+        workspace = torch.empty(need.value, dtype=torch.uint8, device=input.device)
+    if lossSum is None:
+        lossSum = torch.zeros(1, dtype=torch.float32, device=input.device)
+    tptr, tstride = None, 0
+    if targets is not None:
+        _, tstride = _vector_info(targets, CoopVecComponentType.Float16, "targets")
+        tptr = targets.data_ptr()
+    _check(lib.cvMlpTrainStep(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride, tptr, tstride,
+                              float(lossScale), batch, lossSum.data_ptr(), workspace.data_ptr(),
+                              workspace.numel() * workspace.element_size()))
+    return workspace, lossSum

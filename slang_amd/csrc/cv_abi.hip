@@ -381,16 +381,80 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     return fromHip(e, "cvMlpForward launch");
 }
 
-CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc*, uint32_t, size_t* outBytes)
+CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes)
 {
-    if (outBytes) *outBytes = 0;
-    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpTrainStep: not implemented yet");
+    (void)batch;
+    if (!outBytes) return fail(CV_E_INVALID_ARG, "cvMlpTrainStepWorkspaceSize: outBytes is null");
+    *outBytes = 0;
+    cv::MlpArgs a;
+    memset(&a, 0, sizeof(a));
+    CvResult rc = fillMlpLayers("cvMlpTrainStepWorkspaceSize", mlp, a.layers);
+    if (CV_FAILED(rc)) return rc;
+    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights");
+    a.numLayers = mlp->numLayers;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const size_t n = cv::trainWorkspaceBytes(a, cus);
+    if (!n) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: no fused specialisation for these layer sizes");
+    *outBytes = n;
+    return CV_OK;
 }
 
-CV_API CvResult cvMlpTrainStep(void*, const CvMlpDesc*, const void*, size_t, const void*, size_t, float,
-                               uint32_t, float*, void*, size_t)
+CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
+                               const void* targets, size_t targetStride, float lossScale, uint32_t batch,
+                               float* lossSum, void* workspace, size_t workspaceBytes)
 {
-    return fail(CV_E_NOT_IMPLEMENTED, "cvMlpTrainStep: not implemented yet");
+    cv::TrainLaunch t;
+    memset(&t, 0, sizeof(t));
+    CvResult rc = fillMlpLayers("cvMlpTrainStep", mlp, t.mlp.layers);
+    if (CV_FAILED(rc)) return rc;
+    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights");
+    if (mlp->gradType != CV_FLOAT16 && mlp->gradType != CV_FLOAT32)
+        return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: gradType %d (supported: FLOAT16, FLOAT32)", mlp->gradType);
+    const int L = mlp->numLayers;
+    if (L < 2) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: needs at least two layers");
+    if (batch == 0) return CV_OK;
+    if (!input || !workspace) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: null input/workspace");
+    if ((uintptr_t)input % 2 || inputStride % 2 || (uintptr_t)targets % 2 || targetStride % 2 || (uintptr_t)workspace % 16 ||
+        (uintptr_t)lossSum % 4)
+        return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: misaligned input/targets/workspace/lossSum");
+    if (batch > 1 && (inputStride < (size_t)mlp->layers[0].inputSize * 2 ||
+                      (targets && targetStride < (size_t)mlp->layers[L - 1].outputSize * 2)))
+        return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: vector stride smaller than the vector");
+    const uint32_t gEsz = cv::elemSize(mlp->gradType);
+    for (int l = 0; l < L; ++l) {
+        const CvMlpLayer& ly = mlp->layers[l];
+        if (ly.leakySlope < 0.f || ly.leakySlope >= 1.f)
+            if (ly.activation == CV_ACT_LEAKY_RELU) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: leakySlope must be in [0,1)", l);
+        t.wGrad[l] = (uint8_t*)ly.weightsGrad;
+        t.bGrad[l] = (uint8_t*)ly.biasesGrad;
+        if (ly.weightsGrad) {
+            if (ly.gradLayout < 0 || ly.gradLayout > 3 || !cv::layoutSupports(mlp->gradType, ly.gradLayout))
+                return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: layer %d: component type %d has no layout %d", l, mlp->gradType, ly.gradLayout);
+            t.gradShape[l] = cv::MatrixShape{(uint32_t)ly.outputSize, (uint32_t)ly.inputSize, mlp->gradType, ly.gradLayout,
+                                             isOptimal(ly.gradLayout) ? 0 : (size_t)ly.gradStride};
+            if (cv::matrixSize(t.gradShape[l]) == 0) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: gradStride %u smaller than a row/column", l, ly.gradStride);
+            if ((uintptr_t)ly.weightsGrad % gEsz || ly.gradStride % gEsz) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: weightsGrad misaligned", l);
+        }
+        if ((uintptr_t)ly.biasesGrad % gEsz) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: biasesGrad misaligned", l);
+    }
+    t.mlp.numLayers = L;
+    t.mlp.in = (const uint8_t*)input;
+    t.mlp.inStride = inputStride;
+    t.mlp.batch = batch;
+    t.mlp.inAlign = alignOf(input, inputStride);
+    t.targets = (const uint8_t*)targets;
+    t.targetStride = targetStride;
+    t.lossScale = lossScale;
+    t.gradCt = mlp->gradType;
+    t.lossSum = lossSum;
+    t.workspace = (float*)workspace;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const size_t need = cv::trainWorkspaceBytes(t.mlp, cus);
+    if (!need) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: no fused specialisation for these layer sizes");
+    if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvMlpTrainStep: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+    return fromHip(cv::launchMlpTrain((hipStream_t)stream, t, cus), "cvMlpTrainStep launch");
 }
 
 } // extern "C"

@@ -54,6 +54,25 @@ struct MlpArgs {
 // hipErrorInvalidValue when no built-in specialisation covers the layer shapes
 hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 
+// ---- fused training step ------------------------------------------------------------------
+struct TrainLaunch {
+    MlpArgs mlp;                 // layers, input, batch
+    const uint8_t* targets;      // fp16 [batch][lastOut] or nullptr
+    uint64_t targetStride;
+    float lossScale;
+    // gradient destinations, per layer
+    uint8_t* wGrad[kMaxMlpLayers];
+    uint8_t* bGrad[kMaxMlpLayers];
+    MatrixShape gradShape[kMaxMlpLayers];
+    int32_t gradCt;
+    float* lossSum;
+    float* workspace;            // partials
+};
+// Bytes of workspace the training step needs for this network on a device with numCUs compute
+// units; 0 when no built-in specialisation covers the layer shapes.
+size_t trainWorkspaceBytes(const MlpArgs& shapes, int numCUs);
+hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCUs);
+
 // ---- layout conversion --------------------------------------------------------------------
 struct ConvertItem {
     const uint8_t* src;

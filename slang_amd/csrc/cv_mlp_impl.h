@@ -186,8 +186,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 #pragma unroll
             for (int kt = 0; kt < Net::kt(l); ++kt)
                 Mma::decode(&ldsW[((Net::fragBase(l) + t * Net::kt(l) + kt) * 64 + lane) * RAW], W[l][t][kt]);
-            const u32x2 b = *(const u32x2*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
-            Bs[l][t][0] = b.x; Bs[l][t][1] = b.y;
+            const uint16_t* bp = &ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+            Bs[l][t][0] = (uint32_t)bp[0] | ((uint32_t)bp[1] << 16);
+            Bs[l][t][1] = (uint32_t)bp[2] | ((uint32_t)bp[3] << 16);
         }
     });
 

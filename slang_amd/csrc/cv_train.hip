@@ -1,0 +1,89 @@
+// cv_train.hip -- instantiations and launcher of the fused fp16 training step.
+#include "cv_train_impl.h"
+
+namespace cv {
+
+namespace {
+
+// (input feature tiles, input k-tiles, hidden tiles, hidden layers, output tiles)
+#define CV_TRAIN_SHAPES(X) \
+    X(1, 1, 1, 1, 1) X(1, 1, 1, 2, 1) X(1, 1, 1, 3, 1) \
+    X(1, 1, 2, 2, 1) X(1, 1, 4, 2, 1) X(1, 1, 4, 3, 1) X(1, 1, 4, 4, 1) X(2, 1, 4, 2, 1)
+
+struct Shape { int it0, kt0, ht, nhid, mtl; bool ok; };
+
+Shape classify(const MlpArgs& a)
+{
+    Shape s{0, 0, 0, 0, 0, false};
+    const int L = a.numLayers;
+    if (L < 2) return s;
+    s.it0 = (int)optMT((uint32_t)a.layers[0].in);
+    s.kt0 = (int)optKT((uint32_t)a.layers[0].in, 8);
+    s.ht = (int)optMT((uint32_t)a.layers[0].out);
+    for (int l = 1; l + 1 < L; ++l)
+        if ((int)optMT((uint32_t)a.layers[l].out) != s.ht) return s;
+    s.nhid = L - 1;
+    s.mtl = (int)optMT((uint32_t)a.layers[L - 1].out);
+    s.ok = true;
+    return s;
+}
+
+template <class Net>
+hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
+{
+    TrainArgs ta;
+    ta.mlp = t.mlp;
+    ta.targets = t.targets;
+    ta.targetStride = t.targetStride;
+    ta.lossScale = t.lossScale;
+    ta.partials = t.workspace;
+    const uint32_t blocks = (uint32_t)numCUs;      // one resident workgroup per compute unit
+    hipLaunchKernelGGL((mlpTrainKernel<Net>), dim3(blocks), dim3(256), 0, stream, ta);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    TrainReduceArgs ra;
+    for (int l = 0; l < Net::L; ++l) {
+        ra.layers[l].wGrad = t.wGrad[l];
+        ra.layers[l].bGrad = t.bGrad[l];
+        ra.layers[l].gradShape = t.gradShape[l];
+        ra.layers[l].in = t.mlp.layers[l].in;
+        ra.layers[l].out = t.mlp.layers[l].out;
+    }
+    ra.numLayers = Net::L;
+    ra.gradCt = t.gradCt;
+    ra.partials = t.workspace;
+    ra.numPartials = blocks;
+    ra.lossSum = t.lossSum;
+    constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
+    hipLaunchKernelGGL((mlpTrainReduceKernel<Net>), dim3((total + 255) / 256), dim3(256), 0, stream, ra);
+    return hipGetLastError();
+}
+
+} // namespace
+
+size_t trainWorkspaceBytes(const MlpArgs& a, int numCUs)
+{
+    const Shape s = classify(a);
+    if (!s.ok) return 0;
+#define CV_X(I0, K0, HT, NH, ML) \
+    if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \
+        return (size_t)numCUs * TrainNet<I0, K0, HT, NH, ML>::partialFloats * sizeof(float);
+    CV_TRAIN_SHAPES(CV_X)
+#undef CV_X
+    return 0;
+}
+
+hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& t, int numCUs)
+{
+    if (t.mlp.batch == 0) return hipSuccess;
+    const Shape s = classify(t.mlp);
+    if (!s.ok) return hipErrorInvalidValue;
+#define CV_X(I0, K0, HT, NH, ML) \
+    if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \
+        return launchNet<TrainNet<I0, K0, HT, NH, ML>>(stream, t, numCUs);
+    CV_TRAIN_SHAPES(CV_X)
+#undef CV_X
+    return hipErrorInvalidValue;
+}
+
+} // namespace cv

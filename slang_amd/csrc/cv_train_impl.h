@@ -1,0 +1,521 @@
+// cv_train_impl.h -- fused forward + backward of the fp16 MLP for gfx950.
+//
+// Replaces what the example's learnGradient kernel does per shader thread
+// (examples/mlp-training-coopvec/kernels.slang:9-27 -> bwd_diff(loss), fflayer.slang:29-58:
+// coopVecOuterProductAccumulate + coopVecReduceSumAccumulate + coopVecMatMul with the transposed
+// weights; the per-thread atomics of those operators are documented at
+// source/slang/hlsl.meta.slang:33200-33224, 33318-33326) by a batch formulation:
+//
+//   - forward and dX = W^T dY run like the fused forward kernel: 16 samples are the N dimension
+//     of an MFMA, the carrier CoopVec<half> stays in VGPRs between layers ("S" orientation:
+//     lane%16 = sample, features over lane groups and registers);
+//   - the weight gradient dW = sum_s dY_s (x) X_s is an MFMA contraction over the batch.  It
+//     needs both operands with the sample index on the k axis ("F" orientation: lane%16 =
+//     feature).  An S fragment is turned into F fragments exactly, by an MFMA against a 0/1
+//     selection matrix (values are copied, not rounded);
+//   - every wave accumulates its share of dW / db in fp32 registers over all of its samples;
+//     at the end the four waves of a workgroup are summed in LDS in a fixed order and written
+//     as one partial per workgroup; a second kernel sums the partials in a fixed order and
+//     adds them to the gradient buffers ("+=", any layout, fp16 or fp32).  No atomics: the
+//     result is bitwise reproducible.
+//
+// Derivative rules follow Slang: max(x,y) sends the whole gradient to the larger operand and
+// half to each at a tie (source/slang/diff.meta.slang:2258-2277).
+#pragma once
+#include <type_traits>
+
+#include "cv_mlp_impl.h"
+
+namespace cv {
+namespace {
+
+// tile bookkeeping on top of UniformNet; IT0 = 16-feature tiles of the network input
+template <int IT0_, int KT0_, int HT_, int NHID_, int MTL_>
+struct TrainNet : UniformNet<KT0_, HT_, NHID_, MTL_> {
+    typedef UniformNet<KT0_, HT_, NHID_, MTL_> Base;
+    static constexpr int IT0 = IT0_;
+    static constexpr int L = Base::L;
+    static constexpr int nOt(int l) { return Base::mt(l); }
+    static constexpr int nIt(int l) { return l == 0 ? IT0_ : Base::mt(l - 1); }
+    static constexpr int ktOut(int l) { return (Base::mt(l) + 1) / 2; }   // S fragments of layer l's output
+    static constexpr int ITMAX = IT0_ > HT_ ? IT0_ : HT_;
+    static constexpr int KOMAX = (Base::MTMAX + 1) / 2;
+    // transposed weights (A operand of dX = W^T dY) exist for layers 1..L-1
+    static constexpr int tFragBase(int l)
+    {
+        int b = 0;
+        for (int i = 1; i < l; ++i) b += Base::mt(i - 1) * ktOut(i);
+        return b;
+    }
+    static constexpr int totalTFrags = tFragBase(L);
+    static constexpr int gradTileBase(int l)
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += nOt(i) * nIt(i);
+        return b;
+    }
+    static constexpr int totalGradTiles = gradTileBase(L);
+    static constexpr int dbTileBase(int l) { return Base::biasBase(l); }
+    static constexpr int totalDbTiles = Base::totalBiasTiles;
+    // floats of one workgroup's partial: dW tiles, db tiles, loss
+    static constexpr int partialFloats = totalGradTiles * 256 + totalDbTiles * 16 + 16;
+};
+
+struct TrainArgs {
+    MlpArgs mlp;                 // layers, input, batch (out/outStride unused)
+    const uint8_t* targets;      // fp16 [batch][lastOut] or nullptr: sin(sum of the inputs)
+    uint64_t targetStride;
+    float lossScale;
+    float* partials;             // [gridDim.x][partialFloats]
+};
+
+struct TrainReduceArgs {
+    struct Layer {
+        uint8_t* wGrad; uint8_t* bGrad;
+        MatrixShape gradShape;   // out x in as the gradient lies in memory
+        int32_t in, out;
+    } layers[kMaxMlpLayers];
+    int32_t numLayers;
+    int32_t gradCt;              // kF16 or kF32, also the type of the bias gradients
+    const float* partials;
+    uint32_t numPartials;
+    float* lossSum;              // optional
+};
+
+// 3-state outcome of max(z, zs) per element, 2 bits: 1 = first operand larger, 2 = second, 0 = tie
+__device__ __forceinline__ uint32_t maxState(half_t z, half_t zs) { return z > zs ? 1u : (z < zs ? 2u : 0u); }
+
+// dz = g * act'(z) in half, from the saved state (see cvo_ref_mlp_train for the scalar statement)
+__device__ __forceinline__ half_t applyActGrad(half_t gv, uint32_t state, int act, float slope)
+{
+    if (act == kActNone) return gv;
+    const half_t halfG = (half_t)(0.5f * (float)gv);
+    const half_t da = state == 1u ? gv : (state == 0u ? halfG : (half_t)0);
+    if (act == kActRelu) return da;            // second operand is the constant 0
+    const half_t db = state == 2u ? gv : (state == 0u ? halfG : (half_t)0);
+    const half_t dbs = (half_t)((float)db * slope);
+    return (half_t)((float)da + (float)dbs);
+}
+
+template <class Net>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlpTrainKernel(const TrainArgs ta)
+{
+    typedef F16Mma Mma;
+    constexpr int L = Net::L;
+    constexpr int FD = 4, RAW = 4, EPL = 8;
+    constexpr int IN_DW = RAW * Net::KT0;
+    const MlpArgs& a = ta.mlp;
+
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[Net::totalFrags * 64 * RAW];
+    __shared__ __attribute__((aligned(16))) uint32_t ldsWT[(Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW];
+    __shared__ __attribute__((aligned(16))) float ldsB[Net::totalBiasTiles * 16];   // biases as fp32
+    __shared__ __attribute__((aligned(16))) float ldsRed[4 * 256];
+
+    // ---- stage W (A operand of the forward pass), W^T (A operand of dX) and biases ----------
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
+        const MlpLayerArgs& ly = a.layers[l];
+        const uint32_t gs = optGS((uint32_t)ly.in);
+        uint16_t* dst = (uint16_t*)(ldsW + Net::fragBase(l) * 64 * RAW);
+        for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
+            const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
+            const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
+            const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
+            const uint32_t q = (uint32_t)(kt * EPL + s), col = g * gs + q;
+            const bool valid = row < (uint32_t)ly.out && q < gs && col < (uint32_t)ly.in;
+            dst[e] = valid ? *(const uint16_t*)(ly.w + elemOffset(ly.shape, row, col)) : (uint16_t)0;
+        }
+        if constexpr (l > 0) {
+            // rows of W^T are this layer's inputs (tiled like the previous layer's outputs),
+            // its k axis are this layer's outputs
+            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l), ROWSI = 4 * MTI;
+            const uint32_t gso = 4u * MT;
+            uint16_t* dt = (uint16_t*)(ldsWT + Net::tFragBase(l) * 64 * RAW);
+            for (int e = threadIdx.x; e < MTI * KTO * 64 * EPL; e += 256) {
+                const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
+                const int kt = f % KTO, t = f / KTO, g = lane >> 4, p = lane & 15;
+                const uint32_t irow = (uint32_t)((p >> 2) * ROWSI + 4 * t + (p & 3));
+                const uint32_t q = (uint32_t)(kt * EPL + s), ocol = g * gso + q;
+                const bool valid = irow < (uint32_t)ly.in && q < gso && ocol < (uint32_t)ly.out;
+                dt[e] = valid ? *(const uint16_t*)(ly.w + elemOffset(ly.shape, ocol, irow)) : (uint16_t)0;
+            }
+        }
+        for (int e = threadIdx.x; e < MT * 16; e += 256) {
+            const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
+            const int row = g * ROWS + 4 * t + r;
+            float v = 0.f;
+            if (ly.bias && row < ly.out) v = (float)((const half_t*)ly.bias)[row];
+            ldsB[(Net::biasBase(l) + t) * 16 + 4 * g + r] = v;
+        }
+    });
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, n = lane & 15;
+
+    // 0/1 selection fragments: column q of half h picks k-slot (group q/4, slot 4h + q%4)
+    uint32_t Isel[2][FD];
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int d = 0; d < FD; ++d) {
+            const int s0 = 4 * h + (lane & 3);            // the slot this lane may own
+            const bool mine = g == (n >> 2);
+            const uint32_t lo = (mine && s0 == 2 * d) ? 0x3C00u : 0u;
+            const uint32_t hi = (mine && s0 == 2 * d + 1) ? 0x3C00u : 0u;
+            Isel[h][d] = lo | (hi << 16);
+        }
+    const halfx2 ones2 = {(half_t)1.f, (half_t)1.f};
+
+    // gradient accumulators of this wave
+    floatx4 accW[Net::totalGradTiles];
+    float accB[Net::totalDbTiles];
+#pragma unroll
+    for (int i = 0; i < Net::totalGradTiles; ++i) accW[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < Net::totalDbTiles; ++i) accB[i] = 0.f;
+    float lossAcc = 0.f;
+
+    // ---- per-lane constants ----------------------------------------------------------------
+    const int in0 = a.layers[0].in;
+    const uint32_t gs0 = optGS((uint32_t)in0);
+    const int colBase = (int)(g * gs0);
+    const int validBytes = min((int)gs0, max(in0 - colBase, 0)) * 2;
+    const bool vecLoad = validBytes == IN_DW * 4 && a.inAlign >= 16u;
+    const int outDim = a.layers[L - 1].out;
+    constexpr int OROWS = 4 * Net::MTL;
+
+    constexpr uint32_t TILE = 32;                 // two 16-sample tiles = one k-tile of dW
+    const uint32_t numTiles = (a.batch + TILE - 1) / TILE;
+    const uint32_t tileStride = gridDim.x * 4;
+    const uint8_t* inLane = a.in + (size_t)colBase * 2;
+    const uint32_t lastSample = a.batch - 1;
+
+    auto loadTile = [&](uint32_t (&buf)[2][IN_DW], uint32_t t) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
+            const uint8_t* p = inLane + (size_t)s * a.inStride;
+            if (vecLoad) {
+#pragma unroll
+                for (int i = 0; i < IN_DW / 4; ++i) {
+                    const u32x4 v = *(const u32x4*)(p + 16 * i);
+                    buf[j][4 * i] = v.x; buf[j][4 * i + 1] = v.y; buf[j][4 * i + 2] = v.z; buf[j][4 * i + 3] = v.w;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) {
+                    uint32_t v = 0;
+                    if (4 * i < validBytes) v = *(const uint16_t*)(p + 4 * i);
+                    if (4 * i + 2 < validBytes) v |= (uint32_t)*(const uint16_t*)(p + 4 * i + 2) << 16;
+                    buf[j][i] = v;
+                }
+            }
+        }
+    };
+
+    // S fragment pair (tiles j = 0,1) -> F fragment of feature tile e = 2*kt + h
+    auto toF = [&](const uint32_t* s0, const uint32_t* s1, int h, uint32_t* frag) {
+        typedef float floatx2 __attribute__((ext_vector_type(2)));
+        const floatx4 z = {0.f, 0.f, 0.f, 0.f};
+        const floatx4 t0 = Mma::mma(s0, Isel[h], z), t1 = Mma::mma(s1, Isel[h], z);
+        frag[0] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{t0[0], t0[1]}, halfx2));
+        frag[1] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{t0[2], t0[3]}, halfx2));
+        frag[2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{t1[0], t1[1]}, halfx2));
+        frag[3] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{t1[2], t1[3]}, halfx2));
+    };
+
+    auto round = [&](const uint32_t (&buf)[2][IN_DW], uint32_t t0) {
+        uint32_t actS[2][Net::KTMAX][FD];           // S fragments of the current layer's input
+        uint32_t xF[L][Net::ITMAX][FD];             // F fragments of every layer's input
+        uint32_t state[L][2];                       // max() outcomes: 2 bits per element, 8 bits per out tile
+        static_assert(Net::MTMAX <= 4, "state packing holds four 16-row tiles");
+        halfx2 yS[2][Net::MTL][2];                  // network output (carrier), tile j, out tile t
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int kt = 0; kt < Net::KT0; ++kt)
+#pragma unroll
+                for (int d = 0; d < FD; ++d) actS[j][kt][d] = buf[j][kt * RAW + d];
+
+        // ---------------- forward ----------------
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int MT = Net::mt(l), KT = Net::kt(l);
+            const int actv = a.layers[l].act;
+            const float slope = a.layers[l].slope;
+            // this layer's input in F orientation, for dW
+#pragma unroll
+            for (int e = 0; e < Net::nIt(l); ++e) toF(actS[0][e / 2], actS[1][e / 2], e & 1, xF[l][e]);
+
+            floatx4 acc[2][MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                const float* bp = &ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+                const floatx4 bv = {bp[0], bp[1], bp[2], bp[3]};
+                acc[0][t] = bv; acc[1][t] = bv;
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const u32x4 wv = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
+                    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+                    acc[0][t] = Mma::mma(w, actS[0][kt], acc[0][t]);
+                    acc[1][t] = Mma::mma(w, actS[1][kt], acc[1][t]);
+                }
+            // carrier: round to fp16, remember the outcome of max(), apply the activation
+            halfx2 car[2][MT][2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    typedef float floatx2 __attribute__((ext_vector_type(2)));
+                    halfx2 z01 = __builtin_convertvector(floatx2{acc[j][t][0], acc[j][t][1]}, halfx2);
+                    halfx2 z23 = __builtin_convertvector(floatx2{acc[j][t][2], acc[j][t][3]}, halfx2);
+                    uint32_t st = 0;
+                    if (actv != kActNone) {
+                        half_t zz[4] = {z01.x, z01.y, z23.x, z23.y};
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const half_t zs = actv == kActRelu ? (half_t)0 : (half_t)((float)zz[r] * slope);
+                            st |= maxState(zz[r], zs) << (2 * r);
+                            zz[r] = zz[r] >= zs ? zz[r] : zs;
+                        }
+                        z01 = halfx2{zz[0], zz[1]}; z23 = halfx2{zz[2], zz[3]};
+                    }
+                    if (t == 0) state[l][j] = st; else state[l][j] |= st << (8 * t);
+                    car[j][t][0] = z01; car[j][t][1] = z23;
+                }
+            if constexpr (l + 1 < L) {
+                constexpr int KTN = Net::kt(l + 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int kt = 0; kt < KTN; ++kt) {
+                        actS[j][kt][0] = __builtin_bit_cast(uint32_t, car[j][2 * kt][0]);
+                        actS[j][kt][1] = __builtin_bit_cast(uint32_t, car[j][2 * kt][1]);
+                        actS[j][kt][2] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, car[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0][0]) : 0u;
+                        actS[j][kt][3] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, car[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0][1]) : 0u;
+                    }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t) { yS[j][t][0] = car[j][t][0]; yS[j][t][1] = car[j][t][1]; }
+            }
+        });
+
+        // ---------------- loss and its gradient (S orientation) ----------------
+        uint32_t bS[2][Net::KOMAX][FD];             // S fragments of dY of the current layer
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t sample = t0 * TILE + 16 * j + n;
+            const bool live = sample < a.batch;
+            float tgtAll = 0.f;
+            if (!ta.targets) {
+                // target = sin(sum of the sample's inputs): every lane group holds a quarter of them
+                float part = 0.f;
+#pragma unroll
+                for (int d = 0; d < IN_DW; ++d) {
+                    const halfx2 v = __builtin_bit_cast(halfx2, buf[j][d]);
+                    part += (float)v.x; part += (float)v.y;
+                }
+                part += __shfl_xor(part, 16);
+                part += __shfl_xor(part, 32);
+                tgtAll = (float)(half_t)sinf(part);
+            }
+            half_t dz[Net::MTL][4];
+#pragma unroll
+            for (int t = 0; t < Net::MTL; ++t) {
+                const half_t yv[4] = {yS[j][t][0].x, yS[j][t][0].y, yS[j][t][1].x, yS[j][t][1].y};
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = g * OROWS + 4 * t + r;
+                    half_t gv = (half_t)0;
+                    if (live && row < outDim) {
+                        const float tv = ta.targets
+                            ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row) : tgtAll;
+                        const half_t diff = (half_t)((float)yv[r] - tv);
+                        lossAcc += (float)diff * (float)diff;
+                        gv = (half_t)(2.0f * (float)diff * ta.lossScale);
+                    }
+                    dz[t][r] = applyActGrad(gv, (state[L - 1][j] >> (8 * t + 2 * r)) & 3u, a.layers[L - 1].act, a.layers[L - 1].slope);
+                }
+            }
+#pragma unroll
+            for (int kt = 0; kt < Net::ktOut(L - 1); ++kt) {
+                const halfx2 p0 = {dz[2 * kt][0], dz[2 * kt][1]}, p1 = {dz[2 * kt][2], dz[2 * kt][3]};
+                bS[j][kt][0] = __builtin_bit_cast(uint32_t, p0);
+                bS[j][kt][1] = __builtin_bit_cast(uint32_t, p1);
+                if (2 * kt + 1 < Net::MTL) {
+                    const int tt = 2 * kt + 1 < Net::MTL ? 2 * kt + 1 : 0;
+                    const halfx2 q0 = {dz[tt][0], dz[tt][1]}, q1 = {dz[tt][2], dz[tt][3]};
+                    bS[j][kt][2] = __builtin_bit_cast(uint32_t, q0);
+                    bS[j][kt][3] = __builtin_bit_cast(uint32_t, q1);
+                } else {
+                    bS[j][kt][2] = 0u; bS[j][kt][3] = 0u;
+                }
+            }
+        }
+
+        // ---------------- backward ----------------
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = L - 1 - decltype(lc)::value;
+            constexpr int MT = Net::mt(l);
+            // dY in F orientation; bias gradient; weight gradient
+#pragma unroll
+            for (int eo = 0; eo < MT; ++eo) {
+                uint32_t dzF[FD];
+                toF(bS[0][eo / 2], bS[1][eo / 2], eo & 1, dzF);
+                float s = accB[Net::dbTileBase(l) + eo];
+#pragma unroll
+                for (int d = 0; d < FD; ++d) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, dzF[d]), ones2, s, false);
+                accB[Net::dbTileBase(l) + eo] = s;
+#pragma unroll
+                for (int ei = 0; ei < Net::nIt(l); ++ei) {
+                    floatx4& w = accW[Net::gradTileBase(l) + eo * Net::nIt(l) + ei];
+                    w = Mma::mma(dzF, xF[l][ei], w);
+                }
+            }
+            if constexpr (l > 0) {
+                // dX = W^T dY, then through the previous layer's activation
+                constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
+                const int actp = a.layers[l - 1].act;
+                const float slopep = a.layers[l - 1].slope;
+                floatx4 gacc[2][MTI];
+#pragma unroll
+                for (int t = 0; t < MTI; ++t) { gacc[0][t] = floatx4{0.f, 0.f, 0.f, 0.f}; gacc[1][t] = gacc[0][t]; }
+#pragma unroll
+                for (int kt = 0; kt < KTO; ++kt)
+#pragma unroll
+                    for (int t = 0; t < MTI; ++t) {
+                        const u32x4 wv = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
+                        const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+                        gacc[0][t] = Mma::mma(w, bS[0][kt], gacc[0][t]);
+                        gacc[1][t] = Mma::mma(w, bS[1][kt], gacc[1][t]);
+                    }
+                constexpr int KTP = Net::ktOut(l - 1);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    half_t dz[MTI][4];
+#pragma unroll
+                    for (int t = 0; t < MTI; ++t)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            dz[t][r] = applyActGrad((half_t)gacc[j][t][r], (state[l - 1][j] >> (8 * t + 2 * r)) & 3u, actp, slopep);
+#pragma unroll
+                    for (int kt = 0; kt < KTP; ++kt) {
+                        const halfx2 p0 = {dz[2 * kt][0], dz[2 * kt][1]}, p1 = {dz[2 * kt][2], dz[2 * kt][3]};
+                        bS[j][kt][0] = __builtin_bit_cast(uint32_t, p0);
+                        bS[j][kt][1] = __builtin_bit_cast(uint32_t, p1);
+                        if (2 * kt + 1 < MTI) {
+                            const int tt = 2 * kt + 1 < MTI ? 2 * kt + 1 : 0;
+                            const halfx2 q0 = {dz[tt][0], dz[tt][1]}, q1 = {dz[tt][2], dz[tt][3]};
+                            bS[j][kt][2] = __builtin_bit_cast(uint32_t, q0);
+                            bS[j][kt][3] = __builtin_bit_cast(uint32_t, q1);
+                        } else {
+                            bS[j][kt][2] = 0u; bS[j][kt][3] = 0u;
+                        }
+                    }
+                }
+            }
+        });
+    };
+
+    // ---- main loop: every wave strides over rounds of 32 samples -----------------------------
+    {
+        uint32_t tile = blockIdx.x * 4 + wave;
+        if (tile < numTiles) {
+            uint32_t bufA[2][IN_DW], bufB[2][IN_DW];
+            loadTile(bufA, tile);
+            while (true) {
+                const uint32_t t1 = tile + tileStride;
+                loadTile(bufB, t1 < numTiles ? t1 : tile);
+                round(bufA, tile);
+                if (t1 >= numTiles) break;
+                const uint32_t t2 = t1 + tileStride;
+                loadTile(bufA, t2 < numTiles ? t2 : t1);
+                round(bufB, t1);
+                if (t2 >= numTiles) break;
+                tile = t2;
+            }
+        }
+    }
+
+    // ---- workgroup partial: sum the four waves in a fixed order, one tile at a time ----------
+    float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
+#pragma unroll
+    for (int i = 0; i < Net::totalGradTiles; ++i) {
+        *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[i];
+        __syncthreads();
+        const float s = ((ldsRed[threadIdx.x] + ldsRed[256 + threadIdx.x]) + ldsRed[512 + threadIdx.x]) + ldsRed[768 + threadIdx.x];
+        part[i * 256 + threadIdx.x] = s;
+        __syncthreads();
+    }
+    // bias gradients: lane (g,q) holds the sum over its samples; sum the 4 lane groups and 4 waves
+#pragma unroll
+    for (int i = 0; i < Net::totalDbTiles; ++i) {
+        ldsRed[wave * 64 + lane] = accB[i];
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            float s = 0.f;
+            for (int w = 0; w < 4; ++w)
+                for (int gg = 0; gg < 4; ++gg) s += ldsRed[w * 64 + gg * 16 + threadIdx.x];
+            part[Net::totalGradTiles * 256 + i * 16 + threadIdx.x] = s;
+        }
+        __syncthreads();
+    }
+    ldsRed[threadIdx.x] = lossAcc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int i = 0; i < 256; ++i) s += ldsRed[i];
+        part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+    }
+}
+
+// Sums the workgroup partials in a fixed order and adds them to the gradient buffers.
+template <class Net>
+__global__ __launch_bounds__(256) void mlpTrainReduceKernel(const TrainReduceArgs ra)
+{
+    constexpr int L = Net::L;
+    const uint32_t p = blockIdx.x * 256u + threadIdx.x;
+    constexpr uint32_t nW = Net::totalGradTiles * 256, nB = Net::totalDbTiles * 16;
+    if (p >= nW + nB + 1) return;
+    float s = 0.f;
+    for (uint32_t b = 0; b < ra.numPartials; ++b) s += ra.partials[(size_t)b * Net::partialFloats + p];
+    if (p == nW + nB) {
+        if (ra.lossSum) *ra.lossSum = s;
+        return;
+    }
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
+        constexpr uint32_t w0 = Net::gradTileBase(l) * 256, w1 = w0 + MTO * NI * 256;
+        constexpr uint32_t b0 = nW + Net::dbTileBase(l) * 16, b1 = b0 + MTO * 16;
+        const TrainReduceArgs::Layer& ly = ra.layers[l];
+        if (p >= w0 && p < w1) {
+            const uint32_t q = p - w0, tile = q >> 8, ln = (q >> 2) & 63u, r = q & 3u;
+            const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
+            const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
+            const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
+            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) {
+                uint8_t* d = ly.wGrad + elemOffset(ly.gradShape, o, i);
+                if (ra.gradCt == kF32) *(float*)d += s;
+                else *(half_t*)d = (half_t)((float)*(half_t*)d + s);
+            }
+        } else if (p >= b0 && p < b1) {
+            const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
+            const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
+            if (ly.bGrad && o < (uint32_t)ly.out) {
+                if (ra.gradCt == kF32) ((float*)ly.bGrad)[o] += s;
+                else ((half_t*)ly.bGrad)[o] = (half_t)((float)((half_t*)ly.bGrad)[o] + s);
+            }
+        }
+    });
+}
+
+} // namespace
+} // namespace cv

@@ -1,0 +1,190 @@
+"""GPU parity of the fused training step against the fp64-accumulating CPU oracle, through the C-ABI.
+
+Bar (fp16 carrier, fp32 accumulation of the gradients on the GPU, fp64 in the oracle): per layer
+||dW_gpu - dW_ref||_F <= 1e-3 * ||dW_ref||_F (same for db), plus bitwise run-to-run determinism.
+With explicit targets every rounding point of the oracle is reproduced; the residual differences
+are hidden units whose fp32 sum fell within one rounding of an fp16 boundary."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_binding as ob
+from gpu_util import DEV, as_bytes, matrix_in_layout, to_dev
+from slang_amd import coopvec as cv
+from slang_amd.coopvec import Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML, FeedForwardLayer
+
+pytestmark = pytest.mark.gpu
+G = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "coopvec_goldens.json")))
+
+
+def build(specs, grad_ct=CT.Float32, grad_layout=ML.RowMajor, preset=None):
+    layers = []
+    gdt = torch.float32 if grad_ct == CT.Float32 else torch.float16
+    for li, s in enumerate(specs):
+        out, fan_in = s["W"].shape
+        size = cv.getCooperativeVectorMatrixSize(out, fan_in, grad_ct, grad_layout)
+        wg = torch.zeros(size, dtype=torch.uint8, device=DEV)
+        bg = torch.zeros(out, dtype=gdt, device=DEV)
+        if preset is not None:
+            bg += preset
+        layers.append(FeedForwardLayer(fan_in, out, as_bytes(to_dev(s["W"])),
+                                       as_bytes(to_dev(s["b"])) if s["b"] is not None else None,
+                                       ML.RowMajor, fan_in * 2, s["act"], s.get("slope", 0.0),
+                                       wg, bg.view(torch.uint8), grad_layout, 0))
+    return layers
+
+
+def read_grads(layers, specs, grad_ct, grad_layout):
+    dW, dB = [], []
+    npdt = np.float32 if grad_ct == CT.Float32 else np.float16
+    for L, s in zip(layers, specs):
+        out, fan_in = s["W"].shape
+        raw = L.weightsGrad.cpu().numpy()
+        back = np.zeros((out, fan_in), npdt)
+        rc = ob.lib().cvo_layout_convert(ob.ptr(back), out, fan_in, int(grad_ct), ob.ROW, 0, ob.ptr(raw), int(grad_ct),
+                                         int(grad_layout), 0)
+        assert rc == 0
+        dW.append(back.astype(np.float64))
+        dB.append(L.biasesGrad.cpu().numpy().view(npdt).astype(np.float64))
+    return dW, dB
+
+
+def rel_err(a, b):
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30)
+
+
+def make_specs(rng, dims, act=Activation.ReLU, slope=0.0, bias=True):
+    specs = []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = (rng.standard_normal((fo, fi)) * np.sqrt(2.0 / fi)).astype(np.float16)
+        b = rng.uniform(-0.1, 0.1, fo).astype(np.float16) if bias else None
+        last = i == len(dims) - 2
+        specs.append(dict(W=W, b=b, act=int(Activation.NoActivation if last else act), slope=slope))
+    return specs
+
+
+def test_ffn_closed_form_backward():
+    # tests/neural/basic-ilayer-ffn-backward-test.slang: dW1=[-3,4,6,-8], db1=[-2,4], dW2=[6,-7.25], db2=1
+    f, bwd = G["ffn_forward"], G["ffn_backward"]
+    specs = [dict(W=np.array(f["W1"], np.float16), b=np.array(f["b1"], np.float16), act=0),
+             dict(W=np.array(f["W2"], np.float16), b=np.array(f["b2"], np.float16), act=0)]
+    layers = build(specs)
+    x = to_dev(np.array([f["x"]], np.float16))
+    t = to_dev(np.array([[-41.0]], np.float16))          # seed 2*(y - t) = 1 with y = -40.5
+    _, loss = cv.mlpTrainStep(layers, x, t)
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    assert dW[0].tolist() == bwd["dW1"] and dB[0].tolist() == bwd["db1"]
+    assert dW[1].tolist() == bwd["dW2"] and dB[1].tolist() == bwd["db2"]
+    assert loss.item() == 0.25
+
+
+@pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 4096 + 21), ([4, 16, 4], 1000), ([2, 16, 16, 16, 1], 2048),
+                                    ([8, 32, 32, 4], 777), ([20, 64, 64, 8], 1500), ([8, 64, 64, 64, 5], 900)])
+def test_train_step_against_oracle(dims, B):
+    rng = np.random.default_rng(sum(dims) + B)
+    specs = make_specs(rng, dims)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = np.sin(x.astype(np.float32).sum(1, keepdims=True)).astype(np.float16).repeat(dims[-1], 1)
+    t = np.ascontiguousarray(t)
+    layers = build(specs)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l], rB[l]) <= 1e-3, (l, rel_err(dB[l], rB[l]))
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # bitwise determinism, and "+=" semantics: a second step doubles the (fp32) gradients exactly
+    before = [L.weightsGrad.clone() for L in layers]
+    layers2 = build(specs)
+    cv.mlpTrainStep(layers2, to_dev(x), to_dev(t))
+    for a, b in zip(before, layers2):
+        assert torch.equal(a, b.weightsGrad)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    for a, L in zip(before, layers):
+        assert torch.equal(a.view(torch.float32) * 2, L.weightsGrad.view(torch.float32))
+
+
+def test_train_step_sin_target_in_kernel():
+    # the training configuration: 8 -> 64 x4 -> 1, ReLU, He init, inputs U[-1,1]^8, target sin(sum x)
+    rng = np.random.default_rng(5)
+    dims = [8, 64, 64, 64, 64, 1]
+    B = 8192
+    specs = make_specs(rng, dims, bias=False)
+    x = rng.uniform(-1, 1, (B, 8)).astype(np.float16)
+    layers = build(specs, grad_layout=ML.TrainingOptimal)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), None)
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.TrainingOptimal)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, None, 1.0, tie_rule=True)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l], rB[l]) <= 1e-3
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+
+
+def test_train_tie_rule_and_leaky_relu():
+    # a hidden unit at exactly z = 0 gets half of the gradient (diff.meta.slang:2258-2277)
+    specs = [dict(W=np.array([[1.0], [0.5]] + [[0.0]] * 14, np.float16), b=np.array([-1.0, 0.25] + [0.0] * 14, np.float16), act=1),
+             dict(W=np.array([[2.0, 1.0] + [0.0] * 14], np.float16), b=None, act=0)]
+    layers = build(specs)
+    x = to_dev(np.array([[1.0]], np.float16))            # z = [0, 0.75, 0...]: y = 0.75
+    t = to_dev(np.array([[0.25]], np.float16))           # dL/dy = 1
+    cv.mlpTrainStep(layers, x, t)
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, _ = ob.ref_mlp_train(specs, np.array([[1.0]], np.float16), np.array([[0.25]], np.float16), 1.0, True)
+    assert dB[0].tolist() == rB[0].tolist() and dB[0][0] == 1.0 and dB[0][1] == 1.0   # 0.5*2 and 1*1
+    assert dW[0].tolist() == rW[0].tolist()
+    # leaky ReLU network (the example's activation on hidden layers)
+    rng = np.random.default_rng(9)
+    slope = float(np.float16(0.001))
+    specs = make_specs(rng, [4, 16, 4], act=Activation.LeakyReLU, slope=slope)
+    B = 512
+    x = rng.uniform(0, 1, (B, 4)).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, 4)).astype(np.float16)
+    layers = build(specs)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, _ = ob.ref_mlp_train(specs, x, t, 1.0, True)
+    for l in range(2):
+        assert rel_err(dW[l], rW[l]) <= 1e-3 and rel_err(dB[l], rB[l]) <= 1e-3
+
+
+def test_train_fp16_training_optimal_gradients_and_convert():
+    # the example's flow: fp16 TrainingOptimal weight gradients, then one convert call to RowMajor
+    rng = np.random.default_rng(10)
+    dims = [4, 16, 4]
+    specs = make_specs(rng, dims)
+    B = 64
+    x = rng.uniform(0, 1, (B, 4)).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, 4)).astype(np.float16)
+    layers = build(specs, CT.Float16, ML.TrainingOptimal, preset=None)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=1.0 / 64, gradType=CT.Float16)
+    rW, rB, _ = ob.ref_mlp_train(specs, x, t, 1.0 / 64, True)
+    for l, (L, s) in enumerate(zip(layers, specs)):
+        out, fan_in = s["W"].shape
+        row = torch.zeros(out * fan_in * 2, dtype=torch.uint8, device=DEV)
+        size = cv.getCooperativeVectorMatrixSize(out, fan_in, CT.Float16, ML.TrainingOptimal)
+        cv.convertCooperativeVectorMatrix(row, [cv.CooperativeVectorMatrixDesc(out, fan_in, CT.Float16, ML.RowMajor, out * fan_in * 2, 0, fan_in * 2)],
+                                          L.weightsGrad, [cv.CooperativeVectorMatrixDesc(out, fan_in, CT.Float16, ML.TrainingOptimal, size, 0, 0)])
+        got = row.cpu().numpy().view(np.float16).reshape(out, fan_in).astype(np.float64)
+        assert np.max(np.abs(got - rW[l])) <= 2e-3 * np.max(np.abs(rW[l])) + 1e-6
+
+
+def test_train_argument_validation():
+    rng = np.random.default_rng(0)
+    specs = make_specs(rng, [8, 16, 4])
+    layers = build(specs)
+    x = torch.zeros(10, 8, dtype=torch.float16, device=DEV)
+    need = cv.mlpTrainStepWorkspaceSize(layers, 10)
+    assert need > 0
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.mlpTrainStep(layers, x, None, workspace=torch.zeros(need - 16, dtype=torch.uint8, device=DEV))
+    assert e.value.result == cv.SLANG_E_BUFFER_TOO_SMALL
+    specs = make_specs(rng, [8, 16, 64, 4])
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.mlpTrainStepWorkspaceSize(build(specs), 10)
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
