@@ -261,7 +261,58 @@ def workload_c4n(torch, cv, steps, warmup):
     return workload_c4(torch, cv, steps, warmup, flags=1)
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n}
+def workload_c5(torch, cv, steps, warmup):
+    """fp16 training step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, fp32 TrainingOptimal grads."""
+    import numpy as np
+    from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
+                                   FeedForwardLayer)
+    dev = "cuda"
+    dims = [8, 64, 64, 64, 64, 1]
+    B = 1 << 20
+    g = torch.Generator(device=dev); g.manual_seed(20255)
+    layers, host = [], []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = (torch.randn(fo, fi, device=dev, generator=g) * (2.0 / fi) ** 0.5).half()        # He init
+        bias = torch.zeros(fo, dtype=torch.float16, device=dev)
+        gsize = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float32, ML.TrainingOptimal)
+        wg = torch.zeros(gsize, dtype=torch.uint8, device=dev)
+        bg = torch.zeros(fo, dtype=torch.float32, device=dev)
+        last = i == len(dims) - 2
+        layers.append(FeedForwardLayer(fi, fo, W.contiguous().view(torch.uint8).flatten(), bias.view(torch.uint8),
+                                       ML.RowMajor, fi * 2, Activation.NoActivation if last else Activation.ReLU, 0.0,
+                                       wg, bg.view(torch.uint8), ML.TrainingOptimal, 0))
+        host.append((W, bias))
+    x = (torch.rand(B, dims[0], device=dev, generator=g) * 2 - 1).half()
+    ws = torch.empty(cv.mlpTrainStepWorkspaceSize(layers, B), dtype=torch.uint8, device=dev)
+    loss = torch.zeros(1, dtype=torch.float32, device=dev)
+
+    def step():
+        cv.mlpTrainStep(layers, x, None, workspace=ws, lossSum=loss)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+    macs_dx = sum(dims[i] * dims[i + 1] for i in range(1, len(dims) - 1))
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        n = 1 << 11
+        specs = [dict(W=W.cpu().numpy(), b=b.cpu().numpy(), act=1 if i < len(host) - 1 else 0)
+                 for i, (W, b) in enumerate(host)]
+        xs = x[:n].cpu().numpy()
+        t0 = time.perf_counter(); ob.ref_mlp_train(specs, xs, None, 1.0, True); t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d samples, one core; the parity oracle's training step (fp16 carriers, fp32 forward "
+                          "sums, fp64 gradient sums). The Slang CPU target cannot run the example's learnGradient "
+                          "(wave intrinsics and atomics, docs/cpu-target.md:15-21)" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * dims[0] * 2, alg_flops=B * 2 * (2 * macs + macs_dx),
+                bound="mfma", mfma="f16", dtype="f16", kernel="mlpTrainKernel<8-64x4-1> + mlpTrainReduceKernel",
+                config={"workload": "c5: fp16 train step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, "
+                                    "fp32 TrainingOptimal gradients, deterministic reduction", "batch": B, "layers": dims},
+                cpu_baseline=cpu_baseline, key="c5")
+
+
+WORKLOADS = {"c5": workload_c5, "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n}
 
 
 def main(argv=None) -> int:
