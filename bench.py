@@ -32,7 +32,7 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
 # kernel of known size); the summaries are in profiles/.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"c2": 1074875000}   # profiles/matmul_f16_64x64_batch4M.md
 
 
 def ensure_built():
