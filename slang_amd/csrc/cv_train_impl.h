@@ -55,6 +55,13 @@ struct TrainNet : UniformNet<KT0_, HT_, NHID_, MTL_> {
         return b;
     }
     static constexpr int totalGradTiles = gradTileBase(L);
+    static constexpr int xTileBase(int l)
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += nIt(i);
+        return b;
+    }
+    static constexpr int totalXTiles = xTileBase(L);
     static constexpr int dbTileBase(int l) { return Base::biasBase(l); }
     static constexpr int totalDbTiles = Base::totalBiasTiles;
     // floats of one workgroup's partial: dW tiles, db tiles, loss
@@ -82,19 +89,42 @@ struct TrainReduceArgs {
     float* lossSum;              // optional
 };
 
-// 3-state outcome of max(z, zs) per element, 2 bits: 1 = first operand larger, 2 = second, 0 = tie
-__device__ __forceinline__ uint32_t maxState(half_t z, half_t zs) { return z > zs ? 1u : (z < zs ? 2u : 0u); }
+// Gradient multiplier of max(z, zs) with respect to its first operand, per element of a packed
+// fp16 pair: 1 where z wins, 0 where zs wins, 0.5 at a tie (diff.meta.slang:2258-2277).  For the
+// two activations here (zs = 0, or zs = z*slope with 0 <= slope <= 0.5) the outcome is the sign
+// of z.  Two multiplications lift even the smallest subnormal above 1 before the clamp.
+__device__ __forceinline__ halfx2 maxGradMultiplier(halfx2 z)
+{
+    const halfx2 big = {(half_t)65504.f, (half_t)65504.f};
+    const halfx2 one = {(half_t)1.f, (half_t)1.f}, mone = {(half_t)-1.f, (half_t)-1.f};
+    const halfx2 hlf = {(half_t)0.5f, (half_t)0.5f};
+    halfx2 s = z * big;
+    s = s * big;
+    s = __builtin_elementwise_max(__builtin_elementwise_min(s, one), mone);   // sign(z) in {1, 0, -1}
+    return s * hlf + hlf;                                                       // {1, 0.5, 0}
+}
 
-// dz = g * act'(z) in half, from the saved state (see cvo_ref_mlp_train for the scalar statement)
-__device__ __forceinline__ half_t applyActGrad(half_t gv, uint32_t state, int act, float slope)
+// four multipliers in {0, 0.5, 1} <-> four e4m3 bytes (all exactly representable)
+__device__ __forceinline__ uint32_t packMultipliers(halfx2 m01, halfx2 m23)
+{
+    typedef short shortx2 __attribute__((ext_vector_type(2)));
+    shortx2 r = {0, 0};
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, m01, 1.0f, false);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, m23, 1.0f, true);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
+// dz = g * act'(z) on a packed pair, in half: the scalar statement is cvo_ref_mlp_train's.
+//   ReLU  : da = g*m
+//   leaky : da = g*m, db = g*(1-m), dz = da + db*slope   (each product and the sum rounded to fp16)
+__device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, halfx2 slope2)
 {
     if (act == kActNone) return gv;
-    const half_t halfG = (half_t)(0.5f * (float)gv);
-    const half_t da = state == 1u ? gv : (state == 0u ? halfG : (half_t)0);
-    if (act == kActRelu) return da;            // second operand is the constant 0
-    const half_t db = state == 2u ? gv : (state == 0u ? halfG : (half_t)0);
-    const half_t dbs = (half_t)((float)db * slope);
-    return (half_t)((float)da + (float)dbs);
+    const halfx2 da = gv * m;
+    if (act == kActRelu) return da;
+    const halfx2 one = {(half_t)1.f, (half_t)1.f};
+    const halfx2 db = gv * (one - m);
+    return da + db * slope2;
 }
 
 template <class Net>
@@ -110,6 +140,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __shared__ __attribute__((aligned(16))) uint32_t ldsWT[(Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW];
     __shared__ __attribute__((aligned(16))) float ldsB[Net::totalBiasTiles * 16];   // biases as fp32
     __shared__ __attribute__((aligned(16))) float ldsRed[4 * 256];
+    // per-wave parking space for the F-orientation copies of every layer's input
+    __shared__ __attribute__((aligned(16))) uint32_t ldsXF[4 * Net::totalXTiles * 256];
 
     // ---- stage W (A operand of the forward pass), W^T (A operand of dX) and biases ----------
     staticFor<0, L>([&](auto lc) {
@@ -228,10 +260,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     auto round = [&](const uint32_t (&buf)[2][IN_DW], uint32_t t0) {
         uint32_t actS[2][Net::KTMAX][FD];           // S fragments of the current layer's input
-        uint32_t xF[L][Net::ITMAX][FD];             // F fragments of every layer's input
-        uint32_t state[L][2];                       // max() outcomes: 2 bits per element, 8 bits per out tile
-        static_assert(Net::MTMAX <= 4, "state packing holds four 16-row tiles");
+        uint32_t mst[L][2][Net::MTMAX];             // max() gradient multipliers, four e4m3 bytes per out tile
         halfx2 yS[2][Net::MTL][2];                  // network output (carrier), tile j, out tile t
+        uint32_t* myXF = ldsXF + wave * (Net::totalXTiles * 256);
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -244,10 +275,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             constexpr int l = decltype(lc)::value;
             constexpr int MT = Net::mt(l), KT = Net::kt(l);
             const int actv = a.layers[l].act;
-            const float slope = a.layers[l].slope;
-            // this layer's input in F orientation, for dW
+            const half_t sl = (half_t)a.layers[l].slope;
+            const halfx2 slope2 = {sl, sl};
+            const halfx2 zero2 = {(half_t)0, (half_t)0};
+            // this layer's input in F orientation, parked in LDS until the backward pass
 #pragma unroll
-            for (int e = 0; e < Net::nIt(l); ++e) toF(actS[0][e / 2], actS[1][e / 2], e & 1, xF[l][e]);
+            for (int e = 0; e < Net::nIt(l); ++e) {
+                uint32_t f[FD];
+                toF(actS[0][e / 2], actS[1][e / 2], e & 1, f);
+                uint32_t* dst = myXF + (Net::xTileBase(l) + e) * 256 + lane * 4;
+                dst[0] = f[0]; dst[1] = f[1]; dst[2] = f[2]; dst[3] = f[3];
+            }
 
             floatx4 acc[2][MT];
 #pragma unroll
@@ -260,12 +298,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    const u32x4 wv = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
-                    const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+                    const uint32_t* wp = &ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
+                    const uint32_t w[4] = {wp[0], wp[1], wp[2], wp[3]};
                     acc[0][t] = Mma::mma(w, actS[0][kt], acc[0][t]);
                     acc[1][t] = Mma::mma(w, actS[1][kt], acc[1][t]);
                 }
-            // carrier: round to fp16, remember the outcome of max(), apply the activation
+            // carrier: round to fp16, remember the gradient multiplier of max(), apply the activation
             halfx2 car[2][MT][2];
 #pragma unroll
             for (int j = 0; j < 2; ++j)
@@ -274,18 +312,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     typedef float floatx2 __attribute__((ext_vector_type(2)));
                     halfx2 z01 = __builtin_convertvector(floatx2{acc[j][t][0], acc[j][t][1]}, halfx2);
                     halfx2 z23 = __builtin_convertvector(floatx2{acc[j][t][2], acc[j][t][3]}, halfx2);
-                    uint32_t st = 0;
                     if (actv != kActNone) {
-                        half_t zz[4] = {z01.x, z01.y, z23.x, z23.y};
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const half_t zs = actv == kActRelu ? (half_t)0 : (half_t)((float)zz[r] * slope);
-                            st |= maxState(zz[r], zs) << (2 * r);
-                            zz[r] = zz[r] >= zs ? zz[r] : zs;
-                        }
-                        z01 = halfx2{zz[0], zz[1]}; z23 = halfx2{zz[2], zz[3]};
+                        mst[l][j][t] = packMultipliers(maxGradMultiplier(z01), maxGradMultiplier(z23));
+                        const halfx2 s01 = actv == kActRelu ? zero2 : z01 * slope2;
+                        const halfx2 s23 = actv == kActRelu ? zero2 : z23 * slope2;
+                        z01 = __builtin_elementwise_max(z01, s01);
+                        z23 = __builtin_elementwise_max(z23, s23);
                     }
-                    if (t == 0) state[l][j] = st; else state[l][j] |= st << (8 * t);
                     car[j][t][0] = z01; car[j][t][1] = z23;
                 }
             if constexpr (l + 1 < L) {
@@ -307,63 +340,84 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             }
         });
 
+        // decode four multipliers
+        auto multipliers = [&](uint32_t raw, halfx2& m01, halfx2& m23) {
+            m01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw, 1.0f, false);
+            m23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw, 1.0f, true);
+        };
+        // pack the carrier tiles dz[t] (t < MT) of one sample tile into S fragments
+        auto packS = [&](halfx2 (*dz)[2], int MT, int KT, uint32_t (*out)[FD]) {
+#pragma unroll
+            for (int kt = 0; kt < Net::KOMAX; ++kt) {
+                if (kt < KT) {
+                    out[kt][0] = __builtin_bit_cast(uint32_t, dz[2 * kt][0]);
+                    out[kt][1] = __builtin_bit_cast(uint32_t, dz[2 * kt][1]);
+                    out[kt][2] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, dz[2 * kt + 1 < MT ? 2 * kt + 1 : 0][0]) : 0u;
+                    out[kt][3] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, dz[2 * kt + 1 < MT ? 2 * kt + 1 : 0][1]) : 0u;
+                }
+            }
+        };
+
         // ---------------- loss and its gradient (S orientation) ----------------
         uint32_t bS[2][Net::KOMAX][FD];             // S fragments of dY of the current layer
+        {
+            const int actl = a.layers[L - 1].act;
+            const half_t sll = (half_t)a.layers[L - 1].slope;
+            const halfx2 slope2 = {sll, sll};
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint32_t sample = t0 * TILE + 16 * j + n;
-            const bool live = sample < a.batch;
-            float tgtAll = 0.f;
-            if (!ta.targets) {
-                // target = sin(sum of the sample's inputs): every lane group holds a quarter of them
-                float part = 0.f;
+            for (int j = 0; j < 2; ++j) {
+                const uint32_t sample = t0 * TILE + 16 * j + n;
+                const bool live = sample < a.batch;
+                float tgtAll = 0.f;
+                if (!ta.targets) {
+                    // target = sin(sum of the sample's inputs): every lane group holds a quarter of them
+                    float part = 0.f;
 #pragma unroll
-                for (int d = 0; d < IN_DW; ++d) {
-                    const halfx2 v = __builtin_bit_cast(halfx2, buf[j][d]);
-                    part += (float)v.x; part += (float)v.y;
-                }
-                part += __shfl_xor(part, 16);
-                part += __shfl_xor(part, 32);
-                tgtAll = (float)(half_t)sinf(part);
-            }
-            half_t dz[Net::MTL][4];
-#pragma unroll
-            for (int t = 0; t < Net::MTL; ++t) {
-                const half_t yv[4] = {yS[j][t][0].x, yS[j][t][0].y, yS[j][t][1].x, yS[j][t][1].y};
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = g * OROWS + 4 * t + r;
-                    half_t gv = (half_t)0;
-                    if (live && row < outDim) {
-                        const float tv = ta.targets
-                            ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row) : tgtAll;
-                        const half_t diff = (half_t)((float)yv[r] - tv);
-                        lossAcc += (float)diff * (float)diff;
-                        gv = (half_t)(2.0f * (float)diff * ta.lossScale);
+                    for (int d = 0; d < IN_DW; ++d) {
+                        const halfx2 v = __builtin_bit_cast(halfx2, buf[j][d]);
+                        part += (float)v.x; part += (float)v.y;
                     }
-                    dz[t][r] = applyActGrad(gv, (state[L - 1][j] >> (8 * t + 2 * r)) & 3u, a.layers[L - 1].act, a.layers[L - 1].slope);
+                    part += __shfl_xor(part, 16);
+                    part += __shfl_xor(part, 32);
+                    tgtAll = (float)(half_t)sinf(part);
                 }
-            }
+                halfx2 dz[Net::MTL][2];
 #pragma unroll
-            for (int kt = 0; kt < Net::ktOut(L - 1); ++kt) {
-                const halfx2 p0 = {dz[2 * kt][0], dz[2 * kt][1]}, p1 = {dz[2 * kt][2], dz[2 * kt][3]};
-                bS[j][kt][0] = __builtin_bit_cast(uint32_t, p0);
-                bS[j][kt][1] = __builtin_bit_cast(uint32_t, p1);
-                if (2 * kt + 1 < Net::MTL) {
-                    const int tt = 2 * kt + 1 < Net::MTL ? 2 * kt + 1 : 0;
-                    const halfx2 q0 = {dz[tt][0], dz[tt][1]}, q1 = {dz[tt][2], dz[tt][3]};
-                    bS[j][kt][2] = __builtin_bit_cast(uint32_t, q0);
-                    bS[j][kt][3] = __builtin_bit_cast(uint32_t, q1);
-                } else {
-                    bS[j][kt][2] = 0u; bS[j][kt][3] = 0u;
+                for (int t = 0; t < Net::MTL; ++t) {
+                    const half_t yv[4] = {yS[j][t][0].x, yS[j][t][0].y, yS[j][t][1].x, yS[j][t][1].y};
+                    half_t gv[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int row = g * OROWS + 4 * t + r;
+                        gv[r] = (half_t)0;
+                        if (live && row < outDim) {
+                            const float tv = ta.targets
+                                ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row) : tgtAll;
+                            const half_t diff = (half_t)((float)yv[r] - tv);
+                            lossAcc += (float)diff * (float)diff;
+                            gv[r] = (half_t)(2.0f * (float)diff * ta.lossScale);
+                        }
+                    }
+                    halfx2 m01 = {(half_t)1.f, (half_t)1.f}, m23 = m01;
+                    if (actl != kActNone) multipliers(mst[L - 1][j][t], m01, m23);
+                    dz[t][0] = applyActGrad(halfx2{gv[0], gv[1]}, m01, actl, slope2);
+                    dz[t][1] = applyActGrad(halfx2{gv[2], gv[3]}, m23, actl, slope2);
                 }
+                packS(dz, Net::MTL, Net::ktOut(L - 1), bS[j]);
             }
         }
 
         // ---------------- backward ----------------
         staticFor<0, L>([&](auto lc) {
             constexpr int l = L - 1 - decltype(lc)::value;
-            constexpr int MT = Net::mt(l);
+            constexpr int MT = Net::mt(l), NI = Net::nIt(l);
+            // this layer's input in F orientation, back from LDS
+            uint32_t xF[NI][FD];
+#pragma unroll
+            for (int e = 0; e < NI; ++e) {
+                const uint32_t* src = myXF + (Net::xTileBase(l) + e) * 256 + lane * 4;
+                xF[e][0] = src[0]; xF[e][1] = src[1]; xF[e][2] = src[2]; xF[e][3] = src[3];
+            }
             // dY in F orientation; bias gradient; weight gradient
 #pragma unroll
             for (int eo = 0; eo < MT; ++eo) {
@@ -374,16 +428,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 for (int d = 0; d < FD; ++d) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, dzF[d]), ones2, s, false);
                 accB[Net::dbTileBase(l) + eo] = s;
 #pragma unroll
-                for (int ei = 0; ei < Net::nIt(l); ++ei) {
-                    floatx4& w = accW[Net::gradTileBase(l) + eo * Net::nIt(l) + ei];
-                    w = Mma::mma(dzF, xF[l][ei], w);
+                for (int ei = 0; ei < NI; ++ei) {
+                    floatx4& w = accW[Net::gradTileBase(l) + eo * NI + ei];
+                    w = Mma::mma(dzF, xF[ei], w);
                 }
             }
             if constexpr (l > 0) {
                 // dX = W^T dY, then through the previous layer's activation
                 constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
                 const int actp = a.layers[l - 1].act;
-                const float slopep = a.layers[l - 1].slope;
+                const half_t slp = (half_t)a.layers[l - 1].slope;
+                const halfx2 slope2 = {slp, slp};
                 floatx4 gacc[2][MTI];
 #pragma unroll
                 for (int t = 0; t < MTI; ++t) { gacc[0][t] = floatx4{0.f, 0.f, 0.f, 0.f}; gacc[1][t] = gacc[0][t]; }
@@ -391,55 +446,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 for (int kt = 0; kt < KTO; ++kt)
 #pragma unroll
                     for (int t = 0; t < MTI; ++t) {
-                        const u32x4 wv = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
-                        const uint32_t w[4] = {wv.x, wv.y, wv.z, wv.w};
+                        const uint32_t* wp = &ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
+                        const uint32_t w[4] = {wp[0], wp[1], wp[2], wp[3]};
                         gacc[0][t] = Mma::mma(w, bS[0][kt], gacc[0][t]);
                         gacc[1][t] = Mma::mma(w, bS[1][kt], gacc[1][t]);
                     }
-                constexpr int KTP = Net::ktOut(l - 1);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    half_t dz[MTI][4];
+                    halfx2 dz[MTI][2];
 #pragma unroll
-                    for (int t = 0; t < MTI; ++t)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            dz[t][r] = applyActGrad((half_t)gacc[j][t][r], (state[l - 1][j] >> (8 * t + 2 * r)) & 3u, actp, slopep);
-#pragma unroll
-                    for (int kt = 0; kt < KTP; ++kt) {
-                        const halfx2 p0 = {dz[2 * kt][0], dz[2 * kt][1]}, p1 = {dz[2 * kt][2], dz[2 * kt][3]};
-                        bS[j][kt][0] = __builtin_bit_cast(uint32_t, p0);
-                        bS[j][kt][1] = __builtin_bit_cast(uint32_t, p1);
-                        if (2 * kt + 1 < MTI) {
-                            const int tt = 2 * kt + 1 < MTI ? 2 * kt + 1 : 0;
-                            const halfx2 q0 = {dz[tt][0], dz[tt][1]}, q1 = {dz[tt][2], dz[tt][3]};
-                            bS[j][kt][2] = __builtin_bit_cast(uint32_t, q0);
-                            bS[j][kt][3] = __builtin_bit_cast(uint32_t, q1);
-                        } else {
-                            bS[j][kt][2] = 0u; bS[j][kt][3] = 0u;
-                        }
+                    for (int t = 0; t < MTI; ++t) {
+                        typedef float floatx2 __attribute__((ext_vector_type(2)));
+                        const halfx2 g01 = __builtin_convertvector(floatx2{gacc[j][t][0], gacc[j][t][1]}, halfx2);
+                        const halfx2 g23 = __builtin_convertvector(floatx2{gacc[j][t][2], gacc[j][t][3]}, halfx2);
+                        halfx2 m01 = {(half_t)1.f, (half_t)1.f}, m23 = m01;
+                        if (actp != kActNone) multipliers(mst[l - 1][j][t], m01, m23);
+                        dz[t][0] = applyActGrad(g01, m01, actp, slope2);
+                        dz[t][1] = applyActGrad(g23, m23, actp, slope2);
                     }
+                    packS(dz, MTI, Net::ktOut(l - 1), bS[j]);
                 }
             }
         });
     };
 
-    // ---- main loop: every wave strides over rounds of 32 samples -----------------------------
+    // ---- main loop: every wave strides over rounds of 32 samples; the next round's inputs are
+    //      requested before the current round and copied over after it ------------------------
     {
         uint32_t tile = blockIdx.x * 4 + wave;
         if (tile < numTiles) {
-            uint32_t bufA[2][IN_DW], bufB[2][IN_DW];
-            loadTile(bufA, tile);
-            while (true) {
+            uint32_t cur[2][IN_DW], nxt[2][IN_DW];
+            loadTile(cur, tile);
+            for (; tile < numTiles; tile += tileStride) {
                 const uint32_t t1 = tile + tileStride;
-                loadTile(bufB, t1 < numTiles ? t1 : tile);
-                round(bufA, tile);
-                if (t1 >= numTiles) break;
-                const uint32_t t2 = t1 + tileStride;
-                loadTile(bufA, t2 < numTiles ? t2 : t1);
-                round(bufB, t1);
-                if (t2 >= numTiles) break;
-                tile = t2;
+                loadTile(nxt, t1 < numTiles ? t1 : tile);
+                round(cur, tile);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int d = 0; d < IN_DW; ++d) cur[j][d] = nxt[j][d];
             }
         }
     }
