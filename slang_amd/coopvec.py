@@ -395,3 +395,48 @@ def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, target
                               float(lossScale), batch, lossSum.data_ptr(), workspace.data_ptr(),
                               workspace.numel() * workspace.element_size()))
     return workspace, lossSum
+
+
+# ---------------------------------------------------------------------------------------------
+# training operators over a batch
+# ---------------------------------------------------------------------------------------------
+
+def coopVecOuterProductAccumulate(a: torch.Tensor, b: torch.Tensor, matrix: torch.Tensor, matrixOffset: int,
+                                  matrixStride: int, memoryLayout: int, matrixInterpretation: int, *,
+                                  workspace: Optional[torch.Tensor] = None, stream=None) -> None:
+    """coopVecOuterProductAccumulate<T,M,N> (hlsl.meta.slang:33227-33235) for every row of the batch:
+    matrix[i][j] += sum_s a[s][i]*b[s][j], without atomics and bitwise reproducible."""
+    lib = _lib.load()
+    ta, sa = _vector_info(a, CoopVecComponentType.Float16, "a")
+    tb, sb = _vector_info(b, CoopVecComponentType.Float16, "b")
+    if a.shape[0] != b.shape[0] or ta != tb:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "a and b must have the same batch and element type")
+    batch, m, n = a.shape[0], a.shape[1], b.shape[1]
+    if workspace is None:
+        need = ctypes.c_size_t(0)
+        _check(lib.cvOuterProductAccumulateWorkspaceSize(m, n, batch, ctypes.byref(need)))
+        workspace = torch.empty(max(need.value, 16), dtype=torch.uint8, device=a.device)
+    _check(lib.cvOuterProductAccumulate(_stream_handle(stream), a.data_ptr(), sa, m, b.data_ptr(), sb, n, int(ta), batch,
+                                        _buffer_ptr(matrix, "matrix"), int(matrixOffset), int(matrixStride),
+                                        int(memoryLayout), int(matrixInterpretation), workspace.data_ptr(),
+                                        workspace.numel() * workspace.element_size()))
+
+
+def coopVecReduceSumAccumulate(v: torch.Tensor, buffer: torch.Tensor, offset: int, *,
+                               bufferType: Optional[int] = None, workspace: Optional[torch.Tensor] = None,
+                               stream=None) -> None:
+    """coopVecReduceSumAccumulate<T,N> (hlsl.meta.slang:33330-33334) for every row of the batch:
+    buffer[i] += sum_s v[s][i].  The reference's destination type is the vector's type; bufferType
+    Float32 gives the fp32 accumulation buffers the training configuration asks for."""
+    lib = _lib.load()
+    tv, sv = _vector_info(v, CoopVecComponentType.Float16, "v")
+    batch, n = v.shape
+    if bufferType is None:
+        bufferType = tv
+    if workspace is None:
+        need = ctypes.c_size_t(0)
+        _check(lib.cvReduceSumAccumulateWorkspaceSize(n, batch, ctypes.byref(need)))
+        workspace = torch.empty(max(need.value, 16), dtype=torch.uint8, device=v.device)
+    _check(lib.cvReduceSumAccumulate(_stream_handle(stream), v.data_ptr(), sv, n, int(tv), batch,
+                                     _buffer_ptr(buffer, "buffer"), int(offset), int(bufferType),
+                                     workspace.data_ptr(), workspace.numel() * workspace.element_size()))

@@ -277,28 +277,95 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     return fromHip(e, "cvMatMul launch");
 }
 
-CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t, int32_t, uint32_t, size_t* outBytes)
+CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t m, int32_t n, uint32_t batch, size_t* outBytes)
 {
-    if (outBytes) *outBytes = 0;
-    return fail(CV_E_NOT_IMPLEMENTED, "cvOuterProductAccumulate: not implemented yet");
+    if (!outBytes) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulateWorkspaceSize: outBytes is null");
+    *outBytes = 0;
+    if (m <= 0 || n <= 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulateWorkspaceSize: m=%d n=%d", m, n);
+    CvResult rc;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    *outBytes = cv::outerWorkspaceBytes(m, n, batch ? batch : 1, cus);
+    return CV_OK;
 }
 
-CV_API CvResult cvOuterProductAccumulate(void*, const void*, size_t, int32_t, const void*, size_t, int32_t,
-                                         int32_t, uint32_t, void*, size_t, uint32_t, int32_t, int32_t, void*, size_t)
+CV_API CvResult cvOuterProductAccumulate(void* stream, const void* a, size_t aStride, int32_t m,
+                                         const void* b, size_t bStride, int32_t n, int32_t elementType,
+                                         uint32_t batch, void* matrix, size_t matrixOffset, uint32_t matrixStride,
+                                         int32_t layout, int32_t matrixInterpretation, void* workspace,
+                                         size_t workspaceBytes)
 {
-    return fail(CV_E_NOT_IMPLEMENTED, "cvOuterProductAccumulate: not implemented yet");
+    if (m <= 0 || n <= 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: m=%d n=%d", m, n);
+    if (elementType != CV_FLOAT16)
+        return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: vectors must be FLOAT16 (got %d)", elementType);
+    if (cvComponentPackingFactor(matrixInterpretation) != 1)   // static_assert hlsl.meta.slang:33237
+        return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: can't use packed component type in matrixInterpretation");
+    if (matrixInterpretation != CV_FLOAT16 && matrixInterpretation != CV_FLOAT32)
+        return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: matrixInterpretation %d (supported: FLOAT16, FLOAT32)", matrixInterpretation);
+    if (layout < 0 || layout > 3) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: unknown layout %d", layout);
+    if (batch == 0) return CV_OK;
+    if (!a || !b || !matrix || !workspace) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: null argument");
+    if ((uintptr_t)a % 2 || aStride % 2 || (uintptr_t)b % 2 || bStride % 2 || (uintptr_t)workspace % 16)
+        return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: misaligned vectors/workspace");
+    if (batch > 1 && (aStride < (size_t)m * 2 || bStride < (size_t)n * 2))
+        return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: vector stride smaller than the vector");
+    cv::OuterArgs o;
+    memset(&o, 0, sizeof(o));
+    o.a = (const uint8_t*)a; o.b = (const uint8_t*)b; o.aStride = aStride; o.bStride = bStride;
+    o.aAlign = alignOf(a, aStride); o.bAlign = alignOf(b, bStride);
+    o.m = m; o.n = n; o.batch = batch;
+    o.mat = (uint8_t*)matrix + matrixOffset;
+    o.shape = cv::MatrixShape{(uint32_t)m, (uint32_t)n, matrixInterpretation, layout, isOptimal(layout) ? 0 : (size_t)matrixStride};
+    if (cv::matrixSize(o.shape) == 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrixStride %u smaller than a row/column", matrixStride);
+    const uint32_t esz = cv::elemSize(matrixInterpretation);
+    if ((uintptr_t)o.mat % esz || (!isOptimal(layout) && matrixStride % esz)) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrix misaligned");
+    o.partials = (float*)workspace;
+    CvResult rc;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const size_t need = cv::outerWorkspaceBytes(m, n, batch, cus);
+    if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvOuterProductAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+    return fromHip(cv::launchOuterProduct((hipStream_t)stream, o, cus), "cvOuterProductAccumulate launch");
 }
 
-CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t, uint32_t, size_t* outBytes)
+CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t n, uint32_t batch, size_t* outBytes)
 {
-    if (outBytes) *outBytes = 0;
-    return fail(CV_E_NOT_IMPLEMENTED, "cvReduceSumAccumulate: not implemented yet");
+    if (!outBytes) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulateWorkspaceSize: outBytes is null");
+    *outBytes = 0;
+    if (n <= 0) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulateWorkspaceSize: n=%d", n);
+    CvResult rc;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    *outBytes = cv::reduceSumWorkspaceBytes(batch ? batch : 1, cus);
+    return CV_OK;
 }
 
-CV_API CvResult cvReduceSumAccumulate(void*, const void*, size_t, int32_t, int32_t, uint32_t, void*, size_t,
-                                      int32_t, void*, size_t)
+CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStride, int32_t n, int32_t elementType,
+                                      uint32_t batch, void* buffer, size_t offset, int32_t bufferType,
+                                      void* workspace, size_t workspaceBytes)
 {
-    return fail(CV_E_NOT_IMPLEMENTED, "cvReduceSumAccumulate: not implemented yet");
+    if (n <= 0) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: n=%d", n);
+    if (n > 256) return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: n=%d (limit 256)", n);
+    if (elementType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: vectors must be FLOAT16 (got %d)", elementType);
+    if (bufferType != CV_FLOAT16 && bufferType != CV_FLOAT32)
+        return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: bufferType %d (supported: FLOAT16, FLOAT32)", bufferType);
+    if (batch == 0) return CV_OK;
+    if (!v || !buffer || !workspace) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: null argument");
+    const uint32_t esz = cv::elemSize(bufferType);
+    if ((uintptr_t)v % 2 || vStride % 2 || ((uintptr_t)buffer + offset) % esz || (uintptr_t)workspace % 4)
+        return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: misaligned argument");
+    if (batch > 1 && vStride < (size_t)n * 2) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: vector stride smaller than the vector");
+    cv::ReduceSumArgs r;
+    memset(&r, 0, sizeof(r));
+    r.v = (const uint8_t*)v; r.vStride = vStride; r.n = n;
+    r.colsPerGroup = (((n + 3) / 4) + 1) / 2 * 2;
+    r.batch = batch; r.buf = (uint8_t*)buffer + offset; r.bufCt = bufferType; r.partials = (float*)workspace;
+    CvResult rc;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const size_t need = cv::reduceSumWorkspaceBytes(batch, cus);
+    if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvReduceSumAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+    return fromHip(cv::launchReduceSum((hipStream_t)stream, r, cus), "cvReduceSumAccumulate launch");
 }
 
 // Validates the parts of a CvMlpDesc that forward and training share and fills the per-layer

@@ -73,6 +73,32 @@ struct TrainLaunch {
 size_t trainWorkspaceBytes(const MlpArgs& shapes, int numCUs);
 hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCUs);
 
+// ---- batched outer-product / reduce-sum accumulate ---------------------------------------
+struct OuterArgs {
+    const uint8_t* a; const uint8_t* b;   // fp16 [batch][m], [batch][n]
+    uint64_t aStride, bStride;
+    uint32_t aAlign, bAlign;
+    int32_t m, n;
+    uint32_t batch;
+    uint8_t* mat;                          // destination (offset applied)
+    MatrixShape shape;                     // m x n, FLOAT16 or FLOAT32, any layout
+    float* partials;
+};
+size_t outerWorkspaceBytes(int m, int n, uint32_t batch, int numCUs);
+hipError_t launchOuterProduct(hipStream_t stream, const OuterArgs& args, int numCUs);
+
+struct ReduceSumArgs {
+    const uint8_t* v;                      // fp16 [batch][n]
+    uint64_t vStride;
+    int32_t n, colsPerGroup;
+    uint32_t batch;
+    uint8_t* buf;                          // destination (offset applied)
+    int32_t bufCt;                         // kF16 or kF32
+    float* partials;
+};
+size_t reduceSumWorkspaceBytes(uint32_t batch, int numCUs);
+hipError_t launchReduceSum(hipStream_t stream, const ReduceSumArgs& args, int numCUs);
+
 // ---- layout conversion --------------------------------------------------------------------
 struct ConvertItem {
     const uint8_t* src;
