@@ -172,7 +172,7 @@ def workload_c3(torch, cv, steps, warmup):
                 cpu_baseline=cpu_baseline, key="c3")
 
 
-def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std):
+def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std, with_bias=True):
     import numpy as np
     from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
                                    CooperativeVectorMatrixDesc as D, FeedForwardLayer)
@@ -190,9 +190,9 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
         wopt = torch.empty(size, dtype=torch.uint8, device=dev)
         cv.convertCooperativeVectorMatrix(wopt, [D(fo, fi, wtype, ML.InferencingOptimal, size, 0, 0)],
                                           wrow, [D(fo, fi, wtype, ML.RowMajor, fo * fi * esz, 0, fi * esz)])
-        bias = torch.zeros(fo, dtype=torch.float16, device=dev)
+        bias = torch.zeros(fo, dtype=torch.float16, device=dev)      # the configurations have zero / no biases
         last = i == len(dims) - 2
-        layers.append(FeedForwardLayer(fi, fo, wopt, bias.view(torch.uint8), ML.InferencingOptimal, 0,
+        layers.append(FeedForwardLayer(fi, fo, wopt, bias.view(torch.uint8) if with_bias else None, ML.InferencingOptimal, 0,
                                        Activation.NoActivation if last else Activation.ReLU, 0.0))
         host.append((Wt, bias))
     x = x_maker(torch, g, B, dims[0], dev)
@@ -254,7 +254,7 @@ def workload_c4(torch, cv, steps, warmup, flags=0):
                          "c4: e4m3 MLP 32->64->64->8, ReLU, fp16 out, batch 2^24, fused forward, "
                          + ("fp8 matrix pipeline" if flags else "e4m3 decoded to the fp16 matrix pipeline"),
                          lambda torch, g, B, k, dev: (torch.randn(B, k, device=dev, generator=g) * 0.5).to(torch.float8_e4m3fn),
-                         lambda fi: 0.5)
+                         lambda fi: 0.5, with_bias=False)
 
 
 def workload_c4n(torch, cv, steps, warmup):

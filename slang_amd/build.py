@@ -35,6 +35,16 @@ HIPCC_FLAGS = [
 ]
 
 
+# Forward kernels read every MFMA result with the VALU right away, so their MFMAs write VGPRs
+# directly; left to its heuristics the compiler parks results in AGPRs and copies them back.
+# (The training kernel keeps its gradient accumulators in AGPRs and is built without this.)
+PER_FILE_FLAGS = {
+    name: ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+    for name in ("cv_matmul_f16.hip", "cv_matmul_fp8.hip", "cv_matmul_i8.hip",
+                 "cv_mlp_f16.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip")
+}
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):
@@ -59,7 +69,7 @@ def build_library(jobs: int = 8, verbose: bool = False) -> str:
     for src in sources:
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmds.append([hipcc, *HIPCC_FLAGS, "-I", os.path.join(REPO_DIR, "include"), "-c",
+        cmds.append([hipcc, *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src, []), "-I", os.path.join(REPO_DIR, "include"), "-c",
                      os.path.join(CSRC, src), "-o", obj])
     with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         for cmd, _ in zip(cmds, pool.map(_run, cmds)):

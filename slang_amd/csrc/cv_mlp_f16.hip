@@ -1,5 +1,5 @@
 // cv_mlp_f16.hip -- fp16 instantiations of the fused forward MLP, and the dispatcher.
-#include "cv_mlp_impl.h"
+#include "cv_mlp_stream.h"
 
 namespace cv {
 

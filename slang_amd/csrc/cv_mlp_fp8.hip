@@ -1,6 +1,6 @@
 // cv_mlp_fp8.hip -- e4m3 instantiations of the fused forward MLP on the fp16 matrix pipeline
 // (exact decode of weights and of the re-quantised carrier; fp32-grade accumulation).
-#include "cv_mlp_impl.h"
+#include "cv_mlp_stream.h"
 
 namespace cv {
 

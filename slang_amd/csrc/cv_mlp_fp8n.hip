@@ -1,5 +1,5 @@
 // cv_mlp_fp8n.hip -- e4m3 instantiations of the fused forward MLP on the fp8 matrix pipeline.
-#include "cv_mlp_impl.h"
+#include "cv_mlp_stream.h"
 
 namespace cv {
 

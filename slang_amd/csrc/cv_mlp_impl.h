@@ -377,13 +377,19 @@ hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
     return hipGetLastError();
 }
 
+// streaming instantiation for full-width contiguous inputs (cv_mlp_stream.h)
+template <class Mma, class Net> bool mlpStreamEligible(const MlpArgs& a);
+template <class Mma, class Net> hipError_t launchMlpStream(hipStream_t stream, const MlpArgs& a, int numCUs);
+
 // The specialisations built into the library: (input k-tiles, hidden tiles, hidden layers,
 // output tiles).  Dimensions smaller than a tile are padded with zeros at run time.
+#ifndef CV_MLP_SHAPES
 #define CV_MLP_SHAPES(X) \
     X(1, 1, 1, 1) X(1, 1, 2, 1) X(1, 1, 3, 1) \
     X(1, 2, 1, 1) X(1, 2, 2, 1) X(1, 2, 3, 1) X(1, 2, 1, 2) X(1, 2, 2, 2) X(1, 2, 3, 2) \
     X(1, 4, 1, 1) X(1, 4, 2, 1) X(1, 4, 3, 1) X(1, 4, 4, 1) X(1, 4, 2, 4) X(1, 4, 3, 4) \
     X(2, 4, 1, 4) X(2, 4, 2, 4) X(2, 4, 3, 4) X(2, 4, 2, 1)
+#endif
 
 template <class Mma>
 hipError_t dispatchMlp(hipStream_t stream, const MlpArgs& a, int numCUs)
@@ -396,8 +402,11 @@ hipError_t dispatchMlp(hipStream_t stream, const MlpArgs& a, int numCUs)
         if ((int)optMT((uint32_t)a.layers[l].out) != ht) return hipErrorInvalidValue;
     const int mtl = (int)optMT((uint32_t)a.layers[L - 1].out);
 #define CV_X(K0, HT, NH, ML) \
-    if (kt0 <= K0 && (K0 == 1 || kt0 == K0) && ht == HT && L - 1 == NH && mtl == ML) \
-        return launchMlpNet<Mma, UniformNet<K0, HT, NH, ML>>(stream, a, numCUs);
+    if (kt0 <= K0 && (K0 == 1 || kt0 == K0) && ht == HT && L - 1 == NH && mtl == ML) { \
+        typedef UniformNet<K0, HT, NH, ML> N_; \
+        return mlpStreamEligible<Mma, N_>(a) ? launchMlpStream<Mma, N_>(stream, a, numCUs) \
+                                             : launchMlpNet<Mma, N_>(stream, a, numCUs); \
+    }
     CV_MLP_SHAPES(CV_X)
 #undef CV_X
     return hipErrorInvalidValue;
