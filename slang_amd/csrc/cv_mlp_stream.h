@@ -17,6 +17,15 @@
 namespace cv {
 namespace {
 
+// carrier for ReLU / no activation only (the launcher sends leaky-ReLU networks to the general
+// kernel): no per-tile branch in the round loop
+__device__ __forceinline__ void carrierNoLeaky(const floatx4& acc, const CarrierCfg& c, halfx2& h01, halfx2& h23)
+{
+    typedef float floatx2 __attribute__((ext_vector_type(2)));
+    h01 = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[0], acc[1]}, halfx2), c.floor2);
+    h23 = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[2], acc[3]}, halfx2), c.floor2);
+}
+
 template <class Mma, class Net, int NT, int S, bool HAS_BIAS>
 __global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
 {
@@ -190,8 +199,8 @@ __global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
 #pragma unroll
                         for (int kt = 0; kt < KTN; ++kt) {
                             halfx2 lo01, lo23, hi01 = {(half_t)0, (half_t)0}, hi23 = {(half_t)0, (half_t)0};
-                            carrierFromAcc(acc[j][2 * kt], cc[l], lo01, lo23);
-                            if (2 * kt + 1 < MT) carrierFromAcc(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], cc[l], hi01, hi23);
+                            carrierNoLeaky(acc[j][2 * kt], cc[l], lo01, lo23);
+                            if (2 * kt + 1 < MT) carrierNoLeaky(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], cc[l], hi01, hi23);
                             fragFromCarrier<Mma>(lo01, lo23, hi01, hi23, cc[l], act[j][kt]);
                         }
                 } else {
@@ -203,7 +212,7 @@ __global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
 #pragma unroll
                             for (int t = 0; t < MT; ++t) {
                                 halfx2 p0, p1;
-                                carrierFromAcc(acc[j][t], cc[l], p0, p1);
+                                carrierNoLeaky(acc[j][t], cc[l], p0, p1);
                                 const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
                                 o[t] = v;
                             }
@@ -229,6 +238,8 @@ bool mlpStreamEligible(const MlpArgs& a)
 {
     constexpr int ROW_BYTES = 16 * Mma::kRawDW * Net::KT0;
     const int outDim = a.layers[Net::L - 1].out;
+    for (int l = 0; l < Net::L; ++l)
+        if (a.layers[l].act == kActLeakyRelu) return false;
     return a.layers[0].in * Mma::kEsz == ROW_BYTES && a.inStride == (uint64_t)ROW_BYTES &&
            ((uintptr_t)a.in & 15u) == 0 && outDim % (4 * Net::MTL) == 0 && a.outAlign >= 8u &&
            (uint64_t)a.batch * ROW_BYTES >= 16;
@@ -237,7 +248,11 @@ bool mlpStreamEligible(const MlpArgs& a)
 template <class Mma, class Net, bool HAS_BIAS>
 hipError_t launchMlpStreamB(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
+#ifdef CV_MLP_STREAM_NT
+    constexpr int NT = CV_MLP_STREAM_NT;
+#else
     constexpr int NT = (Net::totalFrags * Mma::kFD <= 32) ? 4 : 2;
+#endif
     constexpr int ROW_DW = 4 * Mma::kRawDW * Net::KT0;
     constexpr int S0 = CV_MLP_STREAM_SLOT_DW / (16 * ROW_DW);
     constexpr int S = S0 < NT ? NT : S0 / NT * NT;
