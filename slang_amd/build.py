@@ -37,11 +37,11 @@ HIPCC_FLAGS = [
 
 # Forward kernels read every MFMA result with the VALU right away, so their MFMAs write VGPRs
 # directly; left to its heuristics the compiler parks results in AGPRs and copies them back.
-# (The training kernel keeps its gradient accumulators in AGPRs and is built without this.)
+# (The training kernel pins its gradient accumulators to AGPRs itself.)
 PER_FILE_FLAGS = {
     name: ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
     for name in ("cv_matmul_f16.hip", "cv_matmul_fp8.hip", "cv_matmul_i8.hip",
-                 "cv_mlp_f16.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip")
+                 "cv_mlp_f16.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip", "cv_train.hip", "cv_accum.hip")
 }
 
 

@@ -117,6 +117,17 @@ __device__ __forceinline__ uint32_t packMultipliers(halfx2 m01, halfx2 m23)
 // dz = g * act'(z) on a packed pair, in half: the scalar statement is cvo_ref_mlp_train's.
 //   ReLU  : da = g*m
 //   leaky : da = g*m, db = g*(1-m), dz = da + db*slope   (each product and the sum rounded to fp16)
+// acc += A . B with the accumulator pinned to AGPRs.  The translation unit is built with VGPR
+// destinations for MFMAs (every other MFMA result here is consumed by the VALU at once); the
+// gradient accumulators are only ever touched by MFMAs until the end of the kernel, and there
+// are too many of them for the 256 architectural VGPRs.  The leading s_nop covers a VALU write
+// of an operand immediately before (the compiler does not look inside inline asm).
+__device__ __forceinline__ void accumulateInAgpr(floatx4& acc, const uint32_t* a, const uint32_t* b)
+{
+    const u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+    asm("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(av), "v"(bv));
+}
+
 __device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, halfx2 slope2)
 {
     if (act == kActNone) return gv;
@@ -430,7 +441,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
                 for (int ei = 0; ei < NI; ++ei) {
                     floatx4& w = accW[Net::gradTileBase(l) + eo * NI + ei];
-                    w = Mma::mma(dzF, xF[ei], w);
+                    accumulateInAgpr(w, dzF, xF[ei]);
                 }
             }
             if constexpr (l > 0) {
@@ -488,6 +499,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             }
         }
     }
+
+    // the last MFMAs into the AGPR accumulators must have retired before they are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- workgroup partial: sum the four waves in a fixed order, one tile at a time ----------
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
