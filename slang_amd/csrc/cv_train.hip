@@ -38,7 +38,10 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ta.lossScale = t.lossScale;
     ta.partials = t.workspace;
     const uint32_t blocks = (uint32_t)numCUs;      // one resident workgroup per compute unit
-    hipLaunchKernelGGL((mlpTrainKernel<Net>), dim3(blocks), dim3(256), 0, stream, ta);
+    bool leaky = false;
+    for (int l = 0; l < Net::L; ++l) leaky = leaky || t.mlp.layers[l].act == kActLeakyRelu;
+    if (leaky) hipLaunchKernelGGL((mlpTrainKernel<Net, true>), dim3(blocks), dim3(256), 0, stream, ta);
+    else       hipLaunchKernelGGL((mlpTrainKernel<Net, false>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     TrainReduceArgs ra;

@@ -92,16 +92,15 @@ struct TrainReduceArgs {
 // Gradient multiplier of max(z, zs) with respect to its first operand, per element of a packed
 // fp16 pair: 1 where z wins, 0 where zs wins, 0.5 at a tie (diff.meta.slang:2258-2277).  For the
 // two activations here (zs = 0, or zs = z*slope with 0 <= slope <= 0.5) the outcome is the sign
-// of z.  Two multiplications lift even the smallest subnormal above 1 before the clamp.
+// of z.  clamp(z*BIG*BIG + 0.5, 0, 1): two scalings lift even the smallest subnormal far above
+// 1 (or below -1), zero stays at 0.5.
 __device__ __forceinline__ halfx2 maxGradMultiplier(halfx2 z)
 {
     const halfx2 big = {(half_t)65504.f, (half_t)65504.f};
-    const halfx2 one = {(half_t)1.f, (half_t)1.f}, mone = {(half_t)-1.f, (half_t)-1.f};
+    const halfx2 one = {(half_t)1.f, (half_t)1.f}, zero = {(half_t)0.f, (half_t)0.f};
     const halfx2 hlf = {(half_t)0.5f, (half_t)0.5f};
-    halfx2 s = z * big;
-    s = s * big;
-    s = __builtin_elementwise_max(__builtin_elementwise_min(s, one), mone);   // sign(z) in {1, 0, -1}
-    return s * hlf + hlf;                                                       // {1, 0.5, 0}
+    const halfx2 s = (z * big) * big + hlf;
+    return __builtin_elementwise_min(__builtin_elementwise_max(s, zero), one);   // {1, 0.5, 0}
 }
 
 // four multipliers in {0, 0.5, 1} <-> four e4m3 bytes (all exactly representable)
@@ -128,17 +127,19 @@ __device__ __forceinline__ void accumulateInAgpr(floatx4& acc, const uint32_t* a
     asm("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(av), "v"(bv));
 }
 
+template <bool LEAKY>
 __device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, halfx2 slope2)
 {
     if (act == kActNone) return gv;
     const halfx2 da = gv * m;
-    if (act == kActRelu) return da;
+    if (!LEAKY || act == kActRelu) return da;
     const halfx2 one = {(half_t)1.f, (half_t)1.f};
     const halfx2 db = gv * (one - m);
     return da + db * slope2;
 }
 
-template <class Net>
+// LEAKY = false compiles the leaky-ReLU arithmetic out (networks with only ReLU / no activation)
+template <class Net, bool LEAKY>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlpTrainKernel(const TrainArgs ta)
 {
     typedef F16Mma Mma;
@@ -325,8 +326,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     halfx2 z23 = __builtin_convertvector(floatx2{acc[j][t][2], acc[j][t][3]}, halfx2);
                     if (actv != kActNone) {
                         mst[l][j][t] = packMultipliers(maxGradMultiplier(z01), maxGradMultiplier(z23));
-                        const halfx2 s01 = actv == kActRelu ? zero2 : z01 * slope2;
-                        const halfx2 s23 = actv == kActRelu ? zero2 : z23 * slope2;
+                        const halfx2 s01 = (!LEAKY || actv == kActRelu) ? zero2 : z01 * slope2;
+                        const halfx2 s23 = (!LEAKY || actv == kActRelu) ? zero2 : z23 * slope2;
                         z01 = __builtin_elementwise_max(z01, s01);
                         z23 = __builtin_elementwise_max(z23, s23);
                     }
@@ -411,8 +412,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     }
                     halfx2 m01 = {(half_t)1.f, (half_t)1.f}, m23 = m01;
                     if (actl != kActNone) multipliers(mst[L - 1][j][t], m01, m23);
-                    dz[t][0] = applyActGrad(halfx2{gv[0], gv[1]}, m01, actl, slope2);
-                    dz[t][1] = applyActGrad(halfx2{gv[2], gv[3]}, m23, actl, slope2);
+                    dz[t][0] = applyActGrad<LEAKY>(halfx2{gv[0], gv[1]}, m01, actl, slope2);
+                    dz[t][1] = applyActGrad<LEAKY>(halfx2{gv[2], gv[3]}, m23, actl, slope2);
                 }
                 packS(dz, Net::MTL, Net::ktOut(L - 1), bS[j]);
             }
@@ -472,8 +473,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         const halfx2 g23 = __builtin_convertvector(floatx2{gacc[j][t][2], gacc[j][t][3]}, halfx2);
                         halfx2 m01 = {(half_t)1.f, (half_t)1.f}, m23 = m01;
                         if (actp != kActNone) multipliers(mst[l - 1][j][t], m01, m23);
-                        dz[t][0] = applyActGrad(g01, m01, actp, slope2);
-                        dz[t][1] = applyActGrad(g23, m23, actp, slope2);
+                        dz[t][0] = applyActGrad<LEAKY>(g01, m01, actp, slope2);
+                        dz[t][1] = applyActGrad<LEAKY>(g23, m23, actp, slope2);
                     }
                     packS(dz, MTI, Net::ktOut(l - 1), bS[j]);
                 }
