@@ -38,10 +38,11 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ta.lossScale = t.lossScale;
     ta.partials = t.workspace;
     const uint32_t blocks = (uint32_t)numCUs;      // one resident workgroup per compute unit
-    bool leaky = false;
-    for (int l = 0; l < Net::L; ++l) leaky = leaky || t.mlp.layers[l].act == kActLeakyRelu;
-    if (leaky) hipLaunchKernelGGL((mlpTrainKernel<Net, true>), dim3(blocks), dim3(256), 0, stream, ta);
-    else       hipLaunchKernelGGL((mlpTrainKernel<Net, false>), dim3(blocks), dim3(256), 0, stream, ta);
+    // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
+    bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
+    for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
+    if (plain) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone>), dim3(blocks), dim3(256), 0, stream, ta);
+    else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     TrainReduceArgs ra;

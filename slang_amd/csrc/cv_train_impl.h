@@ -138,13 +138,20 @@ __device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, hal
     return da + db * slope2;
 }
 
-// LEAKY = false compiles the leaky-ReLU arithmetic out (networks with only ReLU / no activation)
-template <class Net, bool LEAKY>
+// HACT / LACT fix the activation of the hidden layers / the last layer at compile time (the round
+// then is straight-line code the scheduler can interleave); -1 reads them from the arguments and
+// keeps the leaky-ReLU arithmetic.
+template <class Net, int HACT, int LACT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlpTrainKernel(const TrainArgs ta)
 {
     typedef F16Mma Mma;
     constexpr int L = Net::L;
     constexpr int FD = 4, RAW = 4, EPL = 8;
+    constexpr bool LEAKY = HACT < 0 || LACT < 0;
+    auto actOf = [&](int l) -> int {
+        const int fixed = (l + 1 < L) ? HACT : LACT;
+        return fixed >= 0 ? fixed : ta.mlp.layers[l].act;
+    };
     constexpr int IN_DW = RAW * Net::KT0;
     const MlpArgs& a = ta.mlp;
 
@@ -286,7 +293,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         staticFor<0, L>([&](auto lc) {
             constexpr int l = decltype(lc)::value;
             constexpr int MT = Net::mt(l), KT = Net::kt(l);
-            const int actv = a.layers[l].act;
+            const int actv = actOf(l);
             const half_t sl = (half_t)a.layers[l].slope;
             const halfx2 slope2 = {sl, sl};
             const halfx2 zero2 = {(half_t)0, (half_t)0};
@@ -306,14 +313,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 const floatx4 bv = {bp[0], bp[1], bp[2], bp[3]};
                 acc[0][t] = bv; acc[1][t] = bv;
             }
+            // all of the layer's A fragments are requested from LDS at once (one exposed LDS
+            // latency per layer instead of one per fragment)
+            uint32_t wf[MT][KT][4];
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
+                    wf[t][kt][0] = v.x; wf[t][kt][1] = v.y; wf[t][kt][2] = v.z; wf[t][kt][3] = v.w;
+                }
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    const uint32_t* wp = &ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
-                    const uint32_t w[4] = {wp[0], wp[1], wp[2], wp[3]};
-                    acc[0][t] = Mma::mma(w, actS[0][kt], acc[0][t]);
-                    acc[1][t] = Mma::mma(w, actS[1][kt], acc[1][t]);
+                    acc[0][t] = Mma::mma(wf[t][kt], actS[0][kt], acc[0][t]);
+                    acc[1][t] = Mma::mma(wf[t][kt], actS[1][kt], acc[1][t]);
                 }
             // carrier: round to fp16, remember the gradient multiplier of max(), apply the activation
             halfx2 car[2][MT][2];
@@ -351,6 +366,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     for (int t = 0; t < MT; ++t) { yS[j][t][0] = car[j][t][0]; yS[j][t][1] = car[j][t][1]; }
             }
         });
+#ifdef CV_TRAIN_SCHED
+        // ask the scheduler for an MFMA : VALU pipeline over the straight-line forward code
+#pragma unroll
+        for (int i = 0; i < CV_TRAIN_SCHED_FWD_N; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, CV_TRAIN_SCHED_FWD_V, 0);
+        }
+#endif
 
         // decode four multipliers
         auto multipliers = [&](uint32_t raw, halfx2& m01, halfx2& m23) {
@@ -373,7 +396,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // ---------------- loss and its gradient (S orientation) ----------------
         uint32_t bS[2][Net::KOMAX][FD];             // S fragments of dY of the current layer
         {
-            const int actl = a.layers[L - 1].act;
+            const int actl = actOf(L - 1);
             const half_t sll = (half_t)a.layers[L - 1].slope;
             const halfx2 slope2 = {sll, sll};
 #pragma unroll
@@ -448,20 +471,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             if constexpr (l > 0) {
                 // dX = W^T dY, then through the previous layer's activation
                 constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
-                const int actp = a.layers[l - 1].act;
+                const int actp = actOf(l - 1);
                 const half_t slp = (half_t)a.layers[l - 1].slope;
                 const halfx2 slope2 = {slp, slp};
                 floatx4 gacc[2][MTI];
 #pragma unroll
                 for (int t = 0; t < MTI; ++t) { gacc[0][t] = floatx4{0.f, 0.f, 0.f, 0.f}; gacc[1][t] = gacc[0][t]; }
+                uint32_t wt[MTI][KTO][4];
+#pragma unroll
+                for (int t = 0; t < MTI; ++t)
+#pragma unroll
+                    for (int kt = 0; kt < KTO; ++kt) {
+                        const u32x4 v = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
+                        wt[t][kt][0] = v.x; wt[t][kt][1] = v.y; wt[t][kt][2] = v.z; wt[t][kt][3] = v.w;
+                    }
 #pragma unroll
                 for (int kt = 0; kt < KTO; ++kt)
 #pragma unroll
                     for (int t = 0; t < MTI; ++t) {
-                        const uint32_t* wp = &ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
-                        const uint32_t w[4] = {wp[0], wp[1], wp[2], wp[3]};
-                        gacc[0][t] = Mma::mma(w, bS[0][kt], gacc[0][t]);
-                        gacc[1][t] = Mma::mma(w, bS[1][kt], gacc[1][t]);
+                        gacc[0][t] = Mma::mma(wt[t][kt], bS[0][kt], gacc[0][t]);
+                        gacc[1][t] = Mma::mma(wt[t][kt], bS[1][kt], gacc[1][t]);
                     }
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -480,6 +509,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 }
             }
         });
+#ifdef CV_TRAIN_SCHED
+#pragma unroll
+        for (int i = 0; i < CV_TRAIN_SCHED_BWD_N; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, CV_TRAIN_SCHED_BWD_V, 0);
+        }
+#endif
     };
 
     // ---- main loop: every wave strides over rounds of 32 samples; the next round's inputs are
