@@ -290,6 +290,52 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 for (int d = 0; d < FD; ++d) actS[j][kt][d] = buf[j][kt * RAW + d];
 
         // ---------------- forward ----------------
+        // The gradient multipliers of layer l are only needed in the backward pass; they are
+        // computed from the saved pre-activations while layer l+1's MFMAs execute (left alone,
+        // the scheduler sinks all of that VALU work into one serial block after the forward pass).
+        halfx2 zprev[2][Net::MTMAX][2];
+        uint32_t wbuf[Net::MTMAX][Net::KTMAX > Net::KOMAX ? Net::KTMAX : Net::KOMAX][4];   // A fragments of the layer at hand
+        uint32_t xbuf[Net::ITMAX][FD];                                                      // F fragments of its input
+        floatx4 bbuf[Net::MTMAX];                                                           // its biases (accumulator seeds)
+        auto loadW = [&](auto lc) {           // forward weights of layer l
+            constexpr int l = decltype(lc)::value;
+#pragma unroll
+            for (int t = 0; t < Net::mt(l); ++t)
+#pragma unroll
+                for (int kt = 0; kt < Net::kt(l); ++kt) {
+                    const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * Net::kt(l) + kt) * 64 + lane) * RAW];
+                    wbuf[t][kt][0] = v.x; wbuf[t][kt][1] = v.y; wbuf[t][kt][2] = v.z; wbuf[t][kt][3] = v.w;
+                }
+#pragma unroll
+            for (int t = 0; t < Net::mt(l); ++t) bbuf[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+        };
+        auto loadWT = [&](auto lc) {          // transposed weights of layer l (l >= 1)
+            constexpr int l = decltype(lc)::value;
+            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
+#pragma unroll
+            for (int t = 0; t < MTI; ++t)
+#pragma unroll
+                for (int kt = 0; kt < KTO; ++kt) {
+                    const u32x4 v = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
+                    wbuf[t][kt][0] = v.x; wbuf[t][kt][1] = v.y; wbuf[t][kt][2] = v.z; wbuf[t][kt][3] = v.w;
+                }
+        };
+        auto loadXF = [&](auto lc) {          // parked F fragments of layer l's input
+            constexpr int l = decltype(lc)::value;
+#pragma unroll
+            for (int e = 0; e < Net::nIt(l); ++e) {
+                const u32x4 v = *(const u32x4*)(myXF + (Net::xTileBase(l) + e) * 256 + lane * 4);
+                xbuf[e][0] = v.x; xbuf[e][1] = v.y; xbuf[e][2] = v.z; xbuf[e][3] = v.w;
+            }
+        };
+        loadW(std::integral_constant<int, 0>{});
+        auto multipliersOf = [&](int l, int MT) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int t = 0; t < Net::MTMAX; ++t)
+                    if (t < MT) mst[l][j][t] = packMultipliers(maxGradMultiplier(zprev[j][t][0]), maxGradMultiplier(zprev[j][t][1]));
+        };
         staticFor<0, L>([&](auto lc) {
             constexpr int l = decltype(lc)::value;
             constexpr int MT = Net::mt(l), KT = Net::kt(l);
@@ -298,38 +344,45 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             const halfx2 slope2 = {sl, sl};
             const halfx2 zero2 = {(half_t)0, (half_t)0};
             // this layer's input in F orientation, parked in LDS until the backward pass
+            {
+                // all selection MFMAs first, then the conversions: no stall on each pair's result
+                floatx4 tt[Net::nIt(l)][2];
+                const floatx4 zf = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int e = 0; e < Net::nIt(l); ++e) {
-                uint32_t f[FD];
-                toF(actS[0][e / 2], actS[1][e / 2], e & 1, f);
-                uint32_t* dst = myXF + (Net::xTileBase(l) + e) * 256 + lane * 4;
-                dst[0] = f[0]; dst[1] = f[1]; dst[2] = f[2]; dst[3] = f[3];
+                for (int e = 0; e < Net::nIt(l); ++e) {
+                    tt[e][0] = Mma::mma(actS[0][e / 2], Isel[e & 1], zf);
+                    tt[e][1] = Mma::mma(actS[1][e / 2], Isel[e & 1], zf);
+                }
+#pragma unroll
+                for (int e = 0; e < Net::nIt(l); ++e) {
+                    typedef float floatx2 __attribute__((ext_vector_type(2)));
+                    u32x4 f;
+                    f.x = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{tt[e][0][0], tt[e][0][1]}, halfx2));
+                    f.y = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{tt[e][0][2], tt[e][0][3]}, halfx2));
+                    f.z = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{tt[e][1][0], tt[e][1][1]}, halfx2));
+                    f.w = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{tt[e][1][2], tt[e][1][3]}, halfx2));
+                    *(u32x4*)(myXF + (Net::xTileBase(l) + e) * 256 + lane * 4) = f;
+                }
             }
 
             floatx4 acc[2][MT];
 #pragma unroll
             for (int t = 0; t < MT; ++t) {
-                const float* bp = &ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
-                const floatx4 bv = {bp[0], bp[1], bp[2], bp[3]};
-                acc[0][t] = bv; acc[1][t] = bv;
+                acc[0][t] = bbuf[t]; acc[1][t] = bbuf[t];
             }
-            // all of the layer's A fragments are requested from LDS at once (one exposed LDS
-            // latency per layer instead of one per fragment)
-            uint32_t wf[MT][KT][4];
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt) {
-                    const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
-                    wf[t][kt][0] = v.x; wf[t][kt][1] = v.y; wf[t][kt][2] = v.z; wf[t][kt][3] = v.w;
-                }
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-                    acc[0][t] = Mma::mma(wf[t][kt], actS[0][kt], acc[0][t]);
-                    acc[1][t] = Mma::mma(wf[t][kt], actS[1][kt], acc[1][t]);
+                    acc[0][t] = Mma::mma(wbuf[t][kt], actS[0][kt], acc[0][t]);
+                    acc[1][t] = Mma::mma(wbuf[t][kt], actS[1][kt], acc[1][t]);
                 }
+            // the MFMAs above have read wbuf: request the next layer's fragments now, so that the
+            // LDS latency is covered by this layer's VALU work (one wave per SIMD: nobody else hides it)
+            if constexpr (l + 1 < L) loadW(std::integral_constant<int, l + 1>{});
+            if constexpr (l > 0) {
+                if (actOf(l - 1) != kActNone) multipliersOf(l - 1, Net::mt(l - 1));
+            }
             // carrier: round to fp16, remember the gradient multiplier of max(), apply the activation
             halfx2 car[2][MT][2];
 #pragma unroll
@@ -340,7 +393,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     halfx2 z01 = __builtin_convertvector(floatx2{acc[j][t][0], acc[j][t][1]}, halfx2);
                     halfx2 z23 = __builtin_convertvector(floatx2{acc[j][t][2], acc[j][t][3]}, halfx2);
                     if (actv != kActNone) {
-                        mst[l][j][t] = packMultipliers(maxGradMultiplier(z01), maxGradMultiplier(z23));
+                        zprev[j][t][0] = z01; zprev[j][t][1] = z23;
                         const halfx2 s01 = (!LEAKY || actv == kActRelu) ? zero2 : z01 * slope2;
                         const halfx2 s23 = (!LEAKY || actv == kActRelu) ? zero2 : z23 * slope2;
                         z01 = __builtin_elementwise_max(z01, s01);
@@ -365,7 +418,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
                     for (int t = 0; t < MT; ++t) { yS[j][t][0] = car[j][t][0]; yS[j][t][1] = car[j][t][1]; }
             }
+            __builtin_amdgcn_sched_barrier(0);
         });
+        if (actOf(L - 1) != kActNone) multipliersOf(L - 1, Net::mt(L - 1));
 #ifdef CV_TRAIN_SCHED
         // ask the scheduler for an MFMA : VALU pipeline over the straight-line forward code
 #pragma unroll
@@ -394,6 +449,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         };
 
         // ---------------- loss and its gradient (S orientation) ----------------
+        loadXF(std::integral_constant<int, L - 1>{});
+        if constexpr (L > 1) loadWT(std::integral_constant<int, L - 1>{});
         uint32_t bS[2][Net::KOMAX][FD];             // S fragments of dY of the current layer
         {
             const int actl = actOf(L - 1);
@@ -446,13 +503,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         staticFor<0, L>([&](auto lc) {
             constexpr int l = L - 1 - decltype(lc)::value;
             constexpr int MT = Net::mt(l), NI = Net::nIt(l);
-            // this layer's input in F orientation, back from LDS
-            uint32_t xF[NI][FD];
-#pragma unroll
-            for (int e = 0; e < NI; ++e) {
-                const uint32_t* src = myXF + (Net::xTileBase(l) + e) * 256 + lane * 4;
-                xF[e][0] = src[0]; xF[e][1] = src[1]; xF[e][2] = src[2]; xF[e][3] = src[3];
-            }
             // dY in F orientation; bias gradient; weight gradient
 #pragma unroll
             for (int eo = 0; eo < MT; ++eo) {
@@ -465,7 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
                 for (int ei = 0; ei < NI; ++ei) {
                     floatx4& w = accW[Net::gradTileBase(l) + eo * NI + ei];
-                    accumulateInAgpr(w, dzF, xF[ei]);
+                    accumulateInAgpr(w, dzF, xbuf[ei]);
                 }
             }
             if constexpr (l > 0) {
@@ -477,21 +527,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 floatx4 gacc[2][MTI];
 #pragma unroll
                 for (int t = 0; t < MTI; ++t) { gacc[0][t] = floatx4{0.f, 0.f, 0.f, 0.f}; gacc[1][t] = gacc[0][t]; }
-                uint32_t wt[MTI][KTO][4];
-#pragma unroll
-                for (int t = 0; t < MTI; ++t)
-#pragma unroll
-                    for (int kt = 0; kt < KTO; ++kt) {
-                        const u32x4 v = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KTO + kt) * 64 + lane) * RAW];
-                        wt[t][kt][0] = v.x; wt[t][kt][1] = v.y; wt[t][kt][2] = v.z; wt[t][kt][3] = v.w;
-                    }
 #pragma unroll
                 for (int kt = 0; kt < KTO; ++kt)
 #pragma unroll
                     for (int t = 0; t < MTI; ++t) {
-                        gacc[0][t] = Mma::mma(wt[t][kt], bS[0][kt], gacc[0][t]);
-                        gacc[1][t] = Mma::mma(wt[t][kt], bS[1][kt], gacc[1][t]);
+                        gacc[0][t] = Mma::mma(wbuf[t][kt], bS[0][kt], gacc[0][t]);
+                        gacc[1][t] = Mma::mma(wbuf[t][kt], bS[1][kt], gacc[1][t]);
                     }
+                // next layer down: its parked input and (if it has one) its transposed weights
+                loadXF(std::integral_constant<int, l - 1>{});
+                if constexpr (l > 1) loadWT(std::integral_constant<int, l - 1>{});
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     halfx2 dz[MTI][2];
