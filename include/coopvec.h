@@ -266,6 +266,19 @@ CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp,
                                float lossScale, uint32_t batch, float* lossSum,
                                void* workspace, size_t workspaceBytes);
 
+/* ------------------------------------------------------------------------------------ */
+/* parameter update of the example                                                      */
+/* ------------------------------------------------------------------------------------ */
+
+/* Replaces the adjustParameters dispatch (examples/mlp-training-coopvec/kernels.slang:29-45,
+ * AdamOptimizer::step adam.slang:20-36, host side mlp-training-coopvec.cpp:238-250) over `count`
+ * fp16 parameters: `states` are AdamState records {half mean; half variance; int iteration}
+ * (8 bytes each), `gradients` fp16 (zeroed by the call; NaN gradients are cleared and skipped,
+ * infinite ones taken as +-10000).  All arithmetic in half, as the Slang source spells it.
+ * The example's constants: beta1 0.9, beta2 0.999, epsilon 1e-7, learningRate 0.01. */
+CV_API CvResult cvAdamStep(void* stream, void* states, void* params, void* gradients, uint32_t count,
+                           float beta1, float beta2, float epsilon, float learningRate);
+
 #ifdef __cplusplus
 }
 #endif

@@ -852,3 +852,35 @@ int cvo_ref_mlp_train(const CvoLayer* layers, int numLayers,
     free(W);
     return 0;
 }
+
+/* ===================================================================================== */
+/* Adam (examples/mlp-training-coopvec/adam.slang:20-36, kernels.slang:29-45)            */
+/* ===================================================================================== */
+
+void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
+                         float beta1f, float beta2f, float epsf, float lrf, int halfMode)
+{
+#define H(x) cvo_f16_to_f32(to_half((x), halfMode))     /* one rounding to half */
+    const float beta1 = H(beta1f), beta2 = H(beta2f), eps = H(epsf), lr = H(lrf);
+    for (uint32_t i = 0; i < count; ++i) {
+        float g = cvo_f16_to_f32(grads[i]);
+        if (g != g) { grads[i] = 0; continue; }                       /* kernels.slang:39-43 */
+        CvoAdamState* st = &states[i];
+        st->iteration++;
+        if (isinf(g)) g = g > 0 ? H(10000.0f) : H(-10000.0f);          /* adam.slang:23-29 */
+        float mean = cvo_f16_to_f32(st->mean), var = cvo_f16_to_f32(st->variance);
+        const float omb1 = H(1.0f - beta1), omb2 = H(1.0f - beta2);
+        mean = H(H(beta1 * mean) + H(omb1 * g));
+        var = H(H(beta2 * var) + H(H(omb2 * g) * g));
+        const float it = H((float)st->iteration);
+        const float meanHat = H(mean / H(1.0f - H(powf(beta1, it))));
+        const float varHat = H(var / H(1.0f - H(powf(beta2, it))));
+        const float denom = H(sqrtf(H(fmaxf(0.0f, varHat) + eps)));
+        const float p = cvo_f16_to_f32(params[i]);
+        params[i] = to_half(p - H(H(lr * meanHat) / denom), halfMode);
+        st->mean = to_half(mean, halfMode);
+        st->variance = to_half(var, halfMode);
+        grads[i] = 0;
+    }
+#undef H
+}

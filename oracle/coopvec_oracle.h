@@ -157,6 +157,17 @@ int cvo_layout_convert(void* dst, uint32_t rows, uint32_t cols, int dstCt, int d
                        size_t dstStride, const void* src, int srcCt, int srcLayout,
                        size_t srcStride);
 
+/* ---- Adam parameter update (examples/mlp-training-coopvec) ----------------------------- */
+/* AdamState of adam.slang:5-10: { half mean; half variance; int iteration } = 8 bytes. */
+typedef struct CvoAdamState { uint16_t mean, variance; int32_t iteration; } CvoAdamState;
+/* One dispatch of adjustParameters (kernels.slang:29-45) + AdamOptimizer::step (adam.slang:20-36)
+ * over `count` fp16 parameters: every operation in half (each result rounded), NaN gradients are
+ * cleared and skipped, infinite ones replaced by +-10000, the gradient is zeroed afterwards.
+ * PARITY UNPINNED against the reference (it has no golden for the optimizer); pinned by the
+ * closed form of the first steps. */
+void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
+                         float beta1, float beta2, float epsilon, float learningRate, int halfMode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -440,3 +440,27 @@ def coopVecReduceSumAccumulate(v: torch.Tensor, buffer: torch.Tensor, offset: in
     _check(lib.cvReduceSumAccumulate(_stream_handle(stream), v.data_ptr(), sv, n, int(tv), batch,
                                      _buffer_ptr(buffer, "buffer"), int(offset), int(bufferType),
                                      workspace.data_ptr(), workspace.numel() * workspace.element_size()))
+
+
+# ---------------------------------------------------------------------------------------------
+# parameter update of the example
+# ---------------------------------------------------------------------------------------------
+
+ADAM_STATE_BYTES = 8    # {half mean; half variance; int iteration}, adam.slang:5-10
+
+
+def adjustParameters(adamStates: torch.Tensor, params: torch.Tensor, gradients: torch.Tensor, count: Optional[int] = None,
+                     *, beta1: float = 0.9, beta2: float = 0.999, epsilon: float = 1e-7, learningRate: float = 0.01,
+                     stream=None) -> None:
+    """The adjustParameters kernel of the example (kernels.slang:29-45): one Adam step in half on
+    `count` fp16 parameters; gradients are zeroed.  adamStates: raw bytes, 8 per parameter."""
+    if count is None:
+        count = params.numel()
+    if params.dtype != torch.float16 or gradients.dtype != torch.float16:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "params and gradients must be fp16")
+    if (adamStates.numel() * adamStates.element_size() < count * ADAM_STATE_BYTES or params.numel() < count
+            or gradients.numel() < count):
+        raise CoopVecError(SLANG_E_BUFFER_TOO_SMALL, "buffers smaller than count")
+    _check(_lib.load().cvAdamStep(_stream_handle(stream), _buffer_ptr(adamStates, "adamStates"),
+                                  _buffer_ptr(params, "params"), _buffer_ptr(gradients, "gradients"), int(count),
+                                  beta1, beta2, epsilon, learningRate))

@@ -8,6 +8,7 @@
 #include <mutex>
 
 #include "../../include/coopvec.h"
+#include "cv_error.h"
 #include "cv_kernels.h"
 
 namespace {
@@ -77,6 +78,17 @@ const Combo kCombos[] = {
 constexpr uint32_t kNumCombos = sizeof(kCombos) / sizeof(kCombos[0]);
 
 } // namespace
+
+namespace cv {
+CvResult failWith(CvResult code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(tlsError, sizeof(tlsError), fmt, ap);
+    va_end(ap);
+    return code;
+}
+} // namespace cv
 
 extern "C" {
 

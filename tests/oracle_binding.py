@@ -203,3 +203,17 @@ def float_parity_violations(got_f16: np.ndarray, ref_f32: np.ndarray, abs_terms:
     if abs_terms is not None:
         tol = np.maximum(tol, abs_terms * np.float32(2.0 ** -18))
     return err > tol
+
+
+# ---- Adam ---------------------------------------------------------------------------------
+ADAM_STATE_DTYPE = np.dtype([("mean", np.uint16), ("variance", np.uint16), ("iteration", np.int32)])
+
+
+def slang_adam_step(states: np.ndarray, params: np.ndarray, grads: np.ndarray, beta1=0.9, beta2=0.999,
+                    epsilon=1e-7, lr=0.01, half_mode=HALF_RNE):
+    """In-place restatement of adjustParameters + AdamOptimizer::step on numpy arrays
+    (states: ADAM_STATE_DTYPE, params/grads: float16)."""
+    L = lib()
+    L.cvo_slang_adam_step.argtypes = [_vp, _vp, _vp, _u32, _f32, _f32, _f32, _f32, _c.c_int]
+    L.cvo_slang_adam_step.restype = None
+    L.cvo_slang_adam_step(ptr(states), ptr(params), ptr(grads), len(params), beta1, beta2, epsilon, lr, half_mode)
