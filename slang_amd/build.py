@@ -81,6 +81,17 @@ def build_library(jobs: int = 8, verbose: bool = False) -> str:
     return LIB_PATH
 
 
+HOST_SRC = os.path.join(PKG_DIR, "host", "mlp_training_host.cpp")
+HOST_BIN = os.path.join(PKG_DIR, "host", "mlp_training_host")
+
+
+def build_host_example() -> str:
+    """Compile the host program that trains the example network through the C-ABI."""
+    _run([_hipcc(), "-O2", "-std=c++17", "-I", os.path.join(REPO_DIR, "include"), HOST_SRC, "-o", HOST_BIN,
+          "-L", PKG_DIR, "-l:" + LIB_NAME, "-Wl,-rpath,$ORIGIN/.."])
+    return HOST_BIN
+
+
 def build_oracle() -> str:
     """Compile the CPU oracle (test infrastructure) with the host C compiler."""
     _run(["make", "-C", ORACLE_DIR, "-B", "libcoopvec_oracle.so"])
@@ -94,6 +105,7 @@ def main(argv=None) -> int:
     ap.add_argument("-v", "--verbose", action="store_true")
     args = ap.parse_args(argv)
     print(build_library(args.jobs, args.verbose))
+    print(build_host_example())
     if args.oracle:
         print(build_oracle())
     return 0

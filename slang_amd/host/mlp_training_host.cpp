@@ -1,0 +1,183 @@
+// mlp_training_host.cpp -- host program that trains the example's 4 -> 16 -> 4 network on MI355X
+// through the C-ABI of include/coopvec.h.
+//
+// Counterpart of examples/mlp-training-coopvec/mlp-training-coopvec.cpp (execute(), :76-262): the
+// same three-segment parameter buffer with 64-byte sub-allocations (:92-126, :265-315), the same
+// seeded initialisation (srand(1072), rand(), the reference's float->half rule, :128-137,
+// :400-425), the same 16 samples (:163-170) and the same per-iteration order (:178-260):
+//   clear the training-optimal gradient segment -> learnGradient -> convert TrainingOptimal to
+//   RowMajor -> adjustParameters (Adam) -> every 10 iterations read back the loss.
+// What the Slang kernels do per thread is done here by cvMlpTrainStep / cvConvertMatrices /
+// cvAdamStep.  The input encoding (x, y, x^2, y^2) (network.slang:35-38) and the ground truth
+// (network.slang:67-75) are evaluated on the host in half, as the shader would.
+//
+//   mlp_training_host [iterations=1000]
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "coopvec.h"
+
+typedef _Float16 NFloat;
+
+static const int kLayerSizes[] = {4, 16, 4};
+static const int kLayerCount = sizeof(kLayerSizes) / sizeof(int) - 1;
+
+#define HIP_OK(x)                                                                      \
+    do {                                                                               \
+        hipError_t e_ = (x);                                                           \
+        if (e_ != hipSuccess) {                                                        \
+            fprintf(stderr, "%s failed: %s\n", #x, hipGetErrorString(e_));             \
+            return 1;                                                                  \
+        }                                                                              \
+    } while (0)
+#define CV_OK_OR_FAIL(x)                                                               \
+    do {                                                                               \
+        CvResult r_ = (x);                                                             \
+        if (CV_FAILED(r_)) {                                                           \
+            fprintf(stderr, "%s failed: %s\n", #x, cvGetLastErrorMessage());           \
+            return 1;                                                                  \
+        }                                                                              \
+    } while (0)
+
+struct LayerAllocation {
+    size_t weightsOffset, weightsSize, biasOffset, biasSize;
+    size_t weightsGradOffset, biasGradOffset, weightsGradTrainingOffset, weightsGradTrainingSize;
+};
+
+// The reference initialises its parameters with this float -> half rule (guard bit added back:
+// ties away from zero, everything below 2^-24 flushed), not with IEEE nearest-even.
+static uint16_t referenceFloatToHalf(float value)
+{
+    uint32_t in;
+    memcpy(&in, &value, 4);
+    uint32_t out = (in >> 16) & 0x8000u;
+    uint32_t mant = (in >> 12) & 0x07ffu;
+    const uint32_t expo = (in >> 23) & 0xffu;
+    if (expo < 103u) return (uint16_t)out;
+    if (expo > 142u) return (uint16_t)(out | 0x7c00u | (uint32_t)(expo == 255u && (in & 0x007fffffu)));
+    if (expo < 113u) {
+        mant |= 0x0800u;
+        return (uint16_t)(out | ((mant >> (114u - expo)) + ((mant >> (113u - expo)) & 1u)));
+    }
+    out |= ((expo - 112u) << 10) | (mant >> 1);
+    return (uint16_t)(out + (mant & 1u));
+}
+
+int main(int argc, char** argv)
+{
+    const int iterations = argc > 1 ? atoi(argv[1]) : 1000;
+
+    // ---- buffer plan: | weights_i bias_i ... | row-major grads ... | training-optimal weight grads |
+    std::vector<LayerAllocation> layers(kLayerCount);
+    size_t bufferSize = 0;
+    auto alloc64 = [&](size_t size) {
+        const size_t offset = bufferSize;
+        bufferSize += (size + 63) / 64 * 64;
+        return offset;
+    };
+    for (int i = 0; i < kLayerCount; i++) {
+        layers[i].weightsSize = (size_t)kLayerSizes[i] * kLayerSizes[i + 1] * sizeof(NFloat);
+        layers[i].weightsOffset = alloc64(layers[i].weightsSize);
+        layers[i].biasSize = (size_t)kLayerSizes[i + 1] * sizeof(NFloat);
+        layers[i].biasOffset = alloc64(layers[i].biasSize);
+    }
+    const size_t gradientOffset = bufferSize;
+    for (int i = 0; i < kLayerCount; i++) {
+        layers[i].weightsGradOffset = alloc64(layers[i].weightsSize);
+        layers[i].biasGradOffset = alloc64(layers[i].biasSize);
+    }
+    const size_t gradientTrainingOffset = bufferSize;
+    for (int i = 0; i < kLayerCount; i++) {
+        CV_OK_OR_FAIL(cvGetMatrixSize(kLayerSizes[i + 1], kLayerSizes[i], CV_FLOAT16, CV_LAYOUT_TRAINING_OPTIMAL, 0,
+                                      &layers[i].weightsGradTrainingSize));
+        layers[i].weightsGradTrainingOffset = alloc64(layers[i].weightsGradTrainingSize);
+    }
+
+    // ---- seeded initial contents, in the reference's order: parameters first, then the inputs
+    std::vector<uint16_t> initParams;
+    srand(1072);
+    for (size_t i = 0; i < bufferSize / sizeof(NFloat); i++)
+        initParams.push_back(referenceFloatToHalf(rand() / (float)RAND_MAX * 2.0f - 1.0f));
+    const int inputCount = 32, sampleCount = inputCount / 2;
+    std::vector<float> inputData;
+    for (int i = 0; i < inputCount; i++) inputData.push_back(rand() / (float)RAND_MAX);
+
+    std::vector<NFloat> encoded(sampleCount * 4), targets(sampleCount * 4);
+    for (int s = 0; s < sampleCount; s++) {
+        const NFloat x = (NFloat)inputData[2 * s], y = (NFloat)inputData[2 * s + 1];
+        const NFloat one = (NFloat)1, two = (NFloat)2, half = (NFloat)0.5f, c12 = (NFloat)1.2f;
+        encoded[4 * s + 0] = x; encoded[4 * s + 1] = y; encoded[4 * s + 2] = x * x; encoded[4 * s + 3] = y * y;
+        targets[4 * s + 0] = (x + y) / (one + y * y);
+        targets[4 * s + 1] = two * x + y;
+        targets[4 * s + 2] = half * x * x + c12 * y;
+        targets[4 * s + 3] = x + half * y * y;
+    }
+
+    uint8_t* params = nullptr;
+    void *adamStates = nullptr, *dEncoded = nullptr, *dTargets = nullptr, *workspace = nullptr;
+    float* dLoss = nullptr;
+    const size_t paramCount = bufferSize / sizeof(NFloat);
+    HIP_OK(hipMalloc((void**)&params, bufferSize));
+    HIP_OK(hipMemcpy(params, initParams.data(), bufferSize, hipMemcpyHostToDevice));
+    HIP_OK(hipMalloc(&adamStates, paramCount * 8));
+    HIP_OK(hipMemset(adamStates, 0, paramCount * 8));
+    HIP_OK(hipMalloc(&dEncoded, encoded.size() * 2));
+    HIP_OK(hipMemcpy(dEncoded, encoded.data(), encoded.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMalloc(&dTargets, targets.size() * 2));
+    HIP_OK(hipMemcpy(dTargets, targets.data(), targets.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMalloc((void**)&dLoss, sizeof(float)));
+    // the gradient segments start from zero (the reference's random fill there would be noise)
+    HIP_OK(hipMemset(params + gradientOffset, 0, bufferSize - gradientOffset));
+
+    // ---- the network: per layer {weights, weightsGrad, biases, biasesGrad} like :146-158
+    CvMlpLayer net[kLayerCount];
+    CvMatrixDesc srcDescs[kLayerCount], dstDescs[kLayerCount];
+    for (int i = 0; i < kLayerCount; i++) {
+        memset(&net[i], 0, sizeof(net[i]));
+        net[i].weights = params + layers[i].weightsOffset;
+        net[i].weightsGrad = params + layers[i].weightsGradTrainingOffset;
+        net[i].biases = params + layers[i].biasOffset;
+        net[i].biasesGrad = params + layers[i].biasGradOffset;
+        net[i].inputSize = kLayerSizes[i];
+        net[i].outputSize = kLayerSizes[i + 1];
+        net[i].weightLayout = CV_LAYOUT_ROW_MAJOR;
+        net[i].weightStride = kLayerSizes[i] * sizeof(NFloat);
+        net[i].gradLayout = CV_LAYOUT_TRAINING_OPTIMAL;
+        net[i].activation = CV_ACT_LEAKY_RELU;              // max(z, z * 0.001h), fflayer.slang:63-65
+        net[i].leakySlope = (float)(NFloat)0.001f;
+        srcDescs[i] = CvMatrixDesc{(uint32_t)kLayerSizes[i + 1], (uint32_t)kLayerSizes[i], CV_FLOAT16,
+                                   CV_LAYOUT_TRAINING_OPTIMAL, layers[i].weightsGradTrainingSize,
+                                   layers[i].weightsGradTrainingOffset, 0};
+        dstDescs[i] = CvMatrixDesc{(uint32_t)kLayerSizes[i + 1], (uint32_t)kLayerSizes[i], CV_FLOAT16,
+                                   CV_LAYOUT_ROW_MAJOR, layers[i].weightsSize, layers[i].weightsGradOffset,
+                                   (size_t)kLayerSizes[i] * sizeof(NFloat)};
+    }
+    CvMlpDesc mlp = {net, kLayerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0};
+    size_t workspaceBytes = 0;
+    CV_OK_OR_FAIL(cvMlpTrainStepWorkspaceSize(&mlp, sampleCount, &workspaceBytes));
+    HIP_OK(hipMalloc(&workspace, workspaceBytes));
+
+    hipStream_t stream = nullptr;
+    for (int k = 0; k < iterations; k++) {
+        HIP_OK(hipMemsetAsync(params + gradientTrainingOffset, 0, bufferSize - gradientTrainingOffset, stream));
+        CV_OK_OR_FAIL(cvMlpTrainStep(stream, &mlp, dEncoded, 4 * sizeof(NFloat), dTargets, 4 * sizeof(NFloat), 1.0f,
+                                     sampleCount, dLoss, workspace, workspaceBytes));
+        CV_OK_OR_FAIL(cvConvertMatrices(stream, params, dstDescs, params, srcDescs, kLayerCount));
+        CV_OK_OR_FAIL(cvAdamStep(stream, adamStates, params, params + gradientOffset,
+                                 (uint32_t)((gradientTrainingOffset - gradientOffset) / sizeof(NFloat)), 0.9f, 0.999f,
+                                 1e-7f, 0.01f));
+        if ((k + 1) % 10 == 0) {
+            float loss = 0.f;
+            HIP_OK(hipStreamSynchronize(stream));
+            HIP_OK(hipMemcpy(&loss, dLoss, sizeof(float), hipMemcpyDeviceToHost));
+            printf("Loss after %d iterations: %f\n", k + 1, loss / sampleCount);
+        }
+    }
+    HIP_OK(hipDeviceSynchronize());
+    return 0;
+}

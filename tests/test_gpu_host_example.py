@@ -1,0 +1,28 @@
+"""Runs the C++ host program (slang_amd/host/mlp_training_host.cpp), the counterpart of
+examples/mlp-training-coopvec/mlp-training-coopvec.cpp, end to end on the GPU: buffer plan, seeded
+init, 1000 x (clear, learnGradient, convert, Adam); the loss it prints must come down."""
+import os
+import re
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(REPO, "slang_amd", "host", "mlp_training_host")
+
+
+def test_example_training_loop_converges():
+    if not os.path.exists(BIN):
+        pytest.skip("host example not built (python -m slang_amd.build)")
+    out = subprocess.run([BIN, "1000"], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr
+    losses = [float(m.group(2)) for m in re.finditer(r"Loss after (\d+) iterations: ([0-9.eE+-]+|nan|inf)", out.stdout)]
+    assert len(losses) == 100
+    assert all(l == l and l < 1e6 for l in losses), losses[:5]
+    first, last = losses[0], min(losses[-10:])
+    print("loss", first, "->", last)
+    assert last < 0.25 * first, (first, last)
+    # bitwise reproducible: the deterministic gradient reduction makes the whole run repeat exactly
+    out2 = subprocess.run([BIN, "200"], capture_output=True, text=True, timeout=120)
+    assert out2.stdout.splitlines() == out.stdout.splitlines()[:20]
