@@ -32,7 +32,13 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
 # kernel of known size); the summaries are in profiles/.  None where not measured.
-MEASURED_TRAFFIC_BYTES = {"c2": 1074875000}   # profiles/matmul_f16_64x64_batch4M.md
+MEASURED_TRAFFIC_BYTES = {
+    "c2": 1074875000,    # profiles/matmul_f16_64x64_batch4M.md
+    "c3": 2685218000,    # profiles/matmul_i8_128x128_batch4M.md
+    "c4": 805497000,     # profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md
+    "c4n": 805497000,
+    "c5": 32583000,      # profiles/mlp_train_8-64x4-1_batch1M.md (training kernel only)
+}
 
 
 def ensure_built():
