@@ -503,8 +503,9 @@ CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* i
     const uint32_t gEsz = cv::elemSize(mlp->gradType);
     for (int l = 0; l < L; ++l) {
         const CvMlpLayer& ly = mlp->layers[l];
-        if (ly.leakySlope < 0.f || ly.leakySlope >= 1.f)
-            if (ly.activation == CV_ACT_LEAKY_RELU) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: leakySlope must be in [0,1)", l);
+        // with 0 <= slope <= 0.5 the outcome of max(z, z*slope) is the sign of z for every fp16 z
+        if (ly.activation == CV_ACT_LEAKY_RELU && !(ly.leakySlope >= 0.f && ly.leakySlope <= 0.5f))
+            return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: leakySlope must be in [0, 0.5]", l);
         t.wGrad[l] = (uint8_t*)ly.weightsGrad;
         t.bGrad[l] = (uint8_t*)ly.biasesGrad;
         if (ly.weightsGrad) {
