@@ -111,7 +111,7 @@ def workload_c2(torch, cv, steps, warmup):
                           "fallback (fp16 accumulate, software half as gcc<12 selects), -O2" % (n, per_core)}
 
     return dict(step=step, samples=B, alg_bytes=B * (K * 2 + M * 2), alg_flops=B * 2 * M * K,
-                bound="hbm", dtype="f16", kernel="matmulKernel<F16Mma,4,2,4,half>",
+                bound="hbm", dtype="f16", kernel="matmulKernel<F16Mma,4,2,2,half,FAST>",
                 config={"workload": "c2: fp16 coopVecMatMulAdd 64x64, batch 2^22, InferencingOptimal weights, "
                                     "fp32 accumulate, fp16 out", "batch": B, "m": M, "k": K,
                         "layout": "InferencingOptimal"},

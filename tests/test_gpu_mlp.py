@@ -175,3 +175,29 @@ def test_mlp_argument_validation():
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), x)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+def test_full_size_e4m3_decoder():
+    # batch 2^24 of the 32 -> 64 -> 64 -> 8 e4m3 decoder: sampled oracle check, layout equality,
+    # determinism, and agreement of the two halves with one full launch (tiling independence)
+    B = 1 << 24
+    rng = np.random.default_rng(77)
+    specs = make_net(rng, [32, 64, 64, 8], CT.FloatE4M3, bias="none", init="half")
+    g = torch.Generator(device=DEV); g.manual_seed(77)
+    x = (torch.randn(B, 32, device=DEV, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    lo = gpu_layers(specs, CT.FloatE4M3, ML.InferencingOptimal)
+    lr = gpu_layers(specs, CT.FloatE4M3, ML.RowMajor)
+    y1 = cv.mlpForward(lo, x, weightType=CT.FloatE4M3)
+    y2 = cv.mlpForward(lr, x, weightType=CT.FloatE4M3)
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    y3 = cv.mlpForward(lo, x, weightType=CT.FloatE4M3)
+    assert torch.equal(y1.view(torch.int16), y3.view(torch.int16))
+    half = B // 2 + 48          # an offset that is not a multiple of the kernel's slot size
+    ya = cv.mlpForward(lo, x[:half], weightType=CT.FloatE4M3)
+    yb = cv.mlpForward(lo, x[half:], weightType=CT.FloatE4M3)
+    assert torch.equal(y1[:half].view(torch.int16), ya.view(torch.int16))
+    assert torch.equal(y1[half:].view(torch.int16), yb.view(torch.int16))
+    idx = torch.from_numpy(np.concatenate([rng.integers(0, B, 8192), [0, 1, B - 2, B - 1]])).to(DEV)
+    xs = x[idx].view(torch.uint8).cpu().numpy()
+    frac, _ = end_to_end_ok(y1[idx].cpu().numpy(), specs, xs, ob.E4M3)
+    assert frac >= 0.999, frac

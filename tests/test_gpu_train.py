@@ -188,3 +188,39 @@ def test_train_argument_validation():
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpTrainStepWorkspaceSize(build(specs), 10)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+def test_full_size_training_step_properties():
+    # the training configuration at its full batch (2^20): bitwise determinism, scaling of the
+    # gradients with the loss scale, and agreement with the oracle on a leading slice
+    rng = np.random.default_rng(2020)
+    dims = [8, 64, 64, 64, 64, 1]
+    B = 1 << 20
+    specs = make_specs(rng, dims, bias=False)
+    g = torch.Generator(device=DEV); g.manual_seed(5)
+    x = (torch.rand(B, 8, device=DEV, generator=g) * 2 - 1).half()
+    la, lb, lc = build(specs), build(specs), build(specs)
+    _, loss_a = cv.mlpTrainStep(la, x, None)
+    _, loss_b = cv.mlpTrainStep(lb, x, None)
+    cv.mlpTrainStep(lc, x, None, lossScale=0.5)
+    for a, b, c in zip(la, lb, lc):
+        assert torch.equal(a.weightsGrad, b.weightsGrad) and torch.equal(a.biasesGrad, b.biasesGrad)
+        # scaling is exact except where a carrier gradient is subnormal in fp16
+        fa, fc = a.weightsGrad.view(torch.float32), c.weightsGrad.view(torch.float32)
+        assert (fa * 0.5 - fc).norm().item() <= 1e-3 * fc.norm().item()
+    assert loss_a.item() == loss_b.item()
+    # the first 4096 samples against the fp64 oracle (same kernel, smaller batch)
+    n = 4096
+    ls = build(specs)
+    cv.mlpTrainStep(ls, x[:n], None)
+    dW, dB = read_grads(ls, specs, CT.Float32, ML.RowMajor)
+    rW, rB, _ = ob.ref_mlp_train(specs, x[:n].cpu().numpy(), None, 1.0, True)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3
+    # additivity over a split of the batch (fp32 sums in a different order: relative 1e-5)
+    l1, l2 = build(specs), build(specs)
+    cv.mlpTrainStep(l1, x[: B // 2], None)
+    cv.mlpTrainStep(l1, x[B // 2:], None)        # "+=" into the same buffers
+    for a, s in zip(la, l1):
+        fa, fs = a.weightsGrad.view(torch.float32), s.weightsGrad.view(torch.float32)
+        assert (fa - fs).norm().item() <= 1e-5 * fa.norm().item()
