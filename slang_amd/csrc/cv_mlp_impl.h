@@ -351,14 +351,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 }
 
 #ifndef CV_MLP_PREFETCH_DW
-#define CV_MLP_PREFETCH_DW 16     // input dwords per lane held in flight per buffer
+#define CV_MLP_PREFETCH_DW 8      // input dwords per lane held in flight per buffer
 #endif
 
 template <class Mma, class Net>
 hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     // tiles pushed through the layers together (independent MFMA chains), limited by registers
-    constexpr int NT = (Net::totalFrags * Mma::kFD <= 32) ? 4 : 2;
+    // (with all weights in registers, wide networks run faster with one tile per round and a
+    // second wave on the SIMD than with two tiles and a single wave: 63 us vs 79 us for 8-64x4-1)
+    constexpr int NT = (Net::totalFrags * Mma::kFD <= 32) ? 4 : (Net::totalFrags * Mma::kFD <= 64 ? 2 : 1);
     constexpr int IN_DW = Mma::kRawDW * Net::KT0;
     constexpr int S0 = CV_MLP_PREFETCH_DW / IN_DW;
     constexpr int S = S0 < NT ? NT : (S0 > 16 ? 16 : S0 / NT * NT);
