@@ -452,11 +452,11 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     if (CV_FAILED(rc)) return rc;
     cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16
                      : (mlp->flags & CV_FLAG_FP8_MATRIX_PIPELINE) ? cv::MmaKind::Fp8Native : cv::MmaKind::Fp8AsF16;
-    const hipError_t e = cv::launchMlpForward((hipStream_t)stream, kind, a, cus);
+    hipError_t e = cv::launchMlpForward((hipStream_t)stream, kind, a, cus);
+    if (e == hipErrorInvalidValue) e = cv::launchMlpGeneric((hipStream_t)stream, kind, a, cus);   // no built-in shape: general kernel
     if (e == hipErrorInvalidValue)
-        return fail(CV_E_NOT_AVAILABLE, "cvMlpForward: no fused specialisation for these layer sizes "
-                    "(needs equal-width hidden layers of at most 64 and one of the built-in tile shapes); "
-                    "chain cvMatMul calls instead");
+        return fail(CV_E_NOT_AVAILABLE, "cvMlpForward: layer sizes beyond the fused kernels (every dimension must be <= 128 "
+                    "and all weights must fit 144 KB of LDS); chain cvMatMul calls instead");
     return fromHip(e, "cvMlpForward launch");
 }
 

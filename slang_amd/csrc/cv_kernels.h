@@ -53,6 +53,8 @@ struct MlpArgs {
 };
 // hipErrorInvalidValue when no built-in specialisation covers the layer shapes
 hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
+// any layer sizes up to 128 (weights read from LDS); hipErrorInvalidValue beyond that
+hipError_t launchMlpGeneric(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 
 // ---- fused training step ------------------------------------------------------------------
 struct TrainLaunch {

@@ -170,11 +170,37 @@ def test_mlp_argument_validation():
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpForward(layers, x)
     assert e.value.result == cv.SLANG_E_INVALID_ARG
-    # hidden layers of different tile widths have no fused specialisation
-    specs = make_net(rng, [8, 16, 64, 4], CT.Float16)
+    # beyond 128 wide there is no fused kernel
+    specs = make_net(rng, [8, 144, 4], CT.Float16)
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), x)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+@pytest.mark.parametrize("wtype", [CT.Float16, CT.FloatE4M3])
+@pytest.mark.parametrize("dims", [[8, 16, 64, 4], [100, 128, 96, 50, 3], [5, 7], [33, 17, 128, 128, 1], [64, 128, 128, 16]])
+def test_general_kernel_for_arbitrary_shapes(dims, wtype):
+    # no built-in tile shape matches these: the general kernel (weights in LDS, run-time sizes)
+    if len(dims) == 2:
+        dims = dims + [dims[-1]]
+    rng = np.random.default_rng(sum(dims) + int(wtype))
+    B = 777
+    act = Activation.LeakyReLU if wtype == CT.Float16 else Activation.ReLU
+    specs = make_net(rng, dims, wtype, act=act, slope=float(np.float16(0.01)), bias="rand",
+                     init="he" if wtype == CT.Float16 else "half")
+    if wtype == CT.Float16:
+        x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+        xd = to_dev(x); xct = ob.F16
+    else:
+        x = ob.encode_e4m3(rng.standard_normal((B, dims[0])) * 0.5)
+        xd = to_dev(x); xct = ob.E4M3
+    for layout in (ML.RowMajor, ML.InferencingOptimal):
+        y = cv.mlpForward(gpu_layers(specs, wtype, layout), xd, weightType=wtype)
+        yc = chain_of_single_layers(specs, xd, wtype)
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    # deeper and wider chains give more hidden units a chance to sit on a rounding boundary
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, xct)
+    assert frac >= 0.99
 
 
 def test_full_size_e4m3_decoder():
