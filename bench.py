@@ -31,13 +31,13 @@ HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
-# kernel of known size); the summaries are in profiles/.  None where not measured.
+# kernel of known size).  None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "c2": 1074875000,    # profiles/matmul_f16_64x64_batch4M.md
-    "c3": 2685218000,    # profiles/matmul_i8_128x128_batch4M.md
-    "c4": 805497000,     # profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md
+    "c2": 1074875000,
+    "c3": 2685218000,
+    "c4": 805497000,
     "c4n": 805497000,
-    "c5": 32583000,      # profiles/mlp_train_8-64x4-1_batch1M.md (training kernel only)
+    "c5": 32583000,      # training kernel only
 }
 
 
@@ -116,11 +116,6 @@ def workload_c2(torch, cv, steps, warmup):
                                     "fp32 accumulate, fp16 out", "batch": B, "m": M, "k": K,
                         "layout": "InferencingOptimal"},
                 extra={"layout_conversion_us": conv_us}, cpu_baseline=cpu_baseline, key="c2")
-
-
-def _time_cpu(fn, per_item, n):
-    t0 = time.perf_counter(); fn(); t1 = time.perf_counter()
-    return n / (t1 - t0)
 
 
 def workload_c3(torch, cv, steps, warmup):
@@ -330,8 +325,8 @@ def main(argv=None) -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (the path is data-parallel over samples; "
-              "see DESIGN.md for how it would shard); use --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (the path is data-parallel over samples: a batch "
+              "shards with replicated weights and one all-reduce of the gradients); use --gpus 1", file=sys.stderr)
         return 2
     ensure_built()
     import torch

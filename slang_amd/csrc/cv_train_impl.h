@@ -421,14 +421,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             __builtin_amdgcn_sched_barrier(0);
         });
         if (actOf(L - 1) != kActNone) multipliersOf(L - 1, Net::mt(L - 1));
-#ifdef CV_TRAIN_SCHED
-        // ask the scheduler for an MFMA : VALU pipeline over the straight-line forward code
-#pragma unroll
-        for (int i = 0; i < CV_TRAIN_SCHED_FWD_N; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, CV_TRAIN_SCHED_FWD_V, 0);
-        }
-#endif
 
         // decode four multipliers
         auto multipliers = [&](uint32_t raw, halfx2& m01, halfx2& m23) {
@@ -554,13 +546,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 }
             }
         });
-#ifdef CV_TRAIN_SCHED
-#pragma unroll
-        for (int i = 0; i < CV_TRAIN_SCHED_BWD_N; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, CV_TRAIN_SCHED_BWD_V, 0);
-        }
-#endif
     };
 
     // ---- main loop: every wave strides over rounds of 32 samples; the next round's inputs are
