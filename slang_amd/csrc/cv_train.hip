@@ -1,5 +1,5 @@
 // cv_train.hip -- instantiations and launcher of the fused fp16 training step.
-#include "cv_train_pipe.h"
+#include "cv_train_impl.h"
 
 namespace cv {
 
@@ -41,15 +41,8 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
-    // wide ReLU networks of three to five layers run as a pipeline of waves (cv_train_pipe.h)
-    constexpr bool pipeShape = Net::HT == 4 && Net::MTL == 1 && Net::L >= 3 && Net::L <= 5;
-    if constexpr (pipeShape) {
-        if (plain) hipLaunchKernelGGL((mlpTrainPipeKernel<Net>), dim3(blocks), dim3(64 * kPipeWaves), 0, stream, ta);
-        else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
-    } else {
-        if (plain) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone>), dim3(blocks), dim3(256), 0, stream, ta);
-        else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
-    }
+    if (plain) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone>), dim3(blocks), dim3(256), 0, stream, ta);
+    else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     TrainReduceArgs ra;
