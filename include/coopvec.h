@@ -266,6 +266,21 @@ CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp,
                                float lossScale, uint32_t batch, float* lossSum,
                                void* workspace, size_t workspaceBytes);
 
+/* cvMlpTrainStep for callers that cannot allocate device memory or carry a workspace around:
+ * code under HIP graph capture, tight training loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  Same arguments, kernels and results (bit for bit) as
+ * cvMlpTrainStep, but the per-workgroup gradient partials go to an array of
+ * CV_NOALLOC_SCRATCH_BYTES that is part of the library's device image (every GPU the library
+ * runs on holds one copy until the process ends).  Networks whose partials do not fit get
+ * CV_E_NOT_AVAILABLE.  The call allocates and frees nothing; the first call on a device looks up
+ * the array's address (make that call outside a graph capture).  All calls on one GPU share the
+ * array: calls that may overlap on one GPU (different streams, different threads) race. */
+#define CV_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
+CV_API CvResult cvMlpTrainStepNoAlloc(void* stream, const CvMlpDesc* mlp,
+                                      const void* input, size_t inputStride,
+                                      const void* targets, size_t targetStride,
+                                      float lossScale, uint32_t batch, float* lossSum);
+
 /* ------------------------------------------------------------------------------------ */
 /* parameter update of the example                                                      */
 /* ------------------------------------------------------------------------------------ */

@@ -109,6 +109,9 @@ SIGNATURES = {
     "cvMlpTrainStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
                                         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float, ctypes.c_uint32,
                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
+    "cvMlpTrainStepNoAlloc": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p,
+                                               ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float,
+                                               ctypes.c_uint32, ctypes.c_void_p]),
     "cvAdamStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                     ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float]),
 }

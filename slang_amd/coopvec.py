@@ -397,6 +397,26 @@ def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, target
     return workspace, lossSum
 
 
+NOALLOC_SCRATCH_BYTES = 16 << 20   # CV_NOALLOC_SCRATCH_BYTES of include/coopvec.h
+
+
+def mlpTrainStepNoAlloc(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor],
+                        lossSum: torch.Tensor, *, lossScale: float = 1.0,
+                        gradType: int = CoopVecComponentType.Float32, stream=None) -> None:
+    """mlpTrainStep for callers that cannot allocate: the gradient partials go to an array inside
+    the library's device image, nothing is allocated (lossSum is the caller's, too).  Calls that
+    overlap on one GPU race on that array."""
+    _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+    tptr, tstride = None, 0
+    if targets is not None:
+        _, tstride = _vector_info(targets, CoopVecComponentType.Float16, "targets")
+        tptr = targets.data_ptr()
+    _check(_lib.load().cvMlpTrainStepNoAlloc(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride,
+                                             tptr, tstride, float(lossScale), input.shape[0],
+                                             lossSum.data_ptr() if lossSum is not None else None))
+
+
 # ---------------------------------------------------------------------------------------------
 # training operators over a batch
 # ---------------------------------------------------------------------------------------------

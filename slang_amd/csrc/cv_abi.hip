@@ -56,6 +56,36 @@ uint32_t alignOf(const void* p, size_t stride)
     return (uint32_t)(v & (~v + 1));
 }
 
+// Scratch of cvMlpTrainStepNoAlloc: the per-workgroup gradient partials of the training step.  Every
+// device the library runs on holds its own copy of this array at its own address; on the host the
+// array's name is only a handle for hipGetSymbolAddress, never a device address.
+static __device__ __align__(256) unsigned char scratch[CV_NOALLOC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device, looked up once per device.
+void* scratchOfCurrentDevice(CvResult* rc)
+{
+    static void* ptr[64];
+    static hipError_t err[64];
+    static std::once_flag once[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= 64) {
+        *rc = fail(CV_E_NOT_AVAILABLE, "no usable HIP device: %s", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::call_once(once[dev], [dev] {
+        void* p = nullptr;
+        err[dev] = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        ptr[dev] = err[dev] == hipSuccess ? p : nullptr;
+    });
+    if (err[dev] != hipSuccess || !ptr[dev]) {
+        *rc = fail(CV_E_INTERNAL_FAIL, "address of the built-in scratch array on device %d: %s", dev, hipGetErrorString(err[dev]));
+        return nullptr;
+    }
+    *rc = CV_OK;
+    return ptr[dev];
+}
+
 bool isOptimal(int layout) { return layout == CV_LAYOUT_INFERENCING_OPTIMAL || layout == CV_LAYOUT_TRAINING_OPTIMAL; }
 
 struct Combo {
@@ -479,44 +509,46 @@ CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch
     return CV_OK;
 }
 
-CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
-                               const void* targets, size_t targetStride, float lossScale, uint32_t batch,
-                               float* lossSum, void* workspace, size_t workspaceBytes)
+// Shared body of cvMlpTrainStep and cvMlpTrainStepNoAlloc; `ownScratch` marks the library's own
+// scratch array, whose fixed size is a limit of the entry point rather than a caller's mistake.
+static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
+                          const void* targets, size_t targetStride, float lossScale, uint32_t batch,
+                          float* lossSum, void* workspace, size_t workspaceBytes, bool ownScratch)
 {
     cv::TrainLaunch t;
     memset(&t, 0, sizeof(t));
-    CvResult rc = fillMlpLayers("cvMlpTrainStep", mlp, t.mlp.layers);
+    CvResult rc = fillMlpLayers(who, mlp, t.mlp.layers);
     if (CV_FAILED(rc)) return rc;
-    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights");
+    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "%s: training needs FLOAT16 weights", who);
     if (mlp->gradType != CV_FLOAT16 && mlp->gradType != CV_FLOAT32)
-        return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: gradType %d (supported: FLOAT16, FLOAT32)", mlp->gradType);
+        return fail(CV_E_NOT_AVAILABLE, "%s: gradType %d (supported: FLOAT16, FLOAT32)", who, mlp->gradType);
     const int L = mlp->numLayers;
-    if (L < 2) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: needs at least two layers");
+    if (L < 2) return fail(CV_E_NOT_AVAILABLE, "%s: needs at least two layers", who);
     if (batch == 0) return CV_OK;
-    if (!input || !workspace) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: null input/workspace");
+    if (!input || !workspace) return fail(CV_E_INVALID_ARG, "%s: null input/workspace", who);
     if ((uintptr_t)input % 2 || inputStride % 2 || (uintptr_t)targets % 2 || targetStride % 2 || (uintptr_t)workspace % 16 ||
         (uintptr_t)lossSum % 4)
-        return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: misaligned input/targets/workspace/lossSum");
+        return fail(CV_E_INVALID_ARG, "%s: misaligned input/targets/workspace/lossSum", who);
     if (batch > 1 && (inputStride < (size_t)mlp->layers[0].inputSize * 2 ||
                       (targets && targetStride < (size_t)mlp->layers[L - 1].outputSize * 2)))
-        return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: vector stride smaller than the vector");
+        return fail(CV_E_INVALID_ARG, "%s: vector stride smaller than the vector", who);
     const uint32_t gEsz = cv::elemSize(mlp->gradType);
     for (int l = 0; l < L; ++l) {
         const CvMlpLayer& ly = mlp->layers[l];
         // with 0 <= slope <= 0.5 the outcome of max(z, z*slope) is the sign of z for every fp16 z
         if (ly.activation == CV_ACT_LEAKY_RELU && !(ly.leakySlope >= 0.f && ly.leakySlope <= 0.5f))
-            return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: leakySlope must be in [0, 0.5]", l);
+            return fail(CV_E_INVALID_ARG, "%s: layer %d: leakySlope must be in [0, 0.5]", who, l);
         t.wGrad[l] = (uint8_t*)ly.weightsGrad;
         t.bGrad[l] = (uint8_t*)ly.biasesGrad;
         if (ly.weightsGrad) {
             if (ly.gradLayout < 0 || ly.gradLayout > 3 || !cv::layoutSupports(mlp->gradType, ly.gradLayout))
-                return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: layer %d: component type %d has no layout %d", l, mlp->gradType, ly.gradLayout);
+                return fail(CV_E_NOT_AVAILABLE, "%s: layer %d: component type %d has no layout %d", who, l, mlp->gradType, ly.gradLayout);
             t.gradShape[l] = cv::MatrixShape{(uint32_t)ly.outputSize, (uint32_t)ly.inputSize, mlp->gradType, ly.gradLayout,
                                              isOptimal(ly.gradLayout) ? 0 : (size_t)ly.gradStride};
-            if (cv::matrixSize(t.gradShape[l]) == 0) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: gradStride %u smaller than a row/column", l, ly.gradStride);
-            if ((uintptr_t)ly.weightsGrad % gEsz || ly.gradStride % gEsz) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: weightsGrad misaligned", l);
+            if (cv::matrixSize(t.gradShape[l]) == 0) return fail(CV_E_INVALID_ARG, "%s: layer %d: gradStride %u smaller than a row/column", who, l, ly.gradStride);
+            if ((uintptr_t)ly.weightsGrad % gEsz || ly.gradStride % gEsz) return fail(CV_E_INVALID_ARG, "%s: layer %d: weightsGrad misaligned", who, l);
         }
-        if ((uintptr_t)ly.biasesGrad % gEsz) return fail(CV_E_INVALID_ARG, "cvMlpTrainStep: layer %d: biasesGrad misaligned", l);
+        if ((uintptr_t)ly.biasesGrad % gEsz) return fail(CV_E_INVALID_ARG, "%s: layer %d: biasesGrad misaligned", who, l);
     }
     t.mlp.numLayers = L;
     t.mlp.in = (const uint8_t*)input;
@@ -532,9 +564,33 @@ CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* i
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     const size_t need = cv::trainWorkspaceBytes(t.mlp, cus);
-    if (!need) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: no fused specialisation for these layer sizes");
-    if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvMlpTrainStep: workspace of %zu bytes, %zu needed", workspaceBytes, need);
-    return fromHip(cv::launchMlpTrain((hipStream_t)stream, t, cus), "cvMlpTrainStep launch");
+    if (!need) return fail(CV_E_NOT_AVAILABLE, "%s: no fused specialisation for these layer sizes", who);
+    if (workspaceBytes < need) {
+        if (ownScratch)
+            return fail(CV_E_NOT_AVAILABLE, "%s: this network needs %zu bytes of scratch, the built-in array holds %zu; "
+                        "use cvMlpTrainStep with a caller-provided workspace", who, need, workspaceBytes);
+        return fail(CV_E_BUFFER_TOO_SMALL, "%s: workspace of %zu bytes, %zu needed", who, workspaceBytes, need);
+    }
+    return fromHip(cv::launchMlpTrain((hipStream_t)stream, t, cus), who);
+}
+
+CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
+                               const void* targets, size_t targetStride, float lossScale, uint32_t batch,
+                               float* lossSum, void* workspace, size_t workspaceBytes)
+{
+    return trainStep("cvMlpTrainStep", stream, mlp, input, inputStride, targets, targetStride, lossScale, batch,
+                     lossSum, workspace, workspaceBytes, false);
+}
+
+CV_API CvResult cvMlpTrainStepNoAlloc(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,
+                                      const void* targets, size_t targetStride, float lossScale, uint32_t batch,
+                                      float* lossSum)
+{
+    CvResult rc;
+    void* ws = scratchOfCurrentDevice(&rc);
+    if (CV_FAILED(rc)) return rc;
+    return trainStep("cvMlpTrainStepNoAlloc", stream, mlp, input, inputStride, targets, targetStride, lossScale,
+                     batch, lossSum, ws, CV_NOALLOC_SCRATCH_BYTES, true);
 }
 
 } // extern "C"
