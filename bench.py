@@ -1,13 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the cooperative-vector hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 
 A "step" is one pass of the hot path over one batch of synthetic, seeded input that already
-lives in HBM.  The default workload is the configuration the headline metric is quoted on:
-a single fp16 coopVecMatMulAdd layer 64x64 (fp32 accumulate, fp16 output) over 2^22 vectors,
-weights in InferencingOptimal layout (the layout conversion is timed separately and reported
-as `layout_conversion_us`).  Prints ONE JSON line.
+lives in HBM.  The headline workload (top-level fields of the JSON line) is the configuration the
+metric is quoted on: a single fp16 coopVecMatMulAdd layer 64x64 (fp32 accumulate, fp16 output) over
+2^22 vectors, weights in InferencingOptimal layout (the layout conversion is timed separately and
+reported as `layout_conversion_us`).  Without --workload every other configuration is timed the same
+way in the same run (W warm-up steps, K timed steps, HIP events on the launch stream) and reported
+under "workloads": c1, c3, c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
+c5 (training step), op / rs (stand-alone outer-product / reduce-sum accumulate).  With --workload
+only that one runs and becomes the headline (profiling runs).  Prints ONE JSON line.
 
 `roofline.achieved` = algorithmic bytes per launch / average kernel duration, the duration
 measured with HIP events on the launch stream around the timed launches.  `cpu_baseline` times
@@ -30,14 +34,14 @@ METRIC = "CoopVec MLP samples/sec (fp16/fp8/int8 fwd, fp16 train step); % MFMA p
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
-# kernel of known size).  None where not measured.
-MEASURED_TRAFFIC_BYTES = {
-    "c2": 1074875000,
-    "c3": 2685218000,
-    "c4": 805497000,
-    "c4n": 805497000,
-    "c5": 32583000,      # training kernel only
+# HBM bytes per launch as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy
+# kernel of known size): not measured by this script, quoted from the committed profile summaries.
+PROFILED_TRAFFIC = {
+    "c2": (1074875000, "profiles/matmul_f16_64x64_batch4M.md"),
+    "c3": (2685218000, "profiles/matmul_i8_128x128_batch4M.md"),
+    "c4": (805497000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
+    "c4n": (805497000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
+    "c5": (32583000, "profiles/mlp_train_8-64x4-1_batch1M.md"),      # training kernel only
 }
 
 
@@ -111,7 +115,7 @@ def workload_c2(torch, cv, steps, warmup):
                           "fallback (fp16 accumulate, software half as gcc<12 selects), -O2" % (n, per_core)}
 
     return dict(step=step, samples=B, alg_bytes=B * (K * 2 + M * 2), alg_flops=B * 2 * M * K,
-                bound="hbm", dtype="f16", kernel="matmulKernel<F16Mma,4,2,2,half,FAST>",
+                bound="hbm", mfma="f16", dtype="f16",
                 config={"workload": "c2: fp16 coopVecMatMulAdd 64x64, batch 2^22, InferencingOptimal weights, "
                                     "fp32 accumulate, fp16 out", "batch": B, "m": M, "k": K,
                         "layout": "InferencingOptimal"},
@@ -166,8 +170,7 @@ def workload_c3(torch, cv, steps, warmup):
                 "sample": "first %d of the 2^22 vectors; C restatement of the Slang CPU-target fallback "
                           "(packed int8, ColumnMajor, int32 accumulate), -O2" % n}
 
-    return dict(step=step, samples=B, alg_bytes=B * (K + M * 4), alg_flops=B * 2 * M * K, bound="hbm", dtype="int8",
-                kernel="matmulKernel<I8Mma,8,2,2,int,fast>",
+    return dict(step=step, samples=B, alg_bytes=B * (K + M * 4), alg_flops=B * 2 * M * K, bound="hbm", mfma="int8", dtype="int8",
                 config={"workload": "c3: int8 coopVecMatMulAdd 128x128 -> int32 + int32 bias, batch 2^22, "
                                     "InferencingOptimal weights", "batch": B, "m": M, "k": K},
                 cpu_baseline=cpu_baseline, key="c3")
@@ -237,7 +240,7 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
                           "layer (fp16 accumulate, software half), -O2" % n}
 
     return dict(step=step, samples=B, alg_bytes=B * (in_bytes + dims[-1] * 2), alg_flops=B * 2 * macs,
-                bound="hbm", dtype=wtype_name, kernel="mlpForwardKernel",
+                bound="hbm", mfma="fp8" if flags else "f16", dtype=wtype_name,
                 config={"workload": desc, "batch": B, "layers": dims}, cpu_baseline=cpu_baseline, key=key)
 
 
@@ -307,13 +310,133 @@ def workload_c5(torch, cv, steps, warmup):
                           "(wave intrinsics and atomics, docs/cpu-target.md:15-21)" % n}
 
     return dict(step=step, samples=B, alg_bytes=B * dims[0] * 2, alg_flops=B * 2 * (2 * macs + macs_dx),
-                bound="mfma", mfma="f16", dtype="f16", kernel="mlpTrainKernel<8-64x4-1> + mlpTrainReduceKernel",
+                bound="mfma", mfma="f16", dtype="f16",
                 config={"workload": "c5: fp16 train step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, "
                                     "fp32 TrainingOptimal gradients, deterministic reduction", "batch": B, "layers": dims},
                 cpu_baseline=cpu_baseline, key="c5")
 
 
-WORKLOADS = {"c5": workload_c5, "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n}
+def workload_op(torch, cv, steps, warmup):
+    """stand-alone coopVecOuterProductAccumulate 64x64 over 2^20 vector pairs, fp32 TrainingOptimal destination."""
+    from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML
+    dev = "cuda"
+    B, M, N = 1 << 20, 64, 64
+    g = torch.Generator(device=dev); g.manual_seed(20256)
+    a = (torch.randn(B, M, device=dev, generator=g) * 0.25).half()
+    b = (torch.rand(B, N, device=dev, generator=g) * 2 - 1).half()
+    size = cv.getCooperativeVectorMatrixSize(M, N, CT.Float32, ML.TrainingOptimal)
+    mat = torch.zeros(size, dtype=torch.uint8, device=dev)
+    import ctypes
+    from slang_amd import _lib
+    need = ctypes.c_size_t(0)
+    _lib.load().cvOuterProductAccumulateWorkspaceSize(M, N, B, ctypes.byref(need))
+    ws = torch.empty(max(need.value, 16), dtype=torch.uint8, device=dev)
+
+    def step():
+        cv.coopVecOuterProductAccumulate(a, b, mat, 0, 0, ML.TrainingOptimal, CT.Float32, workspace=ws)
+
+    def cpu_baseline():
+        import numpy as np
+        import oracle_binding as ob
+        n = 1 << 12
+        an, bn = a[:n].cpu().numpy(), b[:n].cpu().numpy()
+        dst = np.zeros((M, N), np.float16)
+        L = ob.lib()
+        t0 = time.perf_counter()
+        for s_ in range(n):
+            rc = L.cvo_slang_outer_product_accumulate(ob.ptr(an[s_]), M, ob.ptr(bn[s_]), N, ob.F16, ob.ptr(dst), 0,
+                                                      N * 2, ob.ROW, ob.F16, ob.HALF_SLANG)
+            assert rc == 0
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vector pairs, one core; C restatement of the Slang CPU-target fallback "
+                          "(per-thread load-add-store in half, RowMajor), -O2, called per thread from Python" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * (M + N) * 2, alg_flops=B * 2 * M * N, bound="hbm", mfma="f16",
+                dtype="f16", config={"workload": "op: coopVecOuterProductAccumulate 64x64 over 2^20 fp16 vector pairs, "
+                                                 "fp32 TrainingOptimal destination, deterministic reduction",
+                                     "batch": B, "m": M, "n": N}, cpu_baseline=cpu_baseline, key="op")
+
+
+def workload_rs(torch, cv, steps, warmup):
+    """stand-alone coopVecReduceSumAccumulate of 64-vectors over a batch of 2^22, fp32 destination."""
+    from slang_amd.coopvec import CoopVecComponentType as CT
+    dev = "cuda"
+    B, N = 1 << 22, 64
+    g = torch.Generator(device=dev); g.manual_seed(20257)
+    v = (torch.rand(B, N, device=dev, generator=g) * 2 - 1).half()
+    buf = torch.zeros(N, dtype=torch.float32, device=dev)
+    import ctypes
+    from slang_amd import _lib
+    need = ctypes.c_size_t(0)
+    _lib.load().cvReduceSumAccumulateWorkspaceSize(N, B, ctypes.byref(need))
+    ws = torch.empty(max(need.value, 16), dtype=torch.uint8, device=dev)
+
+    def step():
+        cv.coopVecReduceSumAccumulate(v, buf.view(torch.uint8), 0, bufferType=CT.Float32, workspace=ws)
+
+    def cpu_baseline():
+        import numpy as np
+        import oracle_binding as ob
+        n = 1 << 14
+        vn = v[:n].cpu().numpy()
+        dst = np.zeros(N, np.float16)
+        L = ob.lib()
+        t0 = time.perf_counter()
+        for s_ in range(n):
+            assert L.cvo_slang_reduce_sum_accumulate(ob.ptr(vn[s_]), N, ob.F16, ob.ptr(dst), 0, ob.HALF_SLANG) == 0
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vectors, one core; C restatement of the Slang CPU-target fallback (per-thread "
+                          "load-add-store in half), -O2, called per thread from Python" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * N * 2, alg_flops=B * N, bound="hbm", mfma="f16", dtype="f16",
+                config={"workload": "rs: coopVecReduceSumAccumulate of 64-vectors over 2^22 fp16 vectors, fp32 destination",
+                        "batch": B, "n": N}, cpu_baseline=cpu_baseline, key="rs")
+
+
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n,
+             "c5": workload_c5, "op": workload_op, "rs": workload_rs}
+HEADLINE = "c2"
+
+
+def measure(torch, w, steps, warmup, with_cpu):
+    """W untimed warm-up steps, then exactly K timed steps between synchronisations; kernel time from
+    HIP events recorded on the launch stream (torch's current stream is the one handed to the library)."""
+    from slang_amd import _lib
+    step = w["step"]
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        step()
+    ev1.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kernel = _lib.load().cvGetLastKernelName().decode()
+    wall_ms = (t1 - t0) * 1e3 / steps
+    kern_ms = ev0.elapsed_time(ev1) / steps
+    hbm = w["alg_bytes"] / (kern_ms * 1e-3) / 1e9
+    tflops = w["alg_flops"] / (kern_ms * 1e-3) / 1e12
+    mfma_peak = MFMA_PEAK_TFLOPS[w["mfma"]]
+    if w["bound"] == "hbm":
+        achieved, peak, unit = hbm, HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved, peak, unit = tflops, mfma_peak, "TFLOP/s"
+    traffic = PROFILED_TRAFFIC.get(w["key"])
+    roofline = {"bound": w["bound"], "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
+                "traffic": traffic[0] if traffic else None,
+                "traffic_source": (traffic[1] + " (rocprofv3 --pmc, not measured by this run)") if traffic else None,
+                "kernel": kernel, "kernel_ms": kern_ms,
+                "alg_bytes_per_launch": w["alg_bytes"], "alg_flops_per_launch": w["alg_flops"],
+                "hbm_GBps": hbm, "hbm_frac": hbm / HBM_PEAK_GBS,
+                "mfma_TFLOPs": tflops, "mfma_peak_TFLOPs": mfma_peak, "mfma_frac": tflops / mfma_peak}
+    return {"value": w["samples"] / (wall_ms * 1e-3), "unit": "samples/s", "ms_per_step": wall_ms, "dtype": w["dtype"],
+            "config": w["config"], "roofline": roofline,
+            "cpu_baseline": w["cpu_baseline"]() if with_cpu else None, "extra": w.get("extra", {})}
 
 
 def main(argv=None) -> int:
@@ -321,7 +444,8 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=None, choices=sorted(WORKLOADS),
+                    help="run only this workload (default: the headline c2 plus all others under 'workloads')")
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     args = ap.parse_args(argv)
     if args.gpus != 1:
@@ -335,39 +459,30 @@ def main(argv=None) -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 3
     torch.cuda.set_device(0)
-    w = WORKLOADS[args.workload](torch, cv, args.steps, args.warmup)
-    step = w["step"]
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
-        step()
-    ev1.record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / args.steps
-    kern_ms = ev0.elapsed_time(ev1) / args.steps          # HIP events on the launch stream
-    value = w["samples"] / (wall_ms * 1e-3)
-    if w["bound"] == "hbm":
-        achieved = w["alg_bytes"] / (kern_ms * 1e-3) / 1e9
-        peak, unit = HBM_PEAK_GBS, "GB/s"
-    else:
-        achieved = w["alg_flops"] / (kern_ms * 1e-3) / 1e12
-        peak, unit = MFMA_PEAK_TFLOPS[w["mfma"]], "TFLOP/s"
+    head_key = args.workload or HEADLINE
+    others = [] if args.workload else [k for k in WORKLOADS if k != HEADLINE]
+
+    def run(key):
+        w = WORKLOADS[key](torch, cv, args.steps, args.warmup)
+        r = measure(torch, w, args.steps, args.warmup, not args.no_cpu_baseline)
+        del w
+        torch.cuda.empty_cache()
+        return r
+
+    h = run(head_key)
     line = {
-        "metric": METRIC, "value": value, "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic", "config": w["config"],
-        "roofline": {"bound": w["bound"], "achieved": achieved, "peak": peak, "unit": unit,
-                     "frac": achieved / peak, "traffic": MEASURED_TRAFFIC_BYTES.get(w["key"]),
-                     "kernel": w["kernel"], "kernel_ms": kern_ms,
-                     "alg_bytes_per_launch": w["alg_bytes"], "alg_flops_per_launch": w["alg_flops"]},
-        "cpu_baseline": None if args.no_cpu_baseline else w["cpu_baseline"](),
+        "metric": METRIC, "value": h["value"], "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": h["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": h["dtype"], "data": "synthetic", "config": h["config"],
+        "roofline": h["roofline"], "cpu_baseline": h["cpu_baseline"],
     }
-    line.update(w.get("extra", {}))
+    line.update(h["extra"])
+    if others:
+        line["workloads"] = {}
+        for k in others:
+            r = run(k)
+            r.pop("extra")
+            line["workloads"][k] = r
     print(json.dumps(line))
     return 0
 

@@ -17,7 +17,9 @@
  *   - every call is asynchronous on the given stream (a `hipStream_t` passed as void*;
  *     NULL = the default stream) and returns a SlangResult-compatible code
  *     (include/slang.h:1377-1464): 0 = OK, negative = failure; nothing throws;
- *   - calls are thread-compatible: no mutable global state besides a per-thread error string;
+ *   - calls are thread-compatible: the only global state is a per-thread error string and
+ *     per-device caches of immutable device facts (compute-unit count, kernel residency), kept
+ *     in atomics / call_once;
  *   - vectors must start at 16-byte-aligned addresses (hlsl.meta.slang:30761-30764,
  *     30874-30878); matrices and biases at 64-byte-aligned addresses like the example's
  *     sub-allocations (mlp-training-coopvec.cpp:273-279).
@@ -66,6 +68,19 @@ typedef enum CvComponentType {
     CV_COMPONENT_NONE = -1
 } CvComponentType;
 
+/* ---- the host API's numbering of the same types: rhi::CooperativeVectorComponentType
+ *      (include/slang-gfx.h:1748-1765), which is what the example passes to
+ *      getCooperativeVectorMatrixSize and puts into CooperativeVectorMatrixDesc.componentType
+ *      (mlp-training-coopvec.cpp:212,220,308).  It differs from the shader-side numbering above
+ *      (Float16 is 0 there, FLOAT_E4M3 is 0 here): every entry point of this library takes
+ *      CvComponentType, so a caller holding an rhi value converts it first. */
+typedef enum CvRhiComponentType {
+    CV_RHI_FLOAT16 = 0, CV_RHI_FLOAT32 = 1, CV_RHI_FLOAT64 = 2,
+    CV_RHI_SINT8 = 3, CV_RHI_SINT16 = 4, CV_RHI_SINT32 = 5, CV_RHI_SINT64 = 6,
+    CV_RHI_UINT8 = 7, CV_RHI_UINT16 = 8, CV_RHI_UINT32 = 9, CV_RHI_UINT64 = 10,
+    CV_RHI_SINT8_PACKED = 11, CV_RHI_UINT8_PACKED = 12, CV_RHI_FLOAT_E4M3 = 13, CV_RHI_FLOAT_E5M2 = 14
+} CvRhiComponentType;
+
 /* Activation fused behind a matMulAdd.  RELU is max(z, 0) as the neural module defines it
  * (source/standard-modules/neural/activations.slang:25-42); LEAKY_RELU is the example's
  * max(z, z * slope) evaluated in half (examples/mlp-training-coopvec/fflayer.slang:64-65). */
@@ -113,10 +128,17 @@ typedef struct CvCombination {
 CV_API uint32_t cvGetVersion(void);
 /* Message describing the last failure on the calling thread ("" if none). */
 CV_API const char* cvGetLastErrorMessage(void);
+/* Diagnostics: the kernel specialisation(s) the calling thread's last operator call launched
+ * (e.g. "matmulKernel<f16,MT=4,KT=2,NT=2,out=f16,streaming>"); "" before the first launch. */
+CV_API const char* cvGetLastKernelName(void);
 /* Helpers replacing hlsl.meta.slang:32578-32593 / :32596-32633 / :32636-32670. */
 CV_API int32_t cvComponentPackingFactor(int32_t componentType);
 CV_API int32_t cvComponentScalarType(int32_t componentType);      /* SLANG_SCALAR_TYPE_* or -1 */
 CV_API int32_t cvComponentTypeStride(int32_t componentType);      /* bytes, -1 if unknown */
+/* rhi::CooperativeVectorComponentType -> CvComponentType and back; CV_COMPONENT_NONE (-1) for a
+ * value outside the enum. */
+CV_API int32_t cvComponentTypeFromRhi(int32_t rhiComponentType);
+CV_API int32_t cvComponentTypeToRhi(int32_t componentType);
 /* The (type, interpretation) combinations cvMatMul accepts, in the shape a host compares
  * against ICooperativeTypesMetadata (include/slang.h:5231-5273).  Returns the total count;
  * fills at most `capacity` entries. */

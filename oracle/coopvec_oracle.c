@@ -13,6 +13,8 @@
  *       matrix-mul*.slang, outer-product.slang, reduce-sum-accumulate*.slang).
  *   cvo_ref_*                         : pinned (same goldens, fp64 brute force, closed forms
  *       of tests/neural/basic-ilayer-ffn-{forward,backward}-test.slang, finite differences).
+ *   cvo_slang_adam_step               : pinned by multi-step closed forms of Adam (constant
+ *       gradient, impulse response, iteration count, NaN/Inf rules); the reference has no golden.
  *   cvo_layout_* for the two Optimal layouts : PARITY UNPINNED against the reference (the
  *       reference delegates those layouts to the vendor driver); pinned only by invariants.
  */
@@ -857,8 +859,20 @@ int cvo_ref_mlp_train(const CvoLayer* layers, int numLayers,
 /* Adam (examples/mlp-training-coopvec/adam.slang:20-36, kernels.slang:29-45)            */
 /* ===================================================================================== */
 
-void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
-                         float beta1f, float beta2f, float epsf, float lrf, int halfMode)
+/* powNudge1/2 move the fp32 value of pow(beta1, it) / pow(beta2, it) by that many fp32 ulps before
+ * it is rounded to half: pow is the one operation here that maths libraries are allowed to round
+ * differently, and the tests use the nudges to show that a result differing from nudge (0,0) is such
+ * a case. */
+static float nudge_ulps(float v, int n)
+{
+    for (; n > 0; --n) v = nextafterf(v, INFINITY);
+    for (; n < 0; ++n) v = nextafterf(v, -INFINITY);
+    return v;
+}
+
+void cvo_slang_adam_step_nudged(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
+                                float beta1f, float beta2f, float epsf, float lrf, int halfMode,
+                                int powNudge1, int powNudge2)
 {
 #define H(x) cvo_f16_to_f32(to_half((x), halfMode))     /* one rounding to half */
     const float beta1 = H(beta1f), beta2 = H(beta2f), eps = H(epsf), lr = H(lrf);
@@ -873,8 +887,8 @@ void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads
         mean = H(H(beta1 * mean) + H(omb1 * g));
         var = H(H(beta2 * var) + H(H(omb2 * g) * g));
         const float it = H((float)st->iteration);
-        const float meanHat = H(mean / H(1.0f - H(powf(beta1, it))));
-        const float varHat = H(var / H(1.0f - H(powf(beta2, it))));
+        const float meanHat = H(mean / H(1.0f - H(nudge_ulps(powf(beta1, it), powNudge1))));
+        const float varHat = H(var / H(1.0f - H(nudge_ulps(powf(beta2, it), powNudge2))));
         const float denom = H(sqrtf(H(fmaxf(0.0f, varHat) + eps)));
         const float p = cvo_f16_to_f32(params[i]);
         params[i] = to_half(p - H(H(lr * meanHat) / denom), halfMode);
@@ -883,4 +897,10 @@ void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads
         grads[i] = 0;
     }
 #undef H
+}
+
+void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
+                         float beta1f, float beta2f, float epsf, float lrf, int halfMode)
+{
+    cvo_slang_adam_step_nudged(states, params, grads, count, beta1f, beta2f, epsf, lrf, halfMode, 0, 0);
 }

@@ -163,10 +163,19 @@ typedef struct CvoAdamState { uint16_t mean, variance; int32_t iteration; } CvoA
 /* One dispatch of adjustParameters (kernels.slang:29-45) + AdamOptimizer::step (adam.slang:20-36)
  * over `count` fp16 parameters: every operation in half (each result rounded), NaN gradients are
  * cleared and skipped, infinite ones replaced by +-10000, the gradient is zeroed afterwards.
- * PARITY UNPINNED against the reference (it has no golden for the optimizer); pinned by the
- * closed form of the first steps. */
+ * The reference has no golden for the optimizer; pinned by what the mathematics of Adam fixes
+ * over several steps (tests/test_adam.py): a constant gradient g gives bias-corrected moments g and
+ * g^2, so every step moves the parameter by lr*sign(g); one gradient followed by zeros gives the
+ * closed-form decay beta1^(n-1)(1-beta1)/(1-beta1^n) over sqrt of the same in beta2; the iteration
+ * counter; NaN skips, infinities clip. */
 void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
                          float beta1, float beta2, float epsilon, float learningRate, int halfMode);
+/* Same, with the fp32 values of pow(beta1, it) and pow(beta2, it) moved by powNudge1 / powNudge2
+ * ulps before they are rounded to half (pow is the one operation maths libraries may round
+ * differently). */
+void cvo_slang_adam_step_nudged(CvoAdamState* states, uint16_t* params, uint16_t* grads, uint32_t count,
+                                float beta1, float beta2, float epsilon, float learningRate, int halfMode,
+                                int powNudge1, int powNudge2);
 
 #ifdef __cplusplus
 }

@@ -82,9 +82,12 @@ class CvMlpDesc(ctypes.Structure):
 SIGNATURES = {
     "cvGetVersion": (ctypes.c_uint32, []),
     "cvGetLastErrorMessage": (ctypes.c_char_p, []),
+    "cvGetLastKernelName": (ctypes.c_char_p, []),
     "cvComponentPackingFactor": (ctypes.c_int32, [ctypes.c_int32]),
     "cvComponentScalarType": (ctypes.c_int32, [ctypes.c_int32]),
     "cvComponentTypeStride": (ctypes.c_int32, [ctypes.c_int32]),
+    "cvComponentTypeFromRhi": (ctypes.c_int32, [ctypes.c_int32]),
+    "cvComponentTypeToRhi": (ctypes.c_int32, [ctypes.c_int32]),
     "cvQuerySupportedCombinations": (ctypes.c_uint32, [ctypes.POINTER(CvCombination), ctypes.c_uint32]),
     "cvGetMatrixSize": (ctypes.c_int32, [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int32, ctypes.c_int32,
                                          ctypes.c_size_t, ctypes.POINTER(ctypes.c_size_t)]),

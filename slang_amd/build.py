@@ -27,9 +27,13 @@ HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul_f16.hip", "cv_matmul_f
                "cv_matmul_i8.hip", "cv_mlp_f16.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip", "cv_mlp_generic.hip", "cv_train.hip", "cv_accum.hip", "cv_adam.hip"]
 
 # packed-fp32 instructions are switched off on purpose (see the flag below): hipcc would
-# otherwise form v_pk_*_f32 from ordinary float code.
+# otherwise form v_pk_*_f32 from ordinary float code.  -ffp-contract=off: the kernels state every
+# rounding point of the Slang source (each half product and sum rounded on its own); hipcc's default
+# would fuse a rounded product and a following sum into one fma with a single rounding.  Where a
+# fused multiply-add is wanted it is written as one.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fvisibility=hidden", "-fno-strict-aliasing",
+    "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]

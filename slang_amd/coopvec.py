@@ -51,6 +51,41 @@ class CoopVecComponentType(enum.IntEnum):
     UnsignedInt8Packed = 14
 
 
+class RhiCooperativeVectorComponentType(enum.IntEnum):
+    """rhi::CooperativeVectorComponentType (include/slang-gfx.h:1748-1765): the numbering the example's
+    host code holds (mlp-training-coopvec.cpp:212,220,308).  Convert with componentTypeFromRhi before
+    calling into this module, whose functions all take CoopVecComponentType."""
+    Float16 = 0
+    Float32 = 1
+    Float64 = 2
+    SInt8 = 3
+    SInt16 = 4
+    SInt32 = 5
+    SInt64 = 6
+    UInt8 = 7
+    UInt16 = 8
+    UInt32 = 9
+    UInt64 = 10
+    SInt8Packed = 11
+    UInt8Packed = 12
+    FloatE4M3 = 13
+    FloatE5M2 = 14
+
+
+def componentTypeFromRhi(rhiComponentType: int) -> CoopVecComponentType:
+    v = _lib.load().cvComponentTypeFromRhi(int(rhiComponentType))
+    if v < 0:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "not an rhi::CooperativeVectorComponentType: %d" % int(rhiComponentType))
+    return CoopVecComponentType(v)
+
+
+def componentTypeToRhi(componentType: int) -> RhiCooperativeVectorComponentType:
+    v = _lib.load().cvComponentTypeToRhi(int(componentType))
+    if v < 0:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "not a CoopVecComponentType: %d" % int(componentType))
+    return RhiCooperativeVectorComponentType(v)
+
+
 FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.h
 
 

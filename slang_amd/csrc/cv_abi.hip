@@ -14,6 +14,7 @@
 namespace {
 
 thread_local char tlsError[512] = "";
+thread_local char tlsKernel[256] = "";
 
 CvResult fail(CvResult code, const char* fmt, ...)
 {
@@ -118,9 +119,23 @@ CvResult failWith(CvResult code, const char* fmt, ...)
     va_end(ap);
     return code;
 }
+void noteKernel(bool append, const char* fmt, ...)
+{
+    size_t at = 0;
+    if (append) {
+        at = strlen(tlsKernel);
+        if (at + 4 < sizeof(tlsKernel)) { memcpy(tlsKernel + at, " + ", 4); at += 3; }
+    }
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(tlsKernel + at, sizeof(tlsKernel) - at, fmt, ap);
+    va_end(ap);
+}
 } // namespace cv
 
 extern "C" {
+
+CV_API const char* cvGetLastKernelName(void) { return tlsKernel; }
 
 CV_API uint32_t cvGetVersion(void) { return (1u << 16) | 0u; }
 
@@ -155,6 +170,24 @@ CV_API int32_t cvComponentTypeStride(int32_t ct)
 {
     const uint32_t s = cv::elemSize(ct);
     return s ? (int32_t)s : -1;
+}
+
+// rhi::CooperativeVectorComponentType (include/slang-gfx.h:1748-1765), indexed by its value
+static const int32_t kRhiToCv[15] = {
+    CV_FLOAT16, CV_FLOAT32, CV_FLOAT64, CV_SINT8, CV_SINT16, CV_SINT32, CV_SINT64,
+    CV_UINT8, CV_UINT16, CV_UINT32, CV_UINT64, CV_SINT8_PACKED, CV_UINT8_PACKED, CV_FLOAT_E4M3, CV_FLOAT_E5M2,
+};
+
+CV_API int32_t cvComponentTypeFromRhi(int32_t rhi)
+{
+    return (rhi >= 0 && rhi < 15) ? kRhiToCv[rhi] : (int32_t)CV_COMPONENT_NONE;
+}
+
+CV_API int32_t cvComponentTypeToRhi(int32_t ct)
+{
+    for (int32_t i = 0; i < 15; ++i)
+        if (kRhiToCv[i] == ct) return i;
+    return -1;
 }
 
 CV_API uint32_t cvQuerySupportedCombinations(CvCombination* out, uint32_t capacity)

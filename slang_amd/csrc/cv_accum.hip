@@ -15,6 +15,7 @@
 //     order to the destination ("+=", any matrix layout, fp16 or fp32): bitwise reproducible.
 #include "cv_device.h"
 #include "cv_kernels.h"
+#include "cv_error.h"
 
 namespace cv {
 
@@ -212,6 +213,7 @@ hipError_t launchOuterProduct(hipStream_t stream, const OuterArgs& a, int numCUs
     if (a.batch == 0) return hipSuccess;
     const uint32_t gx = outerGridX(a.batch, numCUs);
     const uint32_t blocks = (uint32_t)((a.m + kBlk - 1) / kBlk) * (uint32_t)((a.n + kBlk - 1) / kBlk);
+    noteKernel(false, "outerProductKernel + outerReduceKernel");
     hipLaunchKernelGGL(outerProductKernel, dim3(gx, blocks), dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -229,6 +231,7 @@ hipError_t launchReduceSum(hipStream_t stream, const ReduceSumArgs& a, int numCU
     if (a.batch == 0) return hipSuccess;
     if (a.n > kMaxReduceCols) return hipErrorInvalidValue;
     const uint32_t gx = outerGridX(a.batch * 2, numCUs);
+    noteKernel(false, "reduceSumKernel + reduceSumFinalKernel");
     hipLaunchKernelGGL(reduceSumKernel, dim3(gx), dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

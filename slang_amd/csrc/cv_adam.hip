@@ -54,6 +54,7 @@ extern "C" CV_API CvResult cvAdamStep(void* stream, void* states, void* params, 
     if (!states || !params || !gradients) return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: null argument");
     if ((uintptr_t)states % 4 || (uintptr_t)params % 2 || (uintptr_t)gradients % 2)
         return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: misaligned argument");
+    cv::noteKernel(false, "adamKernel");
     hipLaunchKernelGGL(cv::adamKernel, dim3((count + 255) / 256), dim3(256), 0, (hipStream_t)stream,
                        (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count, beta1, beta2,
                        epsilon, learningRate);

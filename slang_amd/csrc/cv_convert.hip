@@ -8,6 +8,7 @@
 // elements are written; bytes between rows (stride padding) are left alone.
 #include "cv_device.h"
 #include "cv_kernels.h"
+#include "cv_error.h"
 
 namespace cv {
 
@@ -80,6 +81,7 @@ hipError_t launchConvert(hipStream_t stream, const ConvertArgs& args)
     }
     uint32_t bx = (maxSlots + 255u) / 256u;
     if (bx > 1024u) bx = 1024u;
+    noteKernel(false, "convertKernel");
     hipLaunchKernelGGL(convertKernel, dim3(bx, args.count), dim3(256), 0, stream, args);
     return hipGetLastError();
 }

@@ -33,6 +33,7 @@ enum : int { kActNone = 0, kActRelu = 1, kActLeakyRelu = 2 };
 // fragment after decode()), the accumulator type, and D += A.B.
 
 struct F16Mma {
+    static constexpr const char* kName = "f16";
     static constexpr int kEsz = 2, kEpl = 8, kRawDW = 4, kFD = 4;
     static constexpr bool kIsFloat = true;
     typedef floatx4 Acc;
@@ -52,6 +53,7 @@ struct F16Mma {
 // products of one instruction to the largest of them and keeps about 11 bits below it, so sums
 // that cancel carry an absolute error of up to ~2^-12 * sum|terms|.
 struct Fp8NativeMma {
+    static constexpr const char* kName = "e4m3-fp8pipe";
     static constexpr int kEsz = 1, kEpl = 8, kRawDW = 2, kFD = 2;
     static constexpr bool kIsFloat = true;
     typedef floatx4 Acc;
@@ -71,6 +73,7 @@ struct Fp8NativeMma {
 // fp16 matrix pipeline, whose accumulation is fp32-grade.  This is the flavour that meets the
 // fp32-accumulated parity bar for e4m3 matrices.
 struct Fp8AsF16Mma {
+    static constexpr const char* kName = "e4m3-f16pipe";
     static constexpr int kEsz = 1, kEpl = 8, kRawDW = 2, kFD = 4;
     static constexpr bool kIsFloat = true;
     typedef floatx4 Acc;
@@ -88,6 +91,7 @@ struct Fp8AsF16Mma {
 };
 
 struct I8Mma {   // int8 x int8 -> int32
+    static constexpr const char* kName = "i8";
     static constexpr int kEsz = 1, kEpl = 16, kRawDW = 4, kFD = 4;
     static constexpr bool kIsFloat = false;
     typedef intx4 Acc;

@@ -5,4 +5,7 @@
 namespace cv {
 // Records a printf-style message for cvGetLastErrorMessage() on the calling thread; returns `code`.
 CvResult failWith(CvResult code, const char* fmt, ...);
+// Records (printf-style) which kernel a launcher dispatched, for cvGetLastKernelName() on the calling
+// thread.  `append` adds to the current name (" + second kernel") instead of replacing it.
+void noteKernel(bool append, const char* fmt, ...);
 }

@@ -23,6 +23,8 @@
 #pragma once
 #include "cv_device.h"
 #include "cv_kernels.h"
+#include "cv_launch.h"
+#include "cv_error.h"
 
 namespace cv {
 namespace {
@@ -334,23 +336,20 @@ struct TileShape {
 };
 
 template <class Mma, int MT, int KT, typename OutT, bool FAST>
-hipError_t launchOne(hipStream_t stream, const MatMulArgs& a, int numCUs)
+hipError_t launchOne(hipStream_t stream, const MatMulArgs& a, int numCUs, bool tailOfStreaming = false)
 {
     constexpr int NT = TileShape<MT, KT>::NT;
     // Persistent grid: exactly as many workgroups as are resident at once, so that every wave
     // strides over the same number of tiles (a partial second round would run at a fraction of
     // the occupancy).  The residency of a kernel is fixed, so it is queried once.
-    static int blocksPerCU = 0;
-    if (blocksPerCU == 0) {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, matmulKernel<Mma, MT, KT, NT, OutT, FAST>, 256, 0) != hipSuccess || n < 1) n = 1;
-        blocksPerCU = n;
-    }
+    const int blocksPerCU = residentBlocksPerCU<matmulKernel<Mma, MT, KT, NT, OutT, FAST>>(256);
     const uint32_t tile = 16 * NT;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
+    noteKernel(tailOfStreaming, "matmulKernel<%s,MT=%d,KT=%d,NT=%d,out=%dB,%s>", Mma::kName, MT, KT, NT,
+               (int)sizeof(OutT), FAST ? "streaming" : "general");
     hipLaunchKernelGGL((matmulKernel<Mma, MT, KT, NT, OutT, FAST>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
@@ -378,7 +377,7 @@ hipError_t launchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
     t.in += (size_t)whole * a.inStride;
     t.out += (size_t)whole * a.outStride;
     t.batch = a.batch - whole;
-    return launchOne<Mma, MT, KT, OutT, false>(stream, t, numCUs);
+    return launchOne<Mma, MT, KT, OutT, false>(stream, t, numCUs, whole != 0);
 }
 
 template <class Mma, typename OutT>

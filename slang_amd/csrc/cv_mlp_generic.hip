@@ -167,17 +167,13 @@ hipError_t launchGeneric(hipStream_t stream, const MlpArgs& a, int numCUs)
     const uint32_t dwords = ga.biasDwordBase + bias;
     if (dwords > kGenLdsDwords) return hipErrorInvalidValue;
     const size_t ldsBytes = (size_t)dwords * 4;
-    static bool attrSet = false;
-    if (!attrSet) {
-        const hipError_t e = hipFuncSetAttribute((const void*)mlpGenericKernel<Mma>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 (int)(kGenLdsDwords * 4));
-        if (e != hipSuccess) return e;
-        attrSet = true;
-    }
+    const hipError_t ea = allowDynamicLds<mlpGenericKernel<Mma>>((int)(kGenLdsDwords * 4));
+    if (ea != hipSuccess) return ea;
     int perCU = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpGenericKernel<Mma>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
     const uint32_t numTiles = (a.batch + 15) / 16, need = (numTiles + 3) / 4;
     const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
+    noteKernel(false, "mlpGenericKernel<%s>", Mma::kName);
     hipLaunchKernelGGL(mlpGenericKernel<Mma>, dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
     return hipGetLastError();
 }

@@ -20,6 +20,8 @@
 
 #include "cv_device.h"
 #include "cv_kernels.h"
+#include "cv_launch.h"
+#include "cv_error.h"
 
 namespace cv {
 namespace {
@@ -364,17 +366,14 @@ hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
     constexpr int IN_DW = Mma::kRawDW * Net::KT0;
     constexpr int S0 = CV_MLP_PREFETCH_DW / IN_DW;
     constexpr int S = S0 < NT ? NT : (S0 > 16 ? 16 : S0 / NT * NT);
-    static int blocksPerCU = 0;
-    if (blocksPerCU == 0) {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mlpForwardKernel<Mma, Net, NT, S>, 256, 0) != hipSuccess || n < 1) n = 1;
-        blocksPerCU = n;
-    }
+    const int blocksPerCU = residentBlocksPerCU<mlpForwardKernel<Mma, Net, NT, S>>(256);
     const uint32_t tile = 16 * S;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
+    noteKernel(false, "mlpForwardKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d>", Mma::kName, Net::KT0, Net::HT,
+               Net::L - 1, Net::MTL, NT, S);
     hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }

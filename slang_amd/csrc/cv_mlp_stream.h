@@ -256,17 +256,14 @@ hipError_t launchMlpStreamB(hipStream_t stream, const MlpArgs& a, int numCUs)
     constexpr int ROW_DW = 4 * Mma::kRawDW * Net::KT0;
     constexpr int S0 = CV_MLP_STREAM_SLOT_DW / (16 * ROW_DW);
     constexpr int S = S0 < NT ? NT : S0 / NT * NT;
-    static int blocksPerCU = 0;
-    if (blocksPerCU == 0) {
-        int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS>, 256, 0) != hipSuccess || n < 1) n = 1;
-        blocksPerCU = n;
-    }
+    const int blocksPerCU = residentBlocksPerCU<mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS>>(256);
     const uint32_t slot = 16 * S;
     const uint32_t numSlots = (a.batch + slot - 1) / slot;
     const uint32_t blocksNeeded = (numSlots + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
+    noteKernel(false, "mlpStreamKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d,%s>", Mma::kName, Net::KT0, Net::HT,
+               Net::L - 1, Net::MTL, NT, S, HAS_BIAS ? "bias" : "nobias");
     hipLaunchKernelGGL((mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }

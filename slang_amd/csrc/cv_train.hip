@@ -1,5 +1,6 @@
 // cv_train.hip -- instantiations and launcher of the fused fp16 training step.
 #include "cv_train_impl.h"
+#include "cv_error.h"
 
 namespace cv {
 
@@ -41,6 +42,8 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
+    noteKernel(false, "mlpTrainKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s> + mlpTrainReduceKernel", Net::IT0, Net::KT0,
+               Net::HT, Net::L - 1, Net::MTL, plain ? "relu/none" : "runtime-act");
     if (plain) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone>), dim3(blocks), dim3(256), 0, stream, ta);
     else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();

@@ -99,7 +99,7 @@ __device__ __forceinline__ halfx2 maxGradMultiplier(halfx2 z)
     const halfx2 big = {(half_t)65504.f, (half_t)65504.f};
     const halfx2 one = {(half_t)1.f, (half_t)1.f}, zero = {(half_t)0.f, (half_t)0.f};
     const halfx2 hlf = {(half_t)0.5f, (half_t)0.5f};
-    const halfx2 s = (z * big) * big + hlf;
+    const halfx2 s = __builtin_elementwise_fma(z * big, big, hlf);
     return __builtin_elementwise_min(__builtin_elementwise_max(s, zero), one);   // {1, 0.5, 0}
 }
 

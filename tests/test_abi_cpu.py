@@ -184,3 +184,29 @@ def test_library_missing_is_loud(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     with pytest.raises(ImportError):
         _lib.load()
+
+
+def test_rhi_component_type_numbering(lib):
+    # rhi::CooperativeVectorComponentType (include/slang-gfx.h:1748-1765), the values the example's host
+    # code passes (mlp-training-coopvec.cpp:212,220,308), against the shader-side enum this ABI takes
+    rhi_names = ["Float16", "Float32", "Float64", "SInt8", "SInt16", "SInt32", "SInt64", "UInt8", "UInt16",
+                 "UInt32", "UInt64", "SInt8Packed", "UInt8Packed", "FloatE4M3", "FloatE5M2"]
+    slang_names = {"Float16": "Float16", "Float32": "Float32", "Float64": "Float64", "SInt8": "SignedInt8",
+                   "SInt16": "SignedInt16", "SInt32": "SignedInt32", "SInt64": "SignedInt64", "UInt8": "UnsignedInt8",
+                   "UInt16": "UnsignedInt16", "UInt32": "UnsignedInt32", "UInt64": "UnsignedInt64",
+                   "SInt8Packed": "SignedInt8Packed", "UInt8Packed": "UnsignedInt8Packed",
+                   "FloatE4M3": "FloatE4M3", "FloatE5M2": "FloatE5M2"}
+    from slang_amd.coopvec import CoopVecComponentType, RhiCooperativeVectorComponentType
+    for value, name in enumerate(rhi_names):
+        assert RhiCooperativeVectorComponentType[name] == value
+        want = CoopVecComponentType[slang_names[name]]
+        assert lib.cvComponentTypeFromRhi(value) == want
+        assert lib.cvComponentTypeToRhi(int(want)) == value
+    assert lib.cvComponentTypeFromRhi(15) == -1 and lib.cvComponentTypeFromRhi(-1) == -1
+    assert lib.cvComponentTypeToRhi(15) == -1
+    # the example's size query: rhi Float16 (0) must give the fp16 size, not the e4m3 size that the
+    # raw value 0 means on this ABI
+    fp16, raw0 = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert lib.cvGetMatrixSize(16, 4, lib.cvComponentTypeFromRhi(0), 0, 0, ctypes.byref(fp16)) == OK
+    assert lib.cvGetMatrixSize(16, 4, 0, 0, 0, ctypes.byref(raw0)) == OK
+    assert fp16.value == 16 * 4 * 2 and raw0.value == 16 * 4

@@ -1,45 +1,81 @@
-"""The example's Adam update (adam.slang:20-36, kernels.slang:29-45): oracle against the closed
-form of the first steps, GPU kernel against the oracle.  The reference ships no golden for the
-optimizer, so the oracle is pinned by mathematics only (parity unpinned against the reference)."""
+"""The example's Adam update (adam.slang:20-36, kernels.slang:29-45).
+
+The reference ships no golden for the optimizer, so the oracle is pinned by what the mathematics
+of Adam fixes over several steps (bounds stated per test; all arithmetic is fp16, so they are a few
+fp16 roundings wide), and the GPU kernel is then held to the oracle bit for bit -- except where the
+two maths libraries round pow() differently, which the test proves element by element."""
 import numpy as np
 import pytest
 
 import oracle_binding as ob
 
-
-def h(x):
-    return np.float32(np.float16(np.float32(x)))
+LR, B1, B2 = 0.01, 0.9, 0.999
 
 
-def test_oracle_first_step_closed_form():
-    # first step from zero state: mean = (1-b1) g, var = (1-b2) g^2, bias-corrected ratio ~ sign(g):
-    # every parameter moves by about lr against the gradient's sign
-    g = np.array([0.5, -0.25, 2.0, -3.0, 1e-2], np.float16)
-    p = np.array([1.0, 1.0, -1.0, 0.0, 0.5], np.float16)
-    st = np.zeros(5, ob.ADAM_STATE_DTYPE)
-    p0 = p.copy()
-    ob.slang_adam_step(st, p, g.copy())
-    assert (st["iteration"] == 1).all()
-    # step by step in half, as the source spells it
-    b1, b2, eps, lr = h(0.9), h(0.999), h(1e-7), h(0.01)
-    for i in range(5):
-        gi = np.float32(g[i])
-        mean = h(h(b1 * 0) + h(h(1 - b1) * gi))
-        var = h(h(b2 * 0) + h(h(h(1 - b2) * gi) * gi))
-        mhat = h(mean / h(1 - h(np.float32(b1) ** 1)))
-        vhat = h(var / h(1 - h(np.float32(b2) ** 1)))
-        want = np.float16(np.float32(p0[i]) - h(h(lr * mhat) / h(np.sqrt(h(max(np.float32(0), vhat) + eps)))))
-        assert p[i] == want
-        assert abs(float(p0[i]) - float(p[i]) - 0.01 * np.sign(gi)) < 2e-3
-    # NaN gradients are cleared and skipped, infinities clipped to +-10000, gradients zeroed
+def ulp16(v):
+    return float(ob.f16_ulp(np.array([v], np.float32))[0])
+
+
+def test_constant_gradient_moves_by_lr_every_step():
+    # constant g: mean_n = (1-b1^n) g and var_n = (1-b2^n) g^2, so the bias-corrected moments are g
+    # and g^2 at every step and the update is lr*g/(|g|+eps) = lr*sign(g).  This needs the state to
+    # carry over and the correction to use pow(beta, iteration) with the running count: without
+    # carry-over step 2 would move by 0.53*lr, with a constant exponent by 1.34*lr.
+    # Bound: 3 % of lr for the half roundings of mean, variance, both corrections, sqrt and the
+    # quotient (each 2^-11 relative, variance halved by the root) plus the rounding of p itself.
+    # Gradients are chosen so that (1-b2) g^2 is a normal fp16 number: below that the source's own
+    # arithmetic loses the variance to subnormal rounding.
+    g = np.array([0.5, -1.5, 2.0, -3.0, 0.75, -40.0], np.float16)
+    p = np.zeros(6, np.float16)
+    st = np.zeros(6, ob.ADAM_STATE_DTYPE)
+    for n in range(1, 17):
+        before = p.astype(np.float64)
+        ob.slang_adam_step(st, p, g.copy())
+        assert (st["iteration"] == n).all()
+        step = before - p.astype(np.float64)
+        for i in range(6):
+            assert abs(step[i] - LR * np.sign(float(g[i]))) <= 0.03 * LR + ulp16(p[i]), (n, i, step[i])
+
+
+def test_impulse_response_separates_the_two_betas():
+    # one gradient g, then zeros: mean_n = b1^(n-1)(1-b1) g, var_n = b2^(n-1)(1-b2) g^2, so step n moves by
+    #   lr * [b1^(n-1)(1-b1)/(1-b1^n)] / sqrt(b2^(n-1)(1-b2)/(1-b2^n)) * sign(g)
+    # (0.670 lr at n = 2; 0.726 lr if the betas were swapped).  Betas as fp16 values, as the source has them.
+    b1, b2 = float(np.float16(B1)), float(np.float16(B2))
+    g0 = np.array([1.0, -0.5, 8.0], np.float16)
+    p = np.zeros(3, np.float16)
+    st = np.zeros(3, ob.ADAM_STATE_DTYPE)
+    for n in range(1, 9):
+        g = g0.copy() if n == 1 else np.zeros(3, np.float16)
+        before = p.astype(np.float64)
+        ob.slang_adam_step(st, p, g)
+        want = LR * (b1 ** (n - 1) * (1 - b1) / (1 - b1 ** n)) / np.sqrt(b2 ** (n - 1) * (1 - b2) / (1 - b2 ** n))
+        step = before - p.astype(np.float64)
+        for i in range(3):
+            assert abs(step[i] - want * np.sign(float(g0[i]))) <= 0.03 * LR + ulp16(p[i]), (n, i, step[i], want)
+        assert (g == 0).all() and (st["iteration"] == n).all()
+
+
+def test_nan_skips_and_infinities_clip():
+    # kernels.slang:39-43: a NaN gradient is cleared and the parameter's state is left alone (no
+    # iteration, no decay); adam.slang:23-29: +-inf count as +-10000
     g = np.array([np.nan, np.inf, -np.inf, 1.0], np.float16)
     p = np.ones(4, np.float16); st = np.zeros(4, ob.ADAM_STATE_DTYPE)
     ob.slang_adam_step(st, p, g)
     assert (g == 0).all() and st["iteration"].tolist() == [0, 1, 1, 1]
-    # in half, (1-b2)*10000*10000 overflows: variance = inf, so the step itself is 0 -- faithful to
+    # in half, (1-b2)*10000*10000 overflows: variance = inf and the step itself is 0 -- faithful to
     # the source's arithmetic; the state still advances
-    assert p[0] == 1.0 and p[1] == 1.0 and p[2] == 1.0
+    assert p[0] == 1.0 and p[1] == 1.0 and p[2] == 1.0 and p[3] < 1.0
     assert np.isinf(st["variance"][1:3].view(np.float16)).all() and st["mean"][3] != 0
+    # a NaN in the middle of a run: the other steps behave as if it had not been there
+    pa = np.zeros(1, np.float16); sa = np.zeros(1, ob.ADAM_STATE_DTYPE)
+    pb = np.zeros(1, np.float16); sb = np.zeros(1, ob.ADAM_STATE_DTYPE)
+    for n in range(6):
+        ob.slang_adam_step(sa, pa, np.array([0.5], np.float16))
+        if n == 2:
+            ob.slang_adam_step(sb, pb, np.array([np.nan], np.float16))
+        ob.slang_adam_step(sb, pb, np.array([0.5], np.float16))
+    assert pa[0] == pb[0] and sa.tobytes() == sb.tobytes()
 
 
 @pytest.mark.gpu
@@ -52,20 +88,33 @@ def test_gpu_adam_matches_oracle():
     st = np.zeros(n, ob.ADAM_STATE_DTYPE)
     pd = torch.from_numpy(p.copy()).cuda()
     sd = torch.zeros(n * 8, dtype=torch.uint8, device="cuda")
-    mism = 0
+    pow_cases = 0
     for it in range(12):
         g = (rng.standard_normal(n) * 10.0 ** rng.integers(-4, 3, n)).astype(np.float16)
         g[::97] = np.nan; g[5::101] = np.inf; g[7::103] = -np.inf
         gd = torch.from_numpy(g.copy()).cuda()
         cv.adjustParameters(sd, pd, gd)
-        ob.slang_adam_step(st, p, g)
+        # the oracle with pow() as the host library rounds it, and with its fp32 value one or two ulps
+        # to either side for each beta: the only operation the two libraries may round differently
+        variants = {}
+        for n1 in range(-2, 3):
+            for n2 in range(-2, 3):
+                pv, sv, gv = p.copy(), st.copy(), g.copy()
+                ob.slang_adam_step(sv, pv, gv, pow_nudge=(n1, n2))
+                variants[(n1, n2)] = (pv, sv)
         assert (gd.cpu().numpy() == 0).all()
         got = pd.cpu().numpy()
-        # identical arithmetic; only powf may differ by an fp32 ulp between the two maths libraries
-        mism = max(mism, int((got.view(np.uint16) != p.view(np.uint16)).sum()))
-        assert np.max(np.abs(got.astype(np.float32) - p.astype(np.float32))) <= 2e-3
         stg = sd.cpu().numpy().view(ob.ADAM_STATE_DTYPE)
-        assert (stg["iteration"] == st["iteration"]).all()
+        ref_p, ref_s = variants[(0, 0)]
+        # state: no pow() involved, bit-equal always
+        assert stg.tobytes() == ref_s.tobytes()
+        differs = got.view(np.uint16) != ref_p.view(np.uint16)
+        if differs.any():
+            explained = np.zeros(n, bool)
+            for pv, _ in variants.values():
+                explained |= got.view(np.uint16) == pv.view(np.uint16)
+            assert explained[differs].all(), "parameters differ from the oracle beyond the rounding of pow()"
+            pow_cases += int(differs.sum())
         # continue from the GPU's state so that differences do not accumulate in the comparison
         p = got.copy(); st = stg.copy()
-    assert mism <= n // 100
+    assert pow_cases <= n // 100

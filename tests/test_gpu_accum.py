@@ -93,6 +93,27 @@ def test_reduce_sum_against_fp64(N, B):
     assert torch.equal(d, d2)
 
 
+def test_outer_product_infinite_element_stays_within_its_fragment():
+    # One infinite b[s][j].  The reference's per-element a[i]*b[j] (hlsl.meta.slang:33261-33315) makes
+    # column j of the destination non-finite and nothing else.  Here the sample-major -> feature-major
+    # transposition multiplies a fragment of 32 features by a 0/1 selection matrix on the MFMA, and
+    # 0 * Inf = NaN: the columns that share j's 32-feature fragment become NaN as well.  Everything
+    # outside that fragment stays exact.
+    rng = np.random.default_rng(99)
+    M, N, B, j = 64, 64, 1000, 5
+    a = (rng.standard_normal((B, M)) * 0.25).astype(np.float16)
+    b = rng.uniform(-1, 1, (B, N)).astype(np.float16)
+    b[123, j] = np.inf
+    d = torch.zeros(M * N, dtype=torch.float32, device=DEV)
+    cv.coopVecOuterProductAccumulate(to_dev(a), to_dev(b), d.view(torch.uint8), 0, N * 4, ML.RowMajor, CT.Float32)
+    got = d.cpu().numpy().reshape(M, N).astype(np.float64)
+    bad_cols = np.nonzero(~np.isfinite(got).all(axis=0))[0]
+    assert j in bad_cols and len(bad_cols) <= 32
+    ok = np.setdiff1d(np.arange(N), bad_cols)
+    want = a.astype(np.float64).T @ b.astype(np.float64)[:, ok]
+    assert np.linalg.norm(got[:, ok] - want) <= 1e-3 * np.linalg.norm(want)
+
+
 def test_accumulate_argument_validation():
     a = torch.zeros(4, 8, dtype=torch.float16, device=DEV)
     m = torch.zeros(1024, dtype=torch.uint8, device=DEV)

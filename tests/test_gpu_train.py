@@ -153,6 +153,42 @@ def test_train_tie_rule_and_leaky_relu():
         assert rel_err(dW[l], rW[l]) <= 1e-3 and rel_err(dB[l], rB[l]) <= 1e-3
 
 
+def test_train_tie_rule_wide_network():
+    # 8 -> 64 -> 64 -> 1 with ReLU (the kernel instantiation the training configuration uses), one
+    # sample, all values dyadic so that every sum is exact in fp16 and fp32 on both sides.  Layer 0 is
+    # crafted so that hidden unit 0 has z = +0, unit 1 has a negative sum that rounds to -0 in fp16
+    # (-2^-14 * 2^-14), unit 2 is negative and unit 3 positive; Slang's max() rule gives the tied
+    # units half of the gradient whatever the sign of the zero (diff.meta.slang:2258-2277).
+    rng = np.random.default_rng(314)
+    tiny = np.float16(2.0 ** -14)
+    W0 = np.zeros((64, 8), np.float16)
+    W0[1, 0] = -tiny; W0[2, 0] = -1.0; W0[3, 1] = 1.0
+    x = np.zeros((1, 8), np.float16); x[0, 0] = tiny; x[0, 1] = 1.0
+    W1 = rng.choice(np.array([-1, -0.5, -0.25, 0.25, 0.5, 1], np.float16), (64, 64))
+    W1[:4, 3] = [0.0, 0.5, -1.0, 0.25]          # layer 1 gets a tie, two positives and a negative of its own
+    W2 = rng.choice(np.array([-1, -0.5, 0.5, 1], np.float16), (1, 64))
+    specs = [dict(W=W0, b=np.zeros(64, np.float16), act=1), dict(W=W1, b=None, act=1), dict(W=W2, b=None, act=0)]
+    a1 = np.maximum(W1[:, 3].astype(np.float64), 0)
+    y = float((W2.astype(np.float64) @ a1)[0])
+    t = np.array([[y - 0.5]], np.float16)                # dL/dy = 2 * 0.5 = 1
+    assert float(t[0, 0]) == y - 0.5
+    layers = build(specs, grad_layout=ML.TrainingOptimal)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.TrainingOptimal)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
+    assert loss.item() == 0.25 == rloss
+    for l in range(3):
+        assert np.array_equal(dW[l], rW[l]) and np.array_equal(dB[l], rB[l]), l
+    # the rule itself, against the upstream gradient g0 = W1^T dz1 of layer 0's outputs
+    dz1 = W2[0].astype(np.float64) * np.where(W1[:, 3] > 0, 1.0, np.where(W1[:, 3] == 0, 0.5, 0.0))
+    g0 = W1.astype(np.float64).T @ dz1
+    assert dB[0][0] == 0.5 * g0[0] and dB[0][1] == 0.5 * g0[1] and dB[0][2] == 0.0 and dB[0][3] == g0[3]
+    assert g0[0] != 0 and g0[1] != 0 and g0[2] != 0
+    # without the tie rule the oracle disagrees, i.e. the check above has teeth
+    nW, nB, _ = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=False)
+    assert not np.array_equal(nB[0], rB[0])
+
+
 def test_train_fp16_training_optimal_gradients_and_convert():
     # the example's flow: fp16 TrainingOptimal weight gradients, then one convert call to RowMajor
     rng = np.random.default_rng(10)
@@ -199,7 +235,8 @@ def test_full_size_training_step_properties():
     specs = make_specs(rng, dims, bias=False)
     g = torch.Generator(device=DEV); g.manual_seed(5)
     x = (torch.rand(B, 8, device=DEV, generator=g) * 2 - 1).half()
-    la, lb, lc = build(specs), build(specs), build(specs)
+    TO = ML.TrainingOptimal      # the configuration's gradient destinations: fp32 TrainingOptimal
+    la, lb, lc = build(specs, grad_layout=TO), build(specs, grad_layout=TO), build(specs, grad_layout=TO)
     _, loss_a = cv.mlpTrainStep(la, x, None)
     _, loss_b = cv.mlpTrainStep(lb, x, None)
     cv.mlpTrainStep(lc, x, None, lossScale=0.5)
@@ -211,14 +248,14 @@ def test_full_size_training_step_properties():
     assert loss_a.item() == loss_b.item()
     # the first 4096 samples against the fp64 oracle (same kernel, smaller batch)
     n = 4096
-    ls = build(specs)
+    ls = build(specs, grad_layout=TO)
     cv.mlpTrainStep(ls, x[:n], None)
-    dW, dB = read_grads(ls, specs, CT.Float32, ML.RowMajor)
+    dW, dB = read_grads(ls, specs, CT.Float32, TO)
     rW, rB, _ = ob.ref_mlp_train(specs, x[:n].cpu().numpy(), None, 1.0, True)
     for l in range(len(specs)):
         assert rel_err(dW[l], rW[l]) <= 1e-3
     # additivity over a split of the batch (fp32 sums in a different order: relative 1e-5)
-    l1, l2 = build(specs), build(specs)
+    l1 = build(specs, grad_layout=TO)
     cv.mlpTrainStep(l1, x[: B // 2], None)
     cv.mlpTrainStep(l1, x[B // 2:], None)        # "+=" into the same buffers
     for a, s in zip(la, l1):
