@@ -45,7 +45,7 @@ __device__ __forceinline__ void loadQuarter(uint32_t (&dst)[8], const uint8_t* r
 }
 
 // grid: x = persistent workgroups over the batch, y = output block (by * nbx + bx)
-__global__ __launch_bounds__(256) void outerProductKernel(const OuterArgs a)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void outerProductKernel(const OuterArgs a)
 {
     typedef F16Mma Mma;
     __shared__ __attribute__((aligned(16))) float ldsRed[4 * 256];
@@ -82,20 +82,24 @@ __global__ __launch_bounds__(256) void outerProductKernel(const OuterArgs a)
 
     const uint32_t numTiles = (a.batch + 31) / 32;
     const uint32_t lastSample = a.batch - 1;
-    for (uint32_t tile = blockIdx.x * 4 + wave; tile < numTiles; tile += gridDim.x * 4) {
-        // S fragments: lane group g owns columns [16g, 16g+16) of the block, as two 8-slot fragments
-        uint32_t aS[2][8], bS[2][8];
+    const uint32_t tileStride = gridDim.x * 4;
+    // S fragments of a tile of 32 samples: lane group g owns columns [16g, 16g+16) of the block, as
+    // two 8-slot fragments per 16-sample half
+    auto loadTile = [&](uint32_t (&aS)[2][8], uint32_t (&bS)[2][8], uint32_t tile) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const uint32_t s = tile * 32 + 16 * j + n;
-            const uint32_t sc = min(s, lastSample);
+            const uint32_t sc = min(tile * 32 + 16 * j + n, lastSample);
             loadQuarter(aS[j], a.a + (size_t)sc * a.aStride, m0 + 16 * g, a.m, a.aAlign >= 16u);
             loadQuarter(bS[j], a.b + (size_t)sc * a.bStride, n0 + 16 * g, a.n, a.bAlign >= 16u);
-            if (s > lastSample) {      // samples past the end contribute nothing
+        }
+    };
+    auto compute = [&](uint32_t (&aS)[2][8], const uint32_t (&bS)[2][8], uint32_t tile) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            if (tile * 32 + 16 * j + n > lastSample) {      // samples past the end contribute nothing
 #pragma unroll
                 for (int i = 0; i < 8; ++i) aS[j][i] = 0u;
             }
-        }
         uint32_t bF[4][4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) toF(&bS[0][4 * (e / 2)], &bS[1][4 * (e / 2)], e & 1, bF[e]);
@@ -105,6 +109,23 @@ __global__ __launch_bounds__(256) void outerProductKernel(const OuterArgs a)
             toF(&aS[0][4 * (eo / 2)], &aS[1][4 * (eo / 2)], eo & 1, aF);
 #pragma unroll
             for (int ei = 0; ei < 4; ++ei) acc[eo][ei] = Mma::mma(aF, bF[ei], acc[eo][ei]);
+        }
+    };
+    // the next tile's loads are in flight while the current one is contracted
+    {
+        uint32_t tile = blockIdx.x * 4 + wave;
+        if (tile < numTiles) {
+            uint32_t aCur[2][8], bCur[2][8], aNxt[2][8], bNxt[2][8];
+            loadTile(aCur, bCur, tile);
+            for (; tile < numTiles; tile += tileStride) {
+                const uint32_t t1 = tile + tileStride;
+                loadTile(aNxt, bNxt, t1 < numTiles ? t1 : tile);
+                compute(aCur, bCur, tile);
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) { aCur[j][i] = aNxt[j][i]; bCur[j][i] = bNxt[j][i]; }
+            }
         }
     }
 
@@ -121,10 +142,32 @@ __global__ __launch_bounds__(256) void outerProductKernel(const OuterArgs a)
         }
 }
 
-// one thread per element of the (padded) block grid
+// A workgroup owns 64 consecutive values of one block's partial; its four waves each sum a quarter
+// of the partials (eight loads in flight per lane) and wave 0 adds the four sums in a fixed order.
 __global__ __launch_bounds__(256) void outerReduceKernel(const OuterArgs a, uint32_t numPartials)
 {
-    const uint32_t p = blockIdx.x * 256u + threadIdx.x;          // index inside one block's partial
+    __shared__ float red[4 * 64];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t p = blockIdx.x * 64u + lane;                  // index inside one block's partial
+    {
+        const uint32_t per = (numPartials + 3u) / 4u;
+        const uint32_t b0 = wave * per, b1 = min(b0 + per, numPartials);
+        const float* src = a.partials + (size_t)blockIdx.y * numPartials * kOuterPartialFloats + p;
+        float c = 0.f;
+        uint32_t b = b0;
+        for (; b + 8 <= b1; b += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(b + u) * kOuterPartialFloats];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) c += v[u];
+        }
+        for (; b < b1; ++b) c += src[(size_t)b * kOuterPartialFloats];
+        red[wave * 64 + lane] = c;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const float s = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
     const int nbx = (a.n + kBlk - 1) / kBlk;
     const int by = blockIdx.y / nbx, bx = blockIdx.y % nbx;
     const uint32_t tile = p >> 8, ln = (p >> 2) & 63u, r = p & 3u;
@@ -133,9 +176,6 @@ __global__ __launch_bounds__(256) void outerReduceKernel(const OuterArgs a, uint
     const uint32_t row = (uint32_t)by * kBlk + gq * 16u + 4u * eo + r;
     const uint32_t col = (uint32_t)bx * kBlk + (qi >> 2) * 16u + 4u * ei + (qi & 3u);
     if (row >= (uint32_t)a.m || col >= (uint32_t)a.n) return;
-    const float* src = a.partials + (size_t)blockIdx.y * numPartials * kOuterPartialFloats + p;
-    float s = 0.f;
-    for (uint32_t b = 0; b < numPartials; ++b) s += src[(size_t)b * kOuterPartialFloats];
     uint8_t* d = a.mat + elemOffset(a.shape, row, col);
     if (a.shape.ct == kF32) *(float*)d += s;
     else *(half_t*)d = (half_t)((float)*(half_t*)d + s);
@@ -183,20 +223,101 @@ __global__ __launch_bounds__(256) void reduceSumKernel(const ReduceSumArgs a)
     }
 }
 
+// Streaming form for rows of whole 16-byte chunks (n % 8 == 0, 16-byte aligned base and stride): a row
+// is C = n/8 chunks; LP = C rounded up to a power of two lanes share a row, a wave covers 64/LP rows
+// per load, and every lane keeps eight fp32 sums for the eight columns of its chunk.  With a dense
+// batch (stride = 2n) consecutive lanes read consecutive 16-byte pieces of memory.
+constexpr int kRsUnroll = 8;
+__global__ __launch_bounds__(256) void reduceSumStreamKernel(const ReduceSumArgs a, uint32_t lanesPerRow)
+{
+    __shared__ __attribute__((aligned(16))) float ldsRed[4 * 64 * 8];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t chunks = (uint32_t)a.n / 8u;
+    const uint32_t rowsPerLoad = 64u / lanesPerRow;
+    const uint32_t r = lane / lanesPerRow, c = lane % lanesPerRow;
+    const bool active = c < chunks;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+    const uint32_t span = rowsPerLoad * kRsUnroll;                 // rows a wave takes per iteration
+    const uint8_t* base = a.v + (size_t)c * 16u;
+    for (uint64_t row0 = (uint64_t)(blockIdx.x * 4u + wave) * span; row0 < a.batch; row0 += (uint64_t)gridDim.x * 4u * span) {
+        u32x4 v[kRsUnroll];
+#pragma unroll
+        for (int u = 0; u < kRsUnroll; ++u) {
+            const uint64_t s = row0 + (uint64_t)u * rowsPerLoad + r;
+            v[u] = u32x4{0u, 0u, 0u, 0u};
+            if (active && s < a.batch) v[u] = *(const u32x4*)(base + s * a.vStride);
+        }
+#pragma unroll
+        for (int u = 0; u < kRsUnroll; ++u) {
+            const uint32_t dw[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const halfx2 h = __builtin_bit_cast(halfx2, dw[d]);
+                acc[2 * d] += (float)h.x;
+                acc[2 * d + 1] += (float)h.y;
+            }
+        }
+    }
+    // workgroup partial per column: rows of the wave, then the four waves, in a fixed order
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ldsRed[(wave * 64 + lane) * 8 + i] = acc[i];
+    __syncthreads();
+    const uint32_t col = threadIdx.x;
+    if (col < (uint32_t)a.n) {
+        float s = 0.f;
+        for (uint32_t w = 0; w < 4; ++w)
+            for (uint32_t rr = 0; rr < rowsPerLoad; ++rr) s += ldsRed[(w * 64 + rr * lanesPerRow + col / 8u) * 8 + (col & 7u)];
+        a.partials[(size_t)blockIdx.x * kMaxReduceCols + col] = s;
+    }
+}
+
+// 64 columns per workgroup; its four waves each sum a quarter of the partials, wave 0 combines.
 __global__ __launch_bounds__(256) void reduceSumFinalKernel(const ReduceSumArgs a, uint32_t numPartials)
 {
-    const uint32_t col = blockIdx.x * 256u + threadIdx.x;
-    if (col >= (uint32_t)a.n) return;
-    float s = 0.f;
-    for (uint32_t b = 0; b < numPartials; ++b) s += a.partials[(size_t)b * kMaxReduceCols + col];
+    __shared__ float red[4 * 64];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t col = blockIdx.x * 64u + lane;
+    const bool inRange = col < (uint32_t)a.n;
+    {
+        const uint32_t per = (numPartials + 3u) / 4u;
+        const uint32_t b0 = wave * per, b1 = min(b0 + per, numPartials);
+        float c = 0.f;
+        if (inRange) {
+            const float* src = a.partials + col;
+            uint32_t b = b0;
+            for (; b + 8 <= b1; b += 8) {
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(b + u) * kMaxReduceCols];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) c += v[u];
+            }
+            for (; b < b1; ++b) c += src[(size_t)b * kMaxReduceCols];
+        }
+        red[wave * 64 + lane] = c;
+    }
+    __syncthreads();
+    if (wave != 0 || !inRange) return;
+    const float s = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
     if (a.bufCt == kF32) ((float*)a.buf)[col] += s;
     else ((half_t*)a.buf)[col] = (half_t)((float)((half_t*)a.buf)[col] + s);
 }
 
+// persistent workgroups of the streaming reduce-sum kernel: eight per compute unit
+uint32_t reduceStreamGridX(uint32_t batch, int numCUs)
+{
+    const uint32_t need = (batch + 4u * kRsUnroll - 1u) / (4u * kRsUnroll);      // at least one row per wave-iteration
+    const uint32_t cap = 8u * (uint32_t)numCUs;
+    return need < cap ? (need ? need : 1) : cap;
+}
+
 uint32_t outerGridX(uint32_t batch, int numCUs)
 {
+    // two workgroups per compute unit: eight waves whose loads overlap each other's MFMAs
     const uint32_t rounds = (batch + 31) / 32, need = (rounds + 3) / 4;
-    const uint32_t cap = (uint32_t)numCUs;
+    const uint32_t cap = 2u * (uint32_t)numCUs;
     return need < cap ? (need ? need : 1) : cap;
 }
 
@@ -217,25 +338,35 @@ hipError_t launchOuterProduct(hipStream_t stream, const OuterArgs& a, int numCUs
     hipLaunchKernelGGL(outerProductKernel, dim3(gx, blocks), dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(outerReduceKernel, dim3(kOuterPartialFloats / 256, blocks), dim3(256), 0, stream, a, gx);
+    hipLaunchKernelGGL(outerReduceKernel, dim3(kOuterPartialFloats / 64, blocks), dim3(256), 0, stream, a, gx);
     return hipGetLastError();
 }
 
 size_t reduceSumWorkspaceBytes(uint32_t batch, int numCUs)
 {
-    return (size_t)outerGridX(batch * 2, numCUs) * kMaxReduceCols * sizeof(float);
+    const uint32_t gx = max(outerGridX(batch * 2, numCUs), reduceStreamGridX(batch, numCUs));
+    return (size_t)gx * kMaxReduceCols * sizeof(float);
 }
 
 hipError_t launchReduceSum(hipStream_t stream, const ReduceSumArgs& a, int numCUs)
 {
     if (a.batch == 0) return hipSuccess;
     if (a.n > kMaxReduceCols) return hipErrorInvalidValue;
-    const uint32_t gx = outerGridX(a.batch * 2, numCUs);
-    noteKernel(false, "reduceSumKernel + reduceSumFinalKernel");
-    hipLaunchKernelGGL(reduceSumKernel, dim3(gx), dim3(256), 0, stream, a);
+    uint32_t gx;
+    if (a.n % 8 == 0 && ((uintptr_t)a.v & 15u) == 0 && (a.vStride & 15u) == 0) {
+        uint32_t lanesPerRow = 1;
+        while (lanesPerRow < (uint32_t)a.n / 8u) lanesPerRow *= 2;
+        gx = reduceStreamGridX(a.batch, numCUs);
+        noteKernel(false, "reduceSumStreamKernel + reduceSumFinalKernel");
+        hipLaunchKernelGGL(reduceSumStreamKernel, dim3(gx), dim3(256), 0, stream, a, lanesPerRow);
+    } else {
+        gx = outerGridX(a.batch * 2, numCUs);
+        noteKernel(false, "reduceSumKernel + reduceSumFinalKernel");
+        hipLaunchKernelGGL(reduceSumKernel, dim3(gx), dim3(256), 0, stream, a);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(reduceSumFinalKernel, dim3((a.n + 255) / 256), dim3(256), 0, stream, a, gx);
+    hipLaunchKernelGGL(reduceSumFinalKernel, dim3((a.n + 63) / 64), dim3(256), 0, stream, a, gx);
     return hipGetLastError();
 }
 

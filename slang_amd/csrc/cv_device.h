@@ -107,6 +107,26 @@ struct I8Mma {   // int8 x int8 -> int32
     }
 };
 
+// ---- floating-point mode ----------------------------------------------------------------
+// MODE.FP16_OVFL (hardware mode register 1, bit 23).  While it is set, conversions to fp16 and to
+// fp8 clamp an out-of-range result to the largest finite value (65504 / 448) instead of producing
+// inf / NaN.  Measured on gfx950: with the bit set v_cvt_scalef32_pk_fp8_f16 equals the saturating
+// OCP e4m3 quantiser for every one of the 65 536 fp16 inputs (NaN aside), so the explicit clamp to
+// +-448 in front of it can go.  fp32 -> fp16 conversions clamp too while it is set, which is the
+// same thing for a value that is quantised to e4m3 next, but not for a kernel's fp16 output: the
+// bit is cleared around those.
+template <bool ON>
+__device__ __forceinline__ void setFp16OverflowClamp()
+{
+    __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), ON ? 1 : 0);
+}
+
+// Makes `v` pass through this point of the program: nothing that computes v can sink below it and
+// nothing that uses v can rise above it.  Used on both sides of a mode switch, whose ordering
+// against plain arithmetic the optimiser would not keep by itself.
+template <class T>
+__device__ __forceinline__ void pinHere(T& v) { asm volatile("" : "+v"(v)); }
+
 // ---- scalar helpers ---------------------------------------------------------------------
 
 __device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct)

@@ -100,20 +100,25 @@ __device__ __forceinline__ void carrierFromAcc(const floatx4& acc, const Carrier
 }
 
 // fp16 pair x2 -> one dword of four e4m3 bytes (saturating, nearest even: v_cvt_scalef32_pk_fp8_f16
-// rounds like the fp32 route for every fp16 input within +-448)
+// rounds like the fp32 route for every fp16 input within +-448).  MODE_CLAMPS: the caller runs
+// with MODE.FP16_OVFL set, under which the instruction saturates by itself.
+template <bool MODE_CLAMPS = false>
 __device__ __forceinline__ uint32_t quantE4M3x4(halfx2 h01, halfx2 h23, const CarrierCfg& c)
 {
     typedef short shortx2 __attribute__((ext_vector_type(2)));
-    h01 = __builtin_elementwise_min(h01, c.ceil2);
-    h23 = __builtin_elementwise_min(h23, c.ceil2);
-    shortx2 r = {0, 0};
+    if constexpr (!MODE_CLAMPS) {
+        h01 = __builtin_elementwise_min(h01, c.ceil2);
+        h23 = __builtin_elementwise_min(h23, c.ceil2);
+    }
+    // both halves of r are overwritten; starting from a value that is live anyway saves a move
+    shortx2 r = __builtin_bit_cast(shortx2, h01);
     r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h01, 1.0f, false);
     r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h23, 1.0f, true);
     return __builtin_bit_cast(uint32_t, r);
 }
 
 // Two accumulator tiles (already carriers) -> one B fragment of the next layer (8 k-slots per lane).
-template <class Mma>
+template <class Mma, bool MODE_CLAMPS = false>
 __device__ __forceinline__ void fragFromCarrier(halfx2 lo01, halfx2 lo23, halfx2 hi01, halfx2 hi23,
                                                 const CarrierCfg& c, uint32_t* frag)
 {
@@ -122,7 +127,7 @@ __device__ __forceinline__ void fragFromCarrier(halfx2 lo01, halfx2 lo23, halfx2
         frag[2] = __builtin_bit_cast(uint32_t, hi01); frag[3] = __builtin_bit_cast(uint32_t, hi23);
     } else {
         // re-quantise the fp16 carrier to OCP e4m3
-        const uint32_t raw[2] = {quantE4M3x4(lo01, lo23, c), quantE4M3x4(hi01, hi23, c)};
+        const uint32_t raw[2] = {quantE4M3x4<MODE_CLAMPS>(lo01, lo23, c), quantE4M3x4<MODE_CLAMPS>(hi01, hi23, c)};
         Mma::decode(raw, frag);      // e4m3 bytes as they are, or decoded back to fp16 operands
     }
 }

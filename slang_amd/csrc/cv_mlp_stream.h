@@ -26,11 +26,15 @@ __device__ __forceinline__ void carrierNoLeaky(const floatx4& acc, const Carrier
     h23 = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[2], acc[3]}, halfx2), c.floor2);
 }
 
+#ifndef CV_MLP_STREAM_MINWAVES
+#define CV_MLP_STREAM_MINWAVES 1
+#endif
 template <class Mma, class Net, int NT, int S, bool HAS_BIAS>
-__global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STREAM_MINWAVES))) void mlpStreamKernel(const MlpArgs a)
 {
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     constexpr int L = Net::L;
+    constexpr bool QUANT = !std::is_same<Mma, F16Mma>::value;   // e4m3 carrier between layers
     constexpr int IN_DW = RAW * Net::KT0;          // dwords one lane contributes per sample tile
     constexpr int ROW_DW = 4 * IN_DW;              // dwords of one sample's input row
     constexpr int SLOT_DW = S * 16 * ROW_DW;       // dwords of one slot
@@ -166,6 +170,16 @@ __global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
                         raw[2 * i] = v.x; raw[2 * i + 1] = v.y;
                     }
                 }
+                if constexpr (QUANT) {
+                    // from here to the last layer's accumulators the conversions saturate by mode
+                    if (j == 0) {
+#pragma unroll
+                        for (int i = 0; i < IN_DW; ++i) pinHere(raw[i]);
+                        setFp16OverflowClamp<true>();
+                    }
+#pragma unroll
+                    for (int i = 0; i < IN_DW; ++i) pinHere(raw[i]);
+                }
 #pragma unroll
                 for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&raw[kt * RAW], act[j][kt]);
             }
@@ -201,9 +215,21 @@ __global__ __launch_bounds__(256) void mlpStreamKernel(const MlpArgs a)
                             halfx2 lo01, lo23, hi01 = {(half_t)0, (half_t)0}, hi23 = {(half_t)0, (half_t)0};
                             carrierNoLeaky(acc[j][2 * kt], cc[l], lo01, lo23);
                             if (2 * kt + 1 < MT) carrierNoLeaky(acc[j][2 * kt + 1 < MT ? 2 * kt + 1 : 0], cc[l], hi01, hi23);
-                            fragFromCarrier<Mma>(lo01, lo23, hi01, hi23, cc[l], act[j][kt]);
+                            fragFromCarrier<Mma, QUANT>(lo01, lo23, hi01, hi23, cc[l], act[j][kt]);
                         }
                 } else {
+                    if constexpr (QUANT) {
+                        // the network's fp16 output keeps inf for an overflow: mode off before it is formed
+#pragma unroll
+                        for (int j = 0; j < NT; ++j)
+#pragma unroll
+                            for (int t = 0; t < MT; ++t) pinHere(acc[j][t]);
+                        setFp16OverflowClamp<false>();
+#pragma unroll
+                        for (int j = 0; j < NT; ++j)
+#pragma unroll
+                            for (int t = 0; t < MT; ++t) pinHere(acc[j][t]);
+                    }
 #pragma unroll
                     for (int j = 0; j < NT; ++j) {
                         const uint32_t sample = slot * SLOT + 16 * (r0 + j) + n;

@@ -201,6 +201,41 @@ def test_e4m3_decoder_config(flags):
         assert frac >= 0.80, "only %.5f within tolerance" % frac
 
 
+@pytest.mark.parametrize("flags", [0, cv.FLAG_FP8_MATRIX_PIPELINE])
+@pytest.mark.parametrize("B", [4096, 50])       # streaming kernel / tail path
+def test_e4m3_saturation_and_fp16_overflow(flags, B):
+    # hidden sums beyond +-448 saturate when the carrier is re-quantised (also through an fp16
+    # overflow: inf -> 448), while an overflow of the network's own fp16 output stays inf
+    rng = np.random.default_rng(448)
+    dims = [32, 64, 64, 8]
+    specs = make_net(rng, dims, CT.FloatE4M3, act=Activation.NoActivation, bias="none", init="half")
+    for s in specs[:-1]:
+        s["act"] = int(Activation.NoActivation)
+    specs[0]["W"][:8] = ob.encode_e4m3(np.full((8, 32), 448.0))         # rows that overflow fp16 (+)
+    specs[0]["W"][8:16] = ob.encode_e4m3(np.full((8, 32), -448.0))      # ... and (-)
+    specs[0]["W"][16:24] = ob.encode_e4m3(np.full((8, 32), 2.0))        # beyond 448, within fp16
+    specs[2]["W"][0] = ob.encode_e4m3(np.full(64, 448.0))               # output row that can overflow fp16
+    xf = rng.standard_normal((B, 32)) * 0.5
+    xf[::3] = 448.0
+    xf[1::7] = -448.0
+    x = ob.encode_e4m3(xf)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, ML.InferencingOptimal), xd, weightType=CT.FloatE4M3, flags=flags)
+    hid = []
+    yc = chain_of_single_layers(specs, xd, CT.FloatE4M3, flags, hidden=hid)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    ref, acts = ob.ref_mlp_forward(specs, x, ob.E4M3, want_acts=True)
+    got = y.cpu().numpy()
+    assert np.isinf(ref).any() and np.isinf(acts[0]).any()              # the case is exercised
+    assert np.array_equal(np.isinf(got), np.isinf(ref))
+    assert np.array_equal(got[np.isinf(ref)], ref[np.isinf(ref)])       # same sign of inf
+    if flags == 0:
+        fin = np.isfinite(ref)
+        bad = ob.float_parity_violations(got[fin], ref[fin].astype(np.float32),
+                                         (np.abs(acts[1].astype(np.float32)) @ np.abs(ob.decode_e4m3(specs[2]["W"])).T)[fin])
+        assert bad.mean() <= 1e-3
+
+
 def test_mlp_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_net(rng, [8, 16, 4], CT.Float16)
