@@ -84,7 +84,12 @@ typedef enum CvRhiComponentType {
 /* Activation fused behind a matMulAdd.  RELU is max(z, 0) as the neural module defines it
  * (source/standard-modules/neural/activations.slang:25-42); LEAKY_RELU is the example's
  * max(z, z * slope) evaluated in half (examples/mlp-training-coopvec/fflayer.slang:64-65). */
-typedef enum CvActivation { CV_ACT_NONE = 0, CV_ACT_RELU = 1, CV_ACT_LEAKY_RELU = 2 } CvActivation;
+typedef enum CvActivation {
+    CV_ACT_NONE = 0, CV_ACT_RELU = 1, CV_ACT_LEAKY_RELU = 2,
+    /* the remaining activations of the neural module (activations.slang:88-233), evaluated on the
+     * fp16 (or fp32) result element: in fp32, rounded once */
+    CV_ACT_SIGMOID = 3, CV_ACT_TANH = 4, CV_ACT_EXP = 5, CV_ACT_SINE = 6, CV_ACT_SILU = 7, CV_ACT_QUICK_GELU = 8
+} CvActivation;
 
 /* Flags of CvMatMulDesc / CvMlpDesc.
  * By default FLOAT_E4M3 operands are decoded (exactly) to fp16 and multiplied on the fp16
@@ -234,6 +239,42 @@ CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStrid
                                       int32_t elementType, uint32_t batch,
                                       void* buffer, size_t offset, int32_t bufferType,
                                       void* workspace, size_t workspaceBytes);
+
+/* ------------------------------------------------------------------------------------ */
+/* element-wise surface of CoopVec<T,N>                                                  */
+/* ------------------------------------------------------------------------------------ */
+
+/* The per-component operators and math functions Slang declares on CoopVec<T,N>
+ * (arithmetic: slang-ir-lower-coopvec.cpp:113-166; min/max/clamp/step hlsl.meta.slang:32043-32229;
+ * sin..fma :32231-32421) and the neural module's activations (activations.slang), over a batch:
+ *   out[s][i] = op(a[s][i], b[s][i], c[s][i])
+ * elementType is FLOAT16 or FLOAT32 (all operands and the result); FLOAT16 evaluates in fp32 and
+ * rounds once.  Operands an operator does not take are ignored (may be NULL).  `param` is the
+ * slope of CV_OP_LEAKY_RELU.  In-place use (out == a) is allowed. */
+typedef enum CvElementwiseOp {
+    CV_OP_ADD = 0, CV_OP_SUB = 1, CV_OP_MUL = 2, CV_OP_DIV = 3, CV_OP_NEG = 4,
+    CV_OP_MIN = 5, CV_OP_MAX = 6, CV_OP_CLAMP = 7 /* clamp(a, b, c) */, CV_OP_STEP = 8 /* step(edge = a, x = b) */,
+    CV_OP_SIN = 9, CV_OP_COS = 10, CV_OP_EXP = 11, CV_OP_LOG = 12, CV_OP_LOG2 = 13, CV_OP_EXP2 = 14,
+    CV_OP_TANH = 15, CV_OP_ATAN = 16, CV_OP_FMA = 17 /* a*b + c */,
+    CV_OP_RELU = 18, CV_OP_LEAKY_RELU = 19 /* a < 0 ? param*a : a */, CV_OP_SIGMOID = 20, CV_OP_SILU = 21,
+    CV_OP_QUICK_GELU = 22,
+    CV_OP_COUNT = 23
+} CvElementwiseOp;
+
+CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
+                              const void* a, size_t aStride, const void* b, size_t bStride,
+                              const void* c, size_t cStride, void* out, size_t outStride, float param);
+
+/* Reverse-mode derivative of the same operators, by Slang's rules (diff.meta.slang:1948-2470: the
+ * larger operand of max / smaller of min takes dOut and a tie splits it in halves, clamp passes
+ * dOut to x inside [min, max] including the bounds and to the bound it was clamped to otherwise):
+ *   dA[s][i] = d op / d a * dOut[s][i], likewise dB, dC (overwritten, not accumulated).
+ * Gradient outputs that are NULL, or that the operator has no operand for, are skipped. */
+CV_API CvResult cvElementwiseBackward(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
+                                      const void* a, size_t aStride, const void* b, size_t bStride,
+                                      const void* c, size_t cStride, const void* dOut, size_t dOutStride,
+                                      void* dA, size_t dAStride, void* dB, size_t dBStride,
+                                      void* dC, size_t dCStride, float param);
 
 /* ------------------------------------------------------------------------------------ */
 /* fused MLP: the example's FeedForwardLayer chain                                       */

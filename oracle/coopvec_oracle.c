@@ -904,3 +904,126 @@ void cvo_slang_adam_step(CvoAdamState* states, uint16_t* params, uint16_t* grads
 {
     cvo_slang_adam_step_nudged(states, params, grads, count, beta1f, beta2f, epsf, lrf, halfMode, 0, 0);
 }
+
+/* ===================================================================================== */
+/* element-wise surface (hlsl.meta.slang:32043-32421, slang-ir-lower-coopvec.cpp:113-166, */
+/* activations.slang) and its reverse-mode rules (diff.meta.slang:1948-2470)              */
+/* ===================================================================================== */
+
+static double ew_load(const void* p, int ct, size_t i)
+{
+    if (ct == CVO_FLOAT32) return (double)((const float*)p)[i];
+    return (double)cvo_f16_to_f32(((const uint16_t*)p)[i]);
+}
+
+static void ew_store(void* p, int ct, size_t i, double v)
+{
+    if (ct == CVO_FLOAT32) ((float*)p)[i] = (float)v;
+    else ((uint16_t*)p)[i] = cvo_f32_to_f16_rne((float)v);
+}
+
+static double ew_sigmoid(double x)
+{
+    /* activations.slang:101-108: the exp() argument is always <= 0 */
+    const double ex = exp(x >= 0 ? -x : x);
+    return x >= 0 ? 1.0 / (1.0 + ex) : ex / (1.0 + ex);
+}
+
+static int ew_operands(int op)
+{
+    switch (op) {
+    case CVO_OP_ADD: case CVO_OP_SUB: case CVO_OP_MUL: case CVO_OP_DIV: case CVO_OP_MIN: case CVO_OP_MAX: case CVO_OP_STEP: return 2;
+    case CVO_OP_CLAMP: case CVO_OP_FMA: return 3;
+    }
+    return 1;
+}
+
+static const double kLn2 = 0.69314718055994530941723212145818;
+
+int cvo_elementwise(int op, int ct, size_t count, const void* a, const void* b, const void* c, void* out, float param)
+{
+    if (op < 0 || op >= CVO_OP_COUNT || (ct != CVO_FLOAT16 && ct != CVO_FLOAT32)) return -1;
+    const int n = ew_operands(op);
+    for (size_t i = 0; i < count; ++i) {
+        const double x = ew_load(a, ct, i), y = n >= 2 ? ew_load(b, ct, i) : 0, z = n >= 3 ? ew_load(c, ct, i) : 0;
+        double r = x;
+        switch (op) {
+        case CVO_OP_ADD: r = x + y; break;
+        case CVO_OP_SUB: r = x - y; break;
+        case CVO_OP_MUL: r = x * y; break;
+        case CVO_OP_DIV: r = x / y; break;
+        case CVO_OP_NEG: r = -x; break;
+        case CVO_OP_MIN: r = x < y ? x : y; break;                      /* hlsl.meta.slang:32046-32067 */
+        case CVO_OP_MAX: r = x > y ? x : y; break;
+        case CVO_OP_CLAMP: r = fmin(fmax(x, y), z); break;              /* :32094-32111 */
+        case CVO_OP_STEP: r = y >= x ? 1.0 : 0.0; break;                /* step(edge, x), :32210-32229 */
+        case CVO_OP_SIN: r = sin(x); break;
+        case CVO_OP_COS: r = cos(x); break;
+        case CVO_OP_EXP: r = exp(x); break;
+        case CVO_OP_LOG: r = log(x); break;
+        case CVO_OP_LOG2: r = log2(x); break;
+        case CVO_OP_EXP2: r = exp2(x); break;
+        case CVO_OP_TANH: r = tanh(x); break;
+        case CVO_OP_ATAN: r = atan(x); break;
+        case CVO_OP_FMA: r = x * y + z; break;
+        case CVO_OP_RELU: r = x > 0 ? x : 0; break;                     /* activations.slang:25-42 */
+        case CVO_OP_LEAKY_RELU: r = x < 0 ? (double)param * x : x; break; /* :69-74 */
+        case CVO_OP_SIGMOID: r = ew_sigmoid(x); break;
+        case CVO_OP_SILU: r = x * ew_sigmoid(x); break;                 /* :186-193 */
+        case CVO_OP_QUICK_GELU: r = x * ew_sigmoid(1.702 * x); break;   /* :215-223 */
+        }
+        ew_store(out, ct, i, r);
+    }
+    return 0;
+}
+
+int cvo_elementwise_backward(int op, int ct, size_t count, const void* a, const void* b, const void* c,
+                             const void* dOut, void* dA, void* dB, void* dC, float param)
+{
+    if (op < 0 || op >= CVO_OP_COUNT || (ct != CVO_FLOAT16 && ct != CVO_FLOAT32)) return -1;
+    const int n = ew_operands(op);
+    for (size_t i = 0; i < count; ++i) {
+        const double x = ew_load(a, ct, i), y = n >= 2 ? ew_load(b, ct, i) : 0, z = n >= 3 ? ew_load(c, ct, i) : 0;
+        const double g = ew_load(dOut, ct, i);
+        double dx = 0, dy = 0, dz = 0;
+        switch (op) {
+        case CVO_OP_ADD: dx = g; dy = g; break;
+        case CVO_OP_SUB: dx = g; dy = -g; break;
+        case CVO_OP_MUL: dx = y * g; dy = x * g; break;
+        case CVO_OP_DIV: dx = g / y; dy = -x * g / (y * y); break;
+        case CVO_OP_NEG: dx = -g; break;
+        case CVO_OP_MIN:                                                 /* diff.meta.slang:2293-2300 */
+            dx = x < y ? g : (x > y ? 0 : 0.5 * g);
+            dy = y < x ? g : (y > x ? 0 : 0.5 * g);
+            break;
+        case CVO_OP_MAX:                                                 /* :2266-2273 */
+            dx = x > y ? g : (x < y ? 0 : 0.5 * g);
+            dy = y > x ? g : (y < x ? 0 : 0.5 * g);
+            break;
+        case CVO_OP_CLAMP:                                               /* :2413-2421 */
+            dx = (x >= y && x <= z) ? g : 0;
+            dy = x < y ? g : 0;
+            dz = x > z ? g : 0;
+            break;
+        case CVO_OP_STEP: break;
+        case CVO_OP_SIN: dx = cos(x) * g; break;                        /* :2104-2105 */
+        case CVO_OP_COS: dx = -(sin(x) * g); break;                     /* :2108-2112 */
+        case CVO_OP_EXP: dx = exp(x) * g; break;
+        case CVO_OP_LOG: dx = g / x; break;
+        case CVO_OP_LOG2: dx = g / (x * kLn2); break;                   /* :2134-2139 */
+        case CVO_OP_EXP2: dx = exp2(x) * kLn2 * g; break;
+        case CVO_OP_TANH: { const double t = tanh(x); dx = g - t * t * g; break; }   /* :2117-2124 */
+        case CVO_OP_ATAN: dx = g / (x * x + 1.0); break;                /* :2152-2156 */
+        case CVO_OP_FMA: dx = y * g; dy = x * g; dz = g; break;         /* :2441-2446 */
+        case CVO_OP_RELU: dx = x > 0 ? g : (x < 0 ? 0 : 0.5 * g); break;
+        case CVO_OP_LEAKY_RELU: dx = x < 0 ? (double)param * g : g; break;
+        case CVO_OP_SIGMOID: { const double sg = ew_sigmoid(x); dx = sg * (1 - sg) * g; break; }
+        case CVO_OP_SILU: { const double sg = ew_sigmoid(x); dx = (sg + x * sg * (1 - sg)) * g; break; }
+        case CVO_OP_QUICK_GELU: { const double sg = ew_sigmoid(1.702 * x); dx = (sg + 1.702 * x * sg * (1 - sg)) * g; break; }
+        }
+        if (dA) ew_store(dA, ct, i, dx);
+        if (dB && n >= 2) ew_store(dB, ct, i, dy);
+        if (dC && n >= 3) ew_store(dC, ct, i, dz);
+    }
+    return 0;
+}

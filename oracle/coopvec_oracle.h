@@ -177,6 +177,24 @@ void cvo_slang_adam_step_nudged(CvoAdamState* states, uint16_t* params, uint16_t
                                 float beta1, float beta2, float epsilon, float learningRate, int halfMode,
                                 int powNudge1, int powNudge2);
 
+/* ---- element-wise surface ------------------------------------------------------------- */
+/* Operator numbers of the C-ABI's CvElementwiseOp. */
+enum {
+    CVO_OP_ADD = 0, CVO_OP_SUB, CVO_OP_MUL, CVO_OP_DIV, CVO_OP_NEG, CVO_OP_MIN, CVO_OP_MAX, CVO_OP_CLAMP, CVO_OP_STEP,
+    CVO_OP_SIN, CVO_OP_COS, CVO_OP_EXP, CVO_OP_LOG, CVO_OP_LOG2, CVO_OP_EXP2, CVO_OP_TANH, CVO_OP_ATAN, CVO_OP_FMA,
+    CVO_OP_RELU, CVO_OP_LEAKY_RELU, CVO_OP_SIGMOID, CVO_OP_SILU, CVO_OP_QUICK_GELU, CVO_OP_COUNT
+};
+/* out[i] = op(a[i], b[i], c[i]) over `count` elements of type ct (FLOAT16 or FLOAT32), evaluated in
+ * double and rounded once: the per-component functions of CoopVec<T,N> (hlsl.meta.slang:32043-32421)
+ * and the neural module's activations (activations.slang).  Pinned by the primal CHECK values of
+ * tests/autodiff/coopvec.slang (tests/test_oracle_elementwise.py). */
+int cvo_elementwise(int op, int ct, size_t count, const void* a, const void* b, const void* c, void* out, float param);
+/* dA/dB/dC[i] = d op / d operand * dOut[i], by the rules of diff.meta.slang:1948-2470 (ties of min/max
+ * split dOut in halves; clamp passes dOut to x on the closed interval).  Pinned by the gradient CHECK
+ * values of tests/autodiff/coopvec.slang and by central differences. */
+int cvo_elementwise_backward(int op, int ct, size_t count, const void* a, const void* b, const void* c,
+                             const void* dOut, void* dA, void* dB, void* dC, float param);
+
 #ifdef __cplusplus
 }
 #endif

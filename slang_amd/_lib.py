@@ -105,6 +105,14 @@ SIGNATURES = {
     "cvReduceSumAccumulate": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32,
                                                ctypes.c_int32, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t,
                                                ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t]),
+    "cvElementwise": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint32,
+                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float]),
+    "cvElementwiseBackward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_uint32,
+                                               ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                                               ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                                               ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
+                                               ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float]),
     "cvMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
     "cvMlpTrainStepWorkspaceSize": (ctypes.c_int32, [ctypes.POINTER(CvMlpDesc), ctypes.c_uint32,

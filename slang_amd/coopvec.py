@@ -90,9 +90,45 @@ FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.
 
 
 class Activation(enum.IntEnum):
+    """CvActivation: NoActivation..LeakyReLU as the example spells them (fflayer.slang:60-66), the rest
+    the neural module's (source/standard-modules/neural/activations.slang)."""
     NoActivation = 0
     ReLU = 1
     LeakyReLU = 2
+    Sigmoid = 3
+    Tanh = 4
+    Exp = 5
+    Sine = 6
+    SiLU = 7
+    QuickGELU = 8
+
+
+class ElementwiseOp(enum.IntEnum):
+    """CvElementwiseOp: the per-component operators and functions of CoopVec<T,N>
+    (hlsl.meta.slang:32043-32421, slang-ir-lower-coopvec.cpp:113-166) and the neural activations."""
+    Add = 0
+    Sub = 1
+    Mul = 2
+    Div = 3
+    Neg = 4
+    Min = 5
+    Max = 6
+    Clamp = 7
+    Step = 8
+    Sin = 9
+    Cos = 10
+    Exp = 11
+    Log = 12
+    Log2 = 13
+    Exp2 = 14
+    Tanh = 15
+    Atan = 16
+    Fma = 17
+    ReLU = 18
+    LeakyReLU = 19
+    Sigmoid = 20
+    SiLU = 21
+    QuickGELU = 22
 
 
 # SlangResult values (include/slang.h:1400-1464)
@@ -337,6 +373,48 @@ def coopVecMatMulAdd(input: torch.Tensor, inputInterpretation: int, matrix: torc
                                   transpose, matrixStride, M=M, resultType=resultType, out=out,
                                   accumulate=accumulate, activation=activation, leakySlope=leakySlope,
                                   stream=stream, flags=flags)
+
+
+# ---------------------------------------------------------------------------------------------
+# element-wise surface
+# ---------------------------------------------------------------------------------------------
+
+def _ew_operand(t: Optional[torch.Tensor], like: torch.Tensor, what: str):
+    if t is None:
+        return None, 0
+    if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.shape != like.shape or t.dtype != like.dtype:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "%s must be a GPU tensor [batch, N] of the same shape and dtype" % what)
+    return t.data_ptr(), t.stride(0) * t.element_size()
+
+
+def elementwise(op: int, a: torch.Tensor, b: Optional[torch.Tensor] = None, c: Optional[torch.Tensor] = None, *,
+                param: float = 0.0, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """op(a, b, c) per component of every CoopVec of the batch (fp16 or fp32 tensors [batch, N]):
+    e.g. elementwise(ElementwiseOp.Clamp, x, lo, hi) is Slang's clamp(x, lo, hi)."""
+    ct = _TORCH_TO_CT.get(a.dtype)
+    if out is None:
+        out = torch.empty_like(a, memory_format=torch.contiguous_format)
+    pa, sa = _ew_operand(a, a, "a"); pb, sb = _ew_operand(b, a, "b"); pc, sc = _ew_operand(c, a, "c")
+    po, so = _ew_operand(out, a, "out")
+    _check(_lib.load().cvElementwise(_stream_handle(stream), int(op), int(ct) if ct is not None else -1, a.shape[1],
+                                     a.shape[0], pa, sa, pb, sb, pc, sc, po, so, float(param)))
+    return out
+
+
+def elementwiseBackward(op: int, dOut: torch.Tensor, a: torch.Tensor, b: Optional[torch.Tensor] = None,
+                        c: Optional[torch.Tensor] = None, *, param: float = 0.0, stream=None):
+    """Reverse-mode derivative of elementwise(op, a, b, c) by Slang's rules (diff.meta.slang:1948-2470):
+    returns (dA, dB, dC), None for operands the operator does not take."""
+    ct = _TORCH_TO_CT.get(a.dtype)
+    grads = [torch.empty_like(a, memory_format=torch.contiguous_format) if t is not None else None for t in (a, b, c)]
+    pa, sa = _ew_operand(a, a, "a"); pb, sb = _ew_operand(b, a, "b"); pc, sc = _ew_operand(c, a, "c")
+    pg, sg = _ew_operand(dOut, a, "dOut")
+    ptrs = [_ew_operand(g, a, "grad") for g in grads]
+    _check(_lib.load().cvElementwiseBackward(_stream_handle(stream), int(op), int(ct) if ct is not None else -1,
+                                             a.shape[1], a.shape[0], pa, sa, pb, sb, pc, sc, pg, sg,
+                                             ptrs[0][0], ptrs[0][1], ptrs[1][0], ptrs[1][1], ptrs[2][0], ptrs[2][1],
+                                             float(param)))
+    return tuple(grads)
 
 
 # ---------------------------------------------------------------------------------------------

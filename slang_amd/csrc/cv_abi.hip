@@ -283,7 +283,7 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
         return fail(CV_E_INVALID_ARG, "cvMatMul: transpose must be false for RowMajor/ColumnMajor");
     if (d->accumulate && d->activation != CV_ACT_NONE)
         return fail(CV_E_INVALID_ARG, "cvMatMul: accumulate forms take no activation");
-    if (d->activation < CV_ACT_NONE || d->activation > CV_ACT_LEAKY_RELU)
+    if (d->activation < CV_ACT_NONE || d->activation > CV_ACT_QUICK_GELU)
         return fail(CV_E_INVALID_ARG, "cvMatMul: unknown activation %d", d->activation);
     const uint32_t packing = (uint32_t)cvComponentPackingFactor(d->inputInterpretation);
     if (packing != 1 && d->k % 4 != 0)   // fallback rule k == 4*PackedK (hlsl.meta.slang:32846)
@@ -465,7 +465,7 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
             return fail(CV_E_INVALID_ARG, "%s: layer %d takes %d inputs but layer %d produces %d", who, l, L.inputSize, l - 1, mlp->layers[l - 1].outputSize);
         if (L.weightLayout < 0 || L.weightLayout > 3 || !cv::layoutSupports(mlp->weightType, L.weightLayout))
             return fail(CV_E_NOT_AVAILABLE, "%s: layer %d: component type %d has no layout %d", who, l, mlp->weightType, L.weightLayout);
-        if (L.activation < CV_ACT_NONE || L.activation > CV_ACT_LEAKY_RELU)
+        if (L.activation < CV_ACT_NONE || L.activation > CV_ACT_QUICK_GELU)
             return fail(CV_E_INVALID_ARG, "%s: layer %d: unknown activation %d", who, l, L.activation);
         cv::MlpLayerArgs& o = out[l];
         o.w = (const uint8_t*)L.weights;
@@ -568,6 +568,8 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     const uint32_t gEsz = cv::elemSize(mlp->gradType);
     for (int l = 0; l < L; ++l) {
         const CvMlpLayer& ly = mlp->layers[l];
+        if (ly.activation > CV_ACT_LEAKY_RELU)
+            return fail(CV_E_NOT_AVAILABLE, "%s: layer %d: the fused training step differentiates NONE, RELU and LEAKY_RELU only", who, l);
         // with 0 <= slope <= 0.5 the outcome of max(z, z*slope) is the sign of z for every fp16 z
         if (ly.activation == CV_ACT_LEAKY_RELU && !(ly.leakySlope >= 0.f && ly.leakySlope <= 0.5f))
             return fail(CV_E_INVALID_ARG, "%s: layer %d: leakySlope must be in [0, 0.5]", who, l);

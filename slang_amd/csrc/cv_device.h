@@ -25,7 +25,8 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-enum : int { kActNone = 0, kActRelu = 1, kActLeakyRelu = 2 };
+enum : int { kActNone = 0, kActRelu = 1, kActLeakyRelu = 2, kActSigmoid = 3, kActTanh = 4, kActExp = 5,
+             kActSine = 6, kActSilu = 7, kActQuickGelu = 8, kActCount = 9 };
 
 // ---- MFMA flavours ---------------------------------------------------------------------
 // Each flavour describes how elements lie in memory (kEsz bytes each; kEpl k-slots per lane
@@ -149,6 +150,28 @@ __device__ __forceinline__ uint32_t packE4M3Sat(float a, float b)
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
 }
 
+// The neural module's smooth activations (source/standard-modules/neural/activations.slang:88-233)
+// in fp32.  Sigmoid-like ones keep the source's branch that makes the exp() argument <= 0.
+__device__ __forceinline__ float smoothActivation(float x, int act)
+{
+    switch (act) {
+    case kActTanh: return tanhf(x);
+    case kActExp: return expf(x);
+    case kActSine: return sinf(x);
+    case kActSigmoid: {
+        const float ex = expf(x >= 0.f ? -x : x);
+        return x >= 0.f ? 1.f / (1.f + ex) : ex / (1.f + ex); }
+    case kActSilu: {
+        const float ex = expf(x >= 0.f ? -x : x);
+        return x >= 0.f ? x / (1.f + ex) : x * ex / (1.f + ex); }
+    case kActQuickGelu: {
+        const float sx = 1.702f * x;
+        const float ex = expf(sx >= 0.f ? -sx : sx);
+        return sx >= 0.f ? x / (1.f + ex) : x * ex / (1.f + ex); }
+    }
+    return x;
+}
+
 // activation on a value already rounded to fp16 (the carrier type is CoopVec<half>)
 __device__ __forceinline__ half_t activateHalf(half_t z, int act, float slope)
 {
@@ -157,6 +180,7 @@ __device__ __forceinline__ half_t activateHalf(half_t z, int act, float slope)
         const half_t zs = (half_t)((float)z * slope);   // exact product, one rounding
         return z >= zs ? z : zs;
     }
+    if (act >= kActSigmoid) return (half_t)smoothActivation((float)z, act);
     return z;
 }
 

@@ -1,0 +1,274 @@
+// cv_elementwise.hip -- the per-component surface of CoopVec<T,N> over a batch, forward and reverse.
+//
+// Replaces, for a whole dispatch of shader threads at once, the element-wise operators and math
+// functions Slang declares on CoopVec<T,N> -- arithmetic expanded per element by
+// source/slang/slang-ir-lower-coopvec.cpp:113-166; min/max/clamp/step
+// source/slang/hlsl.meta.slang:32043-32229; sin, cos, exp, log, log2, exp2, tanh, atan, fma
+// :32231-32421 -- the activations of the neural module
+// (source/standard-modules/neural/activations.slang), and their reverse-mode derivative rules
+// (source/slang/diff.meta.slang:1948-2470).  Pure streaming: HBM-bound.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "cv_device.h"
+#include "cv_error.h"
+
+namespace cv {
+namespace {
+
+struct EwArgs {
+    const uint8_t* a; const uint8_t* b; const uint8_t* c; const uint8_t* dOut;
+    uint8_t* out; uint8_t* dA; uint8_t* dB; uint8_t* dC;
+    uint64_t aStride, bStride, cStride, dOutStride, outStride, dAStride, dBStride, dCStride;
+    int32_t op, n;
+    uint32_t batch;
+    float param;
+};
+
+enum : int {
+    kOpAdd = 0, kOpSub, kOpMul, kOpDiv, kOpNeg, kOpMin, kOpMax, kOpClamp, kOpStep, kOpSin, kOpCos, kOpExp, kOpLog,
+    kOpLog2, kOpExp2, kOpTanh, kOpAtan, kOpFma, kOpRelu, kOpLeakyRelu, kOpSigmoid, kOpSilu, kOpQuickGelu, kOpCount
+};
+
+__host__ __device__ inline int operandCount(int op)
+{
+    switch (op) {
+    case kOpAdd: case kOpSub: case kOpMul: case kOpDiv: case kOpMin: case kOpMax: case kOpStep: return 2;
+    case kOpClamp: case kOpFma: return 3;
+    }
+    return 1;
+}
+
+__device__ __forceinline__ float evalOp(int op, float a, float b, float c, float param)
+{
+    switch (op) {
+    case kOpAdd: return a + b;
+    case kOpSub: return a - b;
+    case kOpMul: return a * b;
+    case kOpDiv: return a / b;
+    case kOpNeg: return -a;
+    case kOpMin: return fminf(a, b);
+    case kOpMax: return fmaxf(a, b);
+    case kOpClamp: return fminf(fmaxf(a, b), c);
+    case kOpStep: return b >= a ? 1.f : 0.f;            // step(edge, x) = x >= edge
+    case kOpSin: return sinf(a);
+    case kOpCos: return cosf(a);
+    case kOpExp: return expf(a);
+    case kOpLog: return logf(a);
+    case kOpLog2: return log2f(a);
+    case kOpExp2: return exp2f(a);
+    case kOpTanh: return tanhf(a);
+    case kOpAtan: return atanf(a);
+    case kOpFma: return __builtin_fmaf(a, b, c);
+    case kOpRelu: return fmaxf(a, 0.f);
+    case kOpLeakyRelu: return a < 0.f ? param * a : a;  // activations.slang:69-74
+    case kOpSigmoid: return smoothActivation(a, kActSigmoid);
+    case kOpSilu: return smoothActivation(a, kActSilu);
+    case kOpQuickGelu: return smoothActivation(a, kActQuickGelu);
+    }
+    return a;
+}
+
+// d(sigmoid(k x) * x)/dx for k = 1 (SiLU) or 1.702 (QuickGELU): s + k x s (1 - s)
+__device__ __forceinline__ float gatedSigmoidGrad(float x, float k)
+{
+    const float s = smoothActivation(k * x, kActSigmoid);
+    return s + k * x * s * (1.f - s);
+}
+
+// partial derivatives times dOut, by the rules of diff.meta.slang
+__device__ __forceinline__ void gradOp(int op, float a, float b, float c, float g, float param, float& da, float& db, float& dc)
+{
+    da = db = dc = 0.f;
+    switch (op) {
+    case kOpAdd: da = g; db = g; break;
+    case kOpSub: da = g; db = -g; break;
+    case kOpMul: da = b * g; db = a * g; break;
+    case kOpDiv: da = g / b; db = -a * g / (b * b); break;
+    case kOpNeg: da = -g; break;
+    case kOpMin:    // :2293-2300: the smaller operand takes dOut, a tie splits it
+        da = a < b ? g : (a > b ? 0.f : 0.5f * g);
+        db = b < a ? g : (b > a ? 0.f : 0.5f * g);
+        break;
+    case kOpMax:    // :2266-2273
+        da = a > b ? g : (a < b ? 0.f : 0.5f * g);
+        db = b > a ? g : (b < a ? 0.f : 0.5f * g);
+        break;
+    case kOpClamp:  // :2413-2421: x inside [min, max] (bounds included) keeps dOut, otherwise the bound it hit
+        da = (a >= b && a <= c) ? g : 0.f;
+        db = a < b ? g : 0.f;
+        dc = a > c ? g : 0.f;
+        break;
+    case kOpStep: break;
+    case kOpSin: da = cosf(a) * g; break;
+    case kOpCos: da = -(sinf(a) * g); break;
+    case kOpExp: da = expf(a) * g; break;
+    case kOpLog: da = g / a; break;
+    case kOpLog2: da = g / (a * 0.69314718055994530941723212145818f); break;
+    case kOpExp2: da = exp2f(a) * 0.69314718055994530941723212145818f * g; break;
+    case kOpTanh: { const float t = tanhf(a); da = g - t * t * g; break; }     // :2116-2124
+    case kOpAtan: da = g / (a * a + 1.f); break;
+    case kOpFma: da = b * g; db = a * g; dc = g; break;
+    case kOpRelu: da = a > 0.f ? g : (a < 0.f ? 0.f : 0.5f * g); break;       // max(x, 0) by the max rule
+    case kOpLeakyRelu: da = a < 0.f ? param * g : g; break;
+    case kOpSigmoid: { const float s = smoothActivation(a, kActSigmoid); da = s * (1.f - s) * g; break; }
+    case kOpSilu: da = gatedSigmoidGrad(a, 1.f) * g; break;
+    case kOpQuickGelu: da = gatedSigmoidGrad(a, 1.702f) * g; break;
+    }
+}
+
+template <typename T> __device__ __forceinline__ float ld(const uint8_t* p) { return (float)*(const T*)p; }
+template <typename T> __device__ __forceinline__ void st(uint8_t* p, float v) { *(T*)p = (T)v; }
+
+// one thread per element; rows are contiguous, so consecutive lanes touch consecutive addresses
+template <typename T, bool BACKWARD>
+__global__ __launch_bounds__(256) void elementwiseKernel(const EwArgs e)
+{
+    const uint64_t total = (uint64_t)e.batch * (uint32_t)e.n;
+    const int nOps = operandCount(e.op);
+    for (uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256u) {
+        const uint64_t s = idx / (uint32_t)e.n;
+        const uint64_t off = (idx - s * (uint32_t)e.n) * sizeof(T);
+        const float a = ld<T>(e.a + s * e.aStride + off);
+        const float b = nOps >= 2 ? ld<T>(e.b + s * e.bStride + off) : 0.f;
+        const float c = nOps >= 3 ? ld<T>(e.c + s * e.cStride + off) : 0.f;
+        if constexpr (!BACKWARD) {
+            st<T>(e.out + s * e.outStride + off, evalOp(e.op, a, b, c, e.param));
+        } else {
+            const float g = ld<T>(e.dOut + s * e.dOutStride + off);
+            float da, db, dc;
+            gradOp(e.op, a, b, c, g, e.param, da, db, dc);
+            if (e.dA) st<T>(e.dA + s * e.dAStride + off, da);
+            if (e.dB && nOps >= 2) st<T>(e.dB + s * e.dBStride + off, db);
+            if (e.dC && nOps >= 3) st<T>(e.dC + s * e.dCStride + off, dc);
+        }
+    }
+}
+
+// dense rows (stride = n elements) of a unary / binary operator on 16-byte pieces: the whole batch is
+// one flat array
+template <typename T>
+__global__ __launch_bounds__(256) void elementwiseDenseKernel(const EwArgs e, uint64_t pieces)
+{
+    constexpr int PER = 16 / sizeof(T);
+    const int nOps = operandCount(e.op);
+    for (uint64_t p = (uint64_t)blockIdx.x * 256u + threadIdx.x; p < pieces; p += (uint64_t)gridDim.x * 256u) {
+        T va[PER], vb[PER], vc[PER], vo[PER];
+        *(u32x4*)va = *(const u32x4*)(e.a + p * 16u);
+        if (nOps >= 2) *(u32x4*)vb = *(const u32x4*)(e.b + p * 16u);
+        if (nOps >= 3) *(u32x4*)vc = *(const u32x4*)(e.c + p * 16u);
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            vo[i] = (T)evalOp(e.op, (float)va[i], nOps >= 2 ? (float)vb[i] : 0.f, nOps >= 3 ? (float)vc[i] : 0.f, e.param);
+        *(u32x4*)(e.out + p * 16u) = *(const u32x4*)vo;
+    }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+int currentCUs()
+{
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    return n;
+}
+
+CvResult checkCommon(const char* who, int32_t op, int32_t elementType, int32_t n, uint32_t esz)
+{
+    if (op < 0 || op >= kOpCount) return failWith(CV_E_INVALID_ARG, "%s: unknown operator %d", who, op);
+    if (elementType != CV_FLOAT16 && elementType != CV_FLOAT32)
+        return failWith(CV_E_NOT_AVAILABLE, "%s: elementType %d (supported: FLOAT16, FLOAT32)", who, elementType);
+    if (n <= 0) return failWith(CV_E_INVALID_ARG, "%s: n=%d", who, n);
+    (void)esz;
+    return CV_OK;
+}
+
+bool badOperand(const void* p, size_t stride, int32_t n, uint32_t batch, uint32_t esz)
+{
+    return !p || (uintptr_t)p % esz || stride % esz || (batch > 1 && stride < (size_t)n * esz);
+}
+
+} // namespace
+} // namespace cv
+
+extern "C" {
+
+CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
+                              const void* a, size_t aStride, const void* b, size_t bStride,
+                              const void* c, size_t cStride, void* out, size_t outStride, float param)
+{
+    using namespace cv;
+    const uint32_t esz = elementType == CV_FLOAT32 ? 4u : 2u;
+    CvResult rc = checkCommon("cvElementwise", op, elementType, n, esz);
+    if (CV_FAILED(rc)) return rc;
+    if (batch == 0) return CV_OK;
+    const int nOps = operandCount(op);
+    if (badOperand(a, aStride, n, batch, esz) || badOperand(out, outStride, n, batch, esz) ||
+        (nOps >= 2 && badOperand(b, bStride, n, batch, esz)) || (nOps >= 3 && badOperand(c, cStride, n, batch, esz)))
+        return failWith(CV_E_INVALID_ARG, "cvElementwise: null, misaligned or overlapping-row operand (operator %d takes %d)", op, nOps);
+    EwArgs e;
+    memset(&e, 0, sizeof(e));
+    e.a = (const uint8_t*)a; e.b = (const uint8_t*)b; e.c = (const uint8_t*)c; e.out = (uint8_t*)out;
+    e.aStride = aStride; e.bStride = bStride; e.cStride = cStride; e.outStride = outStride;
+    e.op = op; e.n = n; e.batch = batch; e.param = param;
+    const uint64_t total = (uint64_t)batch * (uint32_t)n;
+    const size_t row = (size_t)n * esz;
+    const bool dense = aStride == row && outStride == row && (nOps < 2 || bStride == row) && (nOps < 3 || cStride == row) &&
+                       aligned16(a) && aligned16(out) && (nOps < 2 || aligned16(b)) && (nOps < 3 || aligned16(c)) &&
+                       (total * esz) % 16 == 0;
+    const uint32_t cap = (uint32_t)currentCUs() * 8u;
+    if (dense) {
+        const uint64_t pieces = total * esz / 16u;
+        const uint32_t blocks = (uint32_t)((pieces + 255) / 256 < cap ? (pieces + 255) / 256 : cap);
+        noteKernel(false, "elementwiseDenseKernel<%s>", esz == 2 ? "f16" : "f32");
+        if (esz == 2) hipLaunchKernelGGL(elementwiseDenseKernel<half_t>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, e, pieces);
+        else          hipLaunchKernelGGL(elementwiseDenseKernel<float>, dim3(blocks), dim3(256), 0, (hipStream_t)stream, e, pieces);
+    } else {
+        const uint32_t blocks = (uint32_t)((total + 255) / 256 < cap ? (total + 255) / 256 : cap);
+        noteKernel(false, "elementwiseKernel<%s>", esz == 2 ? "f16" : "f32");
+        if (esz == 2) hipLaunchKernelGGL((elementwiseKernel<half_t, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, e);
+        else          hipLaunchKernelGGL((elementwiseKernel<float, false>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, e);
+    }
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvElementwise launch: %s", hipGetErrorString(err));
+    return CV_OK;
+}
+
+CV_API CvResult cvElementwiseBackward(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
+                                      const void* a, size_t aStride, const void* b, size_t bStride,
+                                      const void* c, size_t cStride, const void* dOut, size_t dOutStride,
+                                      void* dA, size_t dAStride, void* dB, size_t dBStride,
+                                      void* dC, size_t dCStride, float param)
+{
+    using namespace cv;
+    const uint32_t esz = elementType == CV_FLOAT32 ? 4u : 2u;
+    CvResult rc = checkCommon("cvElementwiseBackward", op, elementType, n, esz);
+    if (CV_FAILED(rc)) return rc;
+    if (batch == 0) return CV_OK;
+    const int nOps = operandCount(op);
+    if (badOperand(a, aStride, n, batch, esz) || badOperand(dOut, dOutStride, n, batch, esz) ||
+        (nOps >= 2 && badOperand(b, bStride, n, batch, esz)) || (nOps >= 3 && badOperand(c, cStride, n, batch, esz)) ||
+        (dA && badOperand(dA, dAStride, n, batch, esz)) || (dB && nOps >= 2 && badOperand(dB, dBStride, n, batch, esz)) ||
+        (dC && nOps >= 3 && badOperand(dC, dCStride, n, batch, esz)))
+        return failWith(CV_E_INVALID_ARG, "cvElementwiseBackward: null, misaligned or overlapping-row operand (operator %d takes %d)", op, nOps);
+    EwArgs e;
+    memset(&e, 0, sizeof(e));
+    e.a = (const uint8_t*)a; e.b = (const uint8_t*)b; e.c = (const uint8_t*)c; e.dOut = (const uint8_t*)dOut;
+    e.dA = (uint8_t*)dA; e.dB = (uint8_t*)dB; e.dC = (uint8_t*)dC;
+    e.aStride = aStride; e.bStride = bStride; e.cStride = cStride; e.dOutStride = dOutStride;
+    e.dAStride = dAStride; e.dBStride = dBStride; e.dCStride = dCStride;
+    e.op = op; e.n = n; e.batch = batch; e.param = param;
+    const uint64_t total = (uint64_t)batch * (uint32_t)n;
+    const uint32_t cap = (uint32_t)currentCUs() * 8u;
+    const uint32_t blocks = (uint32_t)((total + 255) / 256 < cap ? (total + 255) / 256 : cap);
+    noteKernel(false, "elementwiseKernel<%s,backward>", esz == 2 ? "f16" : "f32");
+    if (esz == 2) hipLaunchKernelGGL((elementwiseKernel<half_t, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, e);
+    else          hipLaunchKernelGGL((elementwiseKernel<float, true>), dim3(blocks), dim3(256), 0, (hipStream_t)stream, e);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvElementwiseBackward launch: %s", hipGetErrorString(err));
+    return CV_OK;
+}
+
+} // extern "C"

@@ -273,6 +273,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                             float x = acc[t][r];
                             if (a.act == kActRelu) x = x > 0.f ? x : 0.f;
                             else if (a.act == kActLeakyRelu) x = fmaxf(x, x * a.slope);
+                            else if (a.act >= kActSigmoid) x = smoothActivation(x, a.act);
                             pk[4 * t + r] = __builtin_bit_cast(uint32_t, x);
                         }
                     } else {
@@ -362,7 +363,7 @@ hipError_t launchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
     const bool fast = (uint32_t)a.k == 4u * Mma::kEpl * KT && a.m == 16 * MT &&
                       a.inAlign >= (slotBytes % 16 == 0 ? 16u : 8u) &&
                       a.outAlign >= ((4 * MT * sizeof(OutT)) % 16 == 0 ? 16u : 8u) &&
-                      !a.accumulate && a.act != kActLeakyRelu;
+                      !a.accumulate && a.act <= kActRelu;
     if (!fast) return launchOne<Mma, MT, KT, OutT, false>(stream, a, numCUs);
     // whole tiles on the streaming kernel, the ragged tail (< one tile) on the general one
     const uint32_t whole = a.batch / tile * tile;

@@ -126,8 +126,8 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
 #pragma unroll
                 for (int kt = 0; kt < kGenMaxKT; ++kt) {
                     halfx2 lo01 = {(half_t)0, (half_t)0}, lo23 = lo01, hi01 = lo01, hi23 = lo01;
-                    if (2 * kt < MT) carrierFromAcc(acc[2 * kt], cc, lo01, lo23);
-                    if (2 * kt + 1 < MT) carrierFromAcc(acc[2 * kt + 1], cc, hi01, hi23);
+                    if (2 * kt < MT) carrierFromAcc<true>(acc[2 * kt], cc, lo01, lo23);
+                    if (2 * kt + 1 < MT) carrierFromAcc<true>(acc[2 * kt + 1], cc, hi01, hi23);
                     fragFromCarrier<Mma>(lo01, lo23, hi01, hi23, cc, act[kt]);
                 }
             } else {
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
                 for (int t = 0; t < kGenMaxTiles; ++t) {
                     if (t < MT && sample < a.batch) {
                         halfx2 p0, p1;
-                        carrierFromAcc(acc[t], cc, p0, p1);
+                        carrierFromAcc<true>(acc[t], cc, p0, p1);
                         const half_t v[4] = {p0.x, p0.y, p1.x, p1.y};
 #pragma unroll
                         for (int r = 0; r < 4; ++r)

@@ -85,15 +85,18 @@ __device__ __forceinline__ CarrierCfg makeCarrierCfg(int act, float slope)
 
 // accumulators (one 16-row tile, 4 values per lane) -> the carrier CoopVec<half>: round to
 // fp16 (v_cvt_pk_f16_f32, nearest even), then the activation, on packed pairs
+// SMOOTH: the kernel also serves the neural module's smooth activations (only the general kernel
+// does; the specialised ones would carry the transcendental code in every instantiation)
+template <bool SMOOTH = false>
 __device__ __forceinline__ void carrierFromAcc(const floatx4& acc, const CarrierCfg& c, halfx2& h01, halfx2& h23)
 {
     typedef float floatx2 __attribute__((ext_vector_type(2)));
     const floatx2 a01 = {acc[0], acc[1]}, a23 = {acc[2], acc[3]};
     h01 = __builtin_convertvector(a01, halfx2);
     h23 = __builtin_convertvector(a23, halfx2);
-    if (c.act == kActLeakyRelu) {      // max(z, z*slope) in half, fflayer.slang:64-65
-        h01 = halfx2{activateHalf(h01.x, kActLeakyRelu, c.slope), activateHalf(h01.y, kActLeakyRelu, c.slope)};
-        h23 = halfx2{activateHalf(h23.x, kActLeakyRelu, c.slope), activateHalf(h23.y, kActLeakyRelu, c.slope)};
+    if (c.act == kActLeakyRelu || (SMOOTH && c.act >= kActSigmoid)) {   // leaky: max(z, z*slope) in half, fflayer.slang:64-65
+        h01 = halfx2{activateHalf(h01.x, c.act, c.slope), activateHalf(h01.y, c.act, c.slope)};
+        h23 = halfx2{activateHalf(h23.x, c.act, c.slope), activateHalf(h23.y, c.act, c.slope)};
     }
     h01 = __builtin_elementwise_max(h01, c.floor2);
     h23 = __builtin_elementwise_max(h23, c.floor2);
@@ -402,6 +405,8 @@ hipError_t dispatchMlp(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     const int L = a.numLayers;
     if (L < 2) return hipErrorInvalidValue;
+    for (int l = 0; l < L; ++l)
+        if (a.layers[l].act >= kActSigmoid) return hipErrorInvalidValue;     // smooth activations: general kernel
     const int kt0 = (int)optKT((uint32_t)a.layers[0].in, Mma::kEpl);
     const int ht = (int)optMT((uint32_t)a.layers[0].out);
     for (int l = 1; l + 1 < L; ++l)

@@ -226,6 +226,45 @@ def f16_midpoint_distance(z: np.ndarray) -> np.ndarray:
     return np.abs(r - np.floor(r) - 0.5) * ulp
 
 
+# ---- element-wise surface ------------------------------------------------------------------
+
+def _ew_ct(a: np.ndarray) -> int:
+    if a.dtype == np.float32:
+        return F32
+    if a.dtype == np.float16:
+        return F16
+    raise TypeError(a.dtype)
+
+
+def elementwise(op: int, a, b=None, c=None, param: float = 0.0) -> np.ndarray:
+    L = lib()
+    L.cvo_elementwise.argtypes = [_c.c_int, _c.c_int, _sz, _vp, _vp, _vp, _vp, _f32]
+    L.cvo_elementwise.restype = _c.c_int
+    a = np.ascontiguousarray(a)
+    out = np.empty_like(a)
+    ops = [np.ascontiguousarray(x, dtype=a.dtype) if x is not None else None for x in (b, c)]
+    rc = L.cvo_elementwise(int(op), _ew_ct(a), a.size, ptr(a), ptr(ops[0]) if ops[0] is not None else None,
+                           ptr(ops[1]) if ops[1] is not None else None, ptr(out), float(param))
+    assert rc == 0
+    return out
+
+
+def elementwise_backward(op: int, d_out, a, b=None, c=None, param: float = 0.0):
+    L = lib()
+    L.cvo_elementwise_backward.argtypes = [_c.c_int, _c.c_int, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _f32]
+    L.cvo_elementwise_backward.restype = _c.c_int
+    a = np.ascontiguousarray(a)
+    g = np.ascontiguousarray(d_out, dtype=a.dtype)
+    ops = [np.ascontiguousarray(x, dtype=a.dtype) if x is not None else None for x in (b, c)]
+    grads = [np.zeros_like(a), np.zeros_like(a) if ops[0] is not None else None, np.zeros_like(a) if ops[1] is not None else None]
+    rc = L.cvo_elementwise_backward(int(op), _ew_ct(a), a.size, ptr(a), ptr(ops[0]) if ops[0] is not None else None,
+                                    ptr(ops[1]) if ops[1] is not None else None, ptr(g), ptr(grads[0]),
+                                    ptr(grads[1]) if grads[1] is not None else None,
+                                    ptr(grads[2]) if grads[2] is not None else None, float(param))
+    assert rc == 0
+    return tuple(grads)
+
+
 # ---- Adam ---------------------------------------------------------------------------------
 ADAM_STATE_DTYPE = np.dtype([("mean", np.uint16), ("variance", np.uint16), ("iteration", np.int32)])
 
