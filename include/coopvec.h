@@ -298,6 +298,15 @@ typedef struct CvMlpLayer {
     float       leakySlope;
 } CvMlpLayer;
 
+/* Encoding applied to a sample in front of layer 0.
+ * CV_ENCODE_XY_SQUARES is the example's MyNetwork::encodeInput (network.slang:35-38): a sample is a
+ * float2 (x, y) in memory (`uniform float2* inputs`, kernels.slang:12); it is converted to half2
+ * (kernels.slang:19) and layer 0 sees the CoopVec<half,4> (x, y, x*x, y*y), the squares rounded to half.
+ * Needs inputType FLOAT32, FLOAT16 weights and a first layer of 4 inputs.  With this encoding and
+ * targets == NULL, cvMlpTrainStep differentiates the example's own loss (network.slang:58-75): the
+ * squared distance of the 4 outputs from groundtruth(x, y), evaluated in half. */
+typedef enum CvInputEncoding { CV_ENCODE_NONE = 0, CV_ENCODE_XY_SQUARES = 1 } CvInputEncoding;
+
 typedef struct CvMlpDesc {
     const CvMlpLayer* layers;   /* host array */
     int32_t  numLayers;
@@ -307,6 +316,7 @@ typedef struct CvMlpDesc {
     int32_t  outputType;        /* FLOAT16 */
     int32_t  gradType;          /* FLOAT16 or FLOAT32: element type of weightsGrad/biasesGrad */
     uint32_t flags;             /* CV_FLAG_* */
+    int32_t  inputEncoding;     /* CvInputEncoding */
 } CvMlpDesc;
 
 /* y = layer_{n-1}( ... layer_0(x) ): every layer is coopVecMatMulAdd + activation with
@@ -320,7 +330,8 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp,
 /* Forward + reverse pass of loss_s = sum_i (y[s][i] - target[s][i])^2 with seed `lossScale`
  * (the example: bwd_diff(loss)(network, x, y, 1.0h), kernels.slang:20): accumulates
  * sum_s dY (x) X into every layer's weightsGrad and sum_s dY into biasesGrad ("+=").
- * targets == NULL selects target = sin(sum of the sample's inputs) for every output.
+ * targets == NULL selects target = sin(sum of the sample's inputs) for every output (with
+ * inputEncoding CV_ENCODE_XY_SQUARES: the example's groundtruth(x, y)).
  * lossSum (device, optional, one float) is overwritten with sum_s loss_s. */
 CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes);
 CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp,

@@ -75,7 +75,7 @@ class CvMlpDesc(ctypes.Structure):
     _fields_ = [("layers", ctypes.POINTER(CvMlpLayer)), ("numLayers", ctypes.c_int32),
                 ("inputType", ctypes.c_int32), ("weightType", ctypes.c_int32),
                 ("biasType", ctypes.c_int32), ("outputType", ctypes.c_int32),
-                ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32)]
+                ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32), ("inputEncoding", ctypes.c_int32)]
 
 
 # name -> (restype, argtypes); every function include/coopvec.h declares

@@ -439,7 +439,15 @@ class FeedForwardLayer:
     gradStride: int = 0
 
 
-def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int, flags: int):
+class InputEncoding(enum.IntEnum):
+    """CvInputEncoding: XYSquares is the example's MyNetwork::encodeInput (network.slang:35-38) on
+    float2 samples: layer 0 sees (x, y, x*x, y*y) in half."""
+    NoEncoding = 0
+    XYSquares = 1
+
+
+def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int, flags: int,
+              inputEncoding: int = 0):
     arr = (_lib.CvMlpLayer * len(layers))()
     for i, L in enumerate(layers):
         arr[i].weights = _buffer_ptr(L.weights, "weights")
@@ -454,13 +462,15 @@ def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int
     d.layers = arr; d.numLayers = len(layers)
     d.inputType = int(weightType); d.weightType = int(weightType)
     d.biasType = int(CoopVecComponentType.Float16); d.outputType = int(CoopVecComponentType.Float16)
-    d.gradType = int(gradType); d.flags = int(flags)
+    d.gradType = int(gradType); d.flags = int(flags); d.inputEncoding = int(inputEncoding)
+    if inputEncoding:
+        d.inputType = int(CoopVecComponentType.Float32)
     return d, arr
 
 
 def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
                weightType: int = CoopVecComponentType.Float16, out: Optional[torch.Tensor] = None,
-               flags: int = 0, stream=None) -> torch.Tensor:
+               flags: int = 0, inputEncoding: int = 0, stream=None) -> torch.Tensor:
     """network.eval over a batch: every layer is coopVecMatMulAdd + activation with CoopVec<half>
     between layers (network.slang:41-47), fused into one kernel."""
     inCt, inStride = _vector_info(input, weightType, "input")
@@ -468,7 +478,7 @@ def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
     if out is None:
         out = torch.empty((batch, layers[-1].outputSize), dtype=torch.float16, device=input.device)
     _, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
-    d, keep = _mlp_desc(layers, weightType, CoopVecComponentType.Float32, flags)
+    d, keep = _mlp_desc(layers, weightType, CoopVecComponentType.Float32, flags, inputEncoding)
     d.inputType = int(inCt)
     _check(_lib.load().cvMlpForward(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride,
                                     out.data_ptr(), outStride, batch))
@@ -485,14 +495,15 @@ def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
 
 def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor] = None, *,
                  lossScale: float = 1.0, gradType: int = CoopVecComponentType.Float32,
-                 workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None, stream=None):
+                 workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None,
+                 inputEncoding: int = 0, stream=None):
     """learnGradient over a batch (kernels.slang:9-27): forward, bwd_diff of the squared-error loss,
     weight gradients accumulated into every layer's weightsGrad (coopVecOuterProductAccumulate,
     fflayer.slang:35-41) and bias gradients into biasesGrad (coopVecReduceSumAccumulate, :44),
     deterministically.  Returns (workspace, lossSum) so that both can be reused."""
     _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
     batch = input.shape[0]
-    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0, inputEncoding)
     lib = _lib.load()
     if workspace is None:
         need = ctypes.c_size_t(0)

@@ -454,8 +454,15 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
         return fail(CV_E_NOT_AVAILABLE, "%s: weightType %d (supported: FLOAT16, FLOAT_E4M3)", who, mlp->weightType);
     if (mlp->biasType != CV_FLOAT16 || mlp->outputType != CV_FLOAT16)
         return fail(CV_E_NOT_AVAILABLE, "%s: biasType/outputType must be FLOAT16", who);
-    if (mlp->inputType != mlp->weightType)
+    if (mlp->inputEncoding == CV_ENCODE_XY_SQUARES) {
+        if (mlp->inputType != CV_FLOAT32 || mlp->weightType != CV_FLOAT16 || mlp->layers[0].inputSize != 4 || mlp->numLayers < 2)
+            return fail(CV_E_NOT_AVAILABLE, "%s: CV_ENCODE_XY_SQUARES needs FLOAT32 (x, y) samples, FLOAT16 weights, a first "
+                        "layer of 4 inputs and at least two layers", who);
+    } else if (mlp->inputEncoding != CV_ENCODE_NONE) {
+        return fail(CV_E_INVALID_ARG, "%s: unknown inputEncoding %d", who, mlp->inputEncoding);
+    } else if (mlp->inputType != mlp->weightType) {
         return fail(CV_E_NOT_AVAILABLE, "%s: inputType %d must equal weightType %d", who, mlp->inputType, mlp->weightType);
+    }
     const uint32_t wEsz = cv::elemSize(mlp->weightType);
     for (int l = 0; l < mlp->numLayers; ++l) {
         const CvMlpLayer& L = mlp->layers[l];
@@ -492,9 +499,11 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     if (!input || !output) return fail(CV_E_INVALID_ARG, "cvMlpForward: null input/output");
     const uint32_t inEsz = cv::elemSize(mlp->inputType);
     const int L = mlp->numLayers;
+    const bool encoded = mlp->inputEncoding == CV_ENCODE_XY_SQUARES;
+    const size_t sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * inEsz;
     if ((uintptr_t)input % inEsz || inputStride % inEsz || (uintptr_t)output % 2 || outputStride % 2)
         return fail(CV_E_INVALID_ARG, "cvMlpForward: vector address/stride not aligned to the element size");
-    if (batch > 1 && (inputStride < (size_t)mlp->layers[0].inputSize * inEsz || outputStride < (size_t)mlp->layers[L - 1].outputSize * 2))
+    if (batch > 1 && (inputStride < sampleBytes || outputStride < (size_t)mlp->layers[L - 1].outputSize * 2))
         return fail(CV_E_INVALID_ARG, "cvMlpForward: vector stride smaller than the vector");
     if (L == 1) {   // a single layer is the plain operator
         const CvMlpLayer& l0 = mlp->layers[0];
@@ -511,6 +520,7 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     a.in = (const uint8_t*)input; a.out = (uint8_t*)output;
     a.inStride = inputStride; a.outStride = outputStride; a.batch = batch;
     a.inAlign = alignOf(input, inputStride); a.outAlign = alignOf(output, outputStride);
+    a.inEncoding = encoded ? cv::kEncodeXYSquares : cv::kEncodeNone;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16
@@ -559,10 +569,14 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     if (L < 2) return fail(CV_E_NOT_AVAILABLE, "%s: needs at least two layers", who);
     if (batch == 0) return CV_OK;
     if (!input || !workspace) return fail(CV_E_INVALID_ARG, "%s: null input/workspace", who);
-    if ((uintptr_t)input % 2 || inputStride % 2 || (uintptr_t)targets % 2 || targetStride % 2 || (uintptr_t)workspace % 16 ||
-        (uintptr_t)lossSum % 4)
+    const bool encoded = mlp->inputEncoding == CV_ENCODE_XY_SQUARES;
+    const size_t inAlignTo = encoded ? 4 : 2, sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * 2;
+    if ((uintptr_t)input % inAlignTo || inputStride % inAlignTo || (uintptr_t)targets % 2 || targetStride % 2 ||
+        (uintptr_t)workspace % 16 || (uintptr_t)lossSum % 4)
         return fail(CV_E_INVALID_ARG, "%s: misaligned input/targets/workspace/lossSum", who);
-    if (batch > 1 && (inputStride < (size_t)mlp->layers[0].inputSize * 2 ||
+    if (encoded && !targets && mlp->layers[L - 1].outputSize != 4)
+        return fail(CV_E_INVALID_ARG, "%s: the example's loss (targets == NULL with CV_ENCODE_XY_SQUARES) needs 4 outputs", who);
+    if (batch > 1 && (inputStride < sampleBytes ||
                       (targets && targetStride < (size_t)mlp->layers[L - 1].outputSize * 2)))
         return fail(CV_E_INVALID_ARG, "%s: vector stride smaller than the vector", who);
     const uint32_t gEsz = cv::elemSize(mlp->gradType);
@@ -590,6 +604,7 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     t.mlp.inStride = inputStride;
     t.mlp.batch = batch;
     t.mlp.inAlign = alignOf(input, inputStride);
+    t.mlp.inEncoding = encoded ? cv::kEncodeXYSquares : cv::kEncodeNone;
     t.targets = (const uint8_t*)targets;
     t.targetStride = targetStride;
     t.lossScale = lossScale;

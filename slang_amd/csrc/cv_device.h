@@ -128,6 +128,27 @@ __device__ __forceinline__ void setFp16OverflowClamp()
 template <class T>
 __device__ __forceinline__ void pinHere(T& v) { asm volatile("" : "+v"(v)); }
 
+// ---- the example's input encoding ---------------------------------------------------------
+// MyNetwork::encodeInput (examples/mlp-training-coopvec/network.slang:35-38) on a float2 sample
+// converted to half2 (kernels.slang:19): the CoopVec<half,4> (x, y, x*x, y*y) as two packed dwords.
+__device__ __forceinline__ void encodeXYSquares(const uint8_t* sample, uint32_t& xy, uint32_t& squares)
+{
+    const float x = ((const float*)sample)[0], y = ((const float*)sample)[1];
+    const halfx2 h = {(half_t)x, (half_t)y};
+    xy = __builtin_bit_cast(uint32_t, h);
+    squares = __builtin_bit_cast(uint32_t, h * h);
+}
+
+// groundtruth(x, y) of the example (network.slang:67-75), every operation in half
+__device__ __forceinline__ void exampleGroundTruth(half_t x, half_t y, half_t (&gt)[4])
+{
+    const half_t one = (half_t)1.f, two = (half_t)2.f, hlf = (half_t)0.5f, c12 = (half_t)1.2f;
+    gt[0] = (half_t)((x + y) / (half_t)(one + (half_t)(y * y)));
+    gt[1] = (half_t)((half_t)(two * x) + y);
+    gt[2] = (half_t)((half_t)((half_t)(hlf * x) * x) + (half_t)(c12 * y));
+    gt[3] = (half_t)(x + (half_t)((half_t)(hlf * y) * y));
+}
+
 // ---- scalar helpers ---------------------------------------------------------------------
 
 __device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct)

@@ -50,7 +50,9 @@ struct MlpArgs {
     uint64_t inStride, outStride;
     uint32_t batch;
     uint32_t inAlign, outAlign;
+    int32_t inEncoding;     // kEncodeNone, or kEncodeXYSquares: a sample is a float2, layer 0 sees (x, y, x*x, y*y)
 };
+enum : int { kEncodeNone = 0, kEncodeXYSquares = 1 };
 // hipErrorInvalidValue when no built-in specialisation covers the layer shapes
 hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 // any layer sizes up to 128 (weights read from LDS); hipErrorInvalidValue beyond that

@@ -84,7 +84,11 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
                 uint32_t raw[RAW];
 #pragma unroll
                 for (int d = 0; d < RAW; ++d) raw[d] = 0u;
-                if (kt < kt0) {
+                if (a.inEncoding == kEncodeXYSquares) {
+                    if constexpr (RAW >= 2) {
+                        if (kt == 0 && g == 0) encodeXYSquares(p, raw[0], raw[1]);     // a float2 sample -> (x, y, x*x, y*y)
+                    }
+                } else if (kt < kt0) {
 #pragma unroll
                     for (int s = 0; s < EPL; ++s) {
                         const uint32_t q = (uint32_t)(kt * EPL + s);

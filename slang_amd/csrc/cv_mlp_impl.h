@@ -206,7 +206,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const uint32_t gs0 = optGS((uint32_t)a.layers[0].in);
     const int colBase = (int)(g * gs0);
     const int validBytes = min((int)gs0, max(a.layers[0].in - colBase, 0)) * ESZ;
-    const int loadMode = (validBytes == IN_DW * 4 && a.inAlign >= (IN_DW % 4 == 0 ? 16u : 8u)) ? 0
+    const int loadMode = a.inEncoding == kEncodeXYSquares ? 3
+                       : (validBytes == IN_DW * 4 && a.inAlign >= (IN_DW % 4 == 0 ? 16u : 8u)) ? 0
                        : ((validBytes & 3) == 0 && a.inAlign >= 4u) ? 1 : 2;
     constexpr int OROWS = 4 * Net::MTL;
     const int outDim = a.layers[L - 1].out;
@@ -241,7 +242,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         for (int j = 0; j < S; ++j) {
             const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
             const uint8_t* p = inLane + (size_t)s * a.inStride;
-            if (loadMode == 0) {
+            if (loadMode == 3) {
+                // a float2 sample; lane group 0 owns all four encoded inputs
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) buf[j][i] = 0u;
+                if constexpr (IN_DW >= 2) {
+                    if (g == 0) encodeXYSquares(a.in + (size_t)s * a.inStride, buf[j][0], buf[j][1]);
+                }
+            } else if (loadMode == 0) {
                 if constexpr (IN_DW % 4 == 0) {
 #pragma unroll
                     for (int i = 0; i < IN_DW / 4; ++i) {

@@ -248,7 +248,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int j = 0; j < 2; ++j) {
             const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
             const uint8_t* p = inLane + (size_t)s * a.inStride;
-            if (vecLoad) {
+            if (a.inEncoding == kEncodeXYSquares) {
+                // a float2 sample; lane group 0 owns all four encoded inputs
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) buf[j][i] = 0u;
+                if (g == 0) encodeXYSquares(a.in + (size_t)s * a.inStride, buf[j][0], buf[j][1]);
+            } else if (vecLoad) {
 #pragma unroll
                 for (int i = 0; i < IN_DW / 4; ++i) {
                     const u32x4 v = *(const u32x4*)(p + 16 * i);
@@ -453,7 +458,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 const uint32_t sample = t0 * TILE + 16 * j + n;
                 const bool live = sample < a.batch;
                 float tgtAll = 0.f;
-                if (!ta.targets) {
+                half_t gt[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+                const bool exampleLoss = !ta.targets && a.inEncoding == kEncodeXYSquares;
+                if (exampleLoss) {
+                    // the example's loss: groundtruth(x, y); rows 0..3 live in lane group 0, which holds (x, y)
+                    const halfx2 xy = __builtin_bit_cast(halfx2, buf[j][0]);
+                    exampleGroundTruth(xy.x, xy.y, gt);
+                } else if (!ta.targets) {
                     // target = sin(sum of the sample's inputs): every lane group holds a quarter of them
                     float part = 0.f;
 #pragma unroll
@@ -476,7 +487,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         gv[r] = (half_t)0;
                         if (live && row < outDim) {
                             const float tv = ta.targets
-                                ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row) : tgtAll;
+                                ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row)
+                                : (exampleLoss ? (float)gt[row & 3] : tgtAll);
                             const half_t diff = (half_t)((float)yv[r] - tv);
                             lossAcc += (float)diff * (float)diff;
                             gv[r] = (half_t)(2.0f * (float)diff * ta.lossScale);

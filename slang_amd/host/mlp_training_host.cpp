@@ -107,29 +107,18 @@ int main(int argc, char** argv)
     std::vector<float> inputData;
     for (int i = 0; i < inputCount; i++) inputData.push_back(rand() / (float)RAND_MAX);
 
-    std::vector<NFloat> encoded(sampleCount * 4), targets(sampleCount * 4);
-    for (int s = 0; s < sampleCount; s++) {
-        const NFloat x = (NFloat)inputData[2 * s], y = (NFloat)inputData[2 * s + 1];
-        const NFloat one = (NFloat)1, two = (NFloat)2, half = (NFloat)0.5f, c12 = (NFloat)1.2f;
-        encoded[4 * s + 0] = x; encoded[4 * s + 1] = y; encoded[4 * s + 2] = x * x; encoded[4 * s + 3] = y * y;
-        targets[4 * s + 0] = (x + y) / (one + y * y);
-        targets[4 * s + 1] = two * x + y;
-        targets[4 * s + 2] = half * x * x + c12 * y;
-        targets[4 * s + 3] = x + half * y * y;
-    }
-
+    // the float2 samples go to the device as they are (`uniform float2* inputs`, kernels.slang:12): the
+    // training step converts them to half2, encodes (x, y, x*x, y*y) and evaluates groundtruth(x, y) itself
     uint8_t* params = nullptr;
-    void *adamStates = nullptr, *dEncoded = nullptr, *dTargets = nullptr, *workspace = nullptr;
+    void *adamStates = nullptr, *dInputs = nullptr, *workspace = nullptr;
     float* dLoss = nullptr;
     const size_t paramCount = bufferSize / sizeof(NFloat);
     HIP_OK(hipMalloc((void**)&params, bufferSize));
     HIP_OK(hipMemcpy(params, initParams.data(), bufferSize, hipMemcpyHostToDevice));
     HIP_OK(hipMalloc(&adamStates, paramCount * 8));
     HIP_OK(hipMemset(adamStates, 0, paramCount * 8));
-    HIP_OK(hipMalloc(&dEncoded, encoded.size() * 2));
-    HIP_OK(hipMemcpy(dEncoded, encoded.data(), encoded.size() * 2, hipMemcpyHostToDevice));
-    HIP_OK(hipMalloc(&dTargets, targets.size() * 2));
-    HIP_OK(hipMemcpy(dTargets, targets.data(), targets.size() * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMalloc(&dInputs, inputData.size() * sizeof(float)));
+    HIP_OK(hipMemcpy(dInputs, inputData.data(), inputData.size() * sizeof(float), hipMemcpyHostToDevice));
     HIP_OK(hipMalloc((void**)&dLoss, sizeof(float)));
     // the gradient segments start from zero (the reference's random fill there would be noise)
     HIP_OK(hipMemset(params + gradientOffset, 0, bufferSize - gradientOffset));
@@ -157,7 +146,7 @@ int main(int argc, char** argv)
                                    CV_LAYOUT_ROW_MAJOR, layers[i].weightsSize, layers[i].weightsGradOffset,
                                    (size_t)kLayerSizes[i] * sizeof(NFloat)};
     }
-    CvMlpDesc mlp = {net, kLayerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0};
+    CvMlpDesc mlp = {net, kLayerCount, CV_FLOAT32, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_XY_SQUARES};
     size_t workspaceBytes = 0;
     CV_OK_OR_FAIL(cvMlpTrainStepWorkspaceSize(&mlp, sampleCount, &workspaceBytes));
     HIP_OK(hipMalloc(&workspace, workspaceBytes));
@@ -165,8 +154,8 @@ int main(int argc, char** argv)
     hipStream_t stream = nullptr;
     for (int k = 0; k < iterations; k++) {
         HIP_OK(hipMemsetAsync(params + gradientTrainingOffset, 0, bufferSize - gradientTrainingOffset, stream));
-        CV_OK_OR_FAIL(cvMlpTrainStep(stream, &mlp, dEncoded, 4 * sizeof(NFloat), dTargets, 4 * sizeof(NFloat), 1.0f,
-                                     sampleCount, dLoss, workspace, workspaceBytes));
+        CV_OK_OR_FAIL(cvMlpTrainStep(stream, &mlp, dInputs, 2 * sizeof(float), nullptr, 0, 1.0f, sampleCount, dLoss,
+                                     workspace, workspaceBytes));
         CV_OK_OR_FAIL(cvConvertMatrices(stream, params, dstDescs, params, srcDescs, kLayerCount));
         CV_OK_OR_FAIL(cvAdamStep(stream, adamStates, params, params + gradientOffset,
                                  (uint32_t)((gradientTrainingOffset - gradientOffset) / sizeof(NFloat)), 0.9f, 0.999f,
