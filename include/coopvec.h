@@ -277,6 +277,58 @@ CV_API CvResult cvElementwiseBackward(void* stream, int32_t op, int32_t elementT
                                       void* dC, size_t dCStride, float param);
 
 /* ------------------------------------------------------------------------------------ */
+/* input encoders of the neural module                                                  */
+/* ------------------------------------------------------------------------------------ */
+
+/* gridHash<Type, Dimensions> (source/standard-modules/neural/hash-function.slang:134-151) of `batch`
+ * integer grid positions [batch][dimensions] (uint32): out[s] = hash(positions[s]).  Integer work,
+ * bit-exact. */
+typedef enum CvHashType {
+    CV_HASH_PRIME = 0, CV_HASH_COHERENT_PRIME = 1, CV_HASH_REVERSED_PRIME = 2, CV_HASH_RNG = 3, CV_HASH_BASE_CONVERT = 4
+} CvHashType;
+CV_API CvResult cvGridHash(void* stream, int32_t hashType, int32_t dimensions, const void* positions,
+                           size_t positionStride, uint32_t* out, uint32_t batch);
+
+/* PermutoEncoder (source/standard-modules/neural/permuto-encoder.slang): a multi-level hash encoding
+ * on the permutohedral lattice.  CvPermutoLevelInfo mirrors PerLevelInfo (:22-30), CvPermutoDesc the
+ * generic arguments <T, Dimensions, FeatureDimensionPerEntry, Log2HashmapSize, MaxLevels> plus
+ * HyperParameters (:38-42). */
+#define CV_PERMUTO_MAX_DIMS 8
+#define CV_PERMUTO_MAX_LEVELS 16
+typedef struct CvPermutoLevelInfo {
+    uint32_t currentLevelIndex;
+    uint32_t offsetOfFeatureTable;   /* in entries */
+    uint32_t featureTableSize;       /* hashmap size of this level, in entries */
+    float    scale;
+    float    scalesPerDim[CV_PERMUTO_MAX_DIMS];
+    float    shiftsPerDim[CV_PERMUTO_MAX_DIMS];
+} CvPermutoLevelInfo;
+typedef struct CvPermutoDesc {
+    int32_t  dimensions;                 /* 1..8 */
+    int32_t  featureDimensionPerEntry;
+    uint32_t log2HashmapSize;
+    uint32_t maxLevels;                  /* 1..16 */
+    int32_t  elementType;                /* T: FLOAT32 or FLOAT16 -- positions, feature table and output */
+    float    maxLevel;                   /* maxLevelRatio * maxLevels; levels >= maxLevel + 1e-3 encode as zeros */
+    CvPermutoLevelInfo levelInfo[CV_PERMUTO_MAX_LEVELS];
+} CvPermutoDesc;
+
+/* prepareLevelInfo (:339-368) for every level, on the host: fills maxLevel and levelInfo from
+ * dimensions, log2HashmapSize and maxLevels (scale = baseScale * 2^(level * log2PerLevelScale),
+ * per-dimension scales, PCG32 shifts drawn from `seed`). */
+CV_API CvResult cvPermutoPrepareLevels(CvPermutoDesc* desc, float baseScale, float log2PerLevelScale,
+                                       float maxLevelRatio, uint32_t seed);
+/* encode (:240-337): out[s] = the maxLevels * featureDimensionPerEntry interpolated features of
+ * positions[s]; the feature table holds (sum of level sizes) * featureDimensionPerEntry elements. */
+CV_API CvResult cvPermutoEncode(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                const void* featureTable, void* out, size_t outStride, uint32_t batch);
+/* bwd_diff of encode for FLOAT32 data: dPositions[s] (overwritten; may be NULL) and dFeatureTable
+ * (+=, atomic adds like readFeatureValueBwd :222-238; may be NULL). */
+CV_API CvResult cvPermutoEncodeBackward(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                        const void* featureTable, const void* dOut, size_t dOutStride,
+                                        void* dPositions, size_t dPositionStride, void* dFeatureTable, uint32_t batch);
+
+/* ------------------------------------------------------------------------------------ */
 /* fused MLP: the example's FeedForwardLayer chain                                       */
 /* ------------------------------------------------------------------------------------ */
 

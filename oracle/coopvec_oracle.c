@@ -1027,3 +1027,223 @@ int cvo_elementwise_backward(int op, int ct, size_t count, const void* a, const 
     }
     return 0;
 }
+
+/* ===================================================================================== */
+/* grid hashes (source/standard-modules/neural/hash-function.slang)                      */
+/* ===================================================================================== */
+
+typedef struct { uint64_t state, inc; } Pcg32;
+
+static uint32_t pcg_next(Pcg32* r)                                    /* hash-function.slang:35-42 */
+{
+    const uint64_t old = r->state;
+    r->state = old * 0x5851f42d4c957f2dULL + r->inc;
+    const uint32_t xorshifted = (uint32_t)(((old >> 18) ^ old) >> 27);
+    const uint32_t rot = (uint32_t)(old >> 59);
+    return (xorshifted >> rot) | (xorshifted << ((~rot + 1u) & 31u));
+}
+
+static void pcg_init(Pcg32* r, uint64_t initstate, uint64_t initseq)  /* :25-32 */
+{
+    r->state = 0;
+    r->inc = (initseq << 1) | 1u;
+    pcg_next(r);
+    r->state += initstate;
+    pcg_next(r);
+}
+
+static void pcg_advance(Pcg32* r, int64_t delta)                      /* :45-65 */
+{
+    uint64_t curMult = 0x5851f42d4c957f2dULL, curPlus = r->inc, accMult = 1, accPlus = 0;
+    for (uint64_t d = (uint64_t)delta; d > 0; d /= 2) {
+        if (d & 1) { accMult *= curMult; accPlus = accPlus * curMult + curPlus; }
+        curPlus = (curMult + 1) * curPlus;
+        curMult *= curMult;
+    }
+    r->state = accMult * r->state + accPlus;
+}
+
+uint32_t cvo_grid_hash(int type, int dims, const uint32_t* pos)
+{
+    static const uint32_t prime[7] = {1958374283u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
+    static const uint32_t coherent[7] = {1u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
+    static const uint32_t reversed[7] = {2165219737u, 1434869437u, 2097192037u, 3674653429u, 805459861u, 2654435761u, 1958374283u};
+    switch (type) {
+    case 0: case 1: case 2: {                                           /* lcgHash, :69-78 */
+        const uint32_t* f = type == 0 ? prime : type == 1 ? coherent : reversed;
+        uint32_t r = 0;
+        for (int i = 0; i < dims; ++i) r ^= pos[i] * f[i];
+        return r; }
+    case 3: {                                                           /* rngHash, :117-131 */
+        const int bits = 64 / dims;
+        uint64_t step = 0;
+        for (int i = 0; i < dims; ++i) step ^= (uint64_t)pos[i] << (i * bits);
+        Pcg32 rng;
+        pcg_init(&rng, 1337, 1);
+        pcg_advance(&rng, (int64_t)step);
+        return pcg_next(&rng); }
+    case 4: {                                                           /* baseConvertHash, :103-113 */
+        uint32_t k = 0;
+        for (int d = 0; d < dims; ++d) { k += pos[d]; k *= 2531011u; }
+        return k; }
+    }
+    return 0;
+}
+
+/* ===================================================================================== */
+/* permutohedral-lattice encoder (source/standard-modules/neural/permuto-encoder.slang)  */
+/* ===================================================================================== */
+
+void cvo_permuto_prepare_level(uint32_t level, int dims, uint32_t log2HashmapSize, float baseScale,
+                               float log2PerLevelScale, uint32_t seed, CvoPermutoLevel* out)   /* :339-368 */
+{
+    const uint32_t size = 1u << log2HashmapSize;
+    out->currentLevelIndex = level;
+    out->featureTableSize = size;
+    out->offsetOfFeatureTable = level * size;
+    out->scale = baseScale * exp2f((float)level * log2PerLevelScale);
+    Pcg32 rng;
+    pcg_init(&rng, seed, 1);
+    pcg_advance(&rng, (int64_t)(level * (uint32_t)dims));
+    for (int d = 0; d < dims; ++d) {
+        out->scalesPerDim[d] = out->scale * (1.0f / sqrtf((float)((d + 1) * (d + 2))));
+        const float r = (float)pcg_next(&rng) * (1.0f / 4294967296.0f);
+        out->shiftsPerDim[d] = r * 10.0f - 5.0f;
+    }
+}
+
+/* geometry of one (sample, level): elevated point, closest remainder-0 point, rank (:74-152) */
+static void permuto_geometry(int D, const float* pos, const CvoPermutoLevel* lv, float* elevated, int* rem0, int* rank)
+{
+    float sum = 0.0f;
+    for (int dim = D - 1; dim >= 0; --dim) {
+        const float cf = (pos[dim] + lv->shiftsPerDim[dim]) * lv->scalesPerDim[dim];
+        elevated[dim + 1] = sum - (float)(dim + 1) * cf;
+        sum += cf;
+    }
+    elevated[0] = sum;
+    int isum = 0;
+    for (int dim = 0; dim <= D; ++dim) {
+        rank[dim] = 0;
+        const float v = elevated[dim] * (1.0f / (float)(D + 1));
+        const float up = ceilf(v) * (float)(D + 1), down = floorf(v) * (float)(D + 1);
+        rem0[dim] = (up - elevated[dim] < elevated[dim] - down) ? (int)up : (int)down;
+        isum += rem0[dim];
+    }
+    isum /= (D + 1);
+    for (int dim = 0; dim < D; ++dim) {
+        const float di = elevated[dim] - (float)rem0[dim];
+        for (int other = dim + 1; other <= D; ++other) {
+            if (di < elevated[other] - (float)rem0[other]) rank[dim]++;
+            else rank[other]++;
+        }
+    }
+    for (int dim = 0; dim <= D; ++dim) {
+        rank[dim] += isum;
+        if (rank[dim] < 0) { rank[dim] += D + 1; rem0[dim] += D + 1; }
+        else if (rank[dim] > D) { rank[dim] -= D + 1; rem0[dim] -= D + 1; }
+    }
+}
+
+static uint32_t permuto_vertex_index(int D, int F, const CvoPermutoLevel* lv, const int* rem0, const int* rank, int k)
+{
+    uint32_t key[CVO_PERMUTO_MAX_DIMS];
+    for (int dim = 0; dim < D; ++dim) {                                  /* :296-304 */
+        key[dim] = (uint32_t)(rem0[dim] + k);
+        if (rank[dim] > D - k) key[dim] -= (uint32_t)(D + 1);
+    }
+    return lv->offsetOfFeatureTable * (uint32_t)F + (cvo_grid_hash(4, D, key) % lv->featureTableSize) * (uint32_t)F;
+}
+
+static float permuto_tab(const void* table, int ct, size_t i)
+{
+    return ct == CVO_FLOAT32 ? ((const float*)table)[i] : cvo_f16_to_f32(((const uint16_t*)table)[i]);
+}
+static float permuto_round(float v, int ct) { return ct == CVO_FLOAT32 ? v : cvo_f16_to_f32(cvo_f32_to_f16_rne(v)); }
+
+int cvo_permuto_encode(int D, int F, int numLevels, float maxLevel, const CvoPermutoLevel* levels, int ct,
+                       const void* positions, size_t count, const void* table, void* out)
+{
+    if (D < 1 || D > CVO_PERMUTO_MAX_DIMS || F < 1 || numLevels < 1 || (ct != CVO_FLOAT32 && ct != CVO_FLOAT16)) return -1;
+    for (size_t s = 0; s < count; ++s) {
+        float pos[CVO_PERMUTO_MAX_DIMS];
+        for (int d = 0; d < D; ++d) pos[d] = permuto_tab(positions, ct, s * D + d);
+        for (int l = 0; l < numLevels; ++l) {
+            const CvoPermutoLevel* lv = &levels[l];
+            float acc[64];
+            for (int f = 0; f < F; ++f) acc[f] = 0.0f;
+            if (!((float)lv->currentLevelIndex >= maxLevel + 1e-3f)) {   /* :259-262 */
+                float elevated[CVO_PERMUTO_MAX_DIMS + 1], bary[CVO_PERMUTO_MAX_DIMS + 2];
+                int rem0[CVO_PERMUTO_MAX_DIMS + 1], rank[CVO_PERMUTO_MAX_DIMS + 1];
+                permuto_geometry(D, pos, lv, elevated, rem0, rank);
+                for (int i = 0; i <= D + 1; ++i) bary[i] = 0.0f;        /* :166-179 */
+                for (int dim = 0; dim <= D; ++dim) {
+                    const float delta = (elevated[dim] - (float)rem0[dim]) * (1.0f / (float)(D + 1));
+                    bary[D - rank[dim]] += delta;
+                    bary[D + 1 - rank[dim]] -= delta;
+                }
+                bary[0] += 1.0f + bary[D + 1];
+                for (int k = 0; k <= D; ++k) {
+                    const uint32_t idx = permuto_vertex_index(D, F, lv, rem0, rank, k);
+                    const float w = permuto_round(bary[k], ct);          /* T(weight) */
+                    for (int f = 0; f < F; ++f)                          /* += T(weight) * featureVal, in T (:312-316) */
+                        acc[f] = permuto_round(acc[f] + permuto_round(w * permuto_tab(table, ct, idx + f), ct), ct);
+                }
+            }
+            for (int f = 0; f < F; ++f) {
+                const size_t o = s * (size_t)(numLevels * F) + (size_t)lv->currentLevelIndex * F + f;
+                if (ct == CVO_FLOAT32) ((float*)out)[o] = acc[f];
+                else ((uint16_t*)out)[o] = cvo_f32_to_f16_rne(acc[f]);
+            }
+        }
+    }
+    return 0;
+}
+
+/* Reverse mode of the encoder in double: dPositions (overwritten) and dTable (accumulated, like the
+ * reference's atomicAdd, :222-238). */
+int cvo_permuto_encode_backward(int D, int F, int numLevels, float maxLevel, const CvoPermutoLevel* levels,
+                                const float* positions, size_t count, const float* table, const float* dOut,
+                                double* dPositions, double* dTable)
+{
+    if (D < 1 || D > CVO_PERMUTO_MAX_DIMS || F < 1 || numLevels < 1) return -1;
+    for (size_t s = 0; s < count; ++s) {
+        const float* pos = positions + s * D;
+        for (int d = 0; d < D; ++d) dPositions[s * D + d] = 0.0;
+        for (int l = 0; l < numLevels; ++l) {
+            const CvoPermutoLevel* lv = &levels[l];
+            if ((float)lv->currentLevelIndex >= maxLevel + 1e-3f) continue;
+            float elevated[CVO_PERMUTO_MAX_DIMS + 1];
+            int rem0[CVO_PERMUTO_MAX_DIMS + 1], rank[CVO_PERMUTO_MAX_DIMS + 1];
+            permuto_geometry(D, pos, lv, elevated, rem0, rank);
+            double bary[CVO_PERMUTO_MAX_DIMS + 2], dbary[CVO_PERMUTO_MAX_DIMS + 2];
+            for (int i = 0; i <= D + 1; ++i) { bary[i] = 0.0; dbary[i] = 0.0; }
+            for (int dim = 0; dim <= D; ++dim) {
+                const double delta = ((double)elevated[dim] - (double)rem0[dim]) / (double)(D + 1);
+                bary[D - rank[dim]] += delta;
+                bary[D + 1 - rank[dim]] -= delta;
+            }
+            bary[0] += 1.0 + bary[D + 1];
+            const float* g = dOut + s * (size_t)(numLevels * F) + (size_t)lv->currentLevelIndex * F;
+            for (int k = 0; k <= D; ++k) {
+                const uint32_t idx = permuto_vertex_index(D, F, lv, rem0, rank, k);
+                for (int f = 0; f < F; ++f) {
+                    dTable[idx + f] += bary[k] * (double)g[f];
+                    dbary[k] += (double)table[idx + f] * (double)g[f];
+                }
+            }
+            dbary[D + 1] += dbary[0];                                    /* wrap-around term */
+            double delev[CVO_PERMUTO_MAX_DIMS + 1];
+            for (int dim = 0; dim <= D; ++dim)
+                delev[dim] = (dbary[D - rank[dim]] - dbary[D + 1 - rank[dim]]) / (double)(D + 1);
+            /* elevate: e[dim+1] = sum - (dim+1) cf, sum += cf for dim = D-1..0, e[0] = sum */
+            double dsum = delev[0];
+            for (int dim = 0; dim < D; ++dim) {
+                double dcf = dsum - (double)(dim + 1) * delev[dim + 1];
+                dsum += delev[dim + 1];
+                dPositions[s * D + dim] += dcf * (double)lv->scalesPerDim[dim];
+            }
+        }
+    }
+    return 0;
+}

@@ -195,6 +195,33 @@ int cvo_elementwise(int op, int ct, size_t count, const void* a, const void* b, 
 int cvo_elementwise_backward(int op, int ct, size_t count, const void* a, const void* b, const void* c,
                              const void* dOut, void* dA, void* dB, void* dC, float param);
 
+/* ---- grid hashes and the permutohedral encoder of the neural module --------------------- */
+/* gridHash<Type, Dimensions> (hash-function.slang:134-151): type 0 Prime, 1 CoherentPrime,
+ * 2 ReversedPrime, 3 Rng (PCG32, seed 1337), 4 BaseConvert.  Pinned by all 22 values of
+ * tests/neural/hash-function-test.slang. */
+uint32_t cvo_grid_hash(int type, int dims, const uint32_t* pos);
+
+#define CVO_PERMUTO_MAX_DIMS 8
+/* PermutoEncoder::PerLevelInfo (permuto-encoder.slang:22-30) */
+typedef struct CvoPermutoLevel {
+    uint32_t currentLevelIndex, offsetOfFeatureTable, featureTableSize;
+    float scale;
+    float scalesPerDim[CVO_PERMUTO_MAX_DIMS], shiftsPerDim[CVO_PERMUTO_MAX_DIMS];
+} CvoPermutoLevel;
+/* prepareLevelInfo (:339-368).  Pinned by tests/neural/permuto-encoder-precomputed-constants.slang. */
+void cvo_permuto_prepare_level(uint32_t level, int dims, uint32_t log2HashmapSize, float baseScale,
+                               float log2PerLevelScale, uint32_t seed, CvoPermutoLevel* out);
+/* encode (:240-337) of `count` positions [count][D] of type ct (FLOAT32/FLOAT16, also the type of the
+ * feature table and of out [count][numLevels*F]).  Pinned by the 128 forward values of
+ * tests/neural/permuto-reference-data.slang (to that test's own epsilon 0.1). */
+int cvo_permuto_encode(int D, int F, int numLevels, float maxLevel, const CvoPermutoLevel* levels, int ct,
+                       const void* positions, size_t count, const void* table, void* out);
+/* reverse mode for fp32 data, evaluated in double: dPositions [count][D] overwritten, dTable accumulated.
+ * Pinned by EXPECTED_DL_DPOS / EXPECTED_DL_DPARAMS of the same file. */
+int cvo_permuto_encode_backward(int D, int F, int numLevels, float maxLevel, const CvoPermutoLevel* levels,
+                                const float* positions, size_t count, const float* table, const float* dOut,
+                                double* dPositions, double* dTable);
+
 #ifdef __cplusplus
 }
 #endif

@@ -78,6 +78,22 @@ class CvMlpDesc(ctypes.Structure):
                 ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32), ("inputEncoding", ctypes.c_int32)]
 
 
+PERMUTO_MAX_DIMS, PERMUTO_MAX_LEVELS = 8, 16
+
+
+class CvPermutoLevelInfo(ctypes.Structure):
+    _fields_ = [("currentLevelIndex", ctypes.c_uint32), ("offsetOfFeatureTable", ctypes.c_uint32),
+                ("featureTableSize", ctypes.c_uint32), ("scale", ctypes.c_float),
+                ("scalesPerDim", ctypes.c_float * PERMUTO_MAX_DIMS), ("shiftsPerDim", ctypes.c_float * PERMUTO_MAX_DIMS)]
+
+
+class CvPermutoDesc(ctypes.Structure):
+    _fields_ = [("dimensions", ctypes.c_int32), ("featureDimensionPerEntry", ctypes.c_int32),
+                ("log2HashmapSize", ctypes.c_uint32), ("maxLevels", ctypes.c_uint32),
+                ("elementType", ctypes.c_int32), ("maxLevel", ctypes.c_float),
+                ("levelInfo", CvPermutoLevelInfo * PERMUTO_MAX_LEVELS)]
+
+
 # name -> (restype, argtypes); every function include/coopvec.h declares
 SIGNATURES = {
     "cvGetVersion": (ctypes.c_uint32, []),
@@ -113,6 +129,15 @@ SIGNATURES = {
                                                ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
                                                ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t,
                                                ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float]),
+    "cvGridHash": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p, ctypes.c_size_t,
+                                    ctypes.c_void_p, ctypes.c_uint32]),
+    "cvPermutoPrepareLevels": (ctypes.c_int32, [ctypes.POINTER(CvPermutoDesc), ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                                ctypes.c_uint32]),
+    "cvPermutoEncode": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
+    "cvPermutoEncodeBackward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                                 ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
+                                                 ctypes.c_size_t, ctypes.c_void_p, ctypes.c_uint32]),
     "cvMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
     "cvMlpTrainStepWorkspaceSize": (ctypes.c_int32, [ctypes.POINTER(CvMlpDesc), ctypes.c_uint32,

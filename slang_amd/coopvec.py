@@ -418,6 +418,82 @@ def elementwiseBackward(op: int, dOut: torch.Tensor, a: torch.Tensor, b: Optiona
 
 
 # ---------------------------------------------------------------------------------------------
+# input encoders of the neural module
+# ---------------------------------------------------------------------------------------------
+
+class HashType(enum.IntEnum):
+    """hash-function.slang:6-13"""
+    Prime = 0
+    CoherentPrime = 1
+    ReversedPrime = 2
+    Rng = 3
+    BaseConvert = 4
+
+
+def gridHash(hashType: int, positions: torch.Tensor, *, stream=None) -> torch.Tensor:
+    """gridHash<Type, Dimensions> (hash-function.slang:134-151) of integer grid positions [batch, D]."""
+    if positions.dtype not in (torch.int32, getattr(torch, "uint32", torch.int32)) or positions.dim() != 2 or positions.stride(1) != 1:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "positions must be a 32-bit integer GPU tensor [batch, D]")
+    out = torch.empty(positions.shape[0], dtype=torch.int32, device=positions.device)
+    _check(_lib.load().cvGridHash(_stream_handle(stream), int(hashType), positions.shape[1], positions.data_ptr(),
+                                  positions.stride(0) * 4, out.data_ptr(), positions.shape[0]))
+    return out
+
+
+class PermutoEncoder:
+    """PermutoEncoder<T, Dimensions, FeatureDimensionPerEntry, Log2HashmapSize, MaxLevels>
+    (permuto-encoder.slang:8-20) with its HyperParameters prepared as prepareLevelInfo does (:339-368)."""
+
+    def __init__(self, dimensions: int, featureDimensionPerEntry: int, log2HashmapSize: int, maxLevels: int, *,
+                 baseScale: float, log2PerLevelScale: float, maxLevelRatio: float = 1.1, seed: int = 1337,
+                 dtype: torch.dtype = torch.float32):
+        self.desc = _lib.CvPermutoDesc()
+        self.desc.dimensions = dimensions
+        self.desc.featureDimensionPerEntry = featureDimensionPerEntry
+        self.desc.log2HashmapSize = log2HashmapSize
+        self.desc.maxLevels = maxLevels
+        self.desc.elementType = int(_TORCH_TO_CT.get(dtype, -1))
+        self.dtype = dtype
+        _check(_lib.load().cvPermutoPrepareLevels(ctypes.byref(self.desc), baseScale, log2PerLevelScale, maxLevelRatio, seed))
+
+    @property
+    def featureTableElements(self) -> int:
+        return (1 << self.desc.log2HashmapSize) * self.desc.maxLevels * self.desc.featureDimensionPerEntry
+
+    @property
+    def outputSize(self) -> int:
+        return self.desc.maxLevels * self.desc.featureDimensionPerEntry
+
+    def encode(self, positions: torch.Tensor, featureTable: torch.Tensor, *, out: Optional[torch.Tensor] = None, stream=None):
+        """encode (:319-337) of every row of positions [batch, Dimensions]."""
+        if positions.dtype != self.dtype or featureTable.dtype != self.dtype or positions.dim() != 2 or positions.stride(1) != 1:
+            raise CoopVecError(SLANG_E_INVALID_ARG, "positions [batch, D] and featureTable must have the encoder's dtype")
+        if featureTable.numel() < self.featureTableElements or not featureTable.is_contiguous():
+            raise CoopVecError(SLANG_E_BUFFER_TOO_SMALL, "featureTable holds fewer than %d elements" % self.featureTableElements)
+        if out is None:
+            out = torch.empty(positions.shape[0], self.outputSize, dtype=self.dtype, device=positions.device)
+        es = positions.element_size()
+        _check(_lib.load().cvPermutoEncode(_stream_handle(stream), ctypes.byref(self.desc), positions.data_ptr(),
+                                           positions.stride(0) * es, featureTable.data_ptr(), out.data_ptr(),
+                                           out.stride(0) * es, positions.shape[0]))
+        return out
+
+    def backward(self, positions: torch.Tensor, featureTable: torch.Tensor, dOut: torch.Tensor, *,
+                 dFeatureTable: Optional[torch.Tensor] = None, wantPositionGrad: bool = True, stream=None):
+        """bwd_diff of encode: returns (dPositions or None, dFeatureTable); the table gradient is added to."""
+        if dFeatureTable is None:
+            dFeatureTable = torch.zeros_like(featureTable)
+        dPos = torch.empty_like(positions, memory_format=torch.contiguous_format) if wantPositionGrad else None
+        es = positions.element_size()
+        _check(_lib.load().cvPermutoEncodeBackward(_stream_handle(stream), ctypes.byref(self.desc), positions.data_ptr(),
+                                                   positions.stride(0) * es, featureTable.data_ptr(), dOut.data_ptr(),
+                                                   dOut.stride(0) * es, dPos.data_ptr() if dPos is not None else None,
+                                                   dPos.stride(0) * es if dPos is not None else 0,
+                                                   dFeatureTable.data_ptr(), positions.shape[0]))
+        return dPos, dFeatureTable
+
+
+# ---------------------------------------------------------------------------------------------
 # fused MLP: the example's FeedForwardLayer chain
 # ---------------------------------------------------------------------------------------------
 

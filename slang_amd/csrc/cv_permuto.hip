@@ -1,0 +1,413 @@
+// cv_permuto.hip -- input encoders of the neural module in front of the MLP, for gfx950.
+//
+// Replaces, for a whole batch of positions, PermutoEncoder::encode and its reverse mode
+// (source/standard-modules/neural/permuto-encoder.slang:240-337, readFeatureValueBwd :222-238,
+// prepareLevelInfo :339-368) and the grid hashes it is built on
+// (source/standard-modules/neural/hash-function.slang:69-151).  One thread handles one position: it
+// walks the levels, finds the enclosing simplex of the permutohedral lattice, and gathers D+1 hashed
+// feature-table entries per level -- integer hashing plus scattered reads, bound by cache and HBM
+// latency, not by arithmetic.  The reverse pass scatters with atomic adds, as the reference does.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstring>
+
+#include "cv_device.h"
+#include "cv_error.h"
+
+namespace cv {
+namespace {
+
+constexpr int kMaxDims = CV_PERMUTO_MAX_DIMS;
+constexpr int kMaxLevels = CV_PERMUTO_MAX_LEVELS;
+
+// ---- hashes (hash-function.slang) -----------------------------------------------------------
+struct Pcg32 {
+    uint64_t state, inc;
+    __host__ __device__ uint32_t next()                               // :35-42
+    {
+        const uint64_t old = state;
+        state = old * 0x5851f42d4c957f2dULL + inc;
+        const uint32_t xorshifted = (uint32_t)(((old >> 18) ^ old) >> 27);
+        const uint32_t rot = (uint32_t)(old >> 59);
+        return (xorshifted >> rot) | (xorshifted << ((~rot + 1u) & 31u));
+    }
+    __host__ __device__ void init(uint64_t initstate, uint64_t initseq = 1)   // :25-32
+    {
+        state = 0;
+        inc = (initseq << 1) | 1u;
+        next();
+        state += initstate;
+        next();
+    }
+    __host__ __device__ void advance(int64_t delta)                    // :45-65
+    {
+        uint64_t curMult = 0x5851f42d4c957f2dULL, curPlus = inc, accMult = 1, accPlus = 0;
+        for (uint64_t d = (uint64_t)delta; d > 0; d /= 2) {
+            if (d & 1) { accMult *= curMult; accPlus = accPlus * curMult + curPlus; }
+            curPlus = (curMult + 1) * curPlus;
+            curMult *= curMult;
+        }
+        state = accMult * state + accPlus;
+    }
+};
+
+__host__ __device__ inline uint32_t baseConvertHash(const uint32_t* pos, int dims)   // :103-113
+{
+    uint32_t k = 0;
+    for (int d = 0; d < dims; ++d) { k += pos[d]; k *= 2531011u; }
+    return k;
+}
+
+__host__ __device__ inline uint32_t gridHash(int type, const uint32_t* pos, int dims)
+{
+    const uint32_t prime[7] = {1958374283u, 2654435761u, 805459861u, 3674653429u, 2097192037u, 1434869437u, 2165219737u};
+    switch (type) {
+    case CV_HASH_PRIME: case CV_HASH_COHERENT_PRIME: case CV_HASH_REVERSED_PRIME: {   // lcgHash, :69-100
+        uint32_t r = 0;
+        for (int i = 0; i < dims; ++i) {
+            uint32_t f = type == CV_HASH_REVERSED_PRIME ? prime[6 - i] : prime[i];
+            if (type == CV_HASH_COHERENT_PRIME && i == 0) f = 1u;
+            r ^= pos[i] * f;
+        }
+        return r; }
+    case CV_HASH_RNG: {                                                // :117-131
+        const int bits = 64 / dims;
+        uint64_t step = 0;
+        for (int i = 0; i < dims; ++i) step ^= (uint64_t)pos[i] << (i * bits);
+        Pcg32 rng;
+        rng.init(1337);
+        rng.advance((int64_t)step);
+        return rng.next(); }
+    case CV_HASH_BASE_CONVERT: return baseConvertHash(pos, dims);
+    }
+    return 0;
+}
+
+__global__ __launch_bounds__(256) void gridHashKernel(int type, int dims, const uint8_t* pos, uint64_t stride, uint32_t* out, uint32_t batch)
+{
+    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
+    if (s >= batch) return;
+    uint32_t p[7];
+    for (int i = 0; i < dims; ++i) p[i] = ((const uint32_t*)(pos + (size_t)s * stride))[i];
+    out[s] = gridHash(type, p, dims);
+}
+
+// ---- permutohedral lattice --------------------------------------------------------------------
+struct PermutoArgs {
+    CvPermutoDesc desc;
+    const uint8_t* pos; uint64_t posStride;
+    const uint8_t* table;
+    uint8_t* out; uint64_t outStride;
+    const uint8_t* dOut; uint64_t dOutStride;
+    uint8_t* dPos; uint64_t dPosStride;
+    float* dTable;
+    uint32_t batch;
+};
+
+// elevated point, closest remainder-0 point and rank of one position on one level (:74-152)
+template <int D>
+__device__ __forceinline__ void latticeGeometry(const float* pos, const CvPermutoLevelInfo& lv, float* elevated, int* rem0, int* rank)
+{
+    float sum = 0.0f;
+#pragma unroll
+    for (int dim = D - 1; dim >= 0; --dim) {
+        const float cf = (pos[dim] + lv.shiftsPerDim[dim]) * lv.scalesPerDim[dim];
+        elevated[dim + 1] = sum - (float)(dim + 1) * cf;
+        sum += cf;
+    }
+    elevated[0] = sum;
+    int isum = 0;
+#pragma unroll
+    for (int dim = 0; dim <= D; ++dim) {
+        rank[dim] = 0;
+        const float v = elevated[dim] * (1.0f / (float)(D + 1));
+        const float up = ceilf(v) * (float)(D + 1), down = floorf(v) * (float)(D + 1);
+        rem0[dim] = (up - elevated[dim] < elevated[dim] - down) ? (int)up : (int)down;
+        isum += rem0[dim];
+    }
+    isum /= (D + 1);
+#pragma unroll
+    for (int dim = 0; dim < D; ++dim) {
+        const float di = elevated[dim] - (float)rem0[dim];
+#pragma unroll
+        for (int other = dim + 1; other <= D; ++other) {
+            if (di < elevated[other] - (float)rem0[other]) rank[dim]++;
+            else rank[other]++;
+        }
+    }
+#pragma unroll
+    for (int dim = 0; dim <= D; ++dim) {
+        rank[dim] += isum;
+        if (rank[dim] < 0) { rank[dim] += D + 1; rem0[dim] += D + 1; }
+        else if (rank[dim] > D) { rank[dim] -= D + 1; rem0[dim] -= D + 1; }
+    }
+}
+
+// barycentric[k] of the remainder-k vertex (:166-179), without indexing registers by a run-time value
+template <int D>
+__device__ __forceinline__ void barycentricWeights(const float* elevated, const int* rem0, const int* rank, float* bary)
+{
+#pragma unroll
+    for (int i = 0; i <= D + 1; ++i) bary[i] = 0.0f;
+#pragma unroll
+    for (int dim = 0; dim <= D; ++dim) {
+        const float delta = (elevated[dim] - (float)rem0[dim]) * (1.0f / (float)(D + 1));
+#pragma unroll
+        for (int i = 0; i <= D + 1; ++i) {
+            if (i == D - rank[dim]) bary[i] += delta;
+            if (i == D + 1 - rank[dim]) bary[i] -= delta;
+        }
+    }
+    bary[0] += 1.0f + bary[D + 1];
+}
+
+template <int D>
+__device__ __forceinline__ uint32_t vertexIndex(const CvPermutoLevelInfo& lv, int F, const int* rem0, const int* rank, int k)
+{
+    uint32_t key[D];
+#pragma unroll
+    for (int dim = 0; dim < D; ++dim) {                                // :296-304
+        key[dim] = (uint32_t)(rem0[dim] + k);
+        if (rank[dim] > D - k) key[dim] -= (uint32_t)(D + 1);
+    }
+    return lv.offsetOfFeatureTable * (uint32_t)F + (baseConvertHash(key, D) % lv.featureTableSize) * (uint32_t)F;
+}
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void permutoEncodeKernel(const PermutoArgs a)
+{
+    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
+    if (s >= a.batch) return;
+    const int F = a.desc.featureDimensionPerEntry;
+    float pos[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) pos[d] = (float)((const T*)(a.pos + (size_t)s * a.posStride))[d];
+    T* out = (T*)(a.out + (size_t)s * a.outStride);
+    const T* table = (const T*)a.table;
+    for (uint32_t l = 0; l < a.desc.maxLevels; ++l) {
+        const CvPermutoLevelInfo& lv = a.desc.levelInfo[l];
+        T* o = out + lv.currentLevelIndex * F;
+        for (int f = 0; f < F; ++f) o[f] = (T)0.f;
+        if ((float)lv.currentLevelIndex >= a.desc.maxLevel + 1e-3f) continue;   // zero padding beyond maxLevel, :259-262
+        float elevated[D + 1], bary[D + 2];
+        int rem0[D + 1], rank[D + 1];
+        latticeGeometry<D>(pos, lv, elevated, rem0, rank);
+        barycentricWeights<D>(elevated, rem0, rank, bary);
+        for (int f0 = 0; f0 < F; f0 += 4) {                            // four features of the entry at a time
+            T acc[4] = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
+#pragma unroll
+            for (int k = 0; k <= D; ++k) {
+                const uint32_t idx = vertexIndex<D>(lv, F, rem0, rank, k);
+                const T w = (T)bary[k];
+#pragma unroll
+                for (int f = 0; f < 4; ++f)
+                    if (f0 + f < F) acc[f] = (T)(acc[f] + (T)(w * table[idx + f0 + f]));    // in T, vertex by vertex (:312-316)
+            }
+#pragma unroll
+            for (int f = 0; f < 4; ++f)
+                if (f0 + f < F) o[f0 + f] = acc[f];
+        }
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a)
+{
+    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
+    if (s >= a.batch) return;
+    const int F = a.desc.featureDimensionPerEntry;
+    float pos[D], dpos[D];
+#pragma unroll
+    for (int d = 0; d < D; ++d) { pos[d] = ((const float*)(a.pos + (size_t)s * a.posStride))[d]; dpos[d] = 0.f; }
+    const float* table = (const float*)a.table;
+    const float* g = (const float*)(a.dOut + (size_t)s * a.dOutStride);
+    for (uint32_t l = 0; l < a.desc.maxLevels; ++l) {
+        const CvPermutoLevelInfo& lv = a.desc.levelInfo[l];
+        if ((float)lv.currentLevelIndex >= a.desc.maxLevel + 1e-3f) continue;
+        float elevated[D + 1], bary[D + 2], dbary[D + 2];
+        int rem0[D + 1], rank[D + 1];
+        latticeGeometry<D>(pos, lv, elevated, rem0, rank);
+        barycentricWeights<D>(elevated, rem0, rank, bary);
+#pragma unroll
+        for (int i = 0; i <= D + 1; ++i) dbary[i] = 0.f;
+        const float* gl = g + lv.currentLevelIndex * F;
+#pragma unroll
+        for (int k = 0; k <= D; ++k) {
+            const uint32_t idx = vertexIndex<D>(lv, F, rem0, rank, k);
+            for (int f = 0; f < F; ++f) {
+                if (a.dTable) atomicAdd(a.dTable + idx + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
+                dbary[k] += table[idx + f] * gl[f];
+            }
+        }
+        if (!a.dPos) continue;
+        dbary[D + 1] += dbary[0];                                      // the wrap-around term of barycentric[0]
+        float delev[D + 1];
+#pragma unroll
+        for (int dim = 0; dim <= D; ++dim) {
+            float plus = 0.f, minus = 0.f;
+#pragma unroll
+            for (int i = 0; i <= D + 1; ++i) {
+                if (i == D - rank[dim]) plus = dbary[i];
+                if (i == D + 1 - rank[dim]) minus = dbary[i];
+            }
+            delev[dim] = (plus - minus) * (1.0f / (float)(D + 1));
+        }
+        // elevate: e[dim+1] = sum - (dim+1) cf, sum += cf for dim = D-1..0, e[0] = sum
+        float dsum = delev[0];
+#pragma unroll
+        for (int dim = 0; dim < D; ++dim) {
+            const float dcf = dsum - (float)(dim + 1) * delev[dim + 1];
+            dsum += delev[dim + 1];
+            dpos[dim] += dcf * lv.scalesPerDim[dim];
+        }
+    }
+    if (a.dPos) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) ((float*)(a.dPos + (size_t)s * a.dPosStride))[d] = dpos[d];
+    }
+}
+
+template <typename T>
+hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
+{
+    const dim3 grid((a.batch + 255) / 256), block(256);
+    switch (a.desc.dimensions) {
+#define CV_D(N) case N: hipLaunchKernelGGL((permutoEncodeKernel<T, N>), grid, block, 0, stream, a); break;
+    CV_D(1) CV_D(2) CV_D(3) CV_D(4) CV_D(5) CV_D(6) CV_D(7) CV_D(8)
+#undef CV_D
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launchBackward(hipStream_t stream, const PermutoArgs& a)
+{
+    const dim3 grid((a.batch + 255) / 256), block(256);
+    switch (a.desc.dimensions) {
+#define CV_D(N) case N: hipLaunchKernelGGL(permutoBackwardKernel<N>, grid, block, 0, stream, a); break;
+    CV_D(1) CV_D(2) CV_D(3) CV_D(4) CV_D(5) CV_D(6) CV_D(7) CV_D(8)
+#undef CV_D
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+CvResult checkDesc(const char* who, const CvPermutoDesc* d)
+{
+    if (!d) return failWith(CV_E_INVALID_ARG, "%s: desc is null", who);
+    if (d->dimensions < 1 || d->dimensions > kMaxDims) return failWith(CV_E_INVALID_ARG, "%s: dimensions=%d (1..%d)", who, d->dimensions, kMaxDims);
+    if (d->featureDimensionPerEntry < 1 || d->featureDimensionPerEntry > 64)
+        return failWith(CV_E_INVALID_ARG, "%s: featureDimensionPerEntry=%d (1..64)", who, d->featureDimensionPerEntry);
+    if (d->maxLevels < 1 || d->maxLevels > (uint32_t)kMaxLevels) return failWith(CV_E_INVALID_ARG, "%s: maxLevels=%u (1..%d)", who, d->maxLevels, kMaxLevels);
+    if (d->elementType != CV_FLOAT32 && d->elementType != CV_FLOAT16)
+        return failWith(CV_E_NOT_AVAILABLE, "%s: elementType %d (supported: FLOAT32, FLOAT16)", who, d->elementType);
+    for (uint32_t l = 0; l < d->maxLevels; ++l)
+        if (d->levelInfo[l].featureTableSize == 0 || d->levelInfo[l].currentLevelIndex >= d->maxLevels)
+            return failWith(CV_E_INVALID_ARG, "%s: level %u: empty feature table or level index %u out of range", who, l, d->levelInfo[l].currentLevelIndex);
+    return CV_OK;
+}
+
+} // namespace
+} // namespace cv
+
+extern "C" {
+
+CV_API CvResult cvGridHash(void* stream, int32_t hashType, int32_t dimensions, const void* positions, size_t positionStride,
+                           uint32_t* out, uint32_t batch)
+{
+    using namespace cv;
+    if (hashType < CV_HASH_PRIME || hashType > CV_HASH_BASE_CONVERT) return failWith(CV_E_INVALID_ARG, "cvGridHash: unknown hash type %d", hashType);
+    if (dimensions < 1 || dimensions > 7) return failWith(CV_E_INVALID_ARG, "cvGridHash: dimensions=%d (1..7, the prime table of the reference)", dimensions);
+    if (batch == 0) return CV_OK;
+    if (!positions || !out || (uintptr_t)positions % 4 || positionStride % 4 || (uintptr_t)out % 4 ||
+        (batch > 1 && positionStride < (size_t)dimensions * 4))
+        return failWith(CV_E_INVALID_ARG, "cvGridHash: null or misaligned argument");
+    noteKernel(false, "gridHashKernel");
+    hipLaunchKernelGGL(gridHashKernel, dim3((batch + 255) / 256), dim3(256), 0, (hipStream_t)stream, hashType, dimensions,
+                       (const uint8_t*)positions, (uint64_t)positionStride, out, batch);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvGridHash launch: %s", hipGetErrorString(e));
+    return CV_OK;
+}
+
+CV_API CvResult cvPermutoPrepareLevels(CvPermutoDesc* d, float baseScale, float log2PerLevelScale, float maxLevelRatio, uint32_t seed)
+{
+    using namespace cv;
+    if (!d) return failWith(CV_E_INVALID_ARG, "cvPermutoPrepareLevels: desc is null");
+    if (d->dimensions < 1 || d->dimensions > kMaxDims || d->maxLevels < 1 || d->maxLevels > (uint32_t)kMaxLevels || d->log2HashmapSize > 30)
+        return failWith(CV_E_INVALID_ARG, "cvPermutoPrepareLevels: dimensions=%d maxLevels=%u log2HashmapSize=%u", d->dimensions, d->maxLevels, d->log2HashmapSize);
+    const uint32_t size = 1u << d->log2HashmapSize;
+    d->maxLevel = maxLevelRatio * (float)d->maxLevels;
+    for (uint32_t level = 0; level < d->maxLevels; ++level) {          // prepareLevelInfo, permuto-encoder.slang:339-368
+        CvPermutoLevelInfo& lv = d->levelInfo[level];
+        memset(&lv, 0, sizeof(lv));
+        lv.currentLevelIndex = level;
+        lv.featureTableSize = size;
+        lv.offsetOfFeatureTable = level * size;
+        lv.scale = baseScale * exp2f((float)level * log2PerLevelScale);
+        Pcg32 rng;
+        rng.init(seed);
+        rng.advance((int64_t)(level * (uint32_t)d->dimensions));
+        for (int dim = 0; dim < d->dimensions; ++dim) {
+            lv.scalesPerDim[dim] = lv.scale * (1.0f / sqrtf((float)((dim + 1) * (dim + 2))));
+            const float r = (float)rng.next() * (1.0f / 4294967296.0f);
+            lv.shiftsPerDim[dim] = r * 10.0f - 5.0f;
+        }
+    }
+    return CV_OK;
+}
+
+CV_API CvResult cvPermutoEncode(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                const void* featureTable, void* out, size_t outStride, uint32_t batch)
+{
+    using namespace cv;
+    CvResult rc = checkDesc("cvPermutoEncode", desc);
+    if (CV_FAILED(rc)) return rc;
+    if (batch == 0) return CV_OK;
+    const uint32_t esz = desc->elementType == CV_FLOAT32 ? 4u : 2u;
+    const size_t nOut = (size_t)desc->maxLevels * desc->featureDimensionPerEntry;
+    if (!positions || !featureTable || !out || (uintptr_t)positions % esz || positionStride % esz || (uintptr_t)featureTable % esz ||
+        (uintptr_t)out % esz || outStride % esz ||
+        (batch > 1 && (positionStride < (size_t)desc->dimensions * esz || outStride < nOut * esz)))
+        return failWith(CV_E_INVALID_ARG, "cvPermutoEncode: null, misaligned or overlapping-row argument");
+    PermutoArgs a;
+    memset(&a, 0, sizeof(a));
+    a.desc = *desc;
+    a.pos = (const uint8_t*)positions; a.posStride = positionStride; a.table = (const uint8_t*)featureTable;
+    a.out = (uint8_t*)out; a.outStride = outStride; a.batch = batch;
+    noteKernel(false, "permutoEncodeKernel<%s,D=%d>", esz == 4 ? "f32" : "f16", desc->dimensions);
+    const hipError_t e = esz == 4 ? launchEncode<float>((hipStream_t)stream, a) : launchEncode<half_t>((hipStream_t)stream, a);
+    if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvPermutoEncode launch: %s", hipGetErrorString(e));
+    return CV_OK;
+}
+
+CV_API CvResult cvPermutoEncodeBackward(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                        const void* featureTable, const void* dOut, size_t dOutStride,
+                                        void* dPositions, size_t dPositionStride, void* dFeatureTable, uint32_t batch)
+{
+    using namespace cv;
+    CvResult rc = checkDesc("cvPermutoEncodeBackward", desc);
+    if (CV_FAILED(rc)) return rc;
+    if (desc->elementType != CV_FLOAT32)
+        return failWith(CV_E_NOT_AVAILABLE, "cvPermutoEncodeBackward: FLOAT32 data only (the table gradient is accumulated with fp32 atomic adds)");
+    if (batch == 0) return CV_OK;
+    const size_t nOut = (size_t)desc->maxLevels * desc->featureDimensionPerEntry;
+    if (!positions || !featureTable || !dOut || (uintptr_t)positions % 4 || positionStride % 4 || (uintptr_t)featureTable % 4 ||
+        (uintptr_t)dOut % 4 || dOutStride % 4 || (uintptr_t)dPositions % 4 || dPositionStride % 4 || (uintptr_t)dFeatureTable % 4 ||
+        (batch > 1 && (positionStride < (size_t)desc->dimensions * 4 || dOutStride < nOut * 4 ||
+                       (dPositions && dPositionStride < (size_t)desc->dimensions * 4))))
+        return failWith(CV_E_INVALID_ARG, "cvPermutoEncodeBackward: null, misaligned or overlapping-row argument");
+    PermutoArgs a;
+    memset(&a, 0, sizeof(a));
+    a.desc = *desc;
+    a.pos = (const uint8_t*)positions; a.posStride = positionStride; a.table = (const uint8_t*)featureTable;
+    a.dOut = (const uint8_t*)dOut; a.dOutStride = dOutStride;
+    a.dPos = (uint8_t*)dPositions; a.dPosStride = dPositionStride; a.dTable = (float*)dFeatureTable; a.batch = batch;
+    noteKernel(false, "permutoBackwardKernel<D=%d>", desc->dimensions);
+    const hipError_t e = launchBackward((hipStream_t)stream, a);
+    if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvPermutoEncodeBackward launch: %s", hipGetErrorString(e));
+    return CV_OK;
+}
+
+} // extern "C"

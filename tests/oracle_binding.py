@@ -265,6 +265,60 @@ def elementwise_backward(op: int, d_out, a, b=None, c=None, param: float = 0.0):
     return tuple(grads)
 
 
+# ---- grid hashes / permutohedral encoder ---------------------------------------------------
+HASH_PRIME, HASH_COHERENT_PRIME, HASH_REVERSED_PRIME, HASH_RNG, HASH_BASE_CONVERT = range(5)
+PERMUTO_MAX_DIMS = 8
+
+
+class CvoPermutoLevel(_c.Structure):
+    _fields_ = [("currentLevelIndex", _u32), ("offsetOfFeatureTable", _u32), ("featureTableSize", _u32),
+                ("scale", _f32), ("scalesPerDim", _f32 * PERMUTO_MAX_DIMS), ("shiftsPerDim", _f32 * PERMUTO_MAX_DIMS)]
+
+
+def grid_hash(hash_type: int, pos) -> int:
+    L = lib()
+    L.cvo_grid_hash.argtypes = [_c.c_int, _c.c_int, _vp]
+    L.cvo_grid_hash.restype = _u32
+    a = np.ascontiguousarray(pos, dtype=np.uint32)
+    return int(L.cvo_grid_hash(int(hash_type), a.size, ptr(a)))
+
+
+def permuto_levels(dims, log2_hashmap_size, n_levels, base_scale, log2_per_level_scale, seed=1337):
+    L = lib()
+    L.cvo_permuto_prepare_level.argtypes = [_u32, _c.c_int, _u32, _f32, _f32, _u32, _c.POINTER(CvoPermutoLevel)]
+    L.cvo_permuto_prepare_level.restype = None
+    arr = (CvoPermutoLevel * n_levels)()
+    for l in range(n_levels):
+        L.cvo_permuto_prepare_level(l, dims, log2_hashmap_size, base_scale, log2_per_level_scale, seed, _c.byref(arr[l]))
+    return arr
+
+
+def permuto_encode(levels, feat_per_entry, max_level, positions: np.ndarray, table: np.ndarray) -> np.ndarray:
+    L = lib()
+    L.cvo_permuto_encode.argtypes = [_c.c_int, _c.c_int, _c.c_int, _f32, _c.POINTER(CvoPermutoLevel), _c.c_int, _vp, _sz, _vp, _vp]
+    L.cvo_permuto_encode.restype = _c.c_int
+    B, D = positions.shape
+    out = np.zeros((B, len(levels) * feat_per_entry), positions.dtype)
+    rc = L.cvo_permuto_encode(D, feat_per_entry, len(levels), max_level, levels, _ew_ct(positions), ptr(positions), B,
+                              ptr(table), ptr(out))
+    assert rc == 0
+    return out
+
+
+def permuto_encode_backward(levels, feat_per_entry, max_level, positions: np.ndarray, table: np.ndarray, d_out: np.ndarray):
+    L = lib()
+    L.cvo_permuto_encode_backward.argtypes = [_c.c_int, _c.c_int, _c.c_int, _f32, _c.POINTER(CvoPermutoLevel), _vp, _sz,
+                                              _vp, _vp, _vp, _vp]
+    L.cvo_permuto_encode_backward.restype = _c.c_int
+    B, D = positions.shape
+    d_pos = np.zeros((B, D), np.float64)
+    d_table = np.zeros(table.size, np.float64)
+    rc = L.cvo_permuto_encode_backward(D, feat_per_entry, len(levels), max_level, levels, ptr(positions), B, ptr(table),
+                                       ptr(d_out), ptr(d_pos), ptr(d_table))
+    assert rc == 0
+    return d_pos, d_table
+
+
 # ---- Adam ---------------------------------------------------------------------------------
 ADAM_STATE_DTYPE = np.dtype([("mean", np.uint16), ("variance", np.uint16), ("iteration", np.int32)])
 

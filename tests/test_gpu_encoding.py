@@ -78,3 +78,92 @@ def test_encoding_argument_validation():
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpTrainStep(layers, xy, None, inputEncoding=InputEncoding.XYSquares)    # the example's loss has 4 outputs
     assert e.value.result == cv.SLANG_E_INVALID_ARG
+
+
+# ---- grid hashes and the permutohedral encoder ---------------------------------------------------
+import json
+import os
+
+NG = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "neural_goldens.json")))
+
+
+def test_grid_hash_goldens_and_random_positions():
+    # integer work: bit-exact against tests/neural/hash-function-test.slang and the oracle
+    pos = NG["hash"]["positions"]
+    got = []
+    for t in (cv.HashType.Prime, cv.HashType.CoherentPrime, cv.HashType.ReversedPrime, cv.HashType.BaseConvert, cv.HashType.Rng):
+        for d in "1234":
+            p = torch.tensor([pos[d]], dtype=torch.int32, device=DEV)
+            got.append(int(cv.gridHash(t, p).cpu().numpy().view(np.uint32)[0]))
+    p3 = torch.tensor([pos["3"]], dtype=torch.int32, device=DEV)
+    got.append(int(cv.gridHash(cv.HashType.Prime, p3).cpu().numpy().view(np.uint32)[0]))
+    got.append(int(cv.gridHash(cv.HashType.BaseConvert, p3).cpu().numpy().view(np.uint32)[0]))
+    assert got == NG["hash"]["expected"]
+    rng = np.random.default_rng(1)
+    for dims in (1, 2, 3, 5, 7):
+        grid = rng.integers(0, 2 ** 32, (3000, dims), dtype=np.uint64).astype(np.uint32)
+        gd = to_dev(grid.view(np.int32))
+        for t in range(5):
+            want = np.array([ob.grid_hash(t, row) for row in grid[:300]], np.uint32)
+            assert np.array_equal(cv.gridHash(t, gd).cpu().numpy().view(np.uint32)[:300], want), (t, dims)
+
+
+def _reference_setup():
+    from test_oracle_encoders import reference_setup
+    return reference_setup()
+
+
+def test_permuto_encoder_reference_data():
+    # tests/neural/permuto-encoder-test.slang and -backward: the reference's expected values, to its epsilon
+    P = NG["permuto"]; cfg = P["config"]
+    pos, table, levels, max_level = _reference_setup()
+    enc = cv.PermutoEncoder(2, 2, 8, 4, baseScale=cfg["baseScale"], log2PerLevelScale=cfg["log2PerLevelScale"],
+                            maxLevelRatio=cfg["maxLevelRatio"], seed=cfg["seed"])
+    out = enc.encode(to_dev(pos), to_dev(table)).cpu().numpy()
+    want = np.array(P["expectedForward"]).reshape(16, 8)
+    assert np.abs(out[P["verifyPositions"]] - want).max() <= cfg["epsilon"]
+    assert np.array_equal(out, ob.permuto_encode(levels, 2, max_level, pos, table))      # same fp32 operations, same order
+    d_pos, d_table = enc.backward(to_dev(pos), to_dev(table), torch.ones(256, 8, device=DEV))
+    want_pos = np.array(P["expectedDLdPos"]).reshape(16, 2)
+    got_pos = d_pos.cpu().numpy()[P["verifyPositions"]]
+    assert (np.abs(got_pos - want_pos) <= cfg["epsilon"] + 1e-5 * np.abs(want_pos)).all()
+    assert np.abs(d_table.cpu().numpy()[P["verifyParamIndices"]] - np.array(P["expectedDLdParams"])).max() <= cfg["epsilon"]
+
+
+@pytest.mark.parametrize("D,F,levels_n", [(1, 1, 3), (3, 4, 6), (4, 2, 8), (6, 8, 2), (8, 2, 4)])
+def test_permuto_encoder_against_oracle(D, F, levels_n):
+    rng = np.random.default_rng(D * 100 + F)
+    log2 = 10
+    enc = cv.PermutoEncoder(D, F, log2, levels_n, baseScale=2.0, log2PerLevelScale=0.8, maxLevelRatio=0.8, seed=7)
+    levels = ob.permuto_levels(D, log2, levels_n, 2.0, 0.8, 7)
+    max_level = float(np.float32(0.8) * np.float32(levels_n))
+    B = 5000
+    pos = rng.uniform(0, 1, (B, D)).astype(np.float32)
+    table = rng.standard_normal(enc.featureTableElements).astype(np.float32)
+    out = enc.encode(to_dev(pos), to_dev(table)).cpu().numpy()
+    assert np.array_equal(out, ob.permuto_encode(levels, F, max_level, pos, table))
+    g = rng.standard_normal((B, levels_n * F)).astype(np.float32)
+    d_pos, d_table = enc.backward(to_dev(pos), to_dev(table), to_dev(g))
+    r_pos, r_table = ob.permuto_encode_backward(levels, F, max_level, pos, table, g)
+    assert np.linalg.norm(d_pos.cpu().numpy() - r_pos) <= 1e-4 * np.linalg.norm(r_pos)
+    assert np.linalg.norm(d_table.cpu().numpy() - r_table) <= 1e-4 * np.linalg.norm(r_table)
+    # fp16 data: every product and sum rounded to half, as the generic T of the reference does
+    enc16 = cv.PermutoEncoder(D, F, log2, levels_n, baseScale=2.0, log2PerLevelScale=0.8, maxLevelRatio=0.8, seed=7, dtype=torch.float16)
+    p16, t16 = pos.astype(np.float16), table.astype(np.float16)
+    o16 = enc16.encode(to_dev(p16), to_dev(t16)).cpu().numpy()
+    assert np.array_equal(o16, ob.permuto_encode(levels, F, max_level, p16, t16))
+
+
+def test_encoder_feeds_the_mlp():
+    # encode positions, run the decoder MLP on the fp16 features: the neural-texture shape
+    rng = np.random.default_rng(8)
+    enc = cv.PermutoEncoder(3, 2, 12, 8, baseScale=4.0, log2PerLevelScale=1.0, dtype=torch.float16)
+    B = 4096
+    pos = to_dev(rng.uniform(0, 1, (B, 3)).astype(np.float16))
+    table = to_dev((rng.standard_normal(enc.featureTableElements) * 0.5).astype(np.float16))
+    feats = enc.encode(pos, table)
+    specs = make_specs(rng, [16, 64, 64, 3])
+    layers = build(specs)
+    y = cv.mlpForward(layers, feats)
+    ref = ob.ref_mlp_forward(specs, feats.cpu().numpy(), ob.F16)
+    assert (np.abs(y.cpu().numpy().astype(np.float32) - ref.astype(np.float32)) <= 2e-2 * np.abs(ref.astype(np.float32)) + 2e-2).mean() > 0.999
