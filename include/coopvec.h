@@ -408,6 +408,55 @@ CV_API CvResult cvMlpTrainStepNoAlloc(void* stream, const CvMlpDesc* mlp,
                                       float lossScale, uint32_t batch, float* lossSum);
 
 /* ------------------------------------------------------------------------------------ */
+/* the neural module's network parameter block                                          */
+/* ------------------------------------------------------------------------------------ */
+
+/* NetworkParameterLayoutConverter<T, BiasMask, D0, D1, ...>
+ * (source/standard-modules/neural/network-parameter-layout-converter.slang:469-555) and the FFLayer
+ * chain over such a block (layers.slang:34-110).  dims[0..layerCount] are D0..Dn; bit l of biasMask
+ * says whether layer l (D_l -> D_{l+1}) has a bias.
+ *   portable layout: per layer row-major weight[Out][In], then bias[Out] if the layer has one;
+ *   optimal layout : per layer weight envelope [align16(Out)][align16(In)], then a bias slot of
+ *                    align16(Out) elements (reserved for every layer), padding zero.
+ * `order` is the order of the weights inside an envelope: NATIVE is this library's (accumulator-native
+ * 16x16 tiles, i.e. CV_LAYOUT_TRAINING_OPTIMAL per layer: what the fused kernels read and write); the
+ * other three are the reference's SPIR-V, Metal and CUDA orders (:137-172), so that blocks can be
+ * exchanged with those targets. */
+#define CV_NEURAL_MAX_LAYERS 64
+typedef enum CvNeuralWeightOrder {
+    CV_NEURAL_ORDER_NATIVE = 0, CV_NEURAL_ORDER_TILED_ROW_MAJOR = 1, CV_NEURAL_ORDER_PADDED_ROW_MAJOR = 2,
+    CV_NEURAL_ORDER_CUDA_MATRIX_B = 3
+} CvNeuralWeightOrder;
+typedef struct CvNeuralNetworkDesc {
+    int32_t  layerCount;
+    int32_t  dims[CV_NEURAL_MAX_LAYERS + 1];
+    uint64_t biasMask;
+    int32_t  elementType;     /* T: FLOAT32 or FLOAT16 */
+    int32_t  order;           /* CvNeuralWeightOrder */
+} CvNeuralNetworkDesc;
+
+/* ElementCountLogical / ElementCountPhysical (:477-480). */
+CV_API CvResult cvNeuralNetworkSize(const CvNeuralNetworkDesc* net, size_t* elementCountLogical, size_t* elementCountPhysical);
+/* toOptimalLayout (:487-516) / toPortableLayout (:524-553) of the whole block in one launch. */
+CV_API CvResult cvNeuralToOptimalLayout(void* stream, const CvNeuralNetworkDesc* net, const void* portable, void* optimal);
+CV_API CvResult cvNeuralToPortableLayout(void* stream, const CvNeuralNetworkDesc* net, const void* optimal, void* portable);
+/* The FFLayer chain y = Activation_l(W_l x + b_l) (layers.slang:90-110) over a FLOAT16 parameter block,
+ * in the portable (LinearLayout; optimalLayout = 0) or the optimal layout in NATIVE order
+ * (optimalLayout = 1); layer l's bias sits WeightStorageSize elements behind its weights (:93-96).
+ * activations / leakySlopes: one CvActivation / slope per layer (NULL: none).  Served by cvMlpForward. */
+CV_API CvResult cvNeuralMlpForward(void* stream, const CvNeuralNetworkDesc* net, int32_t optimalLayout, const void* params,
+                                   const int32_t* activations, const float* leakySlopes,
+                                   const void* input, size_t inputStride, void* output, size_t outputStride, uint32_t batch);
+/* bwd_diff through the chain with a gradient block laid out like the parameter block (the
+ * DifferentialPtrPair of layers.slang:21-25): gradients are accumulated in FLOAT16 at the same element
+ * offsets.  Served by cvMlpTrainStep (same loss, targets, workspace rules). */
+CV_API CvResult cvNeuralMlpTrainStepWorkspaceSize(const CvNeuralNetworkDesc* net, uint32_t batch, size_t* outBytes);
+CV_API CvResult cvNeuralMlpTrainStep(void* stream, const CvNeuralNetworkDesc* net, int32_t optimalLayout, const void* params,
+                                     void* paramGrads, const int32_t* activations, const float* leakySlopes,
+                                     const void* input, size_t inputStride, const void* targets, size_t targetStride,
+                                     float lossScale, uint32_t batch, float* lossSum, void* workspace, size_t workspaceBytes);
+
+/* ------------------------------------------------------------------------------------ */
 /* parameter update of the example                                                      */
 /* ------------------------------------------------------------------------------------ */
 

@@ -94,6 +94,14 @@ class CvPermutoDesc(ctypes.Structure):
                 ("levelInfo", CvPermutoLevelInfo * PERMUTO_MAX_LEVELS)]
 
 
+NEURAL_MAX_LAYERS = 64
+
+
+class CvNeuralNetworkDesc(ctypes.Structure):
+    _fields_ = [("layerCount", ctypes.c_int32), ("dims", ctypes.c_int32 * (NEURAL_MAX_LAYERS + 1)),
+                ("biasMask", ctypes.c_uint64), ("elementType", ctypes.c_int32), ("order", ctypes.c_int32)]
+
+
 # name -> (restype, argtypes); every function include/coopvec.h declares
 SIGNATURES = {
     "cvGetVersion": (ctypes.c_uint32, []),
@@ -138,6 +146,19 @@ SIGNATURES = {
     "cvPermutoEncodeBackward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
                                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                                  ctypes.c_size_t, ctypes.c_void_p, ctypes.c_uint32]),
+    "cvNeuralNetworkSize": (ctypes.c_int32, [ctypes.POINTER(CvNeuralNetworkDesc), ctypes.POINTER(ctypes.c_size_t),
+                                             ctypes.POINTER(ctypes.c_size_t)]),
+    "cvNeuralToOptimalLayout": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvNeuralNetworkDesc), ctypes.c_void_p, ctypes.c_void_p]),
+    "cvNeuralToPortableLayout": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvNeuralNetworkDesc), ctypes.c_void_p, ctypes.c_void_p]),
+    "cvNeuralMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvNeuralNetworkDesc), ctypes.c_int32, ctypes.c_void_p,
+                                            ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float), ctypes.c_void_p,
+                                            ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
+    "cvNeuralMlpTrainStepWorkspaceSize": (ctypes.c_int32, [ctypes.POINTER(CvNeuralNetworkDesc), ctypes.c_uint32,
+                                                           ctypes.POINTER(ctypes.c_size_t)]),
+    "cvNeuralMlpTrainStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvNeuralNetworkDesc), ctypes.c_int32, ctypes.c_void_p,
+                                              ctypes.c_void_p, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float),
+                                              ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_float,
+                                              ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]),
     "cvMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
                                       ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
     "cvMlpTrainStepWorkspaceSize": (ctypes.c_int32, [ctypes.POINTER(CvMlpDesc), ctypes.c_uint32,

@@ -663,6 +663,100 @@ def coopVecReduceSumAccumulate(v: torch.Tensor, buffer: torch.Tensor, offset: in
 
 
 # ---------------------------------------------------------------------------------------------
+# the neural module's network parameter block
+# ---------------------------------------------------------------------------------------------
+
+class NeuralWeightOrder(enum.IntEnum):
+    """CvNeuralWeightOrder: Native is this library's; the others are the reference's SPIR-V, Metal and
+    CUDA orders (network-parameter-layout-converter.slang:137-172)."""
+    Native = 0
+    TiledRowMajor = 1
+    PaddedRowMajor = 2
+    CudaMatrixB = 3
+
+
+class NetworkParameterLayoutConverter:
+    """NetworkParameterLayoutConverter<T, BiasMask, D0, D1, ...>
+    (network-parameter-layout-converter.slang:469-555) plus the FFLayer chain over the block."""
+
+    def __init__(self, dtype: torch.dtype, biasMask: int, *dims: int, order: int = NeuralWeightOrder.Native):
+        self.desc = _lib.CvNeuralNetworkDesc()
+        self.desc.layerCount = len(dims) - 1
+        for i, d in enumerate(dims):
+            self.desc.dims[i] = d
+        self.desc.biasMask = biasMask
+        self.desc.elementType = int(_TORCH_TO_CT.get(dtype, -1))
+        self.desc.order = int(order)
+        self.dtype = dtype
+        l, p = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _check(_lib.load().cvNeuralNetworkSize(ctypes.byref(self.desc), ctypes.byref(l), ctypes.byref(p)))
+        self.ElementCountLogical, self.ElementCountPhysical = l.value, p.value
+        self.BytesLogical = l.value * torch.empty(0, dtype=dtype).element_size()
+        self.BytesPhysical = p.value * torch.empty(0, dtype=dtype).element_size()
+
+    def _buf(self, t, count, what):
+        if t.dtype != self.dtype or not t.is_cuda or not t.is_contiguous() or t.numel() < count:
+            raise CoopVecError(SLANG_E_BUFFER_TOO_SMALL, "%s must be a contiguous GPU tensor of at least %d %s" % (what, count, self.dtype))
+        return t.data_ptr()
+
+    def toOptimalLayout(self, portable: torch.Tensor, optimal: Optional[torch.Tensor] = None, *, stream=None) -> torch.Tensor:
+        if optimal is None:
+            optimal = torch.empty(self.ElementCountPhysical, dtype=self.dtype, device=portable.device)
+        _check(_lib.load().cvNeuralToOptimalLayout(_stream_handle(stream), ctypes.byref(self.desc),
+                                                   self._buf(portable, self.ElementCountLogical, "portable"),
+                                                   self._buf(optimal, self.ElementCountPhysical, "optimal")))
+        return optimal
+
+    def toPortableLayout(self, optimal: torch.Tensor, portable: Optional[torch.Tensor] = None, *, stream=None) -> torch.Tensor:
+        if portable is None:
+            portable = torch.empty(self.ElementCountLogical, dtype=self.dtype, device=optimal.device)
+        _check(_lib.load().cvNeuralToPortableLayout(_stream_handle(stream), ctypes.byref(self.desc),
+                                                    self._buf(optimal, self.ElementCountPhysical, "optimal"),
+                                                    self._buf(portable, self.ElementCountLogical, "portable")))
+        return portable
+
+    def _acts(self, activations, slopes):
+        n = self.desc.layerCount
+        a = (ctypes.c_int32 * n)(*[int(x) for x in (activations or [0] * n)])
+        s = (ctypes.c_float * n)(*[float(x) for x in (slopes or [0.0] * n)])
+        return a, s
+
+    def eval(self, params: torch.Tensor, input: torch.Tensor, *, optimalLayout: bool, activations=None, leakySlopes=None,
+             out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+        """The FFLayer chain (layers.slang:90-110) over the block, fp16."""
+        _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+        if out is None:
+            out = torch.empty(input.shape[0], self.desc.dims[self.desc.layerCount], dtype=torch.float16, device=input.device)
+        a, s = self._acts(activations, leakySlopes)
+        count = self.ElementCountPhysical if optimalLayout else self.ElementCountLogical
+        _check(_lib.load().cvNeuralMlpForward(_stream_handle(stream), ctypes.byref(self.desc), 1 if optimalLayout else 0,
+                                              self._buf(params, count, "params"), a, s, input.data_ptr(), inStride,
+                                              out.data_ptr(), out.stride(0) * 2, input.shape[0]))
+        return out
+
+    def trainStep(self, params: torch.Tensor, paramGrads: torch.Tensor, input: torch.Tensor, targets: Optional[torch.Tensor], *,
+                  optimalLayout: bool, activations=None, leakySlopes=None, lossScale: float = 1.0, stream=None) -> torch.Tensor:
+        """bwd_diff through the chain; gradients accumulate in `paramGrads`, laid out like `params`."""
+        _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+        a, s = self._acts(activations, leakySlopes)
+        count = self.ElementCountPhysical if optimalLayout else self.ElementCountLogical
+        need = ctypes.c_size_t(0)
+        lib = _lib.load()
+        _check(lib.cvNeuralMlpTrainStepWorkspaceSize(ctypes.byref(self.desc), input.shape[0], ctypes.byref(need)))
+        ws = torch.empty(need.value, dtype=torch.uint8, device=input.device)
+        loss = torch.zeros(1, dtype=torch.float32, device=input.device)
+        tptr, tstride = None, 0
+        if targets is not None:
+            _, tstride = _vector_info(targets, CoopVecComponentType.Float16, "targets")
+            tptr = targets.data_ptr()
+        _check(lib.cvNeuralMlpTrainStep(_stream_handle(stream), ctypes.byref(self.desc), 1 if optimalLayout else 0,
+                                        self._buf(params, count, "params"), self._buf(paramGrads, count, "paramGrads"), a, s,
+                                        input.data_ptr(), inStride, tptr, tstride, float(lossScale), input.shape[0],
+                                        loss.data_ptr(), ws.data_ptr(), need.value))
+        return loss
+
+
+# ---------------------------------------------------------------------------------------------
 # parameter update of the example
 # ---------------------------------------------------------------------------------------------
 
