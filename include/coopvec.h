@@ -65,6 +65,10 @@ typedef enum CvComponentType {
     CV_FLOAT_E4M3 = 0, CV_FLOAT_E5M2 = 1, CV_FLOAT16 = 2, CV_FLOAT32 = 3, CV_FLOAT64 = 4,
     CV_SINT8 = 5, CV_SINT16 = 6, CV_SINT32 = 7, CV_SINT64 = 8, CV_SINT8_PACKED = 9,
     CV_UINT8 = 10, CV_UINT16 = 11, CV_UINT32 = 12, CV_UINT64 = 13, CV_UINT8_PACKED = 14,
+    /* extension: bfloat16 operands (v_mfma_f32_16x16x32_bf16).  Slang's CoopVecComponentType has no
+     * such entry (SLANG_SCALAR_TYPE_BFLOAT16 = 16 exists as a scalar type only, include/slang.h:2155);
+     * accepted by cvMatMul, cvGetMatrixSize and cvConvertMatrices. */
+    CV_BFLOAT16 = 15,
     CV_COMPONENT_NONE = -1
 } CvComponentType;
 

@@ -199,7 +199,7 @@ static int elem_size(int ct)
 {
     switch (ct) {
     case CVO_FLOAT_E4M3: case CVO_FLOAT_E5M2: case CVO_SINT8: case CVO_UINT8: return 1;
-    case CVO_FLOAT16: case CVO_SINT16: case CVO_UINT16: return 2;
+    case CVO_FLOAT16: case CVO_SINT16: case CVO_UINT16: case CVO_BFLOAT16: return 2;
     case CVO_FLOAT32: case CVO_SINT32: case CVO_UINT32: case CVO_SINT8_PACKED:
     case CVO_UINT8_PACKED: return 4;
     case CVO_FLOAT64: case CVO_SINT64: case CVO_UINT64: return 8;
@@ -497,6 +497,7 @@ static int frag_elems_per_lane(int ct)
     case CVO_SINT8: case CVO_UINT8: return 16;        /* v_mfma_i32_16x16x64_i8: 16 B per lane */
     case CVO_FLOAT_E4M3: case CVO_FLOAT_E5M2: return 8; /* v_mfma_f32_16x16x32_fp8: 8 B */
     case CVO_FLOAT16: return 8;                         /* v_mfma_f32_16x16x32_f16: 16 B */
+    case CVO_BFLOAT16: return 8;                        /* v_mfma_f32_16x16x32_bf16: 16 B */
     case CVO_FLOAT32: return 8;
     }
     return -1;
@@ -506,7 +507,7 @@ static int layout_ct_ok(int ct, int layout)
 {
     if (elem_size(ct) < 0 || cvo_component_packing_factor(ct) != 1) return 0;
     if (layout == CVO_INFERENCING_OPTIMAL) return frag_elems_per_lane(ct) > 0;
-    if (layout == CVO_TRAINING_OPTIMAL) return ct == CVO_FLOAT16 || ct == CVO_FLOAT32;
+    if (layout == CVO_TRAINING_OPTIMAL) return ct == CVO_FLOAT16 || ct == CVO_FLOAT32 || ct == CVO_BFLOAT16;
     return layout == CVO_ROW_MAJOR || layout == CVO_COLUMN_MAJOR;
 }
 
@@ -606,6 +607,8 @@ static inline int decode_f32(const uint8_t* p, int ct, float* out)
     case CVO_FLOAT16: { uint16_t h; memcpy(&h, p, 2); *out = cvo_f16_to_f32(h); return 0; }
     case CVO_FLOAT32: { memcpy(out, p, 4); return 0; }
     case CVO_FLOAT_E4M3: { *out = cvo_e4m3_to_f32(*p); return 0; }
+    case CVO_FLOAT_E5M2: { *out = cvo_f16_to_f32((uint16_t)((uint16_t)*p << 8)); return 0; }   /* e5m2 = high byte of binary16 */
+    case CVO_BFLOAT16: { uint16_t h; memcpy(&h, p, 2); *out = bits_f32((uint32_t)h << 16); return 0; } /* bf16 = high half of binary32 */
     case CVO_SINT8: { *out = (float)*(const int8_t*)p; return 0; }
     case CVO_UINT8: { *out = (float)*p; return 0; }
     }

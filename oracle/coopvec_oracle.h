@@ -39,7 +39,9 @@ extern "C" {
 enum {
     CVO_FLOAT_E4M3 = 0, CVO_FLOAT_E5M2 = 1, CVO_FLOAT16 = 2, CVO_FLOAT32 = 3, CVO_FLOAT64 = 4,
     CVO_SINT8 = 5, CVO_SINT16 = 6, CVO_SINT32 = 7, CVO_SINT64 = 8, CVO_SINT8_PACKED = 9,
-    CVO_UINT8 = 10, CVO_UINT16 = 11, CVO_UINT32 = 12, CVO_UINT64 = 13, CVO_UINT8_PACKED = 14
+    CVO_UINT8 = 10, CVO_UINT16 = 11, CVO_UINT32 = 12, CVO_UINT64 = 13, CVO_UINT8_PACKED = 14,
+    /* not in the reference's enum: bfloat16 operands of the matrix cores, the library's extension */
+    CVO_BFLOAT16 = 15
 };
 /* CoopVecMatrixLayout, hlsl.meta.slang:32547-32553 == include/slang.h:948-955 */
 enum { CVO_ROW_MAJOR = 0, CVO_COLUMN_MAJOR = 1, CVO_INFERENCING_OPTIMAL = 2, CVO_TRAINING_OPTIMAL = 3 };

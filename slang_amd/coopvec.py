@@ -33,7 +33,8 @@ class CoopVecMatrixLayout(enum.IntEnum):
 
 
 class CoopVecComponentType(enum.IntEnum):
-    """hlsl.meta.slang:32558-32575"""
+    """hlsl.meta.slang:32558-32575; BFloat16 is this library's extension (the reference knows
+    bfloat16 as a scalar type only, SLANG_SCALAR_TYPE_BFLOAT16, include/slang.h:2155)."""
     FloatE4M3 = 0
     FloatE5M2 = 1
     Float16 = 2
@@ -49,6 +50,7 @@ class CoopVecComponentType(enum.IntEnum):
     UnsignedInt32 = 12
     UnsignedInt64 = 13
     UnsignedInt8Packed = 14
+    BFloat16 = 15
 
 
 class RhiCooperativeVectorComponentType(enum.IntEnum):
@@ -164,6 +166,7 @@ def _stream_handle(stream) -> ctypes.c_void_p:
 
 _TORCH_TO_CT = {
     torch.float16: CoopVecComponentType.Float16,
+    torch.bfloat16: CoopVecComponentType.BFloat16,
     torch.float32: CoopVecComponentType.Float32,
     torch.int8: CoopVecComponentType.SignedInt8,
     torch.uint8: CoopVecComponentType.UnsignedInt8,
@@ -173,12 +176,22 @@ if hasattr(torch, "uint32"):
     _TORCH_TO_CT[torch.uint32] = CoopVecComponentType.UnsignedInt32
 if hasattr(torch, "float8_e4m3fn"):
     _TORCH_TO_CT[torch.float8_e4m3fn] = CoopVecComponentType.FloatE4M3
+if hasattr(torch, "float8_e5m2"):
+    _TORCH_TO_CT[torch.float8_e5m2] = CoopVecComponentType.FloatE5M2
 
 _CT_TO_TORCH = {
     CoopVecComponentType.Float16: torch.float16,
+    CoopVecComponentType.BFloat16: torch.bfloat16,
     CoopVecComponentType.Float32: torch.float32,
     CoopVecComponentType.SignedInt32: torch.int32,
 }
+if hasattr(torch, "uint32"):
+    _CT_TO_TORCH[CoopVecComponentType.UnsignedInt32] = torch.uint32
+
+
+def lastKernelName() -> str:
+    """Name and specialisation of the kernel(s) the last launching call on this thread dispatched."""
+    return _lib.load().cvGetLastKernelName().decode()
 
 
 def componentPackingFactor(componentType: int) -> int:
@@ -275,9 +288,10 @@ def _vector_info(v: torch.Tensor, interpretation: int, what: str):
     ct = _TORCH_TO_CT.get(v.dtype)
     if ct is None:
         raise CoopVecError(SLANG_E_NOT_AVAILABLE, "%s: unsupported element dtype %s" % (what, v.dtype))
-    # a byte tensor interpreted as e4m3 carries e4m3 elements
-    if ct == CoopVecComponentType.UnsignedInt8 and interpretation == CoopVecComponentType.FloatE4M3:
-        ct = CoopVecComponentType.FloatE4M3
+    # a byte tensor interpreted as an 8-bit float carries elements of that type
+    if ct == CoopVecComponentType.UnsignedInt8 and interpretation in (CoopVecComponentType.FloatE4M3,
+                                                                    CoopVecComponentType.FloatE5M2):
+        ct = CoopVecComponentType(interpretation)
     return ct, v.stride(0) * v.element_size()
 
 
@@ -289,8 +303,9 @@ def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpret
     batch = input.shape[0]
     if resultType is None:
         resultType = (CoopVecComponentType.SignedInt32 if inCt in (
-            CoopVecComponentType.SignedInt8, CoopVecComponentType.SignedInt32,
-            CoopVecComponentType.UnsignedInt32) else CoopVecComponentType.Float16)
+            CoopVecComponentType.SignedInt8, CoopVecComponentType.UnsignedInt8, CoopVecComponentType.SignedInt32,
+            CoopVecComponentType.UnsignedInt32) else
+            CoopVecComponentType.BFloat16 if inCt == CoopVecComponentType.BFloat16 else CoopVecComponentType.Float16)
     if out is None:
         if accumulate:
             raise CoopVecError(SLANG_E_INVALID_ARG, "the accumulate forms need `out` (the vector added to)")

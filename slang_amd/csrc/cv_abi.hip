@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <vector>
 
 #include "../../include/coopvec.h"
 #include "cv_error.h"
@@ -89,24 +90,83 @@ void* scratchOfCurrentDevice(CvResult* rc)
 
 bool isOptimal(int layout) { return layout == CV_LAYOUT_INFERENCING_OPTIMAL || layout == CV_LAYOUT_TRAINING_OPTIMAL; }
 
-struct Combo {
-    int32_t inputType, inputInterp; uint32_t packing; int32_t matrixInterp, biasInterp, resultType;
+// What the matMul kernels implement: the matrix-core flavour that serves a combination of
+// (type of the vectors in memory, inputInterpretation, matrixInterpretation, biasInterpretation or
+// CV_COMPONENT_NONE, resultType), or false.  The table of cvQuerySupportedCombinations is this
+// predicate evaluated over every combination, so the two cannot disagree.
+struct ComboKind {
     cv::MmaKind kind;
+    bool inUnsigned, matUnsigned;
 };
 
-// What the kernels implement.  Rows with a bias also cover the bias-less coopVecMatMul.
-const Combo kCombos[] = {
-    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT16, CV_FLOAT16, cv::MmaKind::F16},
-    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT16, CV_FLOAT32, cv::MmaKind::F16},
-    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT16, cv::MmaKind::F16},
-    {CV_FLOAT16,    CV_FLOAT16,      1, CV_FLOAT16,    CV_FLOAT32, CV_FLOAT32, cv::MmaKind::F16},
-    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT16, cv::MmaKind::Fp8AsF16},
-    {CV_FLOAT_E4M3, CV_FLOAT_E4M3,   1, CV_FLOAT_E4M3, CV_FLOAT16, CV_FLOAT32, cv::MmaKind::Fp8AsF16},
-    {CV_SINT8,      CV_SINT8,        1, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
-    {CV_UINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
-    {CV_SINT32,     CV_SINT8_PACKED, 4, CV_SINT8,      CV_SINT32,  CV_SINT32,  cv::MmaKind::I8},
-};
-constexpr uint32_t kNumCombos = sizeof(kCombos) / sizeof(kCombos[0]);
+bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
+{
+    const bool noBias = biasInterp == CV_COMPONENT_NONE;
+    ComboKind k{cv::MmaKind::F16, false, false};
+    const bool f16f32Res = resType == CV_FLOAT16 || resType == CV_FLOAT32;
+    if (matInterp == CV_FLOAT16) {
+        if (inType != CV_FLOAT16 || inInterp != CV_FLOAT16 || !f16f32Res) return false;
+        if (!noBias && biasInterp != CV_FLOAT16 && biasInterp != CV_FLOAT32) return false;
+        k.kind = cv::MmaKind::F16;
+    } else if (matInterp == CV_FLOAT_E4M3) {
+        if (inInterp != CV_FLOAT_E4M3 || !f16f32Res || (!noBias && biasInterp != CV_FLOAT16)) return false;
+        if (inType == CV_FLOAT_E4M3) k.kind = cv::MmaKind::Fp8AsF16;
+        else if (inType == CV_FLOAT16) k.kind = cv::MmaKind::F16VecAsE4M3;   // CoopVec<half> + interpretation
+        else return false;
+    } else if (matInterp == CV_FLOAT_E5M2) {
+        if (inType != CV_FLOAT_E5M2 || inInterp != CV_FLOAT_E5M2 || !f16f32Res || (!noBias && biasInterp != CV_FLOAT16)) return false;
+        k.kind = cv::MmaKind::Bf8AsF16;
+    } else if (matInterp == CV_BFLOAT16) {
+        if (inType != CV_BFLOAT16 || inInterp != CV_BFLOAT16) return false;
+        if (resType != CV_BFLOAT16 && resType != CV_FLOAT32) return false;
+        if (!noBias && biasInterp != CV_BFLOAT16 && biasInterp != CV_FLOAT32) return false;
+        k.kind = cv::MmaKind::Bf16;
+    } else if (matInterp == CV_SINT8 || matInterp == CV_UINT8) {
+        if (resType != CV_SINT32 && resType != CV_UINT32) return false;
+        if (!noBias && biasInterp != CV_SINT32 && biasInterp != CV_UINT32) return false;
+        if (inInterp == CV_SINT8_PACKED || inInterp == CV_UINT8_PACKED) {
+            // four bytes per 32-bit element; the reference's unpacking sign-extends for both packed
+            // kinds (hlsl.meta.slang:32850-32855)
+            if (inType != CV_UINT32 && inType != CV_SINT32) return false;
+        } else if (inInterp == CV_SINT8 || inInterp == CV_UINT8) {
+            if (inType != inInterp) return false;
+            k.inUnsigned = inType == CV_UINT8;
+        } else {
+            return false;
+        }
+        k.matUnsigned = matInterp == CV_UINT8;
+        k.kind = (k.inUnsigned || k.matUnsigned) ? cv::MmaKind::I8AnySign : cv::MmaKind::I8;
+    } else {
+        return false;
+    }
+    if (out) *out = k;
+    return true;
+}
+
+constexpr int32_t kNumComponentTypes = 16;   // CV_FLOAT_E4M3 .. CV_BFLOAT16
+
+// every supported combination that carries a bias (each also covers the bias-less coopVecMatMul)
+const std::vector<CvCombination>& comboTable()
+{
+    static std::vector<CvCombination> table;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        for (int32_t mat = 0; mat < kNumComponentTypes; ++mat)
+            for (int32_t in = 0; in < kNumComponentTypes; ++in)
+                for (int32_t interp = 0; interp < kNumComponentTypes; ++interp)
+                    for (int32_t bias = 0; bias < kNumComponentTypes; ++bias)
+                        for (int32_t res = 0; res < kNumComponentTypes; ++res) {
+                            if (!classifyCombo(in, interp, mat, bias, res, nullptr)) continue;
+                            CvCombination c;
+                            c.inputType = in; c.inputInterpretation = interp;
+                            c.inputPackingFactor = (uint32_t)cvComponentPackingFactor(interp);
+                            c.matrixInterpretation = mat; c.biasInterpretation = bias; c.resultType = res;
+                            c.transpose = 0;
+                            table.push_back(c);
+                        }
+    });
+    return table;
+}
 
 } // namespace
 
@@ -162,6 +222,7 @@ CV_API int32_t cvComponentScalarType(int32_t ct)
     case CV_UINT16: return 13;
     case CV_UINT32: return 4;
     case CV_UINT64: return 6;
+    case CV_BFLOAT16: return 16;
     }
     return -1;
 }
@@ -192,16 +253,9 @@ CV_API int32_t cvComponentTypeToRhi(int32_t ct)
 
 CV_API uint32_t cvQuerySupportedCombinations(CvCombination* out, uint32_t capacity)
 {
-    for (uint32_t i = 0; i < kNumCombos && out && i < capacity; ++i) {
-        out[i].inputType = kCombos[i].inputType;
-        out[i].inputInterpretation = kCombos[i].inputInterp;
-        out[i].inputPackingFactor = kCombos[i].packing;
-        out[i].matrixInterpretation = kCombos[i].matrixInterp;
-        out[i].biasInterpretation = kCombos[i].biasInterp;
-        out[i].resultType = kCombos[i].resultType;
-        out[i].transpose = 0;
-    }
-    return kNumCombos;
+    const std::vector<CvCombination>& table = comboTable();
+    for (size_t i = 0; i < table.size() && out && i < capacity; ++i) out[i] = table[i];
+    return (uint32_t)table.size();
 }
 
 CV_API CvResult cvGetMatrixSize(uint32_t rowCount, uint32_t colCount, int32_t componentType,
@@ -289,14 +343,9 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     if (packing != 1 && d->k % 4 != 0)   // fallback rule k == 4*PackedK (hlsl.meta.slang:32846)
         return fail(CV_E_NOT_AVAILABLE, "cvMatMul: packed input needs k to be a multiple of 4 (k=%d)", d->k);
 
-    const Combo* combo = nullptr;
-    for (uint32_t i = 0; i < kNumCombos; ++i) {
-        const Combo& c = kCombos[i];
-        if (c.inputType == d->inputType && c.inputInterp == d->inputInterpretation &&
-            c.matrixInterp == d->matrixInterpretation && c.resultType == d->resultType &&
-            (!d->bias || c.biasInterp == d->biasInterpretation)) { combo = &c; break; }
-    }
-    if (!combo)
+    ComboKind combo;
+    if (!classifyCombo(d->inputType, d->inputInterpretation, d->matrixInterpretation,
+                       d->bias ? d->biasInterpretation : (int32_t)CV_COMPONENT_NONE, d->resultType, &combo))
         return fail(CV_E_NOT_AVAILABLE,
                     "cvMatMul: unsupported combination input %d as %d, matrix %d, bias %d, result %d",
                     d->inputType, d->inputInterpretation, d->matrixInterpretation,
@@ -306,8 +355,11 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
 
     cv::MatMulArgs a;
     memset(&a, 0, sizeof(a));
-    const uint32_t inEsz = combo->kind == cv::MmaKind::F16 ? 2u : 1u;
-    const uint32_t outEsz = d->resultType == CV_FLOAT16 ? 2u : 4u;
+    // packed vectors are addressed as the bytes they hold; their 32-bit elements must be aligned
+    const uint32_t inEsz = packing != 1 ? 1u : cv::elemSize(d->inputType);
+    const uint32_t outEsz = cv::elemSize(d->resultType);
+    if (packing != 1 && ((uintptr_t)d->input % 4 || d->inputStride % 4))
+        return fail(CV_E_INVALID_ARG, "cvMatMul: packed vectors must be 4-byte aligned");
     if ((uintptr_t)d->input % inEsz || d->inputStride % inEsz || (uintptr_t)d->output % outEsz || d->outputStride % outEsz)
         return fail(CV_E_INVALID_ARG, "cvMatMul: vector address/stride not aligned to the element size");
     if (d->batch > 1 && (d->inputStride < (size_t)d->k * inEsz || d->outputStride < (size_t)d->m * outEsz))
@@ -335,20 +387,24 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     }
     a.outCt = d->resultType;
     a.act = d->activation;
+    if (d->resultType == CV_UINT32 && a.act == CV_ACT_RELU) a.act = CV_ACT_NONE;   // max(u, 0) == u
     a.slope = d->leakySlope;
     a.accumulate = d->accumulate ? 1 : 0;
     a.batch = d->batch;
+    a.inUnsigned = combo.inUnsigned ? 1 : 0;
+    a.matUnsigned = combo.matUnsigned ? 1 : 0;
     a.inAlign = alignOf(d->input, d->inputStride);
     a.outAlign = alignOf(d->output, d->outputStride);
 
     CvResult rc;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    cv::MmaKind kind = combo->kind;
+    cv::MmaKind kind = combo.kind;
     if (kind == cv::MmaKind::Fp8AsF16 && (d->flags & CV_FLAG_FP8_MATRIX_PIPELINE)) kind = cv::MmaKind::Fp8Native;
     const hipError_t e = cv::launchMatMul((hipStream_t)stream, kind, a, cus);
     if (e == hipErrorInvalidValue)
-        return fail(CV_E_NOT_AVAILABLE, "cvMatMul: no kernel specialisation for m=%d k=%d (limits: m<=128; k<=128 fp16/fp8, k<=256 int8)", d->m, d->k);
+        return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d is beyond what one 16-row block of the matrix can keep in LDS "
+                    "(128 KiB: k <= 4096 for 16-bit types, 8192 for 8-bit ones)", d->k);
     return fromHip(e, "cvMatMul launch");
 }
 

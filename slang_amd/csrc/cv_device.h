@@ -91,6 +91,45 @@ struct Fp8AsF16Mma {
     }
 };
 
+// bfloat16 operands (the library's extension type CV_BFLOAT16)
+struct Bf16Mma {
+    static constexpr const char* kName = "bf16";
+    static constexpr int kEsz = 2, kEpl = 8, kRawDW = 4, kFD = 4;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        frag[0] = raw[0]; frag[1] = raw[1]; frag[2] = raw[2]; frag[3] = raw[3];
+    }
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+        u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), c, 0, 0, 0);
+    }
+};
+
+// OCP e5m2 in memory, decoded exactly to fp16 operands: an e5m2 value is the high byte of the
+// binary16 with the same value
+struct Bf8AsF16Mma {
+    static constexpr const char* kName = "e5m2-f16pipe";
+    static constexpr int kEsz = 1, kEpl = 8, kRawDW = 2, kFD = 4;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+        // v_perm_b32: selector 0x0c = constant 0, 0..3 = bytes of the second source
+        frag[0] = __builtin_amdgcn_perm(0u, raw[0], 0x010c000cu);
+        frag[1] = __builtin_amdgcn_perm(0u, raw[0], 0x030c020cu);
+        frag[2] = __builtin_amdgcn_perm(0u, raw[1], 0x010c000cu);
+        frag[3] = __builtin_amdgcn_perm(0u, raw[1], 0x030c020cu);
+    }
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+        return F16Mma::mma(a, b, c);
+    }
+};
+
 struct I8Mma {   // int8 x int8 -> int32
     static constexpr const char* kName = "i8";
     static constexpr int kEsz = 1, kEpl = 16, kRawDW = 4, kFD = 4;
@@ -156,9 +195,14 @@ __device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct)
     switch (ct) {
     case kF16: return (float)*(const half_t*)p;
     case kF32: return *(const float*)p;
+    case kBF16: return __builtin_bit_cast(float, (uint32_t)*(const uint16_t*)p << 16);
     }
     return 0.f;
 }
+
+// bfloat16 as a result element (conversions round to nearest even: v_cvt_pk_bf16_f32)
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 // fp32 -> OCP e4m3, saturating, round to nearest even; two values per call (bytes 0,1)
 __device__ __forceinline__ uint32_t packE4M3Sat(float a, float b)

@@ -25,11 +25,20 @@ struct MatMulArgs {
     int32_t accumulate;
     uint32_t batch;
     uint32_t inAlign, outAlign;   // largest power of two (<= 16) dividing base address and stride
+    uint32_t rowOff;              // first matrix row of the block this launch computes (set by the launcher)
+    int32_t inUnsigned, matUnsigned;   // MmaKind::I8AnySign: which side holds unsigned bytes
 };
 
-enum class MmaKind : int { F16 = 0, Fp8AsF16 = 1, Fp8Native = 2, I8 = 3 };
+enum class MmaKind : int {
+    F16 = 0, Fp8AsF16 = 1, Fp8Native = 2, I8 = 3,
+    Bf16 = 4,            // bfloat16 vectors and matrix
+    Bf8AsF16 = 5,        // e5m2 vectors and matrix, decoded to fp16 operands
+    F16VecAsE4M3 = 6,    // fp16 vectors quantised to e4m3 on load, e4m3 matrix (matMul only)
+    I8AnySign = 7        // signed/unsigned bytes on either side (matMul only)
+};
 
-// Returns hipSuccess, or hipErrorInvalidValue when no specialisation covers (m,k).
+// Returns hipSuccess, or hipErrorInvalidValue when no kernel covers (m,k): k beyond what one
+// 16-row block of the matrix can hold in LDS.
 hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& args, int numCUs);
 
 // ---- fused forward MLP --------------------------------------------------------------------

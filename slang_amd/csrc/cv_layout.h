@@ -34,7 +34,8 @@ namespace cv {
 // CoopVecComponentType values (hlsl.meta.slang:32558-32575)
 enum : int {
     kE4M3 = 0, kE5M2 = 1, kF16 = 2, kF32 = 3, kF64 = 4, kS8 = 5, kS16 = 6, kS32 = 7, kS64 = 8,
-    kS8Packed = 9, kU8 = 10, kU16 = 11, kU32 = 12, kU64 = 13, kU8Packed = 14
+    kS8Packed = 9, kU8 = 10, kU16 = 11, kU32 = 12, kU64 = 13, kU8Packed = 14,
+    kBF16 = 15          // the library's extension: bfloat16
 };
 enum : int { kRowMajor = 0, kColumnMajor = 1, kInferencingOptimal = 2, kTrainingOptimal = 3 };
 
@@ -43,7 +44,7 @@ CV_HD uint32_t elemSize(int ct)
 {
     switch (ct) {
     case kE4M3: case kE5M2: case kS8: case kU8: return 1;
-    case kF16: case kS16: case kU16: return 2;
+    case kF16: case kS16: case kU16: case kBF16: return 2;
     case kF32: case kS32: case kU32: case kS8Packed: case kU8Packed: return 4;
     case kF64: case kS64: case kU64: return 8;
     }
@@ -56,7 +57,7 @@ CV_HD uint32_t fragElemsPerLane(int ct)
     switch (ct) {
     case kS8: case kU8: return 16;                 // v_mfma_i32_16x16x64_i8
     case kE4M3: case kE5M2: return 8;              // v_mfma_f32_16x16x32_fp8_fp8
-    case kF16: case kF32: return 8;                // v_mfma_f32_16x16x32_f16
+    case kF16: case kF32: case kBF16: return 8;    // v_mfma_f32_16x16x32_f16 / _bf16
     }
     return 0;
 }
@@ -67,7 +68,7 @@ CV_HD bool layoutSupports(int ct, int layout)
     switch (layout) {
     case kRowMajor: case kColumnMajor: return true;
     case kInferencingOptimal: return fragElemsPerLane(ct) != 0;
-    case kTrainingOptimal: return ct == kF16 || ct == kF32;
+    case kTrainingOptimal: return ct == kF16 || ct == kF32 || ct == kBF16;
     }
     return false;
 }

@@ -6,14 +6,14 @@ namespace cv {
 
 hipError_t launchMatMulFp8AsF16(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
-    return a.outCt == kF32 ? dispatchShape<Fp8AsF16Mma, float>(stream, a, numCUs)
-                           : dispatchShape<Fp8AsF16Mma, half_t>(stream, a, numCUs);
+    return a.outCt == kF32 ? dispatchShape<VecAsMatrix<Fp8AsF16Mma>, float>(stream, a, numCUs)
+                           : dispatchShape<VecAsMatrix<Fp8AsF16Mma>, half_t>(stream, a, numCUs);
 }
 
 hipError_t launchMatMulFp8Native(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
-    return a.outCt == kF32 ? dispatchShape<Fp8NativeMma, float>(stream, a, numCUs)
-                           : dispatchShape<Fp8NativeMma, half_t>(stream, a, numCUs);
+    return a.outCt == kF32 ? dispatchShape<VecAsMatrix<Fp8NativeMma>, float>(stream, a, numCUs)
+                           : dispatchShape<VecAsMatrix<Fp8NativeMma>, half_t>(stream, a, numCUs);
 }
 
 } // namespace cv

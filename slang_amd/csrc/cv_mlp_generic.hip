@@ -44,17 +44,8 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
         const MlpLayerArgs& ly = a.layers[l];
         const int MT = ga.gl[l].mt, KT = ga.gl[l].kt, ROWS = 4 * MT;
         const uint32_t gs = optGS((uint32_t)ly.in);
-        uint8_t* dst = (uint8_t*)(lds + ga.gl[l].fragBase * 64 * RAW);
-        for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
-            const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
-            const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
-            const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
-            const uint32_t q = (uint32_t)(kt * EPL + s), col = g * gs + q;
-            const bool valid = row < (uint32_t)ly.out && q < gs && col < (uint32_t)ly.in;
-            const size_t off = valid ? elemOffset(ly.shape, row, col) : 0;
-            if constexpr (ESZ == 2) ((uint16_t*)dst)[e] = valid ? *(const uint16_t*)(ly.w + off) : (uint16_t)0;
-            else                    dst[e] = valid ? ly.w[off] : (uint8_t)0;
-        }
+        stageFragments<ESZ, EPL>(lds + ga.gl[l].fragBase * 64 * RAW, ly.w, ly.shape, false, MT, KT, gs,
+                                 (uint32_t)ly.out, (uint32_t)ly.in);
         for (int e = threadIdx.x; e < MT * 16; e += 256) {
             const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
             const int row = g * ROWS + 4 * t + r;

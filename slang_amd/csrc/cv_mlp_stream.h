@@ -52,25 +52,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STRE
         const MlpLayerArgs& ly = a.layers[l];
         const uint32_t gs = optGS((uint32_t)ly.in);
         uint32_t* base = ldsW + Net::fragBase(l) * 64 * RAW;
-        const bool direct = ly.shape.layout == kInferencingOptimal &&
-                            optMT(ly.shape.rows) == (uint32_t)MT && optKT(ly.shape.cols, EPL) == (uint32_t)KT;
-        if (direct) {
-            const u32x2* src = (const u32x2*)ly.w;
-            u32x2* dst = (u32x2*)base;
-            for (int i = threadIdx.x; i < MT * KT * 64 * RAW / 2; i += 256) dst[i] = src[i];
-        } else {
-            uint8_t* dst = (uint8_t*)base;
-            for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
-                const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
-                const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
-                const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
-                const uint32_t q = (uint32_t)(kt * EPL + s), col = g * gs + q;
-                const bool valid = row < (uint32_t)ly.out && q < gs && col < (uint32_t)ly.in;
-                const size_t off = valid ? elemOffset(ly.shape, row, col) : 0;
-                if constexpr (ESZ == 2) ((uint16_t*)dst)[e] = valid ? *(const uint16_t*)(ly.w + off) : (uint16_t)0;
-                else                    dst[e] = valid ? ly.w[off] : (uint8_t)0;
-            }
-        }
+        stageFragments<ESZ, EPL>(base, ly.w, ly.shape, false, MT, KT, gs, (uint32_t)ly.out, (uint32_t)ly.in);
         if constexpr (HAS_BIAS) {
             for (int e = threadIdx.x; e < MT * 16; e += 256) {
                 const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;

@@ -168,29 +168,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
         const MlpLayerArgs& ly = a.layers[l];
         const uint32_t gs = optGS((uint32_t)ly.in);
-        uint16_t* dst = (uint16_t*)(ldsW + Net::fragBase(l) * 64 * RAW);
-        for (int e = threadIdx.x; e < MT * KT * 64 * EPL; e += 256) {
-            const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
-            const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
-            const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
-            const uint32_t q = (uint32_t)(kt * EPL + s), col = g * gs + q;
-            const bool valid = row < (uint32_t)ly.out && q < gs && col < (uint32_t)ly.in;
-            dst[e] = valid ? *(const uint16_t*)(ly.w + elemOffset(ly.shape, row, col)) : (uint16_t)0;
-        }
+        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, gs,
+                               (uint32_t)ly.out, (uint32_t)ly.in);
         if constexpr (l > 0) {
             // rows of W^T are this layer's inputs (tiled like the previous layer's outputs),
             // its k axis are this layer's outputs
-            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l), ROWSI = 4 * MTI;
-            const uint32_t gso = 4u * MT;
-            uint16_t* dt = (uint16_t*)(ldsWT + Net::tFragBase(l) * 64 * RAW);
-            for (int e = threadIdx.x; e < MTI * KTO * 64 * EPL; e += 256) {
-                const int s = e % EPL, lane = (e / EPL) & 63, f = e / (EPL * 64);
-                const int kt = f % KTO, t = f / KTO, g = lane >> 4, p = lane & 15;
-                const uint32_t irow = (uint32_t)((p >> 2) * ROWSI + 4 * t + (p & 3));
-                const uint32_t q = (uint32_t)(kt * EPL + s), ocol = g * gso + q;
-                const bool valid = irow < (uint32_t)ly.in && q < gso && ocol < (uint32_t)ly.out;
-                dt[e] = valid ? *(const uint16_t*)(ly.w + elemOffset(ly.shape, ocol, irow)) : (uint16_t)0;
-            }
+            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
+            stageFragments<2, EPL>(ldsWT + Net::tFragBase(l) * 64 * RAW, ly.w, ly.shape, true, MTI, KTO, 4u * MT,
+                                   (uint32_t)ly.in, (uint32_t)ly.out);
         }
         for (int e = threadIdx.x; e < MT * 16; e += 256) {
             const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;

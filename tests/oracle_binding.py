@@ -14,7 +14,7 @@ ORACLE_DIR = os.path.join(REPO, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libcoopvec_oracle.so")
 
 # CoopVecComponentType / layout values (hlsl.meta.slang:32547-32575)
-E4M3, E5M2, F16, F32, F64, S8, S16, S32, S64, S8P, U8, U16, U32, U64, U8P = range(15)
+E4M3, E5M2, F16, F32, F64, S8, S16, S32, S64, S8P, U8, U16, U32, U64, U8P, BF16 = range(16)
 ROW, COL, INF_OPT, TRAIN_OPT = range(4)
 HALF_RNE, HALF_SLANG = 0, 1
 ACT_NONE, ACT_RELU, ACT_LEAKY = 0, 1, 2
@@ -102,14 +102,45 @@ def ref_matmul_f32(x: np.ndarray, x_ct: int, W_bytes: np.ndarray, w_ct: int, lay
 
 
 def ref_matmul_i32(x: np.ndarray, W_bytes: np.ndarray, layout: int, stride: int, M: int, K: int,
-                   bias: np.ndarray | None = None, transpose: bool = False):
+                   bias: np.ndarray | None = None, transpose: bool = False, x_ct: int = S8, w_ct: int = S8):
     B = x.shape[0]
     out = np.empty((B, M), np.int32)
-    rc = lib().cvo_ref_matmul_i32(ptr(x), x.strides[0], S8, K, ptr(W_bytes), 0, S8, layout, int(transpose),
+    rc = lib().cvo_ref_matmul_i32(ptr(x), x.strides[0], x_ct, K, ptr(W_bytes), 0, w_ct, layout, int(transpose),
                                   stride, M, ptr(bias) if bias is not None else None, 0,
                                   S32 if bias is not None else -1, B, ptr(out))
     assert rc == 0
     return out
+
+
+def slang_matmul(x: np.ndarray, x_ct: int, in_interp: int, k: int, result_ct: int, M: int, W_bytes: np.ndarray,
+                 w_ct: int, layout: int, stride: int, bias: np.ndarray | None = None, bias_ct: int = -1,
+                 half_mode: int = HALF_RNE) -> np.ndarray:
+    """The Slang fallback operator itself (cvo_slang_matmul), one call per row of x.  x holds the
+    vectors as they lie in memory (packed forms: k/4 32-bit elements per row)."""
+    res_np = {F16: np.float16, F32: np.float32, S32: np.int32, U32: np.uint32}[result_ct]
+    B, packedK = x.shape
+    out = np.zeros((B, M), res_np)
+    for b in range(B):
+        rc = lib().cvo_slang_matmul(ptr(x[b]), x_ct, packedK, in_interp, k, ptr(out[b]), result_ct, M, ptr(W_bytes), 0,
+                                    w_ct, layout, 0, stride, ptr(bias) if bias is not None else None, 0,
+                                    bias_ct if bias is not None else -1, 0, half_mode)
+        assert rc == 0
+    return out
+
+
+def bf16_bits(a: np.ndarray) -> np.ndarray:
+    """float32 -> bfloat16 bit patterns (uint16), round to nearest even."""
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def e5m2_to_f32(codes: np.ndarray) -> np.ndarray:
+    """An e5m2 value is the binary16 whose high byte it is."""
+    return (codes.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
 
 
 def make_layers(specs):
