@@ -516,8 +516,12 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
                         "layer of 4 inputs and at least two layers", who);
     } else if (mlp->inputEncoding != CV_ENCODE_NONE) {
         return fail(CV_E_INVALID_ARG, "%s: unknown inputEncoding %d", who, mlp->inputEncoding);
-    } else if (mlp->inputType != mlp->weightType) {
-        return fail(CV_E_NOT_AVAILABLE, "%s: inputType %d must equal weightType %d", who, mlp->inputType, mlp->weightType);
+    } else if (mlp->inputType != mlp->weightType &&
+               !(mlp->inputType == CV_FLOAT16 && mlp->weightType == CV_FLOAT_E4M3)) {
+        // besides vectors stored like the weights: CoopVec<half> with inputInterpretation FloatE4M3,
+        // the form the operator takes on the Slang API (hlsl.meta.slang:32954-32963)
+        return fail(CV_E_NOT_AVAILABLE, "%s: inputType %d must equal weightType %d (or be FLOAT16 for FLOAT_E4M3 weights)",
+                    who, mlp->inputType, mlp->weightType);
     }
     const uint32_t wEsz = cv::elemSize(mlp->weightType);
     for (int l = 0; l < mlp->numLayers; ++l) {
@@ -577,6 +581,7 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     a.inStride = inputStride; a.outStride = outputStride; a.batch = batch;
     a.inAlign = alignOf(input, inputStride); a.outAlign = alignOf(output, outputStride);
     a.inEncoding = encoded ? cv::kEncodeXYSquares : cv::kEncodeNone;
+    a.inHalfAsE4M3 = (mlp->inputType == CV_FLOAT16 && mlp->weightType == CV_FLOAT_E4M3) ? 1 : 0;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16

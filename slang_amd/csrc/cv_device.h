@@ -215,6 +215,20 @@ __device__ __forceinline__ uint32_t packE4M3Sat(float a, float b)
     return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
 }
 
+// four fp16 values (two packed dwords) -> four OCP e4m3 bytes, saturating at +-448, nearest even
+// (v_cvt_scalef32_pk_fp8_f16 rounds like the fp32 route for every fp16 input within the clamp)
+__device__ __forceinline__ uint32_t quantE4M3x4Sat(uint32_t h01bits, uint32_t h23bits)
+{
+    typedef short shortx2 __attribute__((ext_vector_type(2)));
+    const halfx2 lim = {(half_t)448.f, (half_t)448.f};
+    const halfx2 h01 = __builtin_elementwise_min(__builtin_elementwise_max(__builtin_bit_cast(halfx2, h01bits), -lim), lim);
+    const halfx2 h23 = __builtin_elementwise_min(__builtin_elementwise_max(__builtin_bit_cast(halfx2, h23bits), -lim), lim);
+    shortx2 r = __builtin_bit_cast(shortx2, h01);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h01, 1.0f, false);
+    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, h23, 1.0f, true);
+    return __builtin_bit_cast(uint32_t, r);
+}
+
 // The neural module's smooth activations (source/standard-modules/neural/activations.slang:88-233)
 // in fp32.  Sigmoid-like ones keep the source's branch that makes the exp() argument <= 0.
 __device__ __forceinline__ float smoothActivation(float x, int act)

@@ -60,6 +60,7 @@ struct MlpArgs {
     uint32_t batch;
     uint32_t inAlign, outAlign;
     int32_t inEncoding;     // kEncodeNone, or kEncodeXYSquares: a sample is a float2, layer 0 sees (x, y, x*x, y*y)
+    int32_t inHalfAsE4M3;   // e4m3 networks: the vectors in memory are fp16 and are quantised to e4m3 as they are loaded
 };
 enum : int { kEncodeNone = 0, kEncodeXYSquares = 1 };
 // hipErrorInvalidValue when no built-in specialisation covers the layer shapes

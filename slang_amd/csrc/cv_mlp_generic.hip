@@ -85,8 +85,14 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
                         const uint32_t q = (uint32_t)(kt * EPL + s);
                         const uint32_t col = g * gs0 + q;
                         if (q < gs0 && col < (uint32_t)in0) {
-                            if constexpr (ESZ == 2) raw[s / 2] |= (uint32_t)*(const uint16_t*)(p + 2 * col) << (16 * (s & 1));
-                            else                    raw[s / 4] |= (uint32_t)p[col] << (8 * (s & 3));
+                            if constexpr (ESZ == 2) {
+                                raw[s / 2] |= (uint32_t)*(const uint16_t*)(p + 2 * col) << (16 * (s & 1));
+                            } else if (a.inHalfAsE4M3) {   // an fp16 element, quantised to e4m3 (saturating) on the way
+                                const float v = (float)*(const half_t*)(p + 2 * col);
+                                raw[s / 4] |= (packE4M3Sat(v, 0.f) & 0xffu) << (8 * (s & 3));
+                            } else {
+                                raw[s / 4] |= (uint32_t)p[col] << (8 * (s & 3));
+                            }
                         }
                     }
                 }

@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const uint32_t gs0 = optGS((uint32_t)a.layers[0].in);
     const int colBase = (int)(g * gs0);
     const int validBytes = min((int)gs0, max(a.layers[0].in - colBase, 0)) * ESZ;
-    const int loadMode = a.inEncoding == kEncodeXYSquares ? 3
+    const int loadMode = a.inEncoding == kEncodeXYSquares ? 3 : a.inHalfAsE4M3 ? 4
                        : (validBytes == IN_DW * 4 && a.inAlign >= (IN_DW % 4 == 0 ? 16u : 8u)) ? 0
                        : ((validBytes & 3) == 0 && a.inAlign >= 4u) ? 1 : 2;
     constexpr int OROWS = 4 * Net::MTL;
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const uint32_t tileStride = gridDim.x * 4;
     uint32_t tile = blockIdx.x * 4 + wave;
     if (tile >= numTiles) return;
-    const uint8_t* inLane = a.in + (size_t)colBase * ESZ;
+    const uint8_t* inLane = a.in + (size_t)colBase * (a.inHalfAsE4M3 ? 2 : ESZ);
     uint8_t* outLane = a.out + (size_t)rowBase * 2;
     const uint32_t lastSample = a.batch - 1;
 
@@ -231,6 +231,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                 for (int i = 0; i < IN_DW; ++i) buf[j][i] = 0u;
                 if constexpr (IN_DW >= 2) {
                     if (g == 0) encodeXYSquares(a.in + (size_t)s * a.inStride, buf[j][0], buf[j][1]);
+                }
+            } else if (loadMode == 4) {
+                // fp16 vectors of an e4m3 network (CoopVec<half> with inputInterpretation FloatE4M3):
+                // eight halves become the eight e4m3 bytes of one k-tile
+                if constexpr (ESZ == 1) {
+                    const int validElems = validBytes;
+                    const bool whole = validElems == 8 * Net::KT0 && a.inAlign >= 16u;
+#pragma unroll
+                    for (int kt = 0; kt < Net::KT0; ++kt) {
+                        uint32_t h[4];
+                        if (whole) {
+                            const u32x4 v = *(const u32x4*)(p + 16 * kt);
+                            h[0] = v.x; h[1] = v.y; h[2] = v.z; h[3] = v.w;
+                        } else {
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) {
+                                const int e0 = 8 * kt + 2 * d;
+                                const uint32_t lo = e0 < validElems ? ((const uint16_t*)p)[e0] : 0u;
+                                const uint32_t hi = e0 + 1 < validElems ? ((const uint16_t*)p)[e0 + 1] : 0u;
+                                h[d] = lo | (hi << 16);
+                            }
+                        }
+                        buf[j][2 * kt] = quantE4M3x4Sat(h[0], h[1]);
+                        buf[j][2 * kt + 1] = quantE4M3x4Sat(h[2], h[3]);
+                    }
                 }
             } else if (loadMode == 0) {
                 if constexpr (IN_DW % 4 == 0) {

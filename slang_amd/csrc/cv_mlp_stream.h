@@ -246,7 +246,7 @@ bool mlpStreamEligible(const MlpArgs& a)
 {
     constexpr int ROW_BYTES = 16 * Mma::kRawDW * Net::KT0;
     const int outDim = a.layers[Net::L - 1].out;
-    if (a.inEncoding != kEncodeNone) return false;
+    if (a.inEncoding != kEncodeNone || a.inHalfAsE4M3) return false;
     for (int l = 0; l < Net::L; ++l)
         if (a.layers[l].act == kActLeakyRelu) return false;
     return a.layers[0].in * Mma::kEsz == ROW_BYTES && a.inStride == (uint64_t)ROW_BYTES &&

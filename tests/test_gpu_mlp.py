@@ -236,6 +236,28 @@ def test_e4m3_saturation_and_fp16_overflow(flags, B):
         assert bad.mean() <= 1e-3
 
 
+@pytest.mark.parametrize("dims,B", [([32, 64, 64, 8], 4096), ([32, 64, 64, 8], 77), ([20, 48, 24, 5], 300), ([64, 64, 64, 64], 1000)])
+@pytest.mark.parametrize("flags", [0, cv.FLAG_FP8_MATRIX_PIPELINE])
+def test_e4m3_network_with_fp16_vectors(dims, B, flags):
+    # CoopVec<half> + inputInterpretation FloatE4M3: the vectors are quantised (saturating, nearest
+    # even) as they are loaded, so the result is bit for bit that of the pre-quantised bytes
+    rng = np.random.default_rng(sum(dims) + B)
+    specs = make_net(rng, dims, CT.FloatE4M3, bias="none", init="half")
+    xh = (rng.standard_normal((B, dims[0])) * 0.7).astype(np.float16)
+    xh[0, :6] = [1000.0, -1000.0, 464.0, -480.0, 2.0 ** -10, -0.0]
+    xq = ob.encode_e4m3(xh.astype(np.float32))          # the oracle's quantiser
+    for layout in (ML.RowMajor, ML.InferencingOptimal):
+        layers = gpu_layers(specs, CT.FloatE4M3, layout)
+        y_bytes = cv.mlpForward(layers, to_dev(xq), weightType=CT.FloatE4M3, flags=flags)
+        y_half = cv.mlpForward(layers, to_dev(xh), weightType=CT.FloatE4M3, flags=flags)
+        assert torch.equal(y_half.view(torch.int16), y_bytes.view(torch.int16)), cv.lastKernelName()
+    # strided fp16 vectors (the element-wise load path)
+    wide = torch.zeros((B, dims[0] + 3), dtype=torch.float16, device=DEV)
+    wide[:, :dims[0]] = to_dev(xh)
+    y_str = cv.mlpForward(layers, wide[:, :dims[0]], weightType=CT.FloatE4M3, flags=flags)
+    assert torch.equal(y_str.view(torch.int16), y_bytes.view(torch.int16))
+
+
 def test_mlp_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_net(rng, [8, 16, 4], CT.Float16)
