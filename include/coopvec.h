@@ -103,6 +103,9 @@ typedef enum CvActivation {
  * keeps about 11 bits below it, so results that cancel carry an absolute error of up to
  * ~2^-12 * sum|terms|.  No effect on other types. */
 #define CV_FLAG_FP8_MATRIX_PIPELINE 1u
+/* cvMlpTrainStep[WorkspaceSize]: take the layer-by-layer step (the one that serves any layer sizes)
+ * also where a fused kernel exists.  Same rounding points; for cross-checking the two. */
+#define CV_FLAG_LAYERWISE_TRAINING 2u
 
 /* Mirrors the fields the example fills in rhi::CooperativeVectorMatrixDesc
  * (mlp-training-coopvec.cpp:204-225).  `offset` is in bytes from the buffer handed to

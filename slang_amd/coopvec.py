@@ -89,6 +89,7 @@ def componentTypeToRhi(componentType: int) -> RhiCooperativeVectorComponentType:
 
 
 FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.h
+FLAG_LAYERWISE_TRAINING = 2    # CV_FLAG_LAYERWISE_TRAINING
 
 
 class Activation(enum.IntEnum):
@@ -577,8 +578,8 @@ def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
 
 
 def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
-                              gradType: int = CoopVecComponentType.Float32) -> int:
-    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+                              gradType: int = CoopVecComponentType.Float32, flags: int = 0, inputEncoding: int = 0) -> int:
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, flags, inputEncoding)
     out = ctypes.c_size_t(0)
     _check(_lib.load().cvMlpTrainStepWorkspaceSize(ctypes.byref(d), batch, ctypes.byref(out)))
     return out.value
@@ -587,14 +588,14 @@ def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
 def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor] = None, *,
                  lossScale: float = 1.0, gradType: int = CoopVecComponentType.Float32,
                  workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None,
-                 inputEncoding: int = 0, stream=None):
+                 inputEncoding: int = 0, flags: int = 0, stream=None):
     """learnGradient over a batch (kernels.slang:9-27): forward, bwd_diff of the squared-error loss,
     weight gradients accumulated into every layer's weightsGrad (coopVecOuterProductAccumulate,
     fflayer.slang:35-41) and bias gradients into biasesGrad (coopVecReduceSumAccumulate, :44),
     deterministically.  Returns (workspace, lossSum) so that both can be reused."""
     _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
     batch = input.shape[0]
-    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0, inputEncoding)
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, flags, inputEncoding)
     lib = _lib.load()
     if workspace is None:
         need = ctypes.c_size_t(0)

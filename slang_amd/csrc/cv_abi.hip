@@ -596,7 +596,6 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
 
 CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes)
 {
-    (void)batch;
     if (!outBytes) return fail(CV_E_INVALID_ARG, "cvMlpTrainStepWorkspaceSize: outBytes is null");
     *outBytes = 0;
     cv::MlpArgs a;
@@ -604,11 +603,14 @@ CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch
     CvResult rc = fillMlpLayers("cvMlpTrainStepWorkspaceSize", mlp, a.layers);
     if (CV_FAILED(rc)) return rc;
     if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights");
+    if (mlp->numLayers < 2) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: needs at least two layers");
     a.numLayers = mlp->numLayers;
+    a.batch = batch;
+    a.inEncoding = mlp->inputEncoding == CV_ENCODE_XY_SQUARES ? cv::kEncodeXYSquares : cv::kEncodeNone;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    const size_t n = cv::trainWorkspaceBytes(a, cus);
-    if (!n) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: no fused specialisation for these layer sizes");
+    size_t n = (mlp->flags & CV_FLAG_LAYERWISE_TRAINING) ? 0 : cv::trainWorkspaceBytes(a, cus);
+    if (!n) n = cv::trainGeneralWorkspaceBytes(a, cus);   // no fused shape: the layer-by-layer step
     *outBytes = n;
     return CV_OK;
 }
@@ -674,15 +676,20 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     t.workspace = (float*)workspace;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    const size_t need = cv::trainWorkspaceBytes(t.mlp, cus);
-    if (!need) return fail(CV_E_NOT_AVAILABLE, "%s: no fused specialisation for these layer sizes", who);
+    size_t need = (mlp->flags & CV_FLAG_LAYERWISE_TRAINING) ? 0 : cv::trainWorkspaceBytes(t.mlp, cus);
+    const bool fused = need != 0;
+    if (!fused) need = cv::trainGeneralWorkspaceBytes(t.mlp, cus);   // layer by layer, any layer sizes
     if (workspaceBytes < need) {
         if (ownScratch)
             return fail(CV_E_NOT_AVAILABLE, "%s: this network needs %zu bytes of scratch, the built-in array holds %zu; "
                         "use cvMlpTrainStep with a caller-provided workspace", who, need, workspaceBytes);
         return fail(CV_E_BUFFER_TOO_SMALL, "%s: workspace of %zu bytes, %zu needed", who, workspaceBytes, need);
     }
-    return fromHip(cv::launchMlpTrain((hipStream_t)stream, t, cus), who);
+    if (fused) return fromHip(cv::launchMlpTrain((hipStream_t)stream, t, cus), who);
+    const hipError_t e = cv::launchMlpTrainGeneral((hipStream_t)stream, t, cus);
+    if (e == hipErrorInvalidValue)
+        return fail(CV_E_NOT_AVAILABLE, "%s: a layer is wider than the matMul kernels serve (k beyond 4096)", who);
+    return fromHip(e, who);
 }
 
 CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp, const void* input, size_t inputStride,

@@ -86,6 +86,10 @@ struct TrainLaunch {
 // units; 0 when no built-in specialisation covers the layer shapes.
 size_t trainWorkspaceBytes(const MlpArgs& shapes, int numCUs);
 hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCUs);
+// The same step layer by layer through the batched kernels, for any layer sizes: per-layer vectors
+// of the whole batch are parked in the workspace, whose size therefore grows with mlp.batch.
+size_t trainGeneralWorkspaceBytes(const MlpArgs& shapesAndBatch, int numCUs);
+hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& args, int numCUs);
 
 // ---- batched outer-product / reduce-sum accumulate ---------------------------------------
 struct OuterArgs {

@@ -1,0 +1,327 @@
+// cv_train_general.hip -- the training step for networks outside the fused kernel's tile shapes.
+//
+// The same computation as the fused step (the example's learnGradient, kernels.slang:9-27:
+// forward, bwd_diff of the squared-error loss, fflayer.slang:29-58), layer by layer over the
+// whole batch, with the per-layer vectors parked in the caller's workspace instead of registers:
+//
+//   forward   Z_l = W_l X_l + b_l   (batched matMulAdd kernel, fp16 result)
+//             X_{l+1} = act(Z_l)    (element-wise, half arithmetic)
+//   loss      diff = half(y - t), lossSum += diff^2, g = half(2 diff lossScale)
+//   backward  dZ_l = g * act'(Z_l)  (Slang's max rule: whole gradient to the larger operand, half
+//                                    to each at a tie, diff.meta.slang:2258-2277)
+//             db_l += sum_s dZ_l    (batched reduce-sum accumulate kernel)
+//             dW_l += sum_s dZ_l (x) X_l   (batched outer-product accumulate kernel)
+//             g = half(W_l^T dZ_l)  (batched matMul kernel on the transposed matrix)
+//
+// Every rounding point is the fused kernel's (and the oracle's); all reductions run in a fixed
+// order, so the result is bitwise reproducible.  Any layer sizes the matMul kernels serve.
+#include <cstring>
+
+#include "cv_device.h"
+#include "cv_kernels.h"
+#include "cv_error.h"
+
+namespace cv {
+
+namespace {
+
+constexpr size_t kAlign = 256;
+size_t alignUp(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+// Where each per-layer array lives in the workspace (byte offsets).
+struct GeneralPlan {
+    size_t x0;                        // encoded network input (only with an input encoding)
+    size_t z[kMaxMlpLayers];          // pre-activations, fp16 [batch][out_l]
+    size_t act[kMaxMlpLayers];        // activations (== z[l] where the layer has no activation)
+    size_t gA, gB;                    // gradient ping-pong buffers, fp16 [batch][widest layer]
+    size_t lossPartials;              // one float per workgroup of the loss kernel
+    size_t partials;                  // scratch of the accumulate kernels
+    size_t total;
+    uint32_t lossBlocks;
+};
+
+constexpr uint32_t kLossSamplesPerBlock = 1024;
+
+GeneralPlan makePlan(const MlpArgs& a, int numCUs)
+{
+    GeneralPlan p{};
+    const int L = a.numLayers;
+    const size_t batch = a.batch ? a.batch : 1;
+    size_t off = 0;
+    int widest = a.layers[0].in;
+    p.x0 = off;
+    if (a.inEncoding != kEncodeNone) off += alignUp(batch * 4 * 2);
+    for (int l = 0; l < L; ++l) {
+        const size_t bytes = alignUp(batch * (size_t)a.layers[l].out * 2);
+        p.z[l] = off; off += bytes;
+        if (a.layers[l].act == kActNone) p.act[l] = p.z[l];
+        else { p.act[l] = off; off += bytes; }
+        if (a.layers[l].out > widest) widest = a.layers[l].out;
+    }
+    const size_t gBytes = alignUp(batch * (size_t)widest * 2);
+    p.gA = off; off += gBytes;
+    p.gB = off; off += gBytes;
+    p.lossBlocks = (uint32_t)((batch + kLossSamplesPerBlock - 1) / kLossSamplesPerBlock);
+    p.lossPartials = off; off += alignUp((size_t)p.lossBlocks * sizeof(float));
+    size_t part = reduceSumWorkspaceBytes((uint32_t)batch, numCUs);
+    for (int l = 0; l < L; ++l) {
+        const size_t o = outerWorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch, numCUs);
+        if (o > part) part = o;
+    }
+    p.partials = off; off += alignUp(part);
+    p.total = off;
+    return p;
+}
+
+// ---- element-wise kernels ---------------------------------------------------------------------
+
+// float2 samples -> the example's encoded input (x, y, x*x, y*y) in half
+__global__ __launch_bounds__(256) void encodeXYKernel(const uint8_t* in, uint64_t inStride, uint32_t batch, uint32_t* x0)
+{
+    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
+    if (s >= batch) return;
+    uint32_t xy, sq;
+    encodeXYSquares(in + (size_t)s * inStride, xy, sq);
+    x0[2 * s] = xy; x0[2 * s + 1] = sq;
+}
+
+__global__ __launch_bounds__(256) void activationKernel(const half_t* z, half_t* out, size_t count, int act, float slope)
+{
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < count; i += (size_t)gridDim.x * 256u)
+        out[i] = activateHalf(z[i], act, slope);
+}
+
+// dz = g * act'(z), every product and sum rounded to half
+__device__ __forceinline__ half_t activationGrad(half_t g, half_t z, int act, float slope)
+{
+    const half_t halfG = (half_t)(0.5f * (float)g);
+    if (act == kActRelu) return z > (half_t)0 ? g : (z == (half_t)0 ? halfG : (half_t)0);
+    if (act == kActLeakyRelu) {
+        const half_t zs = (half_t)((float)z * slope);
+        half_t da, db;
+        if (z > zs) { da = g; db = (half_t)0; }
+        else if (z < zs) { da = (half_t)0; db = g; }
+        else { da = halfG; db = halfG; }
+        const half_t dbs = (half_t)((float)db * slope);
+        return (half_t)((float)da + (float)dbs);
+    }
+    return g;
+}
+
+__global__ __launch_bounds__(256) void activationGradKernel(const half_t* g, const half_t* z, half_t* dz, size_t count, int act, float slope)
+{
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < count; i += (size_t)gridDim.x * 256u)
+        dz[i] = activationGrad(g[i], z[i], act, slope);
+}
+
+struct LossArgs {
+    const half_t* y;            // network output, [batch][outDim]
+    const half_t* z;            // last layer's pre-activation
+    half_t* dz;                 // gradient at the last layer's pre-activation
+    const uint8_t* targets; uint64_t targetStride;
+    const uint8_t* in; uint64_t inStride;   // network input as the caller passed it
+    int32_t inDim, outDim, inEncoding;
+    int32_t act; float slope;
+    float lossScale;
+    uint32_t batch;
+    float* partials;
+};
+
+// One thread per sample; a workgroup's squared errors are summed in a fixed order.
+__global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
+{
+    __shared__ float red[256];
+    float loss = 0.f;
+    const uint32_t first = blockIdx.x * kLossSamplesPerBlock;
+    for (uint32_t s = first + threadIdx.x; s < min(first + kLossSamplesPerBlock, a.batch); s += 256u) {
+        const uint8_t* xin = a.in + (size_t)s * a.inStride;
+        const bool exampleLoss = !a.targets && a.inEncoding == kEncodeXYSquares;
+        half_t gt[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+        float tgtAll = 0.f;
+        if (exampleLoss) {
+            exampleGroundTruth((half_t)((const float*)xin)[0], (half_t)((const float*)xin)[1], gt);
+        } else if (!a.targets) {
+            // sin(sum of the inputs), summed quarter by quarter like the fused kernel's lane groups
+            const int gs = (int)optGS((uint32_t)a.inDim);
+            float part[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int g = 0; g < 4; ++g)
+                for (int q = 0; q < gs; ++q) {
+                    const int j = g * gs + q;
+                    if (j < a.inDim) part[g] += (float)((const half_t*)xin)[j];
+                }
+            // lane group g adds the partner groups in the order g^1, then the pair sums: (p0+p1)+(p2+p3)
+            tgtAll = (float)(half_t)sinf((part[0] + part[1]) + (part[2] + part[3]));
+        }
+        for (int i = 0; i < a.outDim; ++i) {
+            const size_t e = (size_t)s * a.outDim + i;
+            const float tv = a.targets ? (float)*(const half_t*)(a.targets + (size_t)s * a.targetStride + 2 * i)
+                                       : (exampleLoss ? (float)gt[i & 3] : tgtAll);
+            const half_t diff = (half_t)((float)a.y[e] - tv);
+            loss += (float)diff * (float)diff;
+            const half_t g = (half_t)(2.0f * (float)diff * a.lossScale);
+            a.dz[e] = activationGrad(g, a.z[e], a.act, a.slope);
+        }
+    }
+    red[threadIdx.x] = loss;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) a.partials[blockIdx.x] = red[0];
+}
+
+__global__ __launch_bounds__(64) void lossFinalKernel(const float* partials, uint32_t n, float* lossSum)
+{
+    __shared__ float red[64];
+    float c = 0.f;
+    for (uint32_t i = threadIdx.x; i < n; i += 64u) c += partials[i];
+    red[threadIdx.x] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int i = 0; i < 64; ++i) s += red[i];
+        *lossSum = s;
+    }
+}
+
+uint32_t gridFor(size_t count, int numCUs)
+{
+    const size_t need = (count + 255) / 256, cap = (size_t)numCUs * 8;
+    return (uint32_t)(need < cap ? (need ? need : 1) : cap);
+}
+
+uint32_t alignOfPtr(const void* p, uint64_t stride)
+{
+    uint32_t al = 16;
+    while (al > 1 && (((uintptr_t)p | stride) & (al - 1))) al >>= 1;
+    return al;
+}
+
+} // namespace
+
+size_t trainGeneralWorkspaceBytes(const MlpArgs& a, int numCUs)
+{
+    if (a.numLayers < 2) return 0;
+    return makePlan(a, numCUs).total;
+}
+
+hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int numCUs)
+{
+    const MlpArgs& a = t.mlp;
+    const uint32_t batch = a.batch;
+    if (batch == 0) return hipSuccess;
+    const int L = a.numLayers;
+    if (L < 2) return hipErrorInvalidValue;
+    const GeneralPlan p = makePlan(a, numCUs);
+    uint8_t* ws = (uint8_t*)t.workspace;
+    hipError_t e;
+
+    // ---- network input ------------------------------------------------------------------------
+    const uint8_t* x = a.in;
+    uint64_t xStride = a.inStride;
+    if (a.inEncoding == kEncodeXYSquares) {
+        hipLaunchKernelGGL(encodeXYKernel, dim3((batch + 255) / 256), dim3(256), 0, stream, a.in, a.inStride, batch, (uint32_t*)(ws + p.x0));
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        x = ws + p.x0; xStride = 8;
+    }
+
+    // ---- forward ------------------------------------------------------------------------------
+    const uint8_t* xl[kMaxMlpLayers];
+    uint64_t xlStride[kMaxMlpLayers];
+    for (int l = 0; l < L; ++l) {
+        const MlpLayerArgs& ly = a.layers[l];
+        xl[l] = x; xlStride[l] = xStride;
+        MatMulArgs m;
+        memset(&m, 0, sizeof(m));
+        m.in = x; m.inStride = xStride;
+        m.out = ws + p.z[l]; m.outStride = (uint64_t)ly.out * 2;
+        m.mat = ly.w; m.bias = ly.bias; m.biasCt = kF16;
+        m.shape = ly.shape; m.transpose = 0; m.m = ly.out; m.k = ly.in;
+        m.inCt = kF16; m.outCt = kF16; m.act = kActNone; m.batch = batch;
+        m.inAlign = alignOfPtr(m.in, m.inStride); m.outAlign = alignOfPtr(m.out, m.outStride);
+        if ((e = launchMatMul(stream, MmaKind::F16, m, numCUs)) != hipSuccess) return e;
+        if (ly.act != kActNone) {
+            const size_t count = (size_t)batch * ly.out;
+            hipLaunchKernelGGL(activationKernel, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                               (const half_t*)(ws + p.z[l]), (half_t*)(ws + p.act[l]), count, ly.act, ly.slope);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
+        x = ws + p.act[l]; xStride = (uint64_t)ly.out * 2;
+    }
+
+    // ---- loss and the gradient at the last pre-activation -----------------------------------------
+    {
+        const MlpLayerArgs& ly = a.layers[L - 1];
+        LossArgs la;
+        la.y = (const half_t*)(ws + p.act[L - 1]); la.z = (const half_t*)(ws + p.z[L - 1]);
+        la.dz = (half_t*)(ws + p.gA);
+        la.targets = t.targets; la.targetStride = t.targetStride;
+        la.in = a.in; la.inStride = a.inStride;
+        la.inDim = a.layers[0].in; la.outDim = ly.out; la.inEncoding = a.inEncoding;
+        la.act = ly.act; la.slope = ly.slope; la.lossScale = t.lossScale; la.batch = batch;
+        la.partials = (float*)(ws + p.lossPartials);
+        hipLaunchKernelGGL(lossGradKernel, dim3(p.lossBlocks), dim3(256), 0, stream, la);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if (t.lossSum) {
+            hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(64), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
+    }
+
+    // ---- backward -----------------------------------------------------------------------------
+    size_t dzOff = p.gA, otherOff = p.gB;
+    for (int l = L - 1; l >= 0; --l) {
+        const MlpLayerArgs& ly = a.layers[l];
+        const uint8_t* dz = ws + dzOff;
+        const uint64_t dzStride = (uint64_t)ly.out * 2;
+        if (t.bGrad[l]) {
+            for (int c0 = 0; c0 < ly.out; c0 += 256) {      // the reduce kernel takes up to 256 columns
+                const int n = ly.out - c0 < 256 ? ly.out - c0 : 256;
+                ReduceSumArgs r;
+                memset(&r, 0, sizeof(r));
+                r.v = dz + (size_t)c0 * 2; r.vStride = dzStride; r.n = n;
+                r.colsPerGroup = (((n + 3) / 4) + 1) / 2 * 2;
+                r.batch = batch; r.buf = t.bGrad[l] + (size_t)c0 * elemSize(t.gradCt); r.bufCt = t.gradCt;
+                r.partials = (float*)(ws + p.partials);
+                if ((e = launchReduceSum(stream, r, numCUs)) != hipSuccess) return e;
+            }
+        }
+        if (t.wGrad[l]) {
+            OuterArgs o;
+            memset(&o, 0, sizeof(o));
+            o.a = dz; o.aStride = dzStride; o.aAlign = alignOfPtr(o.a, o.aStride);
+            o.b = xl[l]; o.bStride = xlStride[l]; o.bAlign = alignOfPtr(o.b, o.bStride);
+            o.m = ly.out; o.n = ly.in; o.batch = batch;
+            o.mat = t.wGrad[l]; o.shape = t.gradShape[l];
+            o.partials = (float*)(ws + p.partials);
+            if ((e = launchOuterProduct(stream, o, numCUs)) != hipSuccess) return e;
+        }
+        if (l == 0) break;
+        // g = W^T dZ (rounded to half), then through the previous layer's activation
+        const MlpLayerArgs& prev = a.layers[l - 1];
+        const bool prevAct = prev.act != kActNone;
+        MatMulArgs m;
+        memset(&m, 0, sizeof(m));
+        m.in = dz; m.inStride = dzStride;
+        m.out = ws + otherOff; m.outStride = (uint64_t)ly.in * 2;
+        m.mat = ly.w; m.shape = ly.shape; m.transpose = 1; m.m = ly.in; m.k = ly.out;
+        m.inCt = kF16; m.outCt = kF16; m.act = kActNone; m.batch = batch;
+        m.inAlign = alignOfPtr(m.in, m.inStride); m.outAlign = alignOfPtr(m.out, m.outStride);
+        if ((e = launchMatMul(stream, MmaKind::F16, m, numCUs)) != hipSuccess) return e;
+        if (prevAct) {
+            // in place: element i of dz depends on element i of g only
+            const size_t count = (size_t)batch * ly.in;
+            hipLaunchKernelGGL(activationGradKernel, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                               (const half_t*)(ws + otherOff), (const half_t*)(ws + p.z[l - 1]), (half_t*)(ws + otherOff),
+                               count, prev.act, prev.slope);
+            if ((e = hipGetLastError()) != hipSuccess) return e;
+        }
+        const size_t tmp = dzOff; dzOff = otherOff; otherOff = tmp;
+    }
+    noteKernel(false, "layer-by-layer training step: matmulKernel/activationKernel (forward), lossGradKernel, "
+                      "reduceSum + outerProduct + transposed matmulKernel + activationGradKernel per layer (backward)");
+    return hipSuccess;
+}
+
+} // namespace cv

@@ -210,6 +210,70 @@ def test_train_fp16_training_optimal_gradients_and_convert():
         assert np.max(np.abs(got - rW[l])) <= 2e-3 * np.max(np.abs(rW[l])) + 1e-6
 
 
+@pytest.mark.parametrize("dims,B,act,slope", [
+    ([8, 16, 64, 4], 1500, Activation.ReLU, 0.0),           # hidden widths differ
+    ([20, 48, 24, 5], 700, Activation.ReLU, 0.0),           # the shapes of the general forward kernel's test
+    ([3, 7, 33, 2], 333, Activation.LeakyReLU, 0.25),
+    ([12, 100, 100, 9], 1000, Activation.LeakyReLU, 0.1),
+    ([64, 160, 96, 32], 900, Activation.ReLU, 0.0),         # wider than 128
+    ([8, 64, 64, 64, 64, 1], 2000, Activation.ReLU, 0.0),   # a fused shape, forced through the general step below
+])
+@pytest.mark.parametrize("grad_ct,grad_layout", [(CT.Float32, ML.RowMajor), (CT.Float16, ML.TrainingOptimal)])
+def test_general_training_step_against_oracle(dims, B, act, slope, grad_ct, grad_layout):
+    rng = np.random.default_rng(sum(dims) + B + int(grad_ct))
+    specs = make_specs(rng, dims, act=act, slope=slope)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
+    layers = build(specs, grad_ct, grad_layout)
+    fused_shape = dims == [8, 64, 64, 64, 64, 1]
+    flags = cv.FLAG_LAYERWISE_TRAINING if fused_shape else 0
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), gradType=grad_ct, flags=flags)
+    assert "layer-by-layer" in cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, grad_ct, grad_layout)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
+    tol = 1e-3 if grad_ct == CT.Float32 else 2e-3      # fp16 gradient storage rounds each element once more
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= tol, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l], rB[l]) <= tol, (l, rel_err(dB[l], rB[l]))
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # bitwise determinism
+    layers2 = build(specs, grad_ct, grad_layout)
+    cv.mlpTrainStep(layers2, to_dev(x), to_dev(t), gradType=grad_ct, flags=flags)
+    for a, b in zip(layers, layers2):
+        assert torch.equal(a.weightsGrad, b.weightsGrad) and torch.equal(a.biasesGrad, b.biasesGrad)
+    if fused_shape:
+        # the fused kernel on the same step: same rounding points, only the order of the fp32 sums differs
+        layers3 = build(specs, grad_ct, grad_layout)
+        _, loss3 = cv.mlpTrainStep(layers3, to_dev(x), to_dev(t), gradType=grad_ct)
+        assert "mlpTrainKernel" in cv.lastKernelName()
+        fW, fB = read_grads(layers3, specs, grad_ct, grad_layout)
+        for l in range(len(specs)):
+            assert rel_err(fW[l], dW[l]) <= (1e-4 if grad_ct == CT.Float32 else 1e-3)
+            assert rel_err(fB[l], dB[l]) <= (1e-4 if grad_ct == CT.Float32 else 1e-3)
+        assert abs(loss3.item() - loss.item()) <= 1e-5 * loss.item()
+
+
+def test_general_training_step_tie_rule_and_sin_target():
+    # hidden pre-activations that are exactly zero take half the gradient (Slang's max rule), also on the
+    # layer-by-layer step; targets == None selects sin(sum of the inputs)
+    rng = np.random.default_rng(31)
+    dims = [8, 16, 40, 3]
+    B = 512
+    specs = make_specs(rng, dims, bias=False)
+    specs[0]["W"][:4] = 0                                   # four hidden units of layer 0 are always exactly 0
+    x = rng.uniform(-1, 1, (B, 8)).astype(np.float16)
+    layers = build(specs)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), None)
+    assert "layer-by-layer" in cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, None, 1.0, tie_rule=True)
+    nW, nB, _ = ob.ref_mlp_train(specs, x, None, 1.0, tie_rule=False)
+    assert np.abs(rB[0][:4]).min() > 0 and np.abs(nB[0][:4]).max() == 0      # the rule matters here
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3 and rel_err(dB[l], rB[l]) <= 1e-3
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+
+
 def test_train_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_specs(rng, [8, 16, 4])
@@ -220,9 +284,11 @@ def test_train_argument_validation():
     with pytest.raises(cv.CoopVecError) as e:
         cv.mlpTrainStep(layers, x, None, workspace=torch.zeros(need - 16, dtype=torch.uint8, device=DEV))
     assert e.value.result == cv.SLANG_E_BUFFER_TOO_SMALL
+    # layer sizes outside the fused shapes take the layer-by-layer step, whose workspace grows with the batch
     specs = make_specs(rng, [8, 16, 64, 4])
-    with pytest.raises(cv.CoopVecError) as e:
-        cv.mlpTrainStepWorkspaceSize(build(specs), 10)
+    assert cv.mlpTrainStepWorkspaceSize(build(specs), 4096) > cv.mlpTrainStepWorkspaceSize(build(specs), 16) > 0
+    with pytest.raises(cv.CoopVecError) as e:      # one layer has nothing to chain
+        cv.mlpTrainStepWorkspaceSize(build(make_specs(rng, [8, 4])), 10)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
 
 
