@@ -9,9 +9,11 @@ metric is quoted on: a single fp16 coopVecMatMulAdd layer 64x64 (fp32 accumulate
 2^22 vectors, weights in InferencingOptimal layout (the layout conversion is timed separately and
 reported as `layout_conversion_us`).  Without --workload every other configuration is timed the same
 way in the same run (W warm-up steps, K timed steps, HIP events on the launch stream) and reported
-under "workloads": c1, c3, c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
-c5 (training step), op / rs (stand-alone outer-product / reduce-sum accumulate).  With --workload
-only that one runs and becomes the headline (profiling runs).  Prints ONE JSON line.
+under "workloads": c1, c2b (c2 in bfloat16), c3, c4 (e4m3 decoded to the fp16 matrix pipeline), c4n
+(fp8 matrix pipeline), c5 (training step), op / rs (stand-alone outer-product / reduce-sum
+accumulate).  With --workload only that one runs and becomes the headline (profiling runs; also
+c4h = c4 fed with fp16 vectors, c5g = c5 on the layer-by-layer step, copy = a plain device copy of
+known size for scaling the traffic counters).  Prints ONE JSON line.
 
 `roofline.achieved` = algorithmic bytes per launch / average kernel duration, the duration
 measured with HIP events on the launch stream around the timed launches.  `cpu_baseline` times
@@ -53,21 +55,22 @@ def ensure_built():
     return _lib.load()
 
 
-def workload_c2(torch, cv, steps, warmup):
-    """fp16 64x64 matMulAdd, batch 2^22, InferencingOptimal weights."""
+def workload_c2(torch, cv, steps, warmup, bf16=False):
+    """fp16 (or bfloat16) 64x64 matMulAdd, batch 2^22, InferencingOptimal weights."""
     import numpy as np
     from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML, CooperativeVectorMatrixDesc as D
     dev = "cuda"
     B, M, K = 1 << 22, 64, 64
+    ct, tdt = (CT.BFloat16, torch.bfloat16) if bf16 else (CT.Float16, torch.float16)
     g = torch.Generator(device=dev); g.manual_seed(20251)
-    x = torch.randn(B, K, device=dev, generator=g).half()
-    W = (torch.randn(M, K, device=dev, generator=g) / 8.0).half()
-    b = (torch.rand(M, device=dev, generator=g) * 0.2 - 0.1).half()
+    x = torch.randn(B, K, device=dev, generator=g).to(tdt)
+    W = (torch.randn(M, K, device=dev, generator=g) / 8.0).to(tdt)
+    b = (torch.rand(M, device=dev, generator=g) * 0.2 - 0.1).to(tdt)
     wrow = W.contiguous().view(torch.uint8).flatten()
-    size = cv.getCooperativeVectorMatrixSize(M, K, CT.Float16, ML.InferencingOptimal)
+    size = cv.getCooperativeVectorMatrixSize(M, K, ct, ML.InferencingOptimal)
     wopt = torch.empty(size, dtype=torch.uint8, device=dev)
-    dst = [D(M, K, CT.Float16, ML.InferencingOptimal, size, 0, 0)]
-    src = [D(M, K, CT.Float16, ML.RowMajor, M * K * 2, 0, K * 2)]
+    dst = [D(M, K, ct, ML.InferencingOptimal, size, 0, 0)]
+    src = [D(M, K, ct, ML.RowMajor, M * K * 2, 0, K * 2)]
     cv.convertCooperativeVectorMatrix(wopt, dst, wrow, src)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -77,11 +80,23 @@ def workload_c2(torch, cv, steps, warmup):
     e1.record(); torch.cuda.synchronize()
     conv_us = e0.elapsed_time(e1) / 20 * 1e3
     bb = b.view(torch.uint8)
-    out = torch.empty(B, M, dtype=torch.float16, device=dev)
+    out = torch.empty(B, M, dtype=tdt, device=dev)
 
     def step():
-        cv.coopVecMatMulAdd(x, CT.Float16, wopt, 0, CT.Float16, bb, 0, CT.Float16, ML.InferencingOptimal,
-                            False, 0, M=M, out=out)
+        cv.coopVecMatMulAdd(x, ct, wopt, 0, ct, bb, 0, ct, ML.InferencingOptimal, False, 0, M=M, out=out)
+
+    def cpu_baseline_bf16():
+        import oracle_binding as ob
+        n = 1 << 14
+        xs = x[:n].view(torch.int16).cpu().numpy().view(np.uint16)
+        Wn = W.view(torch.int16).cpu().numpy().view(np.uint8).ravel()
+        bn = b.view(torch.int16).cpu().numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        ob.ref_matmul_f32(xs, ob.BF16, Wn, ob.BF16, ob.ROW, 2 * K, M, K, bn, ob.BF16)
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vectors, one core; the fp32-accumulate parity oracle (the reference has no bfloat16 "
+                          "CoopVec component type, so there is no reference CPU form of this configuration)" % n}
 
     def cpu_baseline():
         import ctypes
@@ -114,12 +129,33 @@ def workload_c2(torch, cv, steps, warmup):
                 "sample": "first %d of the 2^22 vectors (%d per core); C restatement of the Slang CPU-target "
                           "fallback (fp16 accumulate, software half as gcc<12 selects), -O2" % (n, per_core)}
 
+    name = "bf16" if bf16 else "fp16"
     return dict(step=step, samples=B, alg_bytes=B * (K * 2 + M * 2), alg_flops=B * 2 * M * K,
-                bound="hbm", mfma="f16", dtype="f16",
-                config={"workload": "c2: fp16 coopVecMatMulAdd 64x64, batch 2^22, InferencingOptimal weights, "
-                                    "fp32 accumulate, fp16 out", "batch": B, "m": M, "k": K,
+                bound="hbm", mfma="f16", dtype="bf16" if bf16 else "f16",
+                config={"workload": "%s: %s coopVecMatMulAdd 64x64, batch 2^22, InferencingOptimal weights, "
+                                    "fp32 accumulate, %s out" % ("c2b" if bf16 else "c2", name, name), "batch": B, "m": M, "k": K,
                         "layout": "InferencingOptimal"},
-                extra={"layout_conversion_us": conv_us}, cpu_baseline=cpu_baseline, key="c2")
+                extra={"layout_conversion_us": conv_us}, cpu_baseline=cpu_baseline_bf16 if bf16 else cpu_baseline,
+                key="c2b" if bf16 else "c2")
+
+
+def workload_c2b(torch, cv, steps, warmup):
+    return workload_c2(torch, cv, steps, warmup, bf16=True)
+
+
+def workload_copy(torch, cv, steps, warmup):
+    """A plain device-to-device copy of 2^29 bytes (torch's copy kernel): the known-size transfer that
+    the FETCH_SIZE / WRITE_SIZE counters of the profiles are scaled by, and the box's copy ceiling."""
+    n = 1 << 29
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+
+    def step():
+        dst.copy_(src)
+
+    return dict(step=step, samples=n, alg_bytes=2 * n, alg_flops=0, bound="hbm", mfma="f16", dtype="u8",
+                config={"workload": "copy: plain device copy of 2^29 bytes (counter calibration, copy ceiling)", "bytes": n},
+                cpu_baseline=lambda: None, key="copy", kernel="torch copy kernel")
 
 
 def workload_c3(torch, cv, steps, warmup):
@@ -265,7 +301,16 @@ def workload_c4n(torch, cv, steps, warmup):
     return workload_c4(torch, cv, steps, warmup, flags=1)
 
 
-def workload_c5(torch, cv, steps, warmup):
+def workload_c4h(torch, cv, steps, warmup):
+    """c4 in the form the Slang API takes: fp16 vectors with inputInterpretation FloatE4M3 (quantised on load)."""
+    return _mlp_workload(torch, cv, [32, 64, 64, 8], 1 << 24, "fp8", 0, "c4h",
+                         "c4h: e4m3 MLP 32->64->64->8 fed with fp16 vectors (inputInterpretation FloatE4M3, quantised "
+                         "on load), ReLU, fp16 out, batch 2^24, e4m3 decoded to the fp16 matrix pipeline",
+                         lambda torch, g, B, k, dev: (torch.randn(B, k, device=dev, generator=g) * 0.5).half(),
+                         lambda fi: 0.5, with_bias=False)
+
+
+def workload_c5(torch, cv, steps, warmup, flags=0):
     """fp16 training step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, fp32 TrainingOptimal grads."""
     import numpy as np
     from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
@@ -288,11 +333,11 @@ def workload_c5(torch, cv, steps, warmup):
                                        wg, bg.view(torch.uint8), ML.TrainingOptimal, 0))
         host.append((W, bias))
     x = (torch.rand(B, dims[0], device=dev, generator=g) * 2 - 1).half()
-    ws = torch.empty(cv.mlpTrainStepWorkspaceSize(layers, B), dtype=torch.uint8, device=dev)
+    ws = torch.empty(cv.mlpTrainStepWorkspaceSize(layers, B, flags=flags), dtype=torch.uint8, device=dev)
     loss = torch.zeros(1, dtype=torch.float32, device=dev)
 
     def step():
-        cv.mlpTrainStep(layers, x, None, workspace=ws, lossSum=loss)
+        cv.mlpTrainStep(layers, x, None, workspace=ws, lossSum=loss, flags=flags)
 
     macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
     macs_dx = sum(dims[i] * dims[i + 1] for i in range(1, len(dims) - 1))
@@ -311,9 +356,15 @@ def workload_c5(torch, cv, steps, warmup):
 
     return dict(step=step, samples=B, alg_bytes=B * dims[0] * 2, alg_flops=B * 2 * (2 * macs + macs_dx),
                 bound="mfma", mfma="f16", dtype="f16",
-                config={"workload": "c5: fp16 train step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, "
-                                    "fp32 TrainingOptimal gradients, deterministic reduction", "batch": B, "layers": dims},
-                cpu_baseline=cpu_baseline, key="c5")
+                config={"workload": "%s: fp16 train step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, "
+                                    "fp32 TrainingOptimal gradients, deterministic reduction%s"
+                                    % ("c5g" if flags else "c5", ", layer-by-layer step (the one for arbitrary layer sizes)" if flags else ""),
+                        "batch": B, "layers": dims},
+                cpu_baseline=cpu_baseline, key="c5g" if flags else "c5")
+
+
+def workload_c5g(torch, cv, steps, warmup):
+    return workload_c5(torch, cv, steps, warmup, flags=cv.FLAG_LAYERWISE_TRAINING)
 
 
 def workload_op(torch, cv, steps, warmup):
@@ -395,8 +446,11 @@ def workload_rs(torch, cv, steps, warmup):
                         "batch": B, "n": N}, cpu_baseline=cpu_baseline, key="rs")
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4, "c4n": workload_c4n,
-             "c5": workload_c5, "op": workload_op, "rs": workload_rs}
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2b": workload_c2b, "c3": workload_c3, "c4": workload_c4,
+             "c4n": workload_c4n, "c5": workload_c5, "op": workload_op, "rs": workload_rs,
+             # only with --workload: variants and the counter-calibration copy
+             "c4h": workload_c4h, "c5g": workload_c5g, "copy": workload_copy}
+DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4n", "c5", "op", "rs")
 HEADLINE = "c2"
 
 
@@ -416,7 +470,7 @@ def measure(torch, w, steps, warmup, with_cpu):
     ev1.record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    kernel = _lib.load().cvGetLastKernelName().decode()
+    kernel = w.get("kernel") or _lib.load().cvGetLastKernelName().decode()
     wall_ms = (t1 - t0) * 1e3 / steps
     kern_ms = ev0.elapsed_time(ev1) / steps
     hbm = w["alg_bytes"] / (kern_ms * 1e-3) / 1e9
@@ -460,7 +514,7 @@ def main(argv=None) -> int:
         return 3
     torch.cuda.set_device(0)
     head_key = args.workload or HEADLINE
-    others = [] if args.workload else [k for k in WORKLOADS if k != HEADLINE]
+    others = [] if args.workload else list(DEFAULT_RUN)
 
     def run(key):
         w = WORKLOADS[key](torch, cv, args.steps, args.warmup)

@@ -170,12 +170,15 @@ __device__ __forceinline__ void pinHere(T& v) { asm volatile("" : "+v"(v)); }
 // ---- the example's input encoding ---------------------------------------------------------
 // MyNetwork::encodeInput (examples/mlp-training-coopvec/network.slang:35-38) on a float2 sample
 // converted to half2 (kernels.slang:19): the CoopVec<half,4> (x, y, x*x, y*y) as two packed dwords.
-__device__ __forceinline__ void encodeXYSquares(const uint8_t* sample, uint32_t& xy, uint32_t& squares)
+__device__ __forceinline__ void encodeXYSquares(float x, float y, uint32_t& xy, uint32_t& squares)
 {
-    const float x = ((const float*)sample)[0], y = ((const float*)sample)[1];
     const halfx2 h = {(half_t)x, (half_t)y};
     xy = __builtin_bit_cast(uint32_t, h);
     squares = __builtin_bit_cast(uint32_t, h * h);
+}
+__device__ __forceinline__ void encodeXYSquares(const uint8_t* sample, uint32_t& xy, uint32_t& squares)
+{
+    encodeXYSquares(((const float*)sample)[0], ((const float*)sample)[1], xy, squares);
 }
 
 // groundtruth(x, y) of the example (network.slang:67-75), every operation in half

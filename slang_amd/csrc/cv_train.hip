@@ -42,10 +42,16 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
+    // straight-line input loads: float2 samples of the example's encoding, or slices of whole aligned dwords
+    const bool xy = t.mlp.inEncoding == kEncodeXYSquares;
+    const bool dwords = !xy && t.mlp.layers[0].in % 2 == 0 && t.mlp.inAlign >= 4u;
+    const int variant = !plain || !(xy || dwords) ? 0 : xy ? 2 : 1;
     noteKernel(false, "mlpTrainKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s> + mlpTrainReduceKernel", Net::IT0, Net::KT0,
-               Net::HT, Net::L - 1, Net::MTL, plain ? "relu/none" : "runtime-act");
-    if (plain) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone>), dim3(blocks), dim3(256), 0, stream, ta);
-    else       hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1>), dim3(blocks), dim3(256), 0, stream, ta);
+               Net::HT, Net::L - 1, Net::MTL,
+               variant == 0 ? "runtime-act,any-input" : variant == 1 ? "relu/none,dword-input" : "relu/none,xy-input");
+    if (variant == 1)      hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadDwords>), dim3(blocks), dim3(256), 0, stream, ta);
+    else if (variant == 2) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadXY>), dim3(blocks), dim3(256), 0, stream, ta);
+    else                   hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     TrainReduceArgs ra;

@@ -138,10 +138,17 @@ __device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, hal
     return da + db * slope2;
 }
 
+// LOADS selects how the network input is fetched.  kLoadDwords (every lane's slice is whole, 4-byte
+// aligned dwords) and kLoadXY (float2 samples of the example's encoding) are straight-line code: every
+// lane loads from an address that is always valid and masks afterwards, so the requests of the next
+// round stay in flight during the whole current round.  kLoadAny covers everything else with
+// predicated loads, which the round has to wait for.
+enum : int { kLoadDwords = 0, kLoadAny = 1, kLoadXY = 2 };
+
 // HACT / LACT fix the activation of the hidden layers / the last layer at compile time (the round
 // then is straight-line code the scheduler can interleave); -1 reads them from the arguments and
 // keeps the leaky-ReLU arithmetic.
-template <class Net, int HACT, int LACT>
+template <class Net, int HACT, int LACT, int LOADS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlpTrainKernel(const TrainArgs ta)
 {
     typedef F16Mma Mma;
@@ -218,7 +225,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t gs0 = optGS((uint32_t)in0);
     const int colBase = (int)(g * gs0);
     const int validBytes = min((int)gs0, max(in0 - colBase, 0)) * 2;
-    const bool vecLoad = validBytes == IN_DW * 4 && a.inAlign >= 16u;
     const int outDim = a.layers[L - 1].out;
     constexpr int OROWS = 4 * Net::MTL;
 
@@ -228,29 +234,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint8_t* inLane = a.in + (size_t)colBase * 2;
     const uint32_t lastSample = a.batch - 1;
 
-    auto loadTile = [&](uint32_t (&buf)[2][IN_DW], uint32_t t) {
+    // Requests the input registers of one round.  Loads only, no arithmetic on the loaded values: the
+    // round that consumes them runs a whole round later (float2 samples of the example's encoding
+    // stay raw until then, and slices shorter than IN_DW dwords are masked then).
+    auto loadTile = [&](uint32_t (&raw)[2][IN_DW], uint32_t t) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
-            const uint8_t* p = inLane + (size_t)s * a.inStride;
-            if (a.inEncoding == kEncodeXYSquares) {
-                // a float2 sample; lane group 0 owns all four encoded inputs
+            const uint8_t* row = a.in + (size_t)s * a.inStride;
+            const uint8_t* p = row + (size_t)colBase * 2;
+            if constexpr (LOADS == kLoadXY) {
+                // a float2 sample (lane group 0 owns all four encoded inputs; the others discard it)
 #pragma unroll
-                for (int i = 0; i < IN_DW; ++i) buf[j][i] = 0u;
-                if (g == 0) encodeXYSquares(a.in + (size_t)s * a.inStride, buf[j][0], buf[j][1]);
-            } else if (vecLoad) {
+                for (int i = 0; i < IN_DW; ++i) raw[j][i] = i < 2 ? ((const uint32_t*)row)[i] : 0u;
+            } else if constexpr (LOADS == kLoadDwords) {
+                // dwords past the lane's slice are fetched from the start of the row (always valid) and masked later
 #pragma unroll
-                for (int i = 0; i < IN_DW / 4; ++i) {
-                    const u32x4 v = *(const u32x4*)(p + 16 * i);
-                    buf[j][4 * i] = v.x; buf[j][4 * i + 1] = v.y; buf[j][4 * i + 2] = v.z; buf[j][4 * i + 3] = v.w;
-                }
+                for (int i = 0; i < IN_DW; ++i) raw[j][i] = *(const uint32_t*)(4 * i < validBytes ? p + 4 * i : row);
+            } else if (a.inEncoding == kEncodeXYSquares) {
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) raw[j][i] = (i < 2 && g == 0) ? ((const uint32_t*)row)[i] : 0u;
             } else {
 #pragma unroll
                 for (int i = 0; i < IN_DW; ++i) {
                     uint32_t v = 0;
                     if (4 * i < validBytes) v = *(const uint16_t*)(p + 4 * i);
                     if (4 * i + 2 < validBytes) v |= (uint32_t)*(const uint16_t*)(p + 4 * i + 2) << 16;
-                    buf[j][i] = v;
+                    raw[j][i] = v;
                 }
             }
         }
@@ -267,7 +277,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         frag[3] = __builtin_bit_cast(uint32_t, __builtin_convertvector(floatx2{t1[2], t1[3]}, halfx2));
     };
 
-    auto round = [&](const uint32_t (&buf)[2][IN_DW], uint32_t t0) {
+    auto round = [&](const uint32_t (&raw)[2][IN_DW], uint32_t t0) {
+        uint32_t buf[2][IN_DW];                     // the network input as layer 0 sees it
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int d = 0; d < IN_DW; ++d) {
+                if constexpr (LOADS == kLoadDwords) buf[j][d] = 4 * d < validBytes ? raw[j][d] : 0u;
+                else if constexpr (LOADS == kLoadXY) buf[j][d] = 0u;
+                else buf[j][d] = raw[j][d];
+            }
+            if ((LOADS == kLoadXY || a.inEncoding == kEncodeXYSquares) && g == 0)
+                encodeXYSquares(__builtin_bit_cast(float, raw[j][0]), __builtin_bit_cast(float, raw[j][1]), buf[j][0], buf[j][1]);
+        }
         uint32_t actS[2][Net::KTMAX][FD];           // S fragments of the current layer's input
         uint32_t mst[L][2][Net::MTMAX];             // max() gradient multipliers, four e4m3 bytes per out tile
         halfx2 yS[2][Net::MTL][2];                  // network output (carrier), tile j, out tile t
@@ -555,11 +577,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             for (; tile < numTiles; tile += tileStride) {
                 const uint32_t t1 = tile + tileStride;
                 loadTile(nxt, t1 < numTiles ? t1 : tile);
+                // the requests stay above the round (a load may not move across this point) ...
+                asm volatile("" ::: "memory");
                 round(cur, tile);
+                // ... and their results are first touched below it
 #pragma unroll
                 for (int j = 0; j < 2; ++j)
 #pragma unroll
-                    for (int d = 0; d < IN_DW; ++d) cur[j][d] = nxt[j][d];
+                    for (int d = 0; d < IN_DW; ++d) { pinHere(nxt[j][d]); cur[j][d] = nxt[j][d]; }
             }
         }
     }

@@ -37,11 +37,21 @@ def test_no_alloc_matches_workspace_entry_point(dims):
         assert ref_loss.item() == got_loss.item()
 
 
-def test_no_alloc_validates_like_the_workspace_entry_point():
+def test_no_alloc_on_the_layer_by_layer_step_and_its_limit():
+    # layer sizes without a fused kernel take the layer-by-layer step, whose scratch grows with the batch:
+    # a small batch fits the built-in array (same result as cvMlpTrainStep, bit for bit), a large one does not
     rng = np.random.default_rng(1)
-    layers = build(make_specs(rng, [8, 16, 64, 4]))      # no fused specialisation: same error as cvMlpTrainStep
-    x = torch.zeros(10, 8, dtype=torch.float16, device=DEV)
+    specs = make_specs(rng, [8, 16, 64, 4])
+    x = to_dev(rng.uniform(-1, 1, (300, 8)).astype(np.float16))
+    ref_layers, layers = build(specs), build(specs)
+    _, ref_loss = cv.mlpTrainStep(ref_layers, x, None)
     loss = torch.zeros(1, dtype=torch.float32, device=DEV)
+    cv.mlpTrainStepNoAlloc(layers, x, None, loss)
+    for r, g in zip(ref_layers, layers):
+        assert torch.equal(r.weightsGrad, g.weightsGrad) and torch.equal(r.biasesGrad, g.biasesGrad)
+    assert ref_loss.item() == loss.item()
+    big = torch.zeros(1 << 17, 8, dtype=torch.float16, device=DEV)
+    assert cv.mlpTrainStepWorkspaceSize(layers, big.shape[0]) > cv.NOALLOC_SCRATCH_BYTES
     with pytest.raises(cv.CoopVecError) as e:
-        cv.mlpTrainStepNoAlloc(layers, x, None, loss)
+        cv.mlpTrainStepNoAlloc(layers, big, None, loss)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
