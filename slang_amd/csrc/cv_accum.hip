@@ -142,32 +142,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void o
         }
 }
 
-// A workgroup owns 64 consecutive values of one block's partial; its four waves each sum a quarter
-// of the partials (eight loads in flight per lane) and wave 0 adds the four sums in a fixed order.
-__global__ __launch_bounds__(256) void outerReduceKernel(const OuterArgs a, uint32_t numPartials)
+// A workgroup owns 64 consecutive values of one block's partial (see sumPartials).
+__global__ __launch_bounds__(64 * kReduceWaves) void outerReduceKernel(const OuterArgs a, uint32_t numPartials)
 {
-    __shared__ float red[4 * 64];
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t p = blockIdx.x * 64u + lane;                  // index inside one block's partial
-    {
-        const uint32_t per = (numPartials + 3u) / 4u;
-        const uint32_t b0 = wave * per, b1 = min(b0 + per, numPartials);
-        const float* src = a.partials + (size_t)blockIdx.y * numPartials * kOuterPartialFloats + p;
-        float c = 0.f;
-        uint32_t b = b0;
-        for (; b + 8 <= b1; b += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(b + u) * kOuterPartialFloats];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) c += v[u];
-        }
-        for (; b < b1; ++b) c += src[(size_t)b * kOuterPartialFloats];
-        red[wave * 64 + lane] = c;
-    }
-    __syncthreads();
-    if (wave != 0) return;
-    const float s = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
+    __shared__ float red[kReduceWaves * 64];
+    const uint32_t p = blockIdx.x * 64u + (threadIdx.x & 63u);   // index inside one block's partial
+    float s;
+    if (!sumPartials(a.partials + (size_t)blockIdx.y * numPartials * kOuterPartialFloats + p, kOuterPartialFloats,
+                     numPartials, true, red, s)) return;
     const int nbx = (a.n + kBlk - 1) / kBlk;
     const int by = blockIdx.y / nbx, bx = blockIdx.y % nbx;
     const uint32_t tile = p >> 8, ln = (p >> 2) & 63u, r = p & 3u;
@@ -209,17 +191,18 @@ __global__ __launch_bounds__(256) void reduceSumKernel(const ReduceSumArgs a)
     float* part = a.partials + (size_t)blockIdx.x * kMaxReduceCols;
 #pragma unroll
     for (int i = 0; i < 64; ++i) {
-        if (i >= cpl) break;
-        ldsRed[wave * 64 + lane] = acc[i];
-        __syncthreads();
-        if (threadIdx.x < 4) {
-            float s = 0.f;
-            for (int w = 0; w < 4; ++w)
-                for (int k = 0; k < 16; ++k) s += ldsRed[w * 64 + threadIdx.x * 16 + k];
-            const int col = threadIdx.x * cpl + i;
-            if (col < a.n) part[col] = s;
+        if (i < cpl) {      // uniform; every acc[] index stays a compile-time constant
+            ldsRed[wave * 64 + lane] = acc[i];
+            __syncthreads();
+            if (threadIdx.x < 4) {
+                float s = 0.f;
+                for (int w = 0; w < 4; ++w)
+                    for (int k = 0; k < 16; ++k) s += ldsRed[w * 64 + threadIdx.x * 16 + k];
+                const int col = threadIdx.x * cpl + i;
+                if (col < a.n) part[col] = s;
+            }
+            __syncthreads();
         }
-        __syncthreads();
     }
 }
 
@@ -273,34 +256,14 @@ __global__ __launch_bounds__(256) void reduceSumStreamKernel(const ReduceSumArgs
     }
 }
 
-// 64 columns per workgroup; its four waves each sum a quarter of the partials, wave 0 combines.
-__global__ __launch_bounds__(256) void reduceSumFinalKernel(const ReduceSumArgs a, uint32_t numPartials)
+// 64 columns per workgroup (see sumPartials).
+__global__ __launch_bounds__(64 * kReduceWaves) void reduceSumFinalKernel(const ReduceSumArgs a, uint32_t numPartials)
 {
-    __shared__ float red[4 * 64];
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t col = blockIdx.x * 64u + lane;
+    __shared__ float red[kReduceWaves * 64];
+    const uint32_t col = blockIdx.x * 64u + (threadIdx.x & 63u);
     const bool inRange = col < (uint32_t)a.n;
-    {
-        const uint32_t per = (numPartials + 3u) / 4u;
-        const uint32_t b0 = wave * per, b1 = min(b0 + per, numPartials);
-        float c = 0.f;
-        if (inRange) {
-            const float* src = a.partials + col;
-            uint32_t b = b0;
-            for (; b + 8 <= b1; b += 8) {
-                float v[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(b + u) * kMaxReduceCols];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) c += v[u];
-            }
-            for (; b < b1; ++b) c += src[(size_t)b * kMaxReduceCols];
-        }
-        red[wave * 64 + lane] = c;
-    }
-    __syncthreads();
-    if (wave != 0 || !inRange) return;
-    const float s = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
+    float s;
+    if (!sumPartials(a.partials + col, kMaxReduceCols, numPartials, inRange, red, s) || !inRange) return;
     if (a.bufCt == kF32) ((float*)a.buf)[col] += s;
     else ((half_t*)a.buf)[col] = (half_t)((float)((half_t*)a.buf)[col] + s);
 }
@@ -338,7 +301,7 @@ hipError_t launchOuterProduct(hipStream_t stream, const OuterArgs& a, int numCUs
     hipLaunchKernelGGL(outerProductKernel, dim3(gx, blocks), dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(outerReduceKernel, dim3(kOuterPartialFloats / 64, blocks), dim3(256), 0, stream, a, gx);
+    hipLaunchKernelGGL(outerReduceKernel, dim3(kOuterPartialFloats / 64, blocks), dim3(64 * kReduceWaves), 0, stream, a, gx);
     return hipGetLastError();
 }
 
@@ -366,7 +329,7 @@ hipError_t launchReduceSum(hipStream_t stream, const ReduceSumArgs& a, int numCU
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(reduceSumFinalKernel, dim3((a.n + 63) / 64), dim3(256), 0, stream, a, gx);
+    hipLaunchKernelGGL(reduceSumFinalKernel, dim3((a.n + 63) / 64), dim3(64 * kReduceWaves), 0, stream, a, gx);
     return hipGetLastError();
 }
 

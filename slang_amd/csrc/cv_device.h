@@ -191,6 +191,41 @@ __device__ __forceinline__ void exampleGroundTruth(half_t x, half_t y, half_t (&
     gt[3] = (half_t)(x + (half_t)((half_t)(hlf * y) * y));
 }
 
+// ---- final sum over per-workgroup partials ---------------------------------------------------
+// Used by the second-stage kernels of the deterministic reductions.  A workgroup of kReduceWaves
+// waves owns 64 consecutive values; every wave sums a contiguous share of the partials of the
+// calling lane's value (src[b * stride], b < numPartials) with sixteen independent loads in
+// flight, then wave 0 adds the wave sums in a fixed order.  Returns true in the lanes of wave 0
+// (with the total); all threads of the workgroup must call it.
+constexpr int kReduceWaves = 16;
+__device__ __forceinline__ bool sumPartials(const float* src, size_t stride, uint32_t numPartials, bool inRange,
+                                            float* red /* shared, kReduceWaves * 64 floats */, float& total)
+{
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t per = (numPartials + kReduceWaves - 1u) / kReduceWaves;
+    const uint32_t b0 = min(wave * per, numPartials), b1 = min(b0 + per, numPartials);
+    float c = 0.f;
+    if (inRange) {
+        uint32_t b = b0;
+        for (; b + 16 <= b1; b += 16) {
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = src[(size_t)(b + u) * stride];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) c += v[u];
+        }
+        for (; b < b1; ++b) c += src[(size_t)b * stride];
+    }
+    red[wave * 64 + lane] = c;
+    __syncthreads();
+    if (wave != 0) return false;
+    float s = red[lane];
+#pragma unroll
+    for (int w = 1; w < kReduceWaves; ++w) s += red[w * 64 + lane];
+    total = s;
+    return true;
+}
+
 // ---- scalar helpers ---------------------------------------------------------------------
 
 __device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct)

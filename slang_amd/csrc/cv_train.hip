@@ -68,7 +68,7 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ra.numPartials = blocks;
     ra.lossSum = t.lossSum;
     constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
-    hipLaunchKernelGGL((mlpTrainReduceKernel<Net>), dim3((total + 63) / 64), dim3(256), 0, stream, ra);
+    hipLaunchKernelGGL((mlpTrainReduceKernel<Net>), dim3((total + 63) / 64), dim3(64 * kReduceWaves), 0, stream, ra);
     return hipGetLastError();
 }
 

@@ -85,10 +85,19 @@ __global__ __launch_bounds__(256) void encodeXYKernel(const uint8_t* in, uint64_
     x0[2 * s] = xy; x0[2 * s + 1] = sq;
 }
 
+// eight halves per thread and step where the arrays allow it (16-byte accesses), the rest one by one
 __global__ __launch_bounds__(256) void activationKernel(const half_t* z, half_t* out, size_t count, int act, float slope)
 {
-    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < count; i += (size_t)gridDim.x * 256u)
-        out[i] = activateHalf(z[i], act, slope);
+    const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x, nthreads = (size_t)gridDim.x * 256u;
+    const size_t chunks = count / 8;
+    for (size_t c = tid; c < chunks; c += nthreads) {
+        const halfx8 v = ((const halfx8*)z)[c];
+        halfx8 r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = activateHalf(v[i], act, slope);
+        ((halfx8*)out)[c] = r;
+    }
+    for (size_t i = chunks * 8 + tid; i < count; i += nthreads) out[i] = activateHalf(z[i], act, slope);
 }
 
 // dz = g * act'(z), every product and sum rounded to half
@@ -110,8 +119,16 @@ __device__ __forceinline__ half_t activationGrad(half_t g, half_t z, int act, fl
 
 __global__ __launch_bounds__(256) void activationGradKernel(const half_t* g, const half_t* z, half_t* dz, size_t count, int act, float slope)
 {
-    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < count; i += (size_t)gridDim.x * 256u)
-        dz[i] = activationGrad(g[i], z[i], act, slope);
+    const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x, nthreads = (size_t)gridDim.x * 256u;
+    const size_t chunks = count / 8;
+    for (size_t c = tid; c < chunks; c += nthreads) {
+        const halfx8 gv = ((const halfx8*)g)[c], zv = ((const halfx8*)z)[c];
+        halfx8 r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = activationGrad(gv[i], zv[i], act, slope);
+        ((halfx8*)dz)[c] = r;
+    }
+    for (size_t i = chunks * 8 + tid; i < count; i += nthreads) dz[i] = activationGrad(g[i], z[i], act, slope);
 }
 
 struct LossArgs {
@@ -187,7 +204,7 @@ __global__ __launch_bounds__(64) void lossFinalKernel(const float* partials, uin
 
 uint32_t gridFor(size_t count, int numCUs)
 {
-    const size_t need = (count + 255) / 256, cap = (size_t)numCUs * 8;
+    const size_t need = (count / 8 + 255) / 256, cap = (size_t)numCUs * 8;
     return (uint32_t)(need < cap ? (need ? need : 1) : cap);
 }
 

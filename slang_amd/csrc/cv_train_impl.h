@@ -626,37 +626,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
 // Sums the workgroup partials in a fixed order and adds them to the gradient buffers.
 template <class Net>
-__global__ __launch_bounds__(256) void mlpTrainReduceKernel(const TrainReduceArgs ra)
+__global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const TrainReduceArgs ra)
 {
-    // A workgroup owns 64 consecutive values; its four waves each sum a quarter of the partials
-    // (eight independent loads in flight per lane), and wave 0 adds the four sums in a fixed order.
+    // a workgroup owns 64 consecutive values of the partial (see sumPartials)
     constexpr int L = Net::L;
-    __shared__ float red[4 * 64];
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    const uint32_t p = blockIdx.x * 64u + lane;
+    __shared__ float red[kReduceWaves * 64];
+    const uint32_t p = blockIdx.x * 64u + (threadIdx.x & 63u);
     constexpr uint32_t nW = Net::totalGradTiles * 256, nB = Net::totalDbTiles * 16;
     const bool inRange = p < nW + nB + 1;
-    {
-        const uint32_t per = (ra.numPartials + 3u) / 4u;
-        const uint32_t b0 = wave * per, b1 = min(b0 + per, ra.numPartials);
-        float c = 0.f;
-        if (inRange) {
-            const float* src = ra.partials + p;
-            uint32_t b = b0;
-            for (; b + 8 <= b1; b += 8) {
-                float v[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) v[u] = src[(size_t)(b + u) * Net::partialFloats];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) c += v[u];
-            }
-            for (; b < b1; ++b) c += src[(size_t)b * Net::partialFloats];
-        }
-        red[wave * 64 + lane] = c;
-    }
-    __syncthreads();
-    if (wave != 0 || !inRange) return;
-    const float s = ((red[lane] + red[64 + lane]) + red[128 + lane]) + red[192 + lane];
+    float s;
+    if (!sumPartials(ra.partials + p, Net::partialFloats, ra.numPartials, inRange, red, s) || !inRange) return;
     if (p == nW + nB) {
         if (ra.lossSum) *ra.lossSum = s;
         return;
