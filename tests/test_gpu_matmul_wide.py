@@ -240,6 +240,30 @@ def test_e4m3_large_shape_and_limit():
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
 
 
+def test_non_finite_inputs_stay_within_their_sample():
+    # every sample is a column of the matrix-core product: an Inf or NaN element changes that sample's
+    # outputs only, and there it yields what the scalar definition yields (w * Inf, 0 * Inf = NaN, NaN)
+    rng = np.random.default_rng(12)
+    B, M, K = 300, 48, 64
+    x = fp16_inputs(rng, B, K)
+    W = fp16_weights(rng, M, K)
+    W[7, 3] = 0.0                                           # 0 * Inf
+    clean = cv.coopVecMatMul(to_dev(x), CT.Float16, as_bytes(to_dev(W)), 0, CT.Float16, ML.RowMajor, False, 2 * K, M=M,
+                             resultType=CT.Float32).cpu().numpy()
+    xb = x.copy()
+    xb[5, 3] = np.inf
+    xb[9, 0] = np.nan
+    xb[200, 63] = -np.inf
+    got = cv.coopVecMatMul(to_dev(xb), CT.Float16, as_bytes(to_dev(W)), 0, CT.Float16, ML.RowMajor, False, 2 * K, M=M,
+                           resultType=CT.Float32).cpu().numpy()
+    touched = np.zeros(B, bool); touched[[5, 9, 200]] = True
+    assert np.array_equal(got[~touched], clean[~touched])
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = xb[touched].astype(np.float32) @ W.astype(np.float32).T
+    assert np.array_equal(np.isnan(got[touched]), np.isnan(want))
+    assert np.array_equal(got[touched][~np.isnan(want)], want[~np.isnan(want)])      # +-inf where the definition says so
+
+
 def test_query_lists_what_matmul_accepts():
     combos = cv.querySupportedCombinations()
     keys = {(c["inputType"], c["inputInterpretation"], c["matrixInterpretation"], c["resultType"]) for c in combos}
