@@ -1,5 +1,6 @@
 // cv_train.hip -- instantiations and launcher of the fused fp16 training step.
 #include "cv_train_impl.h"
+#include "cv_train_pair.h"
 #include "cv_error.h"
 
 namespace cv {
@@ -49,9 +50,19 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     noteKernel(false, "mlpTrainKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s> + mlpTrainReduceKernel", Net::IT0, Net::KT0,
                Net::HT, Net::L - 1, Net::MTL,
                variant == 0 ? "runtime-act,any-input" : variant == 1 ? "relu/none,dword-input" : "relu/none,xy-input");
-    if (variant == 1)      hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadDwords>), dim3(blocks), dim3(256), 0, stream, ta);
-    else if (variant == 2) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadXY>), dim3(blocks), dim3(256), 0, stream, ta);
-    else                   hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
+    // 64-wide networks with the plain activations run on the two-waves-per-SIMD kernel
+    constexpr bool kPair = Net::HT == 4;
+    if constexpr (kPair) {
+        if (variant != 0)
+            noteKernel(false, "mlpTrainPairKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,relu/none,%s> + mlpTrainReduceKernel", Net::IT0,
+                       Net::KT0, Net::HT, Net::L - 1, Net::MTL, variant == 1 ? "dword-input" : "xy-input");
+        if (variant == 1)      hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords>), dim3(blocks), dim3(512), 0, stream, ta);
+        else if (variant == 2) hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadXY>), dim3(blocks), dim3(512), 0, stream, ta);
+    } else {
+        if (variant == 1)      hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadDwords>), dim3(blocks), dim3(256), 0, stream, ta);
+        else if (variant == 2) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadXY>), dim3(blocks), dim3(256), 0, stream, ta);
+    }
+    if (variant == 0) hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     TrainReduceArgs ra;

@@ -1,0 +1,430 @@
+// cv_train_pair.h -- the fused training step with two waves per SIMD.
+//
+// Same computation and rounding points as mlpTrainKernel (cv_train_impl.h), reorganised so that
+// the dW accumulators of the network are shared by a pair of waves instead of living in one:
+//
+//   - a workgroup is four pairs of waves; a pair takes rounds of 32 samples, wave 0 of the pair
+//     the first 16, wave 1 the other 16.  Forward, loss and dX = W^T dY run per wave on its 16
+//     samples exactly as in the one-wave kernel ("S" orientation: lane%16 = sample);
+//   - every layer input X_l and every dZ_l is also written to LDS as it is produced, as
+//     [32 samples][16 features] tiles of fp16.  The weight gradient dW_l = sum_s dZ_l (x) X_l
+//     needs both with the sample index on the MFMA k axis ("F" orientation: lane%16 = feature):
+//     ds_read_b64_tr_b16 delivers that transposition directly from those tiles (no
+//     selection-matrix MFMAs, no conversions);
+//   - each wave of the pair accumulates half of the dW tiles of every layer over all 32 samples
+//     of the round (its own 16 and its partner's), so a wave holds half of the accumulators
+//     (112 instead of 224 registers for 8-64-64-64-64-1) and two waves fit on a SIMD: the one
+//     covers the other's LDS and MFMA latencies.
+//
+// The waves of a workgroup meet at a barrier once per layer in the backward pass (dZ_l of both
+// halves must be in LDS before either wave contracts over it) and once per round.  Every wave
+// runs the same number of rounds (rounds past the end of the batch are run with all samples
+// masked), so the barriers always match.  Partials and their second-stage reduction are those of
+// the one-wave kernel (mlpTrainReduceKernel): same layout, fixed order, no atomics.
+#pragma once
+#include "cv_train_impl.h"
+
+namespace cv {
+namespace {
+
+// which dW tiles of layer l a wave of parity `par` accumulates
+template <class Net>
+struct PairSplit {
+    static constexpr int L = Net::L;
+    static constexpr bool byOut(int l) { return Net::mt(l) >= 2; }                       // split the out tiles
+    static constexpr bool byIn(int l) { return Net::mt(l) < 2 && Net::nIt(l) >= 2; }      // else split the in tiles
+    static constexpr bool single(int l) { return Net::mt(l) < 2 && Net::nIt(l) < 2; }     // else wave 0 alone
+    static constexpr int ownedOut(int l) { return byOut(l) ? Net::mt(l) / 2 : 1; }
+    static constexpr int ownedIn(int l) { return byIn(l) ? Net::nIt(l) / 2 : Net::nIt(l); }
+    static constexpr int locTiles(int l) { return ownedOut(l) * ownedIn(l); }
+    static constexpr int locBase(int l)
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += locTiles(i);
+        return b;
+    }
+    static constexpr int totalLoc = locBase(L);
+    static constexpr int locDbBase(int l)
+    {
+        int b = 0;
+        for (int i = 0; i < l; ++i) b += ownedOut(i);
+        return b;
+    }
+    static constexpr int totalLocDb = locDbBase(L);
+};
+
+// LDS tile of one 16-feature group over the 32 samples of a round, 1 KB, in 8-byte chunks of four
+// features: chunk c (features 4c..4c+3) of sample s sits at chunk index c*32 + (s ^ 4c).  With that
+// swizzle both access patterns are free of bank conflicts: a 16-lane group writes one chunk column
+// of 16 samples (16 consecutive chunks), and reads, transposed, the four chunks of four consecutive
+// samples (chunk indices 4((j^c)%4) + r modulo 16, all different).
+constexpr int kPairTileDW = 256;
+__device__ __forceinline__ int pairChunkDW(int sample, int c) { return (c * 32 + (sample ^ (4 * c))) * 2; }
+
+// Transposed read of one F fragment (feature = lane%16, k-slots = 8 samples) from such a tile.
+// Lane 16g+i receives feature i of samples 4g..4g+3 (first instruction) and 16+4g..16+4g+3 (second):
+// within a 16-lane group, lane q hands in the address of the 8-byte chunk (sample 4g + q/4, features
+// 4(q%4)..), and the instruction returns to lane i element r = half i%4 of the chunk of lane 4r + i/4.
+__device__ __forceinline__ void readF(const uint32_t* tile, int g, int n, uint32_t* frag)
+{
+    typedef short shortx4 __attribute__((ext_vector_type(4)));
+    typedef shortx4 __attribute__((address_space(3))) * LdsPtr;
+    const uint32_t* p0 = tile + pairChunkDW(4 * g + (n >> 2), n & 3);
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)p0);
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p0 + 32));      // samples + 16
+    const u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
+    frag[0] = a.x; frag[1] = a.y; frag[2] = b.x; frag[3] = b.y;
+}
+
+// ReLU on the hidden layers, none on the last one (the launcher sends everything else to the
+// one-wave kernel); LOADS as in mlpTrainKernel.
+template <class Net, int LOADS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlpTrainPairKernel(const TrainArgs ta)
+{
+    typedef F16Mma Mma;
+    typedef PairSplit<Net> Split;
+    constexpr int L = Net::L;
+    constexpr int FD = 4, RAW = 4, EPL = 8;
+    constexpr int IN_DW = RAW * Net::KT0;
+    const MlpArgs& a = ta.mlp;
+
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[Net::totalFrags * 64 * RAW];
+    __shared__ __attribute__((aligned(16))) uint32_t ldsWT[(Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW];
+    __shared__ __attribute__((aligned(16))) float ldsB[Net::totalBiasTiles * 16];
+    // per pair: every layer's input of the round, and two alternating slots for dZ
+    __shared__ __attribute__((aligned(16))) uint32_t ldsX[4 * Net::totalXTiles * kPairTileDW];
+    __shared__ __attribute__((aligned(16))) uint32_t ldsDZ[4 * 2 * Net::MTMAX * kPairTileDW];
+    static_assert(4 * Net::totalXTiles * kPairTileDW >= 8 * 256, "the final reduction reuses ldsX");
+
+    // ---- stage W, W^T and biases ----------------------------------------------------------------
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
+        const MlpLayerArgs& ly = a.layers[l];
+        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, optGS((uint32_t)ly.in),
+                               (uint32_t)ly.out, (uint32_t)ly.in);
+        if constexpr (l > 0) {
+            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
+            stageFragments<2, EPL>(ldsWT + Net::tFragBase(l) * 64 * RAW, ly.w, ly.shape, true, MTI, KTO, 4u * MT,
+                                   (uint32_t)ly.in, (uint32_t)ly.out);
+        }
+        for (int e = threadIdx.x; e < MT * 16; e += blockDim.x) {
+            const int t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
+            const int row = gg * ROWS + 4 * t + r;
+            float v = 0.f;
+            if (ly.bias && row < ly.out) v = (float)((const half_t*)ly.bias)[row];
+            ldsB[(Net::biasBase(l) + t) * 16 + 4 * gg + r] = v;
+        }
+    });
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pair = wave >> 1, par = wave & 1;
+    const int g = lane >> 4, n = lane & 15;
+    const halfx2 ones2 = {(half_t)1.f, (half_t)1.f};
+
+    floatx4 accW[Split::totalLoc];
+    float accB[Split::totalLocDb];
+#pragma unroll
+    for (int i = 0; i < Split::totalLoc; ++i) accW[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < Split::totalLocDb; ++i) accB[i] = 0.f;
+    float lossAcc = 0.f;
+
+    // ---- per-lane constants ----------------------------------------------------------------------
+    const int in0 = a.layers[0].in;
+    const uint32_t gs0 = optGS((uint32_t)in0);
+    const int colBase = (int)(g * gs0);
+    const int validBytes = min((int)gs0, max(in0 - colBase, 0)) * 2;
+    const int outDim = a.layers[L - 1].out;
+    constexpr int OROWS = 4 * Net::MTL;
+
+    const uint32_t numRounds = (a.batch + 31u) / 32u;
+    const uint32_t roundsPerPair = (numRounds + gridDim.x * 4u - 1u) / (gridDim.x * 4u);   // the same for every wave
+    const uint32_t lastSample = a.batch - 1;
+    uint32_t* myX = ldsX + pair * (Net::totalXTiles * kPairTileDW);
+    uint32_t* myDZ = ldsDZ + pair * (2 * Net::MTMAX * kPairTileDW);
+    // where this lane puts its four halves of a tile (S fragment half: sample 16*par+n, rows 4g..4g+3) ...
+    const int putDW = pairChunkDW(16 * par + n, g);
+
+    auto loadTile = [&](uint32_t (&raw)[IN_DW], uint32_t r) {
+        const uint32_t s = min(r * 32u + 16u * par + n, lastSample);
+        const uint8_t* row = a.in + (size_t)s * a.inStride;
+        const uint8_t* p = row + (size_t)colBase * 2;
+        if constexpr (LOADS == kLoadXY) {
+#pragma unroll
+            for (int i = 0; i < IN_DW; ++i) raw[i] = i < 2 ? ((const uint32_t*)row)[i] : 0u;
+        } else {
+#pragma unroll
+            for (int i = 0; i < IN_DW; ++i) raw[i] = *(const uint32_t*)(4 * i < validBytes ? p + 4 * i : row);
+        }
+    };
+
+    // one S fragment (8 k-slots) -> the two tiles it belongs to
+    auto putS = [&](uint32_t* tiles, int e0, int tilesInLayer, const uint32_t* frag) {
+        *(u32x2*)(tiles + e0 * kPairTileDW + putDW) = u32x2{frag[0], frag[1]};
+        if (e0 + 1 < tilesInLayer) *(u32x2*)(tiles + (e0 + 1) * kPairTileDW + putDW) = u32x2{frag[2], frag[3]};
+    };
+
+    auto round = [&](const uint32_t (&raw)[IN_DW], uint32_t r) {
+        const uint32_t sample = r * 32u + 16u * par + n;
+        const bool live = sample < a.batch;
+        uint32_t buf[IN_DW];
+#pragma unroll
+        for (int d = 0; d < IN_DW; ++d) {
+            if constexpr (LOADS == kLoadDwords) buf[d] = 4 * d < validBytes ? raw[d] : 0u;
+            else buf[d] = 0u;
+        }
+        if constexpr (LOADS == kLoadXY) {
+            if (g == 0) encodeXYSquares(__builtin_bit_cast(float, raw[0]), __builtin_bit_cast(float, raw[1]), buf[0], buf[1]);
+        }
+        uint32_t actS[Net::KTMAX][FD];
+        uint32_t mst[L][Net::MTMAX];              // max() gradient multipliers, four e4m3 bytes per out tile
+        halfx2 yS[Net::MTL][2];
+#pragma unroll
+        for (int kt = 0; kt < Net::KT0; ++kt)
+#pragma unroll
+            for (int d = 0; d < FD; ++d) actS[kt][d] = buf[kt * RAW + d];
+
+        // ---------------- forward ----------------
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int MT = Net::mt(l), KT = Net::kt(l);
+            constexpr bool relu = l + 1 < L;
+            // this layer's input, for the dW contraction of the backward pass
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+                if (2 * kt < Net::nIt(l)) putS(myX + Net::xTileBase(l) * kPairTileDW, 2 * kt, Net::nIt(l), actS[kt]);
+
+            floatx4 acc[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) {
+                    const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
+                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                    acc[t] = Mma::mma(w, actS[kt], acc[t]);
+                }
+            halfx2 car[MT][2];
+            const halfx2 zero2 = {(half_t)0, (half_t)0};
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                typedef float floatx2 __attribute__((ext_vector_type(2)));
+                halfx2 z01 = __builtin_convertvector(floatx2{acc[t][0], acc[t][1]}, halfx2);
+                halfx2 z23 = __builtin_convertvector(floatx2{acc[t][2], acc[t][3]}, halfx2);
+                if constexpr (relu) {
+                    mst[l][t] = packMultipliers(maxGradMultiplier(z01), maxGradMultiplier(z23));
+                    z01 = __builtin_elementwise_max(z01, zero2);
+                    z23 = __builtin_elementwise_max(z23, zero2);
+                }
+                car[t][0] = z01; car[t][1] = z23;
+            }
+            if constexpr (l + 1 < L) {
+                constexpr int KTN = Net::kt(l + 1);
+#pragma unroll
+                for (int kt = 0; kt < KTN; ++kt) {
+                    actS[kt][0] = __builtin_bit_cast(uint32_t, car[2 * kt][0]);
+                    actS[kt][1] = __builtin_bit_cast(uint32_t, car[2 * kt][1]);
+                    actS[kt][2] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, car[2 * kt + 1 < MT ? 2 * kt + 1 : 0][0]) : 0u;
+                    actS[kt][3] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, car[2 * kt + 1 < MT ? 2 * kt + 1 : 0][1]) : 0u;
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < MT; ++t) { yS[t][0] = car[t][0]; yS[t][1] = car[t][1]; }
+            }
+        });
+
+        auto multipliers = [&](uint32_t rawm, halfx2& m01, halfx2& m23) {
+            m01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(rawm, 1.0f, false);
+            m23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(rawm, 1.0f, true);
+        };
+        auto packS = [&](halfx2 (*dz)[2], int MT, int KT, uint32_t (*out)[FD]) {
+#pragma unroll
+            for (int kt = 0; kt < Net::KOMAX; ++kt) {
+                if (kt < KT) {
+                    out[kt][0] = __builtin_bit_cast(uint32_t, dz[2 * kt][0]);
+                    out[kt][1] = __builtin_bit_cast(uint32_t, dz[2 * kt][1]);
+                    out[kt][2] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, dz[2 * kt + 1 < MT ? 2 * kt + 1 : 0][0]) : 0u;
+                    out[kt][3] = (2 * kt + 1 < MT) ? __builtin_bit_cast(uint32_t, dz[2 * kt + 1 < MT ? 2 * kt + 1 : 0][1]) : 0u;
+                }
+            }
+        };
+
+        // ---------------- loss and its gradient (S orientation) ----------------
+        uint32_t bS[Net::KOMAX][FD];                // S fragments of dZ of the current layer
+        {
+            float tgtAll = 0.f;
+            half_t gt[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+            const bool exampleLoss = !ta.targets && LOADS == kLoadXY;
+            if (exampleLoss) {
+                const halfx2 xy = __builtin_bit_cast(halfx2, buf[0]);
+                exampleGroundTruth(xy.x, xy.y, gt);
+            } else if (!ta.targets) {
+                float part = 0.f;
+#pragma unroll
+                for (int d = 0; d < IN_DW; ++d) {
+                    const halfx2 v = __builtin_bit_cast(halfx2, buf[d]);
+                    part += (float)v.x; part += (float)v.y;
+                }
+                part += __shfl_xor(part, 16);
+                part += __shfl_xor(part, 32);
+                tgtAll = (float)(half_t)sinf(part);
+            }
+            halfx2 dz[Net::MTL][2];
+#pragma unroll
+            for (int t = 0; t < Net::MTL; ++t) {
+                const half_t yv[4] = {yS[t][0].x, yS[t][0].y, yS[t][1].x, yS[t][1].y};
+                half_t gv[4];
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int row = g * OROWS + 4 * t + rr;
+                    gv[rr] = (half_t)0;
+                    if (live && row < outDim) {
+                        const float tv = ta.targets
+                            ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row)
+                            : (exampleLoss ? (float)gt[row & 3] : tgtAll);
+                        const half_t diff = (half_t)((float)yv[rr] - tv);
+                        lossAcc += (float)diff * (float)diff;
+                        gv[rr] = (half_t)(2.0f * (float)diff * ta.lossScale);
+                    }
+                }
+                dz[t][0] = halfx2{gv[0], gv[1]};       // the last layer has no activation
+                dz[t][1] = halfx2{gv[2], gv[3]};
+            }
+            packS(dz, Net::MTL, Net::ktOut(L - 1), bS);
+        }
+
+        // ---------------- backward ----------------
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = L - 1 - decltype(lc)::value;
+            constexpr int MT = Net::mt(l), NI = Net::nIt(l), KO = Net::ktOut(l);
+            uint32_t* slot = myDZ + (l & 1) * (Net::MTMAX * kPairTileDW);
+#pragma unroll
+            for (int kt = 0; kt < KO; ++kt) putS(slot, 2 * kt, MT, bS[kt]);
+
+            // dX = W^T dZ needs only this wave's own dZ: it runs ahead of the barrier, which gives the
+            // partner time to arrive, and its MFMAs cover the transposed reads of the dW part
+            floatx4 gacc[l > 0 ? Net::mt(l > 0 ? l - 1 : 0) : 1];
+            if constexpr (l > 0) {
+                constexpr int MTI = Net::mt(l - 1);
+#pragma unroll
+                for (int t = 0; t < MTI; ++t) gacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kt = 0; kt < KO; ++kt)
+#pragma unroll
+                    for (int t = 0; t < MTI; ++t) {
+                        const u32x4 v = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KO + kt) * 64 + lane) * RAW];
+                        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+                        gacc[t] = Mma::mma(w, bS[kt], gacc[t]);
+                    }
+            }
+            __syncthreads();      // dZ_l (and, long since, X_l) of both halves of the round are in LDS
+
+            // dW_l and db_l: this wave's share of the tiles, over all 32 samples of the round
+            {
+                constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l);
+                const int eo0 = Split::byOut(l) ? par * OO : 0;
+                const int ei0 = Split::byIn(l) ? par * OI : 0;
+                const bool active = !Split::single(l) || par == 0;
+                if (active) {
+                    uint32_t xF[OI][FD];
+#pragma unroll
+                    for (int ei = 0; ei < OI; ++ei) readF(myX + (Net::xTileBase(l) + ei0 + ei) * kPairTileDW, g, n, xF[ei]);
+#pragma unroll
+                    for (int eo = 0; eo < OO; ++eo) {
+                        uint32_t dzF[FD];
+                        readF(slot + (eo0 + eo) * kPairTileDW, g, n, dzF);
+                        if (Split::byOut(l) || par == 0) {
+                            float s = accB[Split::locDbBase(l) + eo];
+#pragma unroll
+                            for (int d = 0; d < FD; ++d) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, dzF[d]), ones2, s, false);
+                            accB[Split::locDbBase(l) + eo] = s;
+                        }
+#pragma unroll
+                        for (int ei = 0; ei < OI; ++ei) accumulateInAgpr(accW[Split::locBase(l) + eo * OI + ei], dzF, xF[ei]);
+                    }
+                }
+            }
+
+            if constexpr (l > 0) {
+                // through the previous layer's activation (ReLU on every hidden layer)
+                constexpr int MTI = Net::mt(l - 1);
+                halfx2 dz[MTI][2];
+#pragma unroll
+                for (int t = 0; t < MTI; ++t) {
+                    typedef float floatx2 __attribute__((ext_vector_type(2)));
+                    const halfx2 g01 = __builtin_convertvector(floatx2{gacc[t][0], gacc[t][1]}, halfx2);
+                    const halfx2 g23 = __builtin_convertvector(floatx2{gacc[t][2], gacc[t][3]}, halfx2);
+                    halfx2 m01, m23;
+                    multipliers(mst[l - 1][t], m01, m23);
+                    dz[t][0] = g01 * m01;
+                    dz[t][1] = g23 * m23;
+                }
+                packS(dz, MTI, Net::ktOut(l - 1), bS);
+            }
+        });
+        __syncthreads();          // nobody reads this round's tiles any more: the next round may overwrite them
+    };
+
+    // ---- main loop ---------------------------------------------------------------------------------
+    {
+        uint32_t cur[IN_DW], nxt[IN_DW];
+        uint32_t r = blockIdx.x * 4u + pair;
+        loadTile(cur, r);
+        for (uint32_t k = 0; k < roundsPerPair; ++k, r += gridDim.x * 4u) {
+            loadTile(nxt, r + gridDim.x * 4u);
+            asm volatile("" ::: "memory");        // the requests stay above the round ...
+            round(cur, r);
+#pragma unroll
+            for (int d = 0; d < IN_DW; ++d) { pinHere(nxt[d]); cur[d] = nxt[d]; }   // ... their results are first touched below it
+        }
+    }
+
+    // the last MFMAs into the AGPR accumulators must have retired before they are read
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
+    float* ldsRed = (float*)ldsX;                 // 8 waves x 256 floats
+    float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
+    const int rpar = threadIdx.x >> 8, ridx = threadIdx.x & 255;      // the parity / element this thread sums
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l), NI = Net::nIt(l);
+#pragma unroll
+        for (int j = 0; j < OO * OI; ++j) {
+            *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[Split::locBase(l) + j];
+            __syncthreads();
+            const float s = ((ldsRed[(0 + rpar) * 256 + ridx] + ldsRed[(2 + rpar) * 256 + ridx]) + ldsRed[(4 + rpar) * 256 + ridx]) +
+                            ldsRed[(6 + rpar) * 256 + ridx];
+            const int eo = (Split::byOut(l) ? rpar * OO : 0) + j / OI, ei = (Split::byIn(l) ? rpar * OI : 0) + j % OI;
+            if (!Split::single(l) || rpar == 0) part[(Net::gradTileBase(l) + eo * NI + ei) * 256 + ridx] = s;
+            __syncthreads();
+        }
+#pragma unroll
+        for (int j = 0; j < OO; ++j) {
+            ldsRed[wave * 64 + lane] = accB[Split::locDbBase(l) + j];
+            __syncthreads();
+            if (threadIdx.x < 32) {
+                const int p2 = threadIdx.x >> 4, q = threadIdx.x & 15;
+                float s = 0.f;
+                for (int w = 0; w < 4; ++w)
+                    for (int gg = 0; gg < 4; ++gg) s += ldsRed[(2 * w + p2) * 64 + gg * 16 + q];
+                const int eo = (Split::byOut(l) ? p2 * OO : 0) + j;
+                if (Split::byOut(l) || p2 == 0) part[Net::totalGradTiles * 256 + (Net::dbTileBase(l) + eo) * 16 + q] = s;
+            }
+            __syncthreads();
+        }
+    });
+    ldsRed[threadIdx.x] = lossAcc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int i = 0; i < 512; ++i) s += ldsRed[i];
+        part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+    }
+}
+
+} // namespace
+} // namespace cv

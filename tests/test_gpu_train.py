@@ -245,7 +245,7 @@ def test_general_training_step_against_oracle(dims, B, act, slope, grad_ct, grad
         # the fused kernel on the same step: same rounding points, only the order of the fp32 sums differs
         layers3 = build(specs, grad_ct, grad_layout)
         _, loss3 = cv.mlpTrainStep(layers3, to_dev(x), to_dev(t), gradType=grad_ct)
-        assert "mlpTrainKernel" in cv.lastKernelName()
+        assert "mlpTrain" in cv.lastKernelName() and "layer-by-layer" not in cv.lastKernelName()
         fW, fB = read_grads(layers3, specs, grad_ct, grad_layout)
         for l in range(len(specs)):
             assert rel_err(fW[l], dW[l]) <= (1e-4 if grad_ct == CT.Float32 else 1e-3)
