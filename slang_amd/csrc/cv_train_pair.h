@@ -14,7 +14,9 @@
 //   - each wave of the pair accumulates half of the dW tiles of every layer over all 32 samples
 //     of the round (its own 16 and its partner's), so a wave holds half of the accumulators
 //     (112 instead of 224 registers for 8-64-64-64-64-1) and two waves fit on a SIMD: the one
-//     covers the other's LDS and MFMA latencies.
+//     covers the other's LDS and MFMA latencies.  The accumulators are ordinary VGPRs here: a
+//     kernel that names no AGPR may use all 256 registers of its share as VGPRs, while one that
+//     does gets them split evenly, which is too few VGPRs for the rest of the round.
 //
 // The waves of a workgroup meet at a barrier once per layer in the backward pass (dZ_l of both
 // halves must be in LDS before either wave contracts over it) and once per round.  Every wave
@@ -88,13 +90,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int IN_DW = RAW * Net::KT0;
     const MlpArgs& a = ta.mlp;
 
-    __shared__ __attribute__((aligned(16))) uint32_t ldsW[Net::totalFrags * 64 * RAW];
-    __shared__ __attribute__((aligned(16))) uint32_t ldsWT[(Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW];
-    __shared__ __attribute__((aligned(16))) float ldsB[Net::totalBiasTiles * 16];
-    // per pair: every layer's input of the round, and two alternating slots for dZ
-    __shared__ __attribute__((aligned(16))) uint32_t ldsX[4 * Net::totalXTiles * kPairTileDW];
-    __shared__ __attribute__((aligned(16))) uint32_t ldsDZ[4 * 2 * Net::MTMAX * kPairTileDW];
-    static_assert(4 * Net::totalXTiles * kPairTileDW >= 8 * 256, "the final reduction reuses ldsX");
+    // One LDS array, carved by hand: the weights and biases come first so that every read of them is
+    // the lane's base address plus an immediate offset (the 16-bit offset field reaches 64 KB; arrays
+    // placed beyond that by the compiler cost an address register per fragment).
+    constexpr int W_DW = Net::totalFrags * 64 * RAW;
+    constexpr int WT_DW = (Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW;
+    constexpr int B_DW = Net::totalBiasTiles * 16;
+    constexpr int X_DW = 4 * Net::totalXTiles * kPairTileDW;          // per pair: every layer's input of the round
+    constexpr int DZ_DW = 4 * 2 * Net::MTMAX * kPairTileDW;           // per pair: two alternating slots for dZ
+    static_assert(X_DW >= 8 * 256, "the final reduction reuses the X tiles");
+    static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
+    __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW];
+    uint32_t* const ldsW = lds;
+    uint32_t* const ldsWT = lds + W_DW;
+    float* const ldsB = (float*)(lds + W_DW + WT_DW);
+    uint32_t* const ldsX = lds + W_DW + WT_DW + B_DW;
+    uint32_t* const ldsDZ = ldsX + X_DW;
 
     // ---- stage W, W^T and biases ----------------------------------------------------------------
     staticFor<0, L>([&](auto lc) {
@@ -196,17 +207,25 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int kt = 0; kt < KT; ++kt)
                 if (2 * kt < Net::nIt(l)) putS(myX + Net::xTileBase(l) * kPairTileDW, 2 * kt, Net::nIt(l), actS[kt]);
 
+            // all of the layer's fragments are requested before the first MFMA: a wave has one partner on
+            // its SIMD to cover an LDS round trip, not enough to wait for every fragment on its own
             floatx4 acc[MT];
-#pragma unroll
-            for (int t = 0; t < MT; ++t) acc[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+            uint32_t wf[KT][MT][4];
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
                     const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
-                    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-                    acc[t] = Mma::mma(w, actS[kt], acc[t]);
+                    wf[kt][t][0] = v.x; wf[kt][t][1] = v.y; wf[kt][t][2] = v.z; wf[kt][t][3] = v.w;
                 }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) acc[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+            __builtin_amdgcn_sched_group_barrier(0x100, KT * MT + MT, 0);     // the LDS reads ...
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                for (int t = 0; t < MT; ++t) acc[t] = Mma::mma(wf[kt][t], actS[kt], acc[t]);
+            __builtin_amdgcn_sched_group_barrier(0x008, KT * MT, 0);          // ... then the MFMAs
             halfx2 car[MT][2];
             const halfx2 zero2 = {(half_t)0, (half_t)0};
 #pragma unroll
@@ -311,14 +330,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 constexpr int MTI = Net::mt(l - 1);
 #pragma unroll
                 for (int t = 0; t < MTI; ++t) gacc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+                uint32_t wf[KO][MTI][4];
 #pragma unroll
                 for (int kt = 0; kt < KO; ++kt)
 #pragma unroll
                     for (int t = 0; t < MTI; ++t) {
                         const u32x4 v = *(const u32x4*)&ldsWT[((Net::tFragBase(l) + t * KO + kt) * 64 + lane) * RAW];
-                        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-                        gacc[t] = Mma::mma(w, bS[kt], gacc[t]);
+                        wf[kt][t][0] = v.x; wf[kt][t][1] = v.y; wf[kt][t][2] = v.z; wf[kt][t][3] = v.w;
                     }
+                __builtin_amdgcn_sched_group_barrier(0x100, KO * MTI, 1);
+#pragma unroll
+                for (int kt = 0; kt < KO; ++kt)
+#pragma unroll
+                    for (int t = 0; t < MTI; ++t) gacc[t] = Mma::mma(wf[kt][t], bS[kt], gacc[t]);
+                __builtin_amdgcn_sched_group_barrier(0x008, KO * MTI, 1);
             }
             __syncthreads();      // dZ_l (and, long since, X_l) of both halves of the round are in LDS
 
@@ -343,7 +368,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                             accB[Split::locDbBase(l) + eo] = s;
                         }
 #pragma unroll
-                        for (int ei = 0; ei < OI; ++ei) accumulateInAgpr(accW[Split::locBase(l) + eo * OI + ei], dzF, xF[ei]);
+                        for (int ei = 0; ei < OI; ++ei) {
+                            floatx4& w = accW[Split::locBase(l) + eo * OI + ei];
+                            w = Mma::mma(dzF, xF[ei], w);
+                        }
                     }
                 }
             }
@@ -381,9 +409,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int d = 0; d < IN_DW; ++d) { pinHere(nxt[d]); cur[d] = nxt[d]; }   // ... their results are first touched below it
         }
     }
-
-    // the last MFMAs into the AGPR accumulators must have retired before they are read
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
     float* ldsRed = (float*)ldsX;                 // 8 waves x 256 floats
