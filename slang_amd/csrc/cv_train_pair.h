@@ -56,12 +56,19 @@ struct PairSplit {
 };
 
 // LDS tile of one 16-feature group over the 32 samples of a round, 1 KB, in 8-byte chunks of four
-// features: chunk c (features 4c..4c+3) of sample s sits at chunk index c*32 + (s ^ 4c).  With that
-// swizzle both access patterns are free of bank conflicts: a 16-lane group writes one chunk column
-// of 16 samples (16 consecutive chunks), and reads, transposed, the four chunks of four consecutive
-// samples (chunk indices 4((j^c)%4) + r modulo 16, all different).
+// features: chunk c (features 4c..4c+3) of sample s sits at chunk index 32c + (s ^ k_c), k = {0, 24, 12, 20}.
+// With that swizzle both access patterns are free of bank conflicts whether the LDS serves 16 or 32
+// lanes of an 8-byte access per pass: a 16-lane group writes one chunk column of 16 consecutive
+// samples (a permutation of 16 consecutive slots; the columns c and c+1 of the neighbouring group
+// land in the other half of the 32 slots), and reads, transposed, the four chunks of four
+// consecutive samples (four different 4-slot blocks modulo 16, and for two neighbouring groups
+// eight different ones modulo 32).
 constexpr int kPairTileDW = 256;
-__device__ __forceinline__ int pairChunkDW(int sample, int c) { return (c * 32 + (sample ^ (4 * c))) * 2; }
+__device__ __forceinline__ int pairChunkDW(int sample, int c)
+{
+    const int k = (0x14 << 24 | 0x0c << 16 | 0x18 << 8 | 0x00) >> (8 * c) & 0xff;
+    return (c * 32 + (sample ^ k)) * 2;
+}
 
 // Transposed read of one F fragment (feature = lane%16, k-slots = 8 samples) from such a tile.
 // Lane 16g+i receives feature i of samples 4g..4g+3 (first instruction) and 16+4g..16+4g+3 (second):
@@ -71,9 +78,8 @@ __device__ __forceinline__ void readF(const uint32_t* tile, int g, int n, uint32
 {
     typedef short shortx4 __attribute__((ext_vector_type(4)));
     typedef shortx4 __attribute__((address_space(3))) * LdsPtr;
-    const uint32_t* p0 = tile + pairChunkDW(4 * g + (n >> 2), n & 3);
-    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)p0);
-    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(p0 + 32));      // samples + 16
+    const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(tile + pairChunkDW(4 * g + (n >> 2), n & 3)));
+    const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(tile + pairChunkDW(16 + 4 * g + (n >> 2), n & 3)));
     const u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
     frag[0] = a.x; frag[1] = a.y; frag[2] = b.x; frag[3] = b.y;
 }
@@ -190,7 +196,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (g == 0) encodeXYSquares(__builtin_bit_cast(float, raw[0]), __builtin_bit_cast(float, raw[1]), buf[0], buf[1]);
         }
         uint32_t actS[Net::KTMAX][FD];
-        uint32_t mst[L][Net::MTMAX];              // max() gradient multipliers, four e4m3 bytes per out tile
+        halfx2 zs[L][Net::MTMAX][2];              // pre-activations of the hidden layers: the backward pass derives
+                                                  // the gradient multiplier of max() from them
         halfx2 yS[Net::MTL][2];
 #pragma unroll
         for (int kt = 0; kt < Net::KT0; ++kt)
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 halfx2 z01 = __builtin_convertvector(floatx2{acc[t][0], acc[t][1]}, halfx2);
                 halfx2 z23 = __builtin_convertvector(floatx2{acc[t][2], acc[t][3]}, halfx2);
                 if constexpr (relu) {
-                    mst[l][t] = packMultipliers(maxGradMultiplier(z01), maxGradMultiplier(z23));
+                    zs[l][t][0] = z01; zs[l][t][1] = z23;
                     z01 = __builtin_elementwise_max(z01, zero2);
                     z23 = __builtin_elementwise_max(z23, zero2);
                 }
@@ -255,10 +262,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         });
 
-        auto multipliers = [&](uint32_t rawm, halfx2& m01, halfx2& m23) {
-            m01 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(rawm, 1.0f, false);
-            m23 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(rawm, 1.0f, true);
-        };
         auto packS = [&](halfx2 (*dz)[2], int MT, int KT, uint32_t (*out)[FD]) {
 #pragma unroll
             for (int kt = 0; kt < Net::KOMAX; ++kt) {
@@ -385,10 +388,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     typedef float floatx2 __attribute__((ext_vector_type(2)));
                     const halfx2 g01 = __builtin_convertvector(floatx2{gacc[t][0], gacc[t][1]}, halfx2);
                     const halfx2 g23 = __builtin_convertvector(floatx2{gacc[t][2], gacc[t][3]}, halfx2);
-                    halfx2 m01, m23;
-                    multipliers(mst[l - 1][t], m01, m23);
-                    dz[t][0] = g01 * m01;
-                    dz[t][1] = g23 * m23;
+                    dz[t][0] = g01 * maxGradMultiplier(zs[l - 1][t][0]);
+                    dz[t][1] = g23 * maxGradMultiplier(zs[l - 1][t][1]);
                 }
                 packS(dz, MTI, Net::ktOut(l - 1), bS);
             }
