@@ -10,7 +10,9 @@
 //   - the slot is dropped into a per-wave LDS buffer and read back in MFMA operand order
 //     (lane (g,n): its quarter of sample n), NT tiles at a time, in a rolled loop: small code,
 //     few live registers, 2-4 waves per SIMD;
-//   - biases are compiled out when no layer has one.
+//   - biases are compiled out when no layer has one;
+//   - IN_HALF (e4m3 networks): the rows in memory are fp16 vectors (CoopVec<half> with
+//     inputInterpretation FloatE4M3) and are quantised to e4m3 as they are read back from LDS.
 #pragma once
 #include "cv_mlp_impl.h"
 
@@ -29,15 +31,17 @@ __device__ __forceinline__ void carrierNoLeaky(const floatx4& acc, const Carrier
 #ifndef CV_MLP_STREAM_MINWAVES
 #define CV_MLP_STREAM_MINWAVES 1
 #endif
-template <class Mma, class Net, int NT, int S, bool HAS_BIAS>
+template <class Mma, class Net, int NT, int S, bool HAS_BIAS, bool IN_HALF = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STREAM_MINWAVES))) void mlpStreamKernel(const MlpArgs a)
 {
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     constexpr int L = Net::L;
     constexpr bool QUANT = !std::is_same<Mma, F16Mma>::value;   // e4m3 carrier between layers
     constexpr int IN_DW = RAW * Net::KT0;          // dwords one lane contributes per sample tile
-    constexpr int ROW_DW = 4 * IN_DW;              // dwords of one sample's input row
+    constexpr int LANE_DW = IN_HALF ? 2 * IN_DW : IN_DW;   // dwords of a lane's quarter of a row as it lies in memory
+    constexpr int ROW_DW = 4 * LANE_DW;            // dwords of one sample's input row
     constexpr int SLOT_DW = S * 16 * ROW_DW;       // dwords of one slot
+    static_assert(!IN_HALF || (!std::is_same<Mma, F16Mma>::value && Mma::kEsz == 1), "fp16 rows are quantised for e4m3 networks only");
     constexpr int CH = SLOT_DW / 256;              // 1 KB chunks per slot
     static_assert(SLOT_DW % 256 == 0 && S % NT == 0, "slot must be whole 1 KB chunks and whole rounds");
 
@@ -137,30 +141,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STRE
             uint32_t act[NT][Net::KTMAX][FD];
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                const uint32_t* src = myIn + ((r0 + j) * 16 + n) * ROW_DW + g * IN_DW;
-                uint32_t raw[IN_DW];
-                if constexpr (IN_DW % 4 == 0) {
+                const uint32_t* src = myIn + ((r0 + j) * 16 + n) * ROW_DW + g * LANE_DW;
+                uint32_t mem[LANE_DW];
+                if constexpr (LANE_DW % 4 == 0) {
 #pragma unroll
-                    for (int i = 0; i < IN_DW / 4; ++i) {
+                    for (int i = 0; i < LANE_DW / 4; ++i) {
                         const u32x4 v = *(const u32x4*)(src + 4 * i);
-                        raw[4 * i] = v.x; raw[4 * i + 1] = v.y; raw[4 * i + 2] = v.z; raw[4 * i + 3] = v.w;
+                        mem[4 * i] = v.x; mem[4 * i + 1] = v.y; mem[4 * i + 2] = v.z; mem[4 * i + 3] = v.w;
                     }
                 } else {
 #pragma unroll
-                    for (int i = 0; i < IN_DW / 2; ++i) {
+                    for (int i = 0; i < LANE_DW / 2; ++i) {
                         const u32x2 v = *(const u32x2*)(src + 2 * i);
-                        raw[2 * i] = v.x; raw[2 * i + 1] = v.y;
+                        mem[2 * i] = v.x; mem[2 * i + 1] = v.y;
                     }
+                }
+                uint32_t raw[IN_DW];
+                if constexpr (!IN_HALF) {
+#pragma unroll
+                    for (int i = 0; i < IN_DW; ++i) raw[i] = mem[i];
                 }
                 if constexpr (QUANT) {
                     // from here to the last layer's accumulators the conversions saturate by mode
                     if (j == 0) {
 #pragma unroll
-                        for (int i = 0; i < IN_DW; ++i) pinHere(raw[i]);
+                        for (int i = 0; i < LANE_DW; ++i) pinHere(mem[i]);
                         setFp16OverflowClamp<true>();
                     }
 #pragma unroll
-                    for (int i = 0; i < IN_DW; ++i) pinHere(raw[i]);
+                    for (int i = 0; i < LANE_DW; ++i) pinHere(mem[i]);
+                    if constexpr (IN_HALF) {
+                        // four halves -> four e4m3 bytes (saturating by mode, nearest even)
+#pragma unroll
+                        for (int i = 0; i < IN_DW; ++i)
+                            raw[i] = quantE4M3x4<true>(__builtin_bit_cast(halfx2, mem[2 * i]), __builtin_bit_cast(halfx2, mem[2 * i + 1]), cc[0]);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < IN_DW; ++i) raw[i] = mem[i];
+                    }
                 }
 #pragma unroll
                 for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&raw[kt * RAW], act[j][kt]);
@@ -244,17 +262,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STRE
 template <class Mma, class Net>
 bool mlpStreamEligible(const MlpArgs& a)
 {
-    constexpr int ROW_BYTES = 16 * Mma::kRawDW * Net::KT0;
+    const bool inHalf = a.inHalfAsE4M3 != 0;
+    if (inHalf && (std::is_same<Mma, F16Mma>::value || Mma::kEsz != 1)) return false;
+    const int rowBytes = 16 * Mma::kRawDW * Net::KT0 * (inHalf ? 2 : 1);
     const int outDim = a.layers[Net::L - 1].out;
-    if (a.inEncoding != kEncodeNone || a.inHalfAsE4M3) return false;
+    if (a.inEncoding != kEncodeNone) return false;
     for (int l = 0; l < Net::L; ++l)
         if (a.layers[l].act == kActLeakyRelu) return false;
-    return a.layers[0].in * Mma::kEsz == ROW_BYTES && a.inStride == (uint64_t)ROW_BYTES &&
+    return a.layers[0].in * (inHalf ? 2 : Mma::kEsz) == rowBytes && a.inStride == (uint64_t)rowBytes &&
            ((uintptr_t)a.in & 15u) == 0 && outDim % (4 * Net::MTL) == 0 && a.outAlign >= 8u &&
-           (uint64_t)a.batch * ROW_BYTES >= 16;
+           (uint64_t)a.batch * rowBytes >= 16;
 }
 
-template <class Mma, class Net, bool HAS_BIAS>
+template <class Mma, class Net, bool HAS_BIAS, bool IN_HALF>
 hipError_t launchMlpStreamB(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
 #ifdef CV_MLP_STREAM_NT
@@ -262,18 +282,18 @@ hipError_t launchMlpStreamB(hipStream_t stream, const MlpArgs& a, int numCUs)
 #else
     constexpr int NT = (Net::totalFrags * Mma::kFD <= 32) ? 4 : 2;
 #endif
-    constexpr int ROW_DW = 4 * Mma::kRawDW * Net::KT0;
+    constexpr int ROW_DW = 4 * Mma::kRawDW * Net::KT0 * (IN_HALF ? 2 : 1);
     constexpr int S0 = CV_MLP_STREAM_SLOT_DW / (16 * ROW_DW);
     constexpr int S = S0 < NT ? NT : S0 / NT * NT;
-    const int blocksPerCU = residentBlocksPerCU<mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS>>(256);
+    const int blocksPerCU = residentBlocksPerCU<mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS, IN_HALF>>(256);
     const uint32_t slot = 16 * S;
     const uint32_t numSlots = (a.batch + slot - 1) / slot;
     const uint32_t blocksNeeded = (numSlots + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
-    noteKernel(false, "mlpStreamKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d,%s>", Mma::kName, Net::KT0, Net::HT,
-               Net::L - 1, Net::MTL, NT, S, HAS_BIAS ? "bias" : "nobias");
-    hipLaunchKernelGGL((mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS>), dim3(blocks), dim3(256), 0, stream, a);
+    noteKernel(false, "mlpStreamKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d,%s%s>", Mma::kName, Net::KT0, Net::HT,
+               Net::L - 1, Net::MTL, NT, S, HAS_BIAS ? "bias" : "nobias", IN_HALF ? ",fp16-vectors" : "");
+    hipLaunchKernelGGL((mlpStreamKernel<Mma, Net, NT, S, HAS_BIAS, IN_HALF>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -282,8 +302,13 @@ hipError_t launchMlpStream(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     bool hasBias = false;
     for (int l = 0; l < Net::L; ++l) hasBias = hasBias || a.layers[l].bias != nullptr;
-    return hasBias ? launchMlpStreamB<Mma, Net, true>(stream, a, numCUs)
-                   : launchMlpStreamB<Mma, Net, false>(stream, a, numCUs);
+    if constexpr (!std::is_same<Mma, F16Mma>::value && Mma::kEsz == 1) {
+        if (a.inHalfAsE4M3)
+            return hasBias ? launchMlpStreamB<Mma, Net, true, true>(stream, a, numCUs)
+                           : launchMlpStreamB<Mma, Net, false, true>(stream, a, numCUs);
+    }
+    return hasBias ? launchMlpStreamB<Mma, Net, true, false>(stream, a, numCUs)
+                   : launchMlpStreamB<Mma, Net, false, false>(stream, a, numCUs);
 }
 
 } // namespace
