@@ -121,6 +121,11 @@ bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t 
         if (resType != CV_BFLOAT16 && resType != CV_FLOAT32) return false;
         if (!noBias && biasInterp != CV_BFLOAT16 && biasInterp != CV_FLOAT32) return false;
         k.kind = cv::MmaKind::Bf16;
+    } else if (matInterp == CV_FLOAT32) {
+        // the all-fp32 form: CoopVec<float> with a Float32 matrix (hlsl.meta.slang:32870-32872)
+        if (inType != CV_FLOAT32 || inInterp != CV_FLOAT32 || resType != CV_FLOAT32) return false;
+        if (!noBias && biasInterp != CV_FLOAT32) return false;
+        k.kind = cv::MmaKind::F32;
     } else if (matInterp == CV_SINT8 || matInterp == CV_UINT8) {
         if (resType != CV_SINT32 && resType != CV_UINT32) return false;
         if (!noBias && biasInterp != CV_SINT32 && biasInterp != CV_UINT32) return false;
@@ -404,7 +409,7 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     const hipError_t e = cv::launchMatMul((hipStream_t)stream, kind, a, cus);
     if (e == hipErrorInvalidValue)
         return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d is beyond what one 16-row block of the matrix can keep in LDS "
-                    "(128 KiB: k <= 4096 for 16-bit types, 8192 for 8-bit ones)", d->k);
+                    "(128 KiB: k <= 2048 for 32-bit types, 4096 for 16-bit ones, 8192 for 8-bit ones)", d->k);
     return fromHip(e, "cvMatMul launch");
 }
 

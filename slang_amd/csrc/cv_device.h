@@ -109,6 +109,29 @@ struct Bf16Mma {
     }
 };
 
+// fp32 operands on v_mfma_f32_16x16x4_f32.  A fragment keeps the 8 k-slots per lane of the 16-bit
+// flavours (so the InferencingOptimal form of an fp32 matrix is the same arrangement with 4-byte
+// elements): eight instructions, the s-th multiplying slot s of every lane, i.e. the four k
+// values {g*GS + 8*kt + s : g = 0..3}.
+struct F32Mma {
+    static constexpr const char* kName = "f32";
+    static constexpr int kEsz = 4, kEpl = 8, kRawDW = 8, kFD = 8;
+    static constexpr bool kIsFloat = true;
+    typedef floatx4 Acc;
+    static __device__ __forceinline__ void decode(const uint32_t* raw, uint32_t* frag)
+    {
+#pragma unroll
+        for (int d = 0; d < 8; ++d) frag[d] = raw[d];
+    }
+    static __device__ __forceinline__ Acc mma(const uint32_t* a, const uint32_t* b, Acc c)
+    {
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+            c = __builtin_amdgcn_mfma_f32_16x16x4f32(__builtin_bit_cast(float, a[s]), __builtin_bit_cast(float, b[s]), c, 0, 0, 0);
+        return c;
+    }
+};
+
 // OCP e5m2 in memory, decoded exactly to fp16 operands: an e5m2 value is the high byte of the
 // binary16 with the same value
 struct Bf8AsF16Mma {
@@ -192,6 +215,41 @@ __device__ __forceinline__ void exampleGroundTruth(half_t x, half_t y, half_t (&
 }
 
 // ---- final sum over per-workgroup partials ---------------------------------------------------
+// v summed over the four 16-lane groups of a wave (lanes n, n+16, n+32, n+48), in every lane.
+// v_permlane16_swap / v_permlane32_swap exchange rows between two registers; fed the same value
+// twice they leave each lane with both values of its pair, so the exchange costs one VALU
+// instruction and no LDS round trip.  The additions are those of v += shfl_xor(v, 16);
+// v += shfl_xor(v, 32) (each sum has the same two operands).
+// (The second result passes through an empty asm: without it the optimiser replaces it by the first
+// one when the two are added as floats.)
+__device__ __forceinline__ void swapRows16(uint32_t a, uint32_t& x, uint32_t& y)
+{
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(a, a, false, false);
+    x = r.x; y = r.y;
+    asm volatile("" : "+v"(y));
+}
+__device__ __forceinline__ void swapHalves32(uint32_t a, uint32_t& x, uint32_t& y)
+{
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(a, a, false, false);
+    x = r.x; y = r.y;
+    asm volatile("" : "+v"(y));
+}
+__device__ __forceinline__ float sumOverGroups(float v)
+{
+    uint32_t x, y;
+    swapRows16(__builtin_bit_cast(uint32_t, v), x, y);
+    v = __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+    swapHalves32(__builtin_bit_cast(uint32_t, v), x, y);
+    return __builtin_bit_cast(float, x) + __builtin_bit_cast(float, y);
+}
+__device__ __forceinline__ int sumOverGroups(int v)
+{
+    uint32_t x, y;
+    swapRows16((uint32_t)v, x, y);
+    swapHalves32(x + y, x, y);
+    return (int)(x + y);
+}
+
 // Used by the second-stage kernels of the deterministic reductions.  A workgroup of kReduceWaves
 // waves owns 64 consecutive values; every wave sums a contiguous share of the partials of the
 // calling lane's value (src[b * stride], b < numPartials) with sixteen independent loads in

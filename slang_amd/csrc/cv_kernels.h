@@ -34,7 +34,8 @@ enum class MmaKind : int {
     Bf16 = 4,            // bfloat16 vectors and matrix
     Bf8AsF16 = 5,        // e5m2 vectors and matrix, decoded to fp16 operands
     F16VecAsE4M3 = 6,    // fp16 vectors quantised to e4m3 on load, e4m3 matrix (matMul only)
-    I8AnySign = 7        // signed/unsigned bytes on either side (matMul only)
+    I8AnySign = 7,       // signed/unsigned bytes on either side (matMul only)
+    F32 = 8              // fp32 vectors and matrix (matMul only)
 };
 
 // Returns hipSuccess, or hipErrorInvalidValue when no kernel covers (m,k): k beyond what one

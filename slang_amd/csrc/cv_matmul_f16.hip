@@ -10,6 +10,7 @@ hipError_t launchMatMulBf8AsF16(hipStream_t stream, const MatMulArgs& a, int num
 hipError_t launchMatMulBf16(hipStream_t stream, const MatMulArgs& a, int numCUs);
 hipError_t launchMatMulI8(hipStream_t stream, const MatMulArgs& a, int numCUs);
 hipError_t launchMatMulI8AnySign(hipStream_t stream, const MatMulArgs& a, int numCUs);
+hipError_t launchMatMulF32(hipStream_t stream, const MatMulArgs& a, int numCUs);
 
 hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& a, int numCUs)
 {
@@ -25,6 +26,7 @@ hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& a, i
     case MmaKind::Bf16: return launchMatMulBf16(stream, a, numCUs);
     case MmaKind::I8: return launchMatMulI8(stream, a, numCUs);
     case MmaKind::I8AnySign: return launchMatMulI8AnySign(stream, a, numCUs);
+    case MmaKind::F32: return launchMatMulF32(stream, a, numCUs);
     }
     return hipErrorInvalidValue;
 }

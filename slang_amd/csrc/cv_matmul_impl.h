@@ -46,6 +46,9 @@ struct VecAsMatrix : Mma {
     // kStreaming: the flavour also gets the branch-free streaming instantiations (the less common
     // ones run every shape on the general kernel)
     static constexpr bool kStreaming = !std::is_same<Mma, Bf8AsF16Mma>::value;
+    // kAlwaysLarge: every shape runs on matmulLargeKernel (fp32 fragments are too wide to keep a
+    // block of the matrix in registers)
+    static constexpr bool kAlwaysLarge = std::is_same<Mma, F32Mma>::value;
     static __device__ __forceinline__ void decodeIn(const uint32_t* raw, uint32_t* frag) { Mma::decode(raw, frag); }
 };
 
@@ -55,7 +58,7 @@ struct VecAsMatrix : Mma {
 struct F16VecAsE4M3 : Fp8AsF16Mma {
     static constexpr const char* kName = "f16-as-e4m3-f16pipe";
     static constexpr int kInEsz = 2, kInRawDW = 4;
-    static constexpr bool kAnySign = false, kStreaming = false;
+    static constexpr bool kAnySign = false, kStreaming = false, kAlwaysLarge = false;
     static __device__ __forceinline__ uint32_t roundTrip(uint32_t h2)
     {
         typedef short shortx2 __attribute__((ext_vector_type(2)));
@@ -81,7 +84,7 @@ struct F16VecAsE4M3 : Fp8AsF16Mma {
 struct I8AnySign : I8Mma {
     static constexpr const char* kName = "i8-any-sign";
     static constexpr int kInEsz = 1, kInRawDW = 4;
-    static constexpr bool kAnySign = true, kStreaming = true;
+    static constexpr bool kAnySign = true, kStreaming = true, kAlwaysLarge = false;
     static __device__ __forceinline__ void decodeIn(const uint32_t* raw, uint32_t* frag) { I8Mma::decode(raw, frag); }
 };
 
@@ -95,13 +98,6 @@ __device__ __forceinline__ uint32_t signFlipMask(int i, int validBytes)
 {
     const int nb = validBytes - 4 * i;
     return nb >= 4 ? 0x80808080u : nb <= 0 ? 0u : (0x80808080u & ((1u << (8 * nb)) - 1u));
-}
-// sum over the four lane groups (lanes n, n+16, n+32, n+48)
-__device__ __forceinline__ int sumOverGroups(int v)
-{
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
 }
 
 // two fp32 values -> one dword of two 16-bit results
@@ -660,15 +656,17 @@ hipError_t dispatchBlock(hipStream_t stream, const MatMulArgs& a, int numCUs, bo
         default: return launchLarge<Fl, 8, OutT>(stream, a, largeKT, numCUs, append);
         }
     }
-    const int KTs = kt <= 1 ? 1 : kt <= 2 ? 2 : kt <= 4 ? 4 : 0;
-    if (!KTs) return hipErrorInvalidValue;
+    if constexpr (!Fl::kAlwaysLarge) {
+        const int KTs = kt <= 1 ? 1 : kt <= 2 ? 2 : kt <= 4 ? 4 : 0;
+        if (!KTs) return hipErrorInvalidValue;
 #define CV_CASE(M_, K_) \
-    if (MTs == M_ && KTs == K_) return launchShape<Fl, M_, K_, OutT>(stream, a, numCUs, append);
-    CV_CASE(1, 1) CV_CASE(1, 2) CV_CASE(1, 4)
-    CV_CASE(2, 1) CV_CASE(2, 2) CV_CASE(2, 4)
-    CV_CASE(4, 1) CV_CASE(4, 2) CV_CASE(4, 4)
-    CV_CASE(8, 1) CV_CASE(8, 2) CV_CASE(8, 4)
+        if (MTs == M_ && KTs == K_) return launchShape<Fl, M_, K_, OutT>(stream, a, numCUs, append);
+        CV_CASE(1, 1) CV_CASE(1, 2) CV_CASE(1, 4)
+        CV_CASE(2, 1) CV_CASE(2, 2) CV_CASE(2, 4)
+        CV_CASE(4, 1) CV_CASE(4, 2) CV_CASE(4, 4)
+        CV_CASE(8, 1) CV_CASE(8, 2) CV_CASE(8, 4)
 #undef CV_CASE
+    }
     return hipErrorInvalidValue;
 }
 
@@ -680,7 +678,7 @@ hipError_t dispatchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
     const uint32_t kt = optKT((uint32_t)a.k, Fl::kEpl);
     int blockTiles = 8, largeKT = 0;
-    if (kt > 4) {
+    if (kt > 4 || Fl::kAlwaysLarge) {
         largeKT = (int)((kt + kLargeKC - 1) / kLargeKC * kLargeKC);
         const size_t tileBytes = (size_t)largeKT * 64 * Fl::kRawDW * 4;
         while (blockTiles > 1 && blockTiles * tileBytes > (size_t)kLargeLdsBytes) blockTiles /= 2;

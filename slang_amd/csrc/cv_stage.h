@@ -24,8 +24,9 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
                                                bool transposed, int MT, int KT, uint32_t gs, uint32_t rows,
                                                uint32_t cols, uint32_t rowOff = 0, uint32_t xorByte = 0)
 {
-    constexpr int CHUNK = ESZ * EPL;              // bytes of one lane-chunk: 8 or 16
-    static_assert(CHUNK % 8 == 0, "a lane-chunk is one or two 8-byte words");
+    constexpr int CHUNK = ESZ * EPL;              // bytes of one lane-chunk: 8, 16 or 32
+    static_assert(ESZ == 1 || ESZ == 2 || ESZ == 4, "element size");
+    static_assert(CHUNK % 8 == 0, "a lane-chunk is a whole number of 8-byte words");
     const int chunks = MT * KT * 64;
     const bool direct = shape.layout == kInferencingOptimal && !transposed && rowOff == 0 && xorByte == 0 &&
                         optMT(shape.rows) == (uint32_t)MT && optKT(shape.cols, EPL) == (uint32_t)KT &&
@@ -66,8 +67,9 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
                 const bool valid = s < nvalid;
                 const uint8_t* p = !valid ? w : contiguous ? p0 + s * ESZ
                                  : w + (transposed ? elemOffset(shape, col0 + s, r) : elemOffset(shape, r, col0 + s));
-                if constexpr (ESZ == 2) ((uint16_t*)d)[s] = valid ? *(const uint16_t*)p : (uint16_t)0;
-                else                    ((uint8_t*)d)[s] = valid ? (uint8_t)(*p ^ xorByte) : (uint8_t)0;
+                if constexpr (ESZ == 4)      d[s] = valid ? *(const uint32_t*)p : 0u;
+                else if constexpr (ESZ == 2) ((uint16_t*)d)[s] = valid ? *(const uint16_t*)p : (uint16_t)0;
+                else                         ((uint8_t*)d)[s] = valid ? (uint8_t)(*p ^ xorByte) : (uint8_t)0;
             }
         }
     }

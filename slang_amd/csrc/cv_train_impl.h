@@ -479,9 +479,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         const halfx2 v = __builtin_bit_cast(halfx2, buf[j][d]);
                         part += (float)v.x; part += (float)v.y;
                     }
-                    part += __shfl_xor(part, 16);
-                    part += __shfl_xor(part, 32);
-                    tgtAll = (float)(half_t)sinf(part);
+                    tgtAll = (float)(half_t)sinf(sumOverGroups(part));
                 }
                 halfx2 dz[Net::MTL][2];
 #pragma unroll

@@ -18,11 +18,14 @@
 //     kernel that names no AGPR may use all 256 registers of its share as VGPRs, while one that
 //     does gets them split evenly, which is too few VGPRs for the rest of the round.
 //
-// The waves of a workgroup meet at a barrier once per layer in the backward pass (dZ_l of both
-// halves must be in LDS before either wave contracts over it) and once per round.  Every wave
-// runs the same number of rounds (rounds past the end of the batch are run with all samples
-// masked), so the barriers always match.  Partials and their second-stage reduction are those of
-// the one-wave kernel (mlpTrainReduceKernel): same layout, fixed order, no atomics.
+// The two waves of a pair meet once per layer in the backward pass (dZ_l of both halves must be in
+// LDS before either wave contracts over it) and once per round.  Only the pair meets, through a
+// sequence number each wave publishes in LDS (pairPublish, pairAwait), not the workgroup at s_barrier: the four
+// pairs of a workgroup drift apart, so that the two waves of a SIMD, which belong to different
+// pairs, are in different phases of the round and want different units.  Every wave runs the same
+// number of rounds (rounds past the end of the batch are run with all samples masked), so the
+// sequence numbers always match.  Partials and their second-stage reduction are those of the
+// one-wave kernel (mlpTrainReduceKernel): same layout, fixed order, no atomics.
 #pragma once
 #include "cv_train_impl.h"
 
@@ -76,12 +79,44 @@ __device__ __forceinline__ int pairChunkDW(int sample, int c)
 // 4(q%4)..), and the instruction returns to lane i element r = half i%4 of the chunk of lane 4r + i/4.
 __device__ __forceinline__ void readF(const uint32_t* tile, int g, int n, uint32_t* frag)
 {
+#ifdef CV_EXP_NOTR
+    frag[0] = frag[1] = frag[2] = frag[3] = (uint32_t)n; return;
+#endif
     typedef short shortx4 __attribute__((ext_vector_type(4)));
     typedef shortx4 __attribute__((address_space(3))) * LdsPtr;
     const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(tile + pairChunkDW(4 * g + (n >> 2), n & 3)));
     const shortx4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(tile + pairChunkDW(16 + 4 * g + (n >> 2), n & 3)));
     const u32x2 a = __builtin_bit_cast(u32x2, lo), b = __builtin_bit_cast(u32x2, hi);
     frag[0] = a.x; frag[1] = a.y; frag[2] = b.x; frag[3] = b.y;
+}
+
+// Meeting of the two waves of a pair, in two halves.  `mine` and `theirs` are the LDS words of this
+// wave and of its partner; `seq` counts the meetings and is the same in both waves.  A wave
+// publishes the number as soon as its part is done and awaits the partner's as late as it can, with
+// work that needs nothing from the partner in between, so that the number has usually arrived.
+// LDS executes the instructions of one wave in the order they were issued: the tile accesses above
+// pairPublish are complete when the partner sees the number; the compiler is kept from moving LDS
+// accesses across either call.  The wait is bounded: a partner that never arrives (which would be a defect of the kernel)
+// costs a wrong result (the return value says so), not a hung GPU.
+constexpr uint32_t kPairSpinLimit = 1u << 20;
+typedef uint32_t __attribute__((address_space(3))) LdsWord;
+__device__ __forceinline__ void pairPublish(volatile LdsWord* mine, uint32_t seq)
+{
+    asm volatile("" ::: "memory");
+    *mine = seq;
+}
+__device__ __forceinline__ uint32_t pairAwait(const volatile LdsWord* theirs, uint32_t seq)
+{
+    uint32_t spins = 0;
+#pragma nounroll
+    while ((uint32_t)__builtin_amdgcn_readfirstlane((int)*theirs) < seq && spins < kPairSpinLimit) {
+        ++spins;
+#ifdef CV_PAIR_SLEEP
+        __builtin_amdgcn_s_sleep(CV_PAIR_SLEEP);
+#endif
+    }
+    asm volatile("" ::: "memory");
+    return spins / kPairSpinLimit;      // 1 after a time-out
 }
 
 // ReLU on the hidden layers, none on the last one (the launcher sends everything else to the
@@ -105,13 +140,16 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int X_DW = 4 * Net::totalXTiles * kPairTileDW;          // per pair: every layer's input of the round
     constexpr int DZ_DW = 4 * 2 * Net::MTMAX * kPairTileDW;           // per pair: two alternating slots for dZ
     static_assert(X_DW >= 8 * 256, "the final reduction reuses the X tiles");
-    static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
-    __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW];
+    constexpr int FLAG_DW = 8;                                        // per wave: the number of its last meeting
+    static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
+    __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW];
     uint32_t* const ldsW = lds;
     uint32_t* const ldsWT = lds + W_DW;
     float* const ldsB = (float*)(lds + W_DW + WT_DW);
     uint32_t* const ldsX = lds + W_DW + WT_DW + B_DW;
     uint32_t* const ldsDZ = ldsX + X_DW;
+    uint32_t* const ldsFlag = ldsDZ + DZ_DW;
+    if (threadIdx.x < FLAG_DW) ldsFlag[threadIdx.x] = 0u;
 
     // ---- stage W, W^T and biases ----------------------------------------------------------------
     staticFor<0, L>([&](auto lc) {
@@ -136,7 +174,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#ifdef CV_PAIR_SAME_SIMD
+    const int pair = wave & 3, par = wave >> 2;
+    constexpr int kPartnerXor = 4;
+#else
     const int pair = wave >> 1, par = wave & 1;
+    constexpr int kPartnerXor = 1;
+#endif
+    const int slotOfWave = 2 * pair + par;
     const int g = lane >> 4, n = lane & 15;
     const halfx2 ones2 = {(half_t)1.f, (half_t)1.f};
 
@@ -163,6 +208,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint32_t* myDZ = ldsDZ + pair * (2 * Net::MTMAX * kPairTileDW);
     // where this lane puts its four halves of a tile (S fragment half: sample 16*par+n, rows 4g..4g+3) ...
     const int putDW = pairChunkDW(16 * par + n, g);
+    volatile LdsWord* const myFlag = (LdsWord*)(ldsFlag + wave);
+    const volatile LdsWord* const partnerFlag = (LdsWord*)(ldsFlag + (wave ^ kPartnerXor));
+    uint32_t meetings = 0, timeouts = 0;
 
     auto loadTile = [&](uint32_t (&raw)[IN_DW], uint32_t r) {
         const uint32_t s = min(r * 32u + 16u * par + n, lastSample);
@@ -179,11 +227,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // one S fragment (8 k-slots) -> the two tiles it belongs to
     auto putS = [&](uint32_t* tiles, int e0, int tilesInLayer, const uint32_t* frag) {
+#ifdef CV_EXP_NOPUT
+        return;
+#endif
+#ifdef CV_EXP_NOPUTX
+        if (tiles >= myX && tiles < myX + Net::totalXTiles * kPairTileDW) return;
+#endif
+#ifdef CV_EXP_NOPUTDZ
+        if (!(tiles >= myX && tiles < myX + Net::totalXTiles * kPairTileDW)) return;
+#endif
+#ifdef CV_EXP_LINEARPUT
+        *(u32x2*)(tiles + e0 * kPairTileDW + lane * 2) = u32x2{frag[0], frag[1]};
+        if (e0 + 1 < tilesInLayer) *(u32x2*)(tiles + (e0 + 1) * kPairTileDW + lane * 2) = u32x2{frag[2], frag[3]};
+        return;
+#endif
         *(u32x2*)(tiles + e0 * kPairTileDW + putDW) = u32x2{frag[0], frag[1]};
         if (e0 + 1 < tilesInLayer) *(u32x2*)(tiles + (e0 + 1) * kPairTileDW + putDW) = u32x2{frag[2], frag[3]};
     };
 
+#ifdef CV_PAIR_PHASE
+    uint64_t tPrev = __builtin_readcyclecounter(), cyc = 0;
+#define PH(k) { const uint64_t now_ = __builtin_readcyclecounter(); if (CV_PAIR_PHASE == 0 || CV_PAIR_PHASE == (k)) cyc += now_ - tPrev; tPrev = now_; }
+#else
+#define PH(k)
+#endif
     auto round = [&](const uint32_t (&raw)[IN_DW], uint32_t r) {
+        PH(99)
         const uint32_t sample = r * 32u + 16u * par + n;
         const bool live = sample < a.batch;
         uint32_t buf[IN_DW];
@@ -195,6 +264,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (LOADS == kLoadXY) {
             if (g == 0) encodeXYSquares(__builtin_bit_cast(float, raw[0]), __builtin_bit_cast(float, raw[1]), buf[0], buf[1]);
         }
+        // The target of the round's sample when the caller passes none: it depends on the input alone, and
+        // computed here its long dependent chain runs in the shadow of the forward pass.
+        float tgtAll = 0.f;
+        half_t gt[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
+        const bool exampleLoss = !ta.targets && LOADS == kLoadXY;
+        if constexpr (LOADS == kLoadXY) {
+            const halfx2 xy = __builtin_bit_cast(halfx2, buf[0]);
+            exampleGroundTruth(xy.x, xy.y, gt);
+        } else if (!ta.targets) {
+            float part = 0.f;
+#pragma unroll
+            for (int d = 0; d < IN_DW; ++d) {
+                const halfx2 v = __builtin_bit_cast(halfx2, buf[d]);
+                part += (float)v.x; part += (float)v.y;
+            }
+            tgtAll = (float)(half_t)sinf(sumOverGroups(part));
+        }
         uint32_t actS[Net::KTMAX][FD];
         halfx2 zs[L][Net::MTMAX][2];              // pre-activations of the hidden layers: the backward pass derives
                                                   // the gradient multiplier of max() from them
@@ -203,6 +289,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int kt = 0; kt < Net::KT0; ++kt)
 #pragma unroll
             for (int d = 0; d < FD; ++d) actS[kt][d] = buf[kt * RAW + d];
+
+        // the partner has left the previous round (published at its end): the round's tiles may be overwritten
+        timeouts |= pairAwait(partnerFlag, meetings); PH(6)
 
         // ---------------- forward ----------------
         staticFor<0, L>([&](auto lc) {
@@ -222,11 +311,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
+#ifdef CV_EXP_HALFW
+                    if (kt > 0) { for (int d = 0; d < 4; ++d) wf[kt][t][d] = wf[0][t][d]; continue; }
+#endif
                     const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
                     wf[kt][t][0] = v.x; wf[kt][t][1] = v.y; wf[kt][t][2] = v.z; wf[kt][t][3] = v.w;
                 }
 #pragma unroll
+#ifdef CV_EXP_NOBIAS
+            for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#else
             for (int t = 0; t < MT; ++t) acc[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+#endif
             __builtin_amdgcn_sched_group_barrier(0x100, KT * MT + MT, 0);     // the LDS reads ...
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
@@ -262,6 +358,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         });
 
+        PH(1)
         auto packS = [&](halfx2 (*dz)[2], int MT, int KT, uint32_t (*out)[FD]) {
 #pragma unroll
             for (int kt = 0; kt < Net::KOMAX; ++kt) {
@@ -277,23 +374,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         // ---------------- loss and its gradient (S orientation) ----------------
         uint32_t bS[Net::KOMAX][FD];                // S fragments of dZ of the current layer
         {
-            float tgtAll = 0.f;
-            half_t gt[4] = {(half_t)0, (half_t)0, (half_t)0, (half_t)0};
-            const bool exampleLoss = !ta.targets && LOADS == kLoadXY;
-            if (exampleLoss) {
-                const halfx2 xy = __builtin_bit_cast(halfx2, buf[0]);
-                exampleGroundTruth(xy.x, xy.y, gt);
-            } else if (!ta.targets) {
-                float part = 0.f;
-#pragma unroll
-                for (int d = 0; d < IN_DW; ++d) {
-                    const halfx2 v = __builtin_bit_cast(halfx2, buf[d]);
-                    part += (float)v.x; part += (float)v.y;
-                }
-                part += __shfl_xor(part, 16);
-                part += __shfl_xor(part, 32);
-                tgtAll = (float)(half_t)sinf(part);
-            }
             halfx2 dz[Net::MTL][2];
 #pragma unroll
             for (int t = 0; t < Net::MTL; ++t) {
@@ -302,15 +382,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int row = g * OROWS + 4 * t + rr;
-                    gv[rr] = (half_t)0;
-                    if (live && row < outDim) {
-                        const float tv = ta.targets
-                            ? (float)*(const half_t*)(ta.targets + (size_t)sample * ta.targetStride + 2 * row)
-                            : (exampleLoss ? (float)gt[row & 3] : tgtAll);
-                        const half_t diff = (half_t)((float)yv[rr] - tv);
-                        lossAcc += (float)diff * (float)diff;
-                        gv[rr] = (half_t)(2.0f * (float)diff * ta.lossScale);
-                    }
+                    const bool on = live && row < outDim;
+                    float tv = exampleLoss ? (float)gt[rr] : tgtAll;
+                    if (ta.targets)
+                        tv = (float)*(const half_t*)(ta.targets + (size_t)min(sample, lastSample) * ta.targetStride + 2 * (on ? row : 0));
+                    // straight-line: rows past the output and samples past the batch compute, then count for nothing
+                    const half_t diff = (half_t)((float)yv[rr] - tv);
+                    lossAcc += on ? (float)diff * (float)diff : 0.f;
+                    gv[rr] = on ? (half_t)(2.0f * (float)diff * ta.lossScale) : (half_t)0;
                 }
                 dz[t][0] = halfx2{gv[0], gv[1]};       // the last layer has no activation
                 dz[t][1] = halfx2{gv[2], gv[3]};
@@ -318,16 +397,46 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             packS(dz, Net::MTL, Net::ktOut(L - 1), bS);
         }
 
+        PH(2)
         // ---------------- backward ----------------
+        // The dW contraction of a layer is not on the round's chain of dependences (it only feeds the
+        // accumulators), so its operands are requested as soon as both halves of dZ_l are in LDS and its
+        // MFMAs are issued one layer later, behind the dX MFMAs of the layer below: by then the
+        // transposed reads have long arrived, and the MFMAs fill the time in which the partner's half of
+        // the next dZ is awaited.
+        uint32_t xFp[Net::ITMAX][FD], dzFp[Net::MTMAX][FD];      // pending operands: F fragments of X_l and dZ_l
+        auto contract = [&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l);
+#ifdef CV_EXP_NODW
+            return;
+#endif
+            if (!Split::single(l) || par == 0) {
+#pragma unroll
+                for (int eo = 0; eo < OO; ++eo) {
+                    if (Split::byOut(l) || par == 0) {
+                        float s = accB[Split::locDbBase(l) + eo];
+#pragma unroll
+                        for (int d = 0; d < FD; ++d) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, dzFp[eo][d]), ones2, s, false);
+                        accB[Split::locDbBase(l) + eo] = s;
+                    }
+#pragma unroll
+                    for (int ei = 0; ei < OI; ++ei) {
+                        floatx4& w = accW[Split::locBase(l) + eo * OI + ei];
+                        w = Mma::mma(dzFp[eo], xFp[ei], w);
+                    }
+                }
+            }
+        };
         staticFor<0, L>([&](auto lc) {
             constexpr int l = L - 1 - decltype(lc)::value;
             constexpr int MT = Net::mt(l), NI = Net::nIt(l), KO = Net::ktOut(l);
             uint32_t* slot = myDZ + (l & 1) * (Net::MTMAX * kPairTileDW);
 #pragma unroll
             for (int kt = 0; kt < KO; ++kt) putS(slot, 2 * kt, MT, bS[kt]);
+            pairPublish(myFlag, ++meetings);          // this wave's half of dZ_l is in LDS
 
-            // dX = W^T dZ needs only this wave's own dZ: it runs ahead of the barrier, which gives the
-            // partner time to arrive, and its MFMAs cover the transposed reads of the dW part
+            // dX = W^T dZ needs only this wave's own dZ: it runs between the two halves of the meeting
             floatx4 gacc[l > 0 ? Net::mt(l > 0 ? l - 1 : 0) : 1];
             if constexpr (l > 0) {
                 constexpr int MTI = Net::mt(l - 1);
@@ -348,34 +457,20 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     for (int t = 0; t < MTI; ++t) gacc[t] = Mma::mma(wf[kt][t], bS[kt], gacc[t]);
                 __builtin_amdgcn_sched_group_barrier(0x008, KO * MTI, 1);
             }
-            __syncthreads();      // dZ_l (and, long since, X_l) of both halves of the round are in LDS
+            if constexpr (l < L - 1) contract(std::integral_constant<int, (l < L - 1 ? l + 1 : 0)>{});
+            PH(3)
+            timeouts |= pairAwait(partnerFlag, meetings); PH(4)     // the partner's half of dZ_l is in LDS
 
-            // dW_l and db_l: this wave's share of the tiles, over all 32 samples of the round
+            // operands of dW_l and db_l: this wave's share of the tiles, over all 32 samples of the round
             {
                 constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l);
                 const int eo0 = Split::byOut(l) ? par * OO : 0;
                 const int ei0 = Split::byIn(l) ? par * OI : 0;
-                const bool active = !Split::single(l) || par == 0;
-                if (active) {
-                    uint32_t xF[OI][FD];
+                if (!Split::single(l) || par == 0) {
 #pragma unroll
-                    for (int ei = 0; ei < OI; ++ei) readF(myX + (Net::xTileBase(l) + ei0 + ei) * kPairTileDW, g, n, xF[ei]);
+                    for (int ei = 0; ei < OI; ++ei) readF(myX + (Net::xTileBase(l) + ei0 + ei) * kPairTileDW, g, n, xFp[ei]);
 #pragma unroll
-                    for (int eo = 0; eo < OO; ++eo) {
-                        uint32_t dzF[FD];
-                        readF(slot + (eo0 + eo) * kPairTileDW, g, n, dzF);
-                        if (Split::byOut(l) || par == 0) {
-                            float s = accB[Split::locDbBase(l) + eo];
-#pragma unroll
-                            for (int d = 0; d < FD; ++d) s = __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, dzF[d]), ones2, s, false);
-                            accB[Split::locDbBase(l) + eo] = s;
-                        }
-#pragma unroll
-                        for (int ei = 0; ei < OI; ++ei) {
-                            floatx4& w = accW[Split::locBase(l) + eo * OI + ei];
-                            w = Mma::mma(dzF, xF[ei], w);
-                        }
-                    }
+                    for (int eo = 0; eo < OO; ++eo) readF(slot + (eo0 + eo) * kPairTileDW, g, n, dzFp[eo]);
                 }
             }
 
@@ -393,8 +488,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
                 packS(dz, MTI, Net::ktOut(l - 1), bS);
             }
+            PH(5)
         });
-        __syncthreads();          // nobody reads this round's tiles any more: the next round may overwrite them
+        contract(std::integral_constant<int, 0>{});
+        pairPublish(myFlag, ++meetings);          // this wave reads the round's tiles no more
     };
 
     // ---- main loop ---------------------------------------------------------------------------------
@@ -412,6 +509,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
+#ifdef CV_PAIR_PHASE
+    lossAcc = lane == 0 ? (float)cyc : 0.f;
+#endif
+    if (timeouts) lossAcc = __builtin_nanf("");       // a meeting timed out: the step's result is void, and the loss says so
+    __syncthreads();                              // every pair has left its last round: the X tiles are free
     float* ldsRed = (float*)ldsX;                 // 8 waves x 256 floats
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
     const int rpar = threadIdx.x >> 8, ridx = threadIdx.x & 255;      // the parity / element this thread sums
@@ -420,7 +522,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l), NI = Net::nIt(l);
 #pragma unroll
         for (int j = 0; j < OO * OI; ++j) {
-            *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[Split::locBase(l) + j];
+            *(floatx4*)&ldsRed[slotOfWave * 256 + lane * 4] = accW[Split::locBase(l) + j];
             __syncthreads();
             const float s = ((ldsRed[(0 + rpar) * 256 + ridx] + ldsRed[(2 + rpar) * 256 + ridx]) + ldsRed[(4 + rpar) * 256 + ridx]) +
                             ldsRed[(6 + rpar) * 256 + ridx];
@@ -430,7 +532,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
 #pragma unroll
         for (int j = 0; j < OO; ++j) {
-            ldsRed[wave * 64 + lane] = accB[Split::locDbBase(l) + j];
+            ldsRed[slotOfWave * 64 + lane] = accB[Split::locDbBase(l) + j];
             __syncthreads();
             if (threadIdx.x < 32) {
                 const int p2 = threadIdx.x >> 4, q = threadIdx.x & 15;

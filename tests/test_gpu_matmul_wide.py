@@ -186,6 +186,55 @@ def test_bfloat16(M, K):
         assert (got >= 0).all()
 
 
+# ---- fp32 vectors against a Float32 matrix -----------------------------------------------------
+
+@pytest.mark.parametrize("M,K", [(64, 64), (128, 128), (24, 40), (16, 32), (4, 4), (200, 300)])
+def test_float32_matrix(M, K):
+    rng = np.random.default_rng(600 + M + K)
+    B = 500
+    x = rng.standard_normal((B, K)).astype(np.float32)
+    W = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+    b = rng.uniform(-0.5, 0.5, M).astype(np.float32)
+    ref, ab = ob.ref_matmul_f32(x, ob.F32, W.view(np.uint8).ravel(), ob.F32, ob.ROW, 4 * K, M, K, b, ob.F32)
+    ref64 = x.astype(np.float64) @ W.astype(np.float64).T + b
+    bound = (K + 1) * 2.0 ** -23 * ab            # fp32 products and sums, any order
+    assert (np.abs(ref - ref64) <= bound).all()   # the oracle against the definition
+    for layout in (ML.RowMajor, ML.ColumnMajor, ML.InferencingOptimal, ML.TrainingOptimal):
+        wb = to_dev(matrix_in_layout(W, CT.Float32, layout))
+        st = 4 * K if layout == ML.RowMajor else 4 * M
+        y = cv.coopVecMatMulAdd(to_dev(x), CT.Float32, wb, 0, CT.Float32, as_bytes(to_dev(b)), 0, CT.Float32, layout,
+                                False, st, M=M, resultType=CT.Float32)
+        assert y.dtype == torch.float32 and "f32" in cv.lastKernelName()
+        got = y.cpu().numpy()
+        assert (np.abs(got - ref64) <= bound).all(), layout
+        assert not ob.float_parity_violations(got, ref, ab).any()
+    # transposed use (memory holds K x M), ReLU; then the bias-less operator
+    wt = to_dev(matrix_in_layout(np.ascontiguousarray(W.T), CT.Float32, ML.InferencingOptimal))
+    y = cv.coopVecMatMulAdd(to_dev(x), CT.Float32, wt, 0, CT.Float32, as_bytes(to_dev(b)), 0, CT.Float32,
+                            ML.InferencingOptimal, True, 0, M=M, resultType=CT.Float32, activation=Activation.ReLU)
+    assert (np.abs(y.cpu().numpy() - np.maximum(ref64, 0)) <= bound).all()
+    y = cv.coopVecMatMul(to_dev(x), CT.Float32, wt, 0, CT.Float32, ML.InferencingOptimal, True, 0, M=M, resultType=CT.Float32)
+    assert (np.abs(y.cpu().numpy() - (ref64 - b)) <= bound).all()
+
+
+def test_float32_matrix_equals_the_slang_operator_on_exact_data():
+    # small integers: every product and sum is exact in fp32, so any summation order gives the operator's result
+    rng = np.random.default_rng(77)
+    M, K, B = 20, 12, 64
+    x = rng.integers(-8, 9, (B, K)).astype(np.float32)
+    W = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    b = rng.integers(-100, 100, M).astype(np.float32)
+    want = ob.slang_matmul(x, ob.F32, ob.F32, K, ob.F32, M, W.view(np.uint8).ravel(), ob.F32, ob.ROW, 4 * K, b, ob.F32)
+    assert np.array_equal(want, x @ W.T + b)
+    y = cv.coopVecMatMulAdd(to_dev(x), CT.Float32, to_dev(W.view(np.uint8).ravel()), 0, CT.Float32, as_bytes(to_dev(b)), 0,
+                            CT.Float32, ML.RowMajor, False, 4 * K, M=M, resultType=CT.Float32)
+    assert np.array_equal(y.cpu().numpy(), want)
+    # a Float32 matrix takes fp32 vectors only
+    with pytest.raises(cv.CoopVecError):
+        cv.coopVecMatMul(to_dev(x.astype(np.float16)), CT.Float16, to_dev(W.view(np.uint8).ravel()), 0, CT.Float32,
+                         ML.RowMajor, False, 4 * K, M=M)
+
+
 # ---- beyond 128 rows / 128 columns --------------------------------------------------------------
 
 @pytest.mark.parametrize("M,K", [(256, 64), (200, 128), (64, 256), (128, 512), (300, 200), (16, 1024), (520, 72)])
@@ -271,5 +320,6 @@ def test_query_lists_what_matmul_accepts():
                  (CT.UnsignedInt32, CT.UnsignedInt8Packed, CT.SignedInt8, CT.SignedInt32),
                  (CT.Float16, CT.FloatE4M3, CT.FloatE4M3, CT.Float16),
                  (CT.FloatE5M2, CT.FloatE5M2, CT.FloatE5M2, CT.Float16),
-                 (CT.BFloat16, CT.BFloat16, CT.BFloat16, CT.BFloat16)]:
+                 (CT.BFloat16, CT.BFloat16, CT.BFloat16, CT.BFloat16),
+                 (CT.Float32, CT.Float32, CT.Float32, CT.Float32)]:
         assert tuple(int(v) for v in want) in keys

@@ -196,6 +196,23 @@ def test_ref_matmul_goldens_and_fp64():
             assert L.cvo_layout_convert(ob.ptr(buf), M, K, F16, layout, 0, ob.ptr(W), F16, ROW, 0) == 0
             got, ab = ob.ref_matmul_f32(x, F16, buf, F16, layout, 0, M, K, b, F16)
             assert np.max(np.abs(got - want)) <= 1e-5 * max(1.0, np.max(ab))
+    # fp32 vectors against a Float32 matrix, the same way (and the Slang operator itself on data it computes exactly)
+    for (M, K) in [(4, 4), (24, 40), (64, 64)]:
+        x = rng.standard_normal((9, K)).astype(np.float32)
+        W = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+        b = rng.uniform(-0.1, 0.1, M).astype(np.float32)
+        want = x.astype(np.float64) @ W.astype(np.float64).T + b.astype(np.float64)
+        for layout in (ROW, COL, INF_OPT, TRAIN_OPT):
+            size = L.cvo_layout_matrix_size(M, K, F32, layout, 0)
+            buf = np.zeros(size, np.uint8)
+            assert L.cvo_layout_convert(ob.ptr(buf), M, K, F32, layout, 0, ob.ptr(W), F32, ROW, 0) == 0
+            got, ab = ob.ref_matmul_f32(x, F32, buf, F32, layout, 0, M, K, b, F32)
+            assert (np.abs(got - want) <= (K + 1) * 2.0 ** -23 * ab).all()
+    xi = rng.integers(-8, 9, (3, 12)).astype(np.float32)
+    Wi = rng.integers(-8, 9, (20, 12)).astype(np.float32)
+    bi = rng.integers(-100, 100, 20).astype(np.float32)
+    assert np.array_equal(ob.slang_matmul(xi, F32, F32, 12, F32, 20, Wi.view(np.uint8).ravel(), F32, ROW, 48, bi, F32),
+                          xi @ Wi.T + bi)
     # integer path: exact, and wraps like int32 only beyond 2^31 (never at these sizes)
     x = rng.integers(-128, 128, (5, 128), dtype=np.int8)
     W = rng.integers(-127, 128, (128, 128), dtype=np.int8)
