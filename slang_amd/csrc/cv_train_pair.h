@@ -79,9 +79,6 @@ __device__ __forceinline__ int pairChunkDW(int sample, int c)
 // 4(q%4)..), and the instruction returns to lane i element r = half i%4 of the chunk of lane 4r + i/4.
 __device__ __forceinline__ void readF(const uint32_t* tile, int g, int n, uint32_t* frag)
 {
-#ifdef CV_EXP_NOTR
-    frag[0] = frag[1] = frag[2] = frag[3] = (uint32_t)n; return;
-#endif
     typedef short shortx4 __attribute__((ext_vector_type(4)));
     typedef shortx4 __attribute__((address_space(3))) * LdsPtr;
     const shortx4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LdsPtr)(tile + pairChunkDW(4 * g + (n >> 2), n & 3)));
@@ -109,12 +106,7 @@ __device__ __forceinline__ uint32_t pairAwait(const volatile LdsWord* theirs, ui
 {
     uint32_t spins = 0;
 #pragma nounroll
-    while ((uint32_t)__builtin_amdgcn_readfirstlane((int)*theirs) < seq && spins < kPairSpinLimit) {
-        ++spins;
-#ifdef CV_PAIR_SLEEP
-        __builtin_amdgcn_s_sleep(CV_PAIR_SLEEP);
-#endif
-    }
+    while ((uint32_t)__builtin_amdgcn_readfirstlane((int)*theirs) < seq && spins < kPairSpinLimit) ++spins;
     asm volatile("" ::: "memory");
     return spins / kPairSpinLimit;      // 1 after a time-out
 }
@@ -174,14 +166,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#ifdef CV_PAIR_SAME_SIMD
-    const int pair = wave & 3, par = wave >> 2;
-    constexpr int kPartnerXor = 4;
-#else
-    const int pair = wave >> 1, par = wave & 1;
-    constexpr int kPartnerXor = 1;
-#endif
-    const int slotOfWave = 2 * pair + par;
+    const int pair = wave >> 1, par = wave & 1;      // partners sit on neighbouring SIMDs
     const int g = lane >> 4, n = lane & 15;
     const halfx2 ones2 = {(half_t)1.f, (half_t)1.f};
 
@@ -209,7 +194,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // where this lane puts its four halves of a tile (S fragment half: sample 16*par+n, rows 4g..4g+3) ...
     const int putDW = pairChunkDW(16 * par + n, g);
     volatile LdsWord* const myFlag = (LdsWord*)(ldsFlag + wave);
-    const volatile LdsWord* const partnerFlag = (LdsWord*)(ldsFlag + (wave ^ kPartnerXor));
+    const volatile LdsWord* const partnerFlag = (LdsWord*)(ldsFlag + (wave ^ 1));
     uint32_t meetings = 0, timeouts = 0;
 
     auto loadTile = [&](uint32_t (&raw)[IN_DW], uint32_t r) {
@@ -227,32 +212,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // one S fragment (8 k-slots) -> the two tiles it belongs to
     auto putS = [&](uint32_t* tiles, int e0, int tilesInLayer, const uint32_t* frag) {
-#ifdef CV_EXP_NOPUT
-        return;
-#endif
-#ifdef CV_EXP_NOPUTX
-        if (tiles >= myX && tiles < myX + Net::totalXTiles * kPairTileDW) return;
-#endif
-#ifdef CV_EXP_NOPUTDZ
-        if (!(tiles >= myX && tiles < myX + Net::totalXTiles * kPairTileDW)) return;
-#endif
-#ifdef CV_EXP_LINEARPUT
-        *(u32x2*)(tiles + e0 * kPairTileDW + lane * 2) = u32x2{frag[0], frag[1]};
-        if (e0 + 1 < tilesInLayer) *(u32x2*)(tiles + (e0 + 1) * kPairTileDW + lane * 2) = u32x2{frag[2], frag[3]};
-        return;
-#endif
         *(u32x2*)(tiles + e0 * kPairTileDW + putDW) = u32x2{frag[0], frag[1]};
         if (e0 + 1 < tilesInLayer) *(u32x2*)(tiles + (e0 + 1) * kPairTileDW + putDW) = u32x2{frag[2], frag[3]};
     };
 
-#ifdef CV_PAIR_PHASE
-    uint64_t tPrev = __builtin_readcyclecounter(), cyc = 0;
-#define PH(k) { const uint64_t now_ = __builtin_readcyclecounter(); if (CV_PAIR_PHASE == 0 || CV_PAIR_PHASE == (k)) cyc += now_ - tPrev; tPrev = now_; }
-#else
-#define PH(k)
-#endif
     auto round = [&](const uint32_t (&raw)[IN_DW], uint32_t r) {
-        PH(99)
         const uint32_t sample = r * 32u + 16u * par + n;
         const bool live = sample < a.batch;
         uint32_t buf[IN_DW];
@@ -291,7 +255,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int d = 0; d < FD; ++d) actS[kt][d] = buf[kt * RAW + d];
 
         // the partner has left the previous round (published at its end): the round's tiles may be overwritten
-        timeouts |= pairAwait(partnerFlag, meetings); PH(6)
+        timeouts |= pairAwait(partnerFlag, meetings);
 
         // ---------------- forward ----------------
         staticFor<0, L>([&](auto lc) {
@@ -311,18 +275,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
                 for (int t = 0; t < MT; ++t) {
-#ifdef CV_EXP_HALFW
-                    if (kt > 0) { for (int d = 0; d < 4; ++d) wf[kt][t][d] = wf[0][t][d]; continue; }
-#endif
                     const u32x4 v = *(const u32x4*)&ldsW[((Net::fragBase(l) + t * KT + kt) * 64 + lane) * RAW];
                     wf[kt][t][0] = v.x; wf[kt][t][1] = v.y; wf[kt][t][2] = v.z; wf[kt][t][3] = v.w;
                 }
 #pragma unroll
-#ifdef CV_EXP_NOBIAS
-            for (int t = 0; t < MT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#else
             for (int t = 0; t < MT; ++t) acc[t] = *(const floatx4*)&ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
-#endif
             __builtin_amdgcn_sched_group_barrier(0x100, KT * MT + MT, 0);     // the LDS reads ...
 #pragma unroll
             for (int kt = 0; kt < KT; ++kt)
@@ -357,8 +314,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 for (int t = 0; t < MT; ++t) { yS[t][0] = car[t][0]; yS[t][1] = car[t][1]; }
             }
         });
-
-        PH(1)
         auto packS = [&](halfx2 (*dz)[2], int MT, int KT, uint32_t (*out)[FD]) {
 #pragma unroll
             for (int kt = 0; kt < Net::KOMAX; ++kt) {
@@ -396,8 +351,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
             packS(dz, Net::MTL, Net::ktOut(L - 1), bS);
         }
-
-        PH(2)
         // ---------------- backward ----------------
         // The dW contraction of a layer is not on the round's chain of dependences (it only feeds the
         // accumulators), so its operands are requested as soon as both halves of dZ_l are in LDS and its
@@ -408,9 +361,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         auto contract = [&](auto lc) {
             constexpr int l = decltype(lc)::value;
             constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l);
-#ifdef CV_EXP_NODW
-            return;
-#endif
             if (!Split::single(l) || par == 0) {
 #pragma unroll
                 for (int eo = 0; eo < OO; ++eo) {
@@ -458,8 +408,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 __builtin_amdgcn_sched_group_barrier(0x008, KO * MTI, 1);
             }
             if constexpr (l < L - 1) contract(std::integral_constant<int, (l < L - 1 ? l + 1 : 0)>{});
-            PH(3)
-            timeouts |= pairAwait(partnerFlag, meetings); PH(4)     // the partner's half of dZ_l is in LDS
+            timeouts |= pairAwait(partnerFlag, meetings);     // the partner's half of dZ_l is in LDS
 
             // operands of dW_l and db_l: this wave's share of the tiles, over all 32 samples of the round
             {
@@ -488,7 +437,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 }
                 packS(dz, MTI, Net::ktOut(l - 1), bS);
             }
-            PH(5)
         });
         contract(std::integral_constant<int, 0>{});
         pairPublish(myFlag, ++meetings);          // this wave reads the round's tiles no more
@@ -509,9 +457,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
-#ifdef CV_PAIR_PHASE
-    lossAcc = lane == 0 ? (float)cyc : 0.f;
-#endif
     if (timeouts) lossAcc = __builtin_nanf("");       // a meeting timed out: the step's result is void, and the loss says so
     __syncthreads();                              // every pair has left its last round: the X tiles are free
     float* ldsRed = (float*)ldsX;                 // 8 waves x 256 floats
@@ -522,7 +467,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l), NI = Net::nIt(l);
 #pragma unroll
         for (int j = 0; j < OO * OI; ++j) {
-            *(floatx4*)&ldsRed[slotOfWave * 256 + lane * 4] = accW[Split::locBase(l) + j];
+            *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[Split::locBase(l) + j];
             __syncthreads();
             const float s = ((ldsRed[(0 + rpar) * 256 + ridx] + ldsRed[(2 + rpar) * 256 + ridx]) + ldsRed[(4 + rpar) * 256 + ridx]) +
                             ldsRed[(6 + rpar) * 256 + ridx];
@@ -532,7 +477,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         }
 #pragma unroll
         for (int j = 0; j < OO; ++j) {
-            ldsRed[slotOfWave * 64 + lane] = accB[Split::locDbBase(l) + j];
+            ldsRed[wave * 64 + lane] = accB[Split::locDbBase(l) + j];
             __syncthreads();
             if (threadIdx.x < 32) {
                 const int p2 = threadIdx.x >> 4, q = threadIdx.x & 15;
