@@ -46,7 +46,7 @@ PROFILED_TRAFFIC = {
     "c4": (805459000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4n": (805467000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4h": (1342320000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c5": (47851000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
+    "c5": (47832000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
     "op": (285453000, "profiles/outer_product_64x64_batch1M.md"),
     "rs": (537965000, "profiles/reduce_sum_64_batch4M.md"),
     "copy": (1073742000, "profiles/copy_calibration_512MiB.md"),
