@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void reduceSumStreamKernel(const ReduceSumArgs
         for (int u = 0; u < kRsUnroll; ++u) {
             const uint64_t s = row0 + (uint64_t)u * rowsPerLoad + r;
             v[u] = u32x4{0u, 0u, 0u, 0u};
-            if (active && s < a.batch) v[u] = *(const u32x4*)(base + s * a.vStride);
+            if (active && s < a.batch) v[u] = loadStream16(base + s * a.vStride);
         }
 #pragma unroll
         for (int u = 0; u < kRsUnroll; ++u) {

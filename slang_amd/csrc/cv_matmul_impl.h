@@ -175,13 +175,13 @@ __device__ __forceinline__ void storeVec(uint8_t* o, const uint32_t (&pk)[DW])
 #pragma unroll
         for (int i = 0; i < DW / 4; ++i) {
             const u32x4 v = {pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]};
-            ((u32x4*)o)[i] = v;
+            storeStream16(o + 16 * i, v);
         }
     } else {
 #pragma unroll
         for (int i = 0; i < DW / 2; ++i) {
             const u32x2 v = {pk[2 * i], pk[2 * i + 1]};
-            ((u32x2*)o)[i] = v;
+            storeStream8(o + 8 * i, v);
         }
     }
 }
@@ -360,10 +360,25 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 
     // One tile's input registers are loaded a whole tile ahead.  The two buffers swap roles
     // (no register copies: a copy would have to wait for the prefetch it is meant to hide).
+    // LINE_LOADS (streaming kernel, rows of eight 16-byte chunks = one 128-byte line): a load instruction
+    // of the wave covers eight whole rows, the eight lanes {n%8} x {g} x {n/8} of a row taking its
+    // chunks 2g + n/8, which lets the loads be non-temporal (loadStream16).  The first instruction
+    // fetches samples 0..7 of the tile, the second samples 8..15, so a lane ends up with chunk
+    // 2g + n/8 of samples n%8 and 8 + n%8; the fragment it needs (chunks 2g and 2g+1 of sample n) is
+    // completed by one exchange with the lane eight places away in its row (lineSwap, DPP).
+    // (Measured: fp16 64x64 196 -> 188 us together with the non-temporal stores; where a sample's output
+    // is several times its input, as for int8 128x128 with 512-byte rows of int32, the exchange costs
+    // more than the loads gain, so those shapes keep the plain pattern.)
+    constexpr bool LINE_LOADS = FAST && KT == 2 && IRAW == 4 && ROWS * 4 * (int)sizeof(OutT) <= 256;
     auto loadTile = [&](uint32_t (&buf)[NT][SLOT_DW], uint32_t t) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-            if constexpr (FAST) {
+            if constexpr (LINE_LOADS) {
+                const uint8_t* p = a.in + (size_t)(t * TILE + 16 * j + (n & 7)) * a.inStride + (2 * g + (n >> 3)) * 16;
+                const u32x4 v0 = loadStream16(p), v1 = loadStream16(p + (size_t)8 * a.inStride);
+                buf[j][0] = v0.x; buf[j][1] = v0.y; buf[j][2] = v0.z; buf[j][3] = v0.w;
+                buf[j][4] = v1.x; buf[j][5] = v1.y; buf[j][6] = v1.z; buf[j][7] = v1.w;
+            } else if constexpr (FAST) {
                 loadSlotsVec<SLOT_DW>(buf[j], inLane + (size_t)(t * TILE + 16 * j + n) * a.inStride);
             } else {
                 const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
@@ -372,9 +387,24 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
         }
     };
 
-    auto computeStore = [&](const uint32_t (&buf)[NT][SLOT_DW], uint32_t t0) {
+    auto computeStore = [&](const uint32_t (&bufIn)[NT][SLOT_DW], uint32_t t0) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
+            uint32_t slot[SLOT_DW];
+#pragma unroll
+            for (int d = 0; d < SLOT_DW; ++d) slot[d] = bufIn[j][d];
+            if constexpr (LINE_LOADS) {
+                // lanes 0..7 of a row keep their first register (sample n, chunk 2g) and take the partner's
+                // first one (sample n, chunk 2g+1); lanes 8..15 keep their second and take the partner's second
+                constexpr int kRowRor8 = 0x128;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const int r0 = (int)bufIn[j][d], r1 = (int)bufIn[j][4 + d];
+                    slot[4 + d] = (uint32_t)__builtin_amdgcn_update_dpp(r1, r0, kRowRor8, 0xf, 0x3, false);
+                    slot[d] = (uint32_t)__builtin_amdgcn_update_dpp(r0, r1, kRowRor8, 0xf, 0xc, false);
+                }
+            }
+            const uint32_t (&buf)[SLOT_DW] = slot;
             Acc acc[MT];
 #pragma unroll
             for (int t = 0; t < MT; ++t) acc[t] = lo.bias[t];
@@ -386,13 +416,13 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                     uint32_t x[IRAW];
 #pragma unroll
                     for (int d = 0; d < IRAW; ++d) {
-                        x[d] = buf[j][kt * IRAW + d];
+                        x[d] = buf[kt * IRAW + d];
                         if (a.inUnsigned) x[d] ^= FAST ? 0x80808080u : signFlipMask(kt * IRAW + d, validBytes);
                         if (a.matUnsigned) xSum += sumSignedBytes(x[d]);
                     }
                     Fl::decodeIn(x, bfrag);
                 } else {
-                    Fl::decodeIn(&buf[j][kt * IRAW], bfrag);
+                    Fl::decodeIn(&buf[kt * IRAW], bfrag);
                 }
 #pragma unroll
                 for (int t = 0; t < MT; ++t) acc[t] = Fl::mma(afrag[t][kt], bfrag, acc[t]);
@@ -443,7 +473,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                     for (int i = 0; i < ROW_DW / 16; ++i) {
                         const int c = i * 64 + lane, srow = c / CPR, ch = c % CPR;
                         const u32x4 v = *(const u32x4*)(st + srow * (ROW_DW + 4) + ch * 4);
-                        *(u32x4*)(tileOut + (size_t)srow * a.outStride + ch * 16) = v;
+                        storeStream16(tileOut + (size_t)srow * a.outStride + ch * 16, v);
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
