@@ -302,19 +302,8 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 
     const uint32_t gs = optGS((uint32_t)a.k);   // k-slots owned by one lane group
 
-    stageFragments<ESZ, EPL>(ldsW, a.mat, a.shape, a.transpose != 0, MT, KT, gs, (uint32_t)a.m, (uint32_t)a.k,
-                             a.rowOff, (Fl::kAnySign && a.matUnsigned) ? 0x80u : 0u);
-    __syncthreads();
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, n = lane & 15;
-
-    uint32_t afrag[MT][KT][FD];
-#pragma unroll
-    for (int t = 0; t < MT; ++t)
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-            Fl::decode(&ldsW[((t * KT + kt) * 64 + lane) * RAW], afrag[t][kt]);
 
     // ---- per-lane constants -------------------------------------------------------------
     const int rowBase = g * ROWS;
@@ -326,20 +315,6 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     LaneOut<Fl, MT> lo;
     loadBias<Fl, MT>(lo, a, rowBase);
     const int validRows = lo.validRows;
-    if constexpr (Fl::kAnySign) {
-        if (a.inUnsigned) {
-            int rowSum[MT];
-#pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                rowSum[t] = 0;
-#pragma unroll
-                for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-                    for (int d = 0; d < FD; ++d) rowSum[t] += sumSignedBytes(afrag[t][kt][d]);
-            }
-            addUnsignedRowTerm<Fl, MT>(lo, rowSum, a, g);
-        }
-    }
     // ReLU as a lower bound: max(z, 0) when on, max(z, -inf) = z when off (FAST path)
     const float reluFloor = a.act == kActRelu ? 0.f : -__builtin_inff();
     const int reluFloorI = a.act == kActRelu ? 0 : (int)0x80000000;
@@ -352,7 +327,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     const uint32_t numTiles = FAST ? a.batch / TILE : (a.batch + TILE - 1) / TILE;
     const uint32_t tileStride = gridDim.x * 4;
     uint32_t tile = blockIdx.x * 4 + wave;
-    if (tile >= numTiles) return;
+    const bool haveTile = tile < numTiles;     // (no early return: every wave takes part in staging the matrix)
 
     const uint8_t* inLane = a.in + (size_t)colBase * IESZ;
     uint8_t* outLane = a.out + (size_t)rowBase * sizeof(OutT);
@@ -387,6 +362,36 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
         }
     };
 
+    // The first tile's vectors are requested before the matrix is staged: their trip to HBM and the
+    // staging overlap.
+    uint32_t bufA[NT][SLOT_DW], bufB[NT][SLOT_DW];
+    if (haveTile) loadTile(bufA, tile);
+
+    stageFragments<ESZ, EPL>(ldsW, a.mat, a.shape, a.transpose != 0, MT, KT, gs, (uint32_t)a.m, (uint32_t)a.k,
+                             a.rowOff, (Fl::kAnySign && a.matUnsigned) ? 0x80u : 0u);
+    __syncthreads();
+
+    uint32_t afrag[MT][KT][FD];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+            Fl::decode(&ldsW[((t * KT + kt) * 64 + lane) * RAW], afrag[t][kt]);
+
+    if constexpr (Fl::kAnySign) {
+        if (a.inUnsigned) {
+            int rowSum[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+                rowSum[t] = 0;
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+                    for (int d = 0; d < FD; ++d) rowSum[t] += sumSignedBytes(afrag[t][kt][d]);
+            }
+            addUnsignedRowTerm<Fl, MT>(lo, rowSum, a, g);
+        }
+    }
     auto computeStore = [&](const uint32_t (&bufIn)[NT][SLOT_DW], uint32_t t0) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
@@ -488,9 +493,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
         }
     };
 
-    uint32_t bufA[NT][SLOT_DW], bufB[NT][SLOT_DW];
-    loadTile(bufA, tile);
-    while (true) {
+    while (haveTile) {
         // a prefetch past the end re-reads a valid tile instead of branching around the loads
         const uint32_t t1 = tile + tileStride;
         loadTile(bufB, t1 < numTiles ? t1 : tile);
