@@ -40,15 +40,15 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 # scaled by a copy of known size): not measured by this script, quoted from the committed profile summaries.
 PROFILED_TRAFFIC = {
     "c1": (717000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
-    "c2": (1074949000, "profiles/matmul_f16_64x64_batch4M.md"),
-    "c2b": (1074893000, "profiles/matmul_bf16_64x64_batch4M.md"),
-    "c3": (2685219000, "profiles/matmul_i8_128x128_batch4M.md"),
+    "c2": (1084790000, "profiles/matmul_f16_64x64_batch4M.md"),
+    "c2b": (1084793000, "profiles/matmul_bf16_64x64_batch4M.md"),
+    "c3": (2684680000, "profiles/matmul_i8_128x128_batch4M.md"),
     "c4": (805459000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4n": (805467000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4h": (1342320000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c5": (47832000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
     "op": (285453000, "profiles/outer_product_64x64_batch1M.md"),
-    "rs": (537965000, "profiles/reduce_sum_64_batch4M.md"),
+    "rs": (537966000, "profiles/reduce_sum_64_batch4M.md"),
     "copy": (1073742000, "profiles/copy_calibration_512MiB.md"),
 }
 
