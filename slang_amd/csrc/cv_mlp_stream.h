@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STRE
             // clamp the last, partial slot to the end of the input (those samples are not stored)
             uint64_t off = (uint64_t)sl * (SLOT_DW * 4) + (uint64_t)c * 1024 + (uint64_t)lane * 16;
             off = off + 16 <= totalBytes ? off : totalBytes - 16;
-            const u32x4 v = *(const u32x4*)(a.in + off);
+            const u32x4 v = loadStream16(a.in + off);
             stg[c][0] = v.x; stg[c][1] = v.y; stg[c][2] = v.z; stg[c][3] = v.w;
         }
     };
