@@ -287,6 +287,20 @@ def test_e4m3_large_shape_and_limit():
         cv.coopVecMatMul(torch.zeros((4, K2), dtype=torch.float16, device=DEV), CT.Float16,
                          torch.zeros(16 * K2 * 2, dtype=torch.uint8, device=DEV), 0, CT.Float16, ML.RowMajor, False, 2 * K2, M=16)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+    # fp32: the widest k (2048) works, one more k-tile does not
+    K3, M3 = 2048, 20
+    x3 = rng.standard_normal((50, K3)).astype(np.float32)
+    W3 = (rng.standard_normal((M3, K3)) / np.sqrt(K3)).astype(np.float32)
+    y3 = cv.coopVecMatMul(to_dev(x3), CT.Float32, as_bytes(to_dev(W3)), 0, CT.Float32, ML.RowMajor, False, 4 * K3, M=M3,
+                          resultType=CT.Float32)
+    want3 = x3.astype(np.float64) @ W3.astype(np.float64).T
+    ab3 = np.abs(x3).astype(np.float64) @ np.abs(W3).astype(np.float64).T
+    assert (np.abs(y3.cpu().numpy() - want3) <= (K3 + 1) * 2.0 ** -23 * ab3).all()
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.coopVecMatMul(torch.zeros((4, K3 + 16), dtype=torch.float32, device=DEV), CT.Float32,
+                         torch.zeros(16 * (K3 + 16) * 4, dtype=torch.uint8, device=DEV), 0, CT.Float32, ML.RowMajor, False,
+                         4 * (K3 + 16), M=16, resultType=CT.Float32)
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
 
 
 def test_non_finite_inputs_stay_within_their_sample():
