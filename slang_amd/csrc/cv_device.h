@@ -217,10 +217,10 @@ __device__ __forceinline__ void exampleGroundTruth(half_t x, half_t y, half_t (&
 // ---- final sum over per-workgroup partials ---------------------------------------------------
 // Streamed vectors (every byte is touched once per launch) go past the caches with non-temporal
 // accesses: measured on an MI355X, a plain 512 MiB copy runs at 5.5-5.8 TB/s with ordinary 16-byte
-// accesses and at 6.1-6.4 TB/s with non-temporal loads and stores.  The loads only where one
-// instruction of a wave covers whole 128-byte lines: a line fetched in two halves by two
-// non-temporal instructions is fetched twice (the batched matMul, whose lanes read 16 bytes at a
-// 32-byte pitch, lost 4 % with them and keeps ordinary loads).
+// accesses and at 6.1-6.4 TB/s with non-temporal loads and stores.  Only where one instruction of
+// a wave covers whole 128-byte lines: a line fetched in two halves by two non-temporal loads is
+// fetched twice (lanes reading 16 bytes at a 32-byte pitch lost 4 % with them), and non-temporal
+// stores of 16-byte pieces at a 128-byte pitch ran at 0.4 TB/s where ordinary ones reach 3 TB/s.
 __device__ __forceinline__ u32x4 loadStream16(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
 __device__ __forceinline__ u32x2 loadStream8(const void* p) { return __builtin_nontemporal_load((const u32x2*)p); }
 __device__ __forceinline__ void storeStream16(void* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }

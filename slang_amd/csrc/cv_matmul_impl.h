@@ -175,13 +175,13 @@ __device__ __forceinline__ void storeVec(uint8_t* o, const uint32_t (&pk)[DW])
 #pragma unroll
         for (int i = 0; i < DW / 4; ++i) {
             const u32x4 v = {pk[4 * i], pk[4 * i + 1], pk[4 * i + 2], pk[4 * i + 3]};
-            storeStream16(o + 16 * i, v);
+            ((u32x4*)o)[i] = v;
         }
     } else {
 #pragma unroll
         for (int i = 0; i < DW / 2; ++i) {
             const u32x2 v = {pk[2 * i], pk[2 * i + 1]};
-            storeStream8(o + 8 * i, v);
+            ((u32x2*)o)[i] = v;
         }
     }
 }
@@ -280,7 +280,9 @@ __device__ __forceinline__ void addUnsignedRowTerm(LaneOut<Fl, MT>& lo, int (&ro
     }
 }
 
-template <class Fl, int MT, int KT, int NT, typename OutT, bool FAST>
+// LINES (streaming kernel only): the vectors on both sides are whole, aligned 128-byte lines, which the
+// kernel then reads and writes with non-temporal accesses.
+template <class Fl, int MT, int KT, int NT, typename OutT, bool FAST, bool LINES = false>
 __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
 {
     constexpr int EPL = Fl::kEpl, FD = Fl::kFD, ESZ = Fl::kEsz, RAW = Fl::kRawDW;
@@ -344,7 +346,7 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
     // (Measured: fp16 64x64 196 -> 188 us together with the non-temporal stores; where a sample's output
     // is several times its input, as for int8 128x128 with 512-byte rows of int32, the exchange costs
     // more than the loads gain, so those shapes keep the plain pattern.)
-    constexpr bool LINE_LOADS = FAST && KT == 2 && IRAW == 4 && ROWS * 4 * (int)sizeof(OutT) <= 256;
+    constexpr bool LINE_LOADS = FAST && LINES && KT == 2 && IRAW == 4 && ROWS * 4 * (int)sizeof(OutT) <= 256;
     auto loadTile = [&](uint32_t (&buf)[NT][SLOT_DW], uint32_t t) {
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
@@ -478,7 +480,9 @@ __global__ __launch_bounds__(256) void matmulKernel(const MatMulArgs a)
                     for (int i = 0; i < ROW_DW / 16; ++i) {
                         const int c = i * 64 + lane, srow = c / CPR, ch = c % CPR;
                         const u32x4 v = *(const u32x4*)(st + srow * (ROW_DW + 4) + ch * 4);
-                        storeStream16(tileOut + (size_t)srow * a.outStride + ch * 16, v);
+                        uint8_t* dst = tileOut + (size_t)srow * a.outStride + ch * 16;
+                        if constexpr (LINES) storeStream16(dst, v);      // in pieces of lines such stores crawl
+                        else *(u32x4*)dst = v;
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
@@ -609,22 +613,22 @@ struct TileShape {
     static constexpr int NT = (MT * KT <= 8) ? CV_MATMUL_NT_SMALL : (MT * KT <= 16 ? 2 : 1);
 };
 
-template <class Fl, int MT, int KT, typename OutT, bool FAST>
+template <class Fl, int MT, int KT, typename OutT, bool FAST, bool LINES = false>
 hipError_t launchOne(hipStream_t stream, const MatMulArgs& a, int numCUs, bool append)
 {
     constexpr int NT = TileShape<MT, KT>::NT;
     // Persistent grid: exactly as many workgroups as are resident at once, so that every wave
     // strides over the same number of tiles (a partial second round would run at a fraction of
     // the occupancy).  The residency of a kernel is fixed, so it is queried once.
-    const int blocksPerCU = residentBlocksPerCU<matmulKernel<Fl, MT, KT, NT, OutT, FAST>>(256);
+    const int blocksPerCU = residentBlocksPerCU<matmulKernel<Fl, MT, KT, NT, OutT, FAST, LINES>>(256);
     const uint32_t tile = 16 * NT;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
     noteKernel(append, "matmulKernel<%s,MT=%d,KT=%d,NT=%d,out=%dB,%s>", Fl::kName, MT, KT, NT,
-               (int)sizeof(OutT), FAST ? "streaming" : "general");
-    hipLaunchKernelGGL((matmulKernel<Fl, MT, KT, NT, OutT, FAST>), dim3(blocks), dim3(256), 0, stream, a);
+               (int)sizeof(OutT), LINES ? "streaming,lines" : FAST ? "streaming" : "general");
+    hipLaunchKernelGGL((matmulKernel<Fl, MT, KT, NT, OutT, FAST, LINES>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -646,7 +650,16 @@ hipError_t launchShape(hipStream_t stream, const MatMulArgs& a, int numCUs, bool
         if (whole) {
             MatMulArgs b = a;
             b.batch = whole;
-            const hipError_t e = launchOne<Fl, MT, KT, OutT, true>(stream, b, numCUs, append);
+            // rows of whole 128-byte lines on both sides (and an output row that leaves through the LDS transpose)
+            constexpr bool kLinesShape = 16 * MT * sizeof(OutT) >= 128;
+            const bool lines = kLinesShape && (((uintptr_t)a.in | a.inStride | (uintptr_t)a.out | a.outStride) & 127u) == 0;
+            hipError_t e;
+            if constexpr (kLinesShape) {
+                e = lines ? launchOne<Fl, MT, KT, OutT, true, true>(stream, b, numCUs, append)
+                          : launchOne<Fl, MT, KT, OutT, true, false>(stream, b, numCUs, append);
+            } else {
+                e = launchOne<Fl, MT, KT, OutT, true, false>(stream, b, numCUs, append);
+            }
             if (e != hipSuccess) return e;
         }
         if (whole == a.batch) return hipSuccess;
