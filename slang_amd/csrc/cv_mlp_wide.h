@@ -1,0 +1,321 @@
+// cv_mlp_wide.h -- fused forward MLP on 32-sample tiles (v_mfma_f32_32x32x16_f16) for e4m3
+// networks whose input rows are 32 contiguous bytes and whose hidden layers are 32 or 64 wide.
+//
+// Why a second tiling.  Between two layers of an e4m3 network every hidden value passes
+// fp32 -> fp16 -> ReLU -> e4m3 -> fp16, one vector-ALU instruction per pair of values and step, and
+// that per-element work, not memory or the matrix pipeline, is what bounds the kernel: measured on
+// gfx950 a SIMD issues one ordinary VALU instruction per ~4.3 cycles, a conversion *to* fp8 per
+// ~8.3 cycles, and an MFMA with 128-bit operands also occupies the VALU port: ~8.7 cycles for
+// v_mfma_f32_16x16x32_f16 but only ~7.3 cycles for v_mfma_f32_32x32x16_f16, which does twice the
+// multiply-adds.  On 32-sample tiles the matrix instructions of a network therefore cost less than
+// half the issue time (16 instead of 28 per 32 samples for 32-64-64-8), and the input can be
+// loaded straight in operand order (no staging through LDS):
+//
+//   lane l = 32*h + n belongs to sample n of the tile and to half h;
+//   D = W . X^T per 32-row tile T: register r of lane (n,h) is row 8*(r/4) + 4*h + r%4;
+//   as B operand of k-step s, lane (n,h) supplies k-slots 8*h .. 8*h+7 of that step.
+//
+// The rows of a hidden layer are ordered so that registers 8*(s%2) .. 8*(s%2)+7 of tile s/2 are,
+// after conversion to packed fp16, exactly the B operand of k-step s of the next layer (no
+// cross-lane movement), and so that the 8-element chunks of k meet the accumulator in the same
+// order as in the 16-sample kernels: chunk (kt, g) there is chunk (s, h) = (2*kt + g/2, g%2) here.
+#pragma once
+#include "cv_mlp_impl.h"
+
+namespace cv {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// hidden unit computed by MFMA row rho of 32-row tile T (H = hidden width / 32)
+__host__ __device__ constexpr int wideUnitOfRow(int H, int T, int rho)
+{
+    return (2 * (rho / 16) + (rho % 8) / 4) * (8 * H) + 8 * T + 4 * ((rho % 16) / 8) + rho % 4;
+}
+// hidden unit consumed by element e of half h in k-step s
+__host__ __device__ constexpr int wideUnitOfSlot(int H, int s, int h, int e)
+{
+    return (2 * (s % 2) + h) * (8 * H) + 8 * (s / 2) + e;
+}
+
+__device__ __forceinline__ floatx16 mfma32(const uint32_t* a, const uint32_t* b, floatx16 c)
+{
+    const u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, av), __builtin_bit_cast(halfx8, bv), c, 0, 0, 0);
+}
+
+// One fragment = 64 lanes x 8 e4m3 bytes: lane (rho, h) holds W[rowOf(T, rho)][colOf(s, h, e)], e < 8.
+template <class RowFn, class ColFn>
+__device__ __forceinline__ void stageWideFragments(uint32_t* dst, const MlpLayerArgs& ly, int tiles, int steps, RowFn rowOf, ColFn colOf)
+{
+    for (int c = threadIdx.x; c < tiles * steps * 64; c += blockDim.x) {
+        const int lane = c & 63, f = c >> 6, s = f % steps, T = f / steps, rho = lane & 31, h = lane >> 5;
+        const int row = rowOf(T, rho);
+        uint32_t lo = 0, hi = 0;
+#pragma nounroll
+        for (int e = 0; e < 8; ++e) {
+            const int col = colOf(s, h, e);
+            uint32_t v = 0;
+            if (row < ly.out && col < ly.in) v = ly.w[elemOffset(ly.shape, (uint32_t)row, (uint32_t)col)];
+            if (e < 4) lo |= v << (8 * e); else hi |= v << (8 * (e - 4));
+        }
+        dst[2 * c] = lo; dst[2 * c + 1] = hi;
+    }
+}
+
+// H: hidden width / 32 (1 or 2); NH: hidden layers; OQ: groups of 8 output rows (1, 2 or 4).
+// Hidden layers are ReLU; the last layer's activation (none or ReLU) is read from the arguments.
+//
+// Work distribution.  A SIMD favours its oldest wave: with a fixed share of tiles per wave the oldest
+// wave of every SIMD is done in less than half of the kernel's time and the SIMD limps through the
+// rest with fewer and fewer waves (measured: wave 0 alive for 140 us of 311 us).  So one workgroup
+// fills a whole compute unit (WAVES waves) and its waves draw pairs of tiles from a counter in LDS;
+// all of them stay busy until the compute unit's share is used up.
+template <int H, int NH, int OQ, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
+{
+    constexpr int KS = 2 * H;                       // k-steps of a hidden vector
+    constexpr int F0 = H * 2, FH = H * KS, FL = KS; // fragments of layer 0, of a hidden->hidden layer, of the last layer
+    constexpr int TOTAL = F0 + (NH - 1) * FH + FL;
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[TOTAL * 64 * 2];
+    __shared__ uint32_t nextClaim;
+    if (threadIdx.x == 0) nextClaim = 0;
+
+    // ---- weights into LDS in operand order ---------------------------------------------------
+    stageWideFragments(ldsW, a.layers[0], H, 2,
+                       [](int T, int rho) { return wideUnitOfRow(H, T, rho); },
+                       [](int s, int h, int e) { return 16 * s + 8 * h + e; });
+#pragma unroll
+    for (int l = 1; l < NH; ++l)
+        stageWideFragments(ldsW + (F0 + (l - 1) * FH) * 128, a.layers[l], H, KS,
+                           [](int T, int rho) { return wideUnitOfRow(H, T, rho); },
+                           [](int s, int h, int e) { return wideUnitOfSlot(H, s, h, e); });
+    stageWideFragments(ldsW + (F0 + (NH - 1) * FH) * 128, a.layers[NH], 1, KS,
+                       [](int, int rho) { return rho; },
+                       [](int s, int h, int e) { return wideUnitOfSlot(H, s, h, e); });
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, h = lane >> 5;
+
+    uint32_t W0[H][2][4], WH[NH > 1 ? NH - 1 : 1][H][KS][4], WL[KS][4];
+    auto loadFrag = [&](int frag, uint32_t* dst) { Fp8AsF16Mma::decode(&ldsW[(frag * 64 + lane) * 2], dst); };
+#pragma unroll
+    for (int T = 0; T < H; ++T)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) loadFrag(T * 2 + s, W0[T][s]);
+#pragma unroll
+    for (int l = 1; l < NH; ++l)
+#pragma unroll
+        for (int T = 0; T < H; ++T)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) loadFrag(F0 + (l - 1) * FH + T * KS + s, WH[l - 1][T][s]);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) loadFrag(F0 + (NH - 1) * FH + s, WL[s]);
+
+    const uint32_t numTiles = (a.batch + 31u) / 32u, fullTiles = a.batch / 32u;
+    const uint32_t numPairs = (numTiles + 1u) / 2u;
+    const uint32_t numGroups = (uint32_t)__builtin_amdgcn_readfirstlane((int)gridDim.x);
+    // the c-th claim of this workgroup is pair c * numGroups + blockIdx.x (tiles 2*pair, 2*pair + 1)
+    auto claim = [&]() -> uint32_t {
+        uint32_t c = 0;
+        if (lane == 0) c = __hip_atomic_fetch_add(&nextClaim, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)c) * numGroups + blockIdx.x;
+    };
+    uint32_t pair = claim();
+    if (pair >= numPairs) return;
+    const uint32_t inLane = (uint32_t)n * 32u + (uint32_t)h * 16u;
+    const uint32_t outLane = (uint32_t)n * (uint32_t)a.outStride + (uint32_t)h * 8u;
+    const uint64_t totalBytes = (uint64_t)a.batch * 32u;
+    const bool lastRelu = a.layers[NH].act == kActRelu;
+    const int outDim = a.layers[NH].out;
+    const halfx2 zero2 = {(half_t)0.f, (half_t)0.f};
+
+    // a tile's 1 KB of input, 16 bytes per lane, in one fully coalesced instruction.  Only the last
+    // tile can be partial; its lanes beyond the end of the input read the last 16 bytes instead.
+    const uint32_t lastTile = numTiles - 1u;
+    uint32_t tailLane = inLane;
+    {
+        const uint64_t room = totalBytes - 16u - (uint64_t)lastTile * 1024u;    // rows are 32 bytes: never negative
+        if ((uint64_t)inLane > room) tailLane = (uint32_t)room;
+    }
+    // The input loads are issued and awaited by hand.  With the loads under its own control the compiler
+    // waits for *every* outstanding access at the top of the loop (also for the store it has just
+    // issued), which exposes the whole memory latency once per round.  Here a slot's four registers
+    // are written by a load that the compiler does not know about.  The statement that consumes a slot
+    // first waits until at most one younger access is outstanding (the other slot's load is always
+    // younger and loads return in order, so the slot's own load has landed whatever else is pending),
+    // takes the rows out, and then refills the same registers for the next pair of tiles.  Between two
+    // such statements a slot is only passed along untouched: the kernel must compile without register
+    // spills, and nothing may copy a slot while its load is on the way (both hold for every
+    // instantiation below; the bit-exact tests at full batch would show a stale register).
+    auto issue = [&](u32x4& slot, uint32_t t) {
+        t = t < lastTile ? t : lastTile;
+        const uint8_t* base = a.in + (uint64_t)t * 1024u;
+        const uint32_t voff = t < fullTiles ? inLane : tailLane;
+        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(slot) : "v"(voff), "s"(base) : "memory");
+    };
+    // bytes [0,8) and [16,24) of a row go to half 0, [8,16) and [24,32) to half 1 (k-steps 0 and 1):
+    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
+    auto consume = [&](u32x4& slot, uint32_t t, uint32_t (&B0)[4], uint32_t (&B1)[4]) {
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(slot) : "n"(1) : "memory");
+        const u32x2 r0 = __builtin_amdgcn_permlane32_swap(slot.x, slot.z, false, false);
+        const u32x2 r1 = __builtin_amdgcn_permlane32_swap(slot.y, slot.w, false, false);
+        uint32_t lo[2] = {r0.x, r1.x}, hi[2] = {r0.y, r1.y};
+        // the slot's registers are free from here on: the refill must not start before the rows are taken out
+        pinHere(lo[0]); pinHere(lo[1]); pinHere(hi[0]); pinHere(hi[1]);
+        issue(slot, t);
+        Fp8AsF16Mma::decode(lo, B0);
+        Fp8AsF16Mma::decode(hi, B1);
+    };
+
+    // Two tiles travel through the layers half a layer apart: while the vector ALU converts one tile's
+    // accumulators into the next layer's operands, the matrix pipeline works on the other tile.
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    uint32_t B[2][KS][4];
+    floatx16 acc[2][H];
+
+    auto firstLayer = [&](int j) {
+#pragma unroll
+        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][0], B[j][0], zero16);
+#pragma unroll
+        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][1], B[j][1], acc[j][T]);
+    };
+    // accumulators -> fp16 -> ReLU -> e4m3 -> fp16 operands of the next layer
+    auto carrier = [&](int j) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int T = s / 2, r0 = 8 * (s % 2);
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            typedef short shortx2 __attribute__((ext_vector_type(2)));
+            halfx2 p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                p[i] = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[j][T][r0 + 2 * i], acc[j][T][r0 + 2 * i + 1]}, halfx2), zero2);
+            uint32_t q[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                shortx2 r = __builtin_bit_cast(shortx2, p[2 * i]);
+                r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, p[2 * i], 1.0f, false);
+                r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, p[2 * i + 1], 1.0f, true);
+                q[i] = __builtin_bit_cast(uint32_t, r);
+            }
+            Fp8AsF16Mma::decode(q, B[j][s]);
+        }
+    };
+    auto hiddenLayer = [&](int l, int j) {
+#pragma unroll
+        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][0], B[j][0], zero16);
+#pragma unroll
+        for (int s = 1; s < KS; ++s)
+#pragma unroll
+            for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][s], B[j][s], acc[j][T]);
+    };
+    auto lastLayer = [&](int j) {      // result in acc[j][0]
+        acc[j][0] = mfma32(WL[0], B[j][0], zero16);
+#pragma unroll
+        for (int s = 1; s < KS; ++s) acc[j][0] = mfma32(WL[s], B[j][s], acc[j][0]);
+    };
+    auto storeTile = [&](int j, uint32_t t) {
+        const floatx16 o = acc[j][0];
+        const uint32_t sample = t * 32u + (uint32_t)n;
+        uint8_t* obase = a.out + (uint64_t)t * 32u * a.outStride;
+#pragma unroll
+        for (int q = 0; q < OQ; ++q) {
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            if (sample < a.batch && 8 * q + 4 * h < outDim) {
+                halfx2 p0 = __builtin_convertvector(floatx2{o[4 * q], o[4 * q + 1]}, halfx2);
+                halfx2 p1 = __builtin_convertvector(floatx2{o[4 * q + 2], o[4 * q + 3]}, halfx2);
+                if (lastRelu) {
+                    p0 = __builtin_elementwise_max(p0, zero2);
+                    p1 = __builtin_elementwise_max(p1, zero2);
+                }
+                const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
+                *(u32x2*)(obase + (outLane + 16u * q)) = v;
+            }
+        }
+    };
+    auto pinOperands = [&]() {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { pinHere(B[j][0][i]); pinHere(B[j][1][i]); }
+    };
+
+    u32x4 pf[2];
+    issue(pf[0], 2u * pair);
+    issue(pf[1], 2u * pair + 1u);
+    while (true) {
+        const uint32_t next = claim();      // beyond the end: its loads are redirected to the last tile and never used
+        consume(pf[0], 2u * next, B[0][0], B[0][1]);
+        consume(pf[1], 2u * next + 1u, B[1][0], B[1][1]);
+        // from here to the last layer's accumulators the conversions saturate by mode
+        pinOperands();
+        setFp16OverflowClamp<true>();
+        pinOperands();
+        firstLayer(0);
+        firstLayer(1);
+#pragma unroll
+        for (int l = 1; l < NH; ++l) {
+            carrier(0); hiddenLayer(l, 0);
+            carrier(1); hiddenLayer(l, 1);
+        }
+        carrier(0); lastLayer(0);
+        carrier(1); lastLayer(1);
+        // the network's fp16 output keeps inf for an overflow: mode off before it is formed
+        pinHere(acc[0][0]); pinHere(acc[1][0]);
+        setFp16OverflowClamp<false>();
+        pinHere(acc[0][0]); pinHere(acc[1][0]);
+        storeTile(0, 2u * pair);
+        storeTile(1, 2u * pair + 1u);
+        if (next >= numPairs) return;
+        pair = next;
+    }
+}
+
+// true when mlpWideKernel can take this call: e4m3 bytes in memory, 32 contiguous bytes per input
+// row, ReLU hidden layers of exactly 32 or 64 units without biases, at most 32 outputs in whole
+// groups of four with 8-byte aligned rows
+inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
+{
+    const int L = a.numLayers;
+    if (L < 2 || L > 4 || a.inHalfAsE4M3 || a.inEncoding != kEncodeNone) return false;
+    if (a.layers[0].in != 32 || a.inStride != 32u || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0) return false;
+    const int width = a.layers[0].out;
+    if (width != 32 && width != 64) return false;
+    for (int l = 0; l < L; ++l) {
+        if (a.layers[l].bias != nullptr) return false;
+        if (l + 1 < L && (a.layers[l].out != width || a.layers[l].act != kActRelu)) return false;
+        if (l > 0 && a.layers[l].in != width) return false;
+    }
+    const int outDim = a.layers[L - 1].out;
+    if (a.layers[L - 1].act != kActNone && a.layers[L - 1].act != kActRelu) return false;
+    if (outDim > 32 || outDim % 4 != 0 || a.outAlign < 8u || a.outStride >= (1u << 26)) return false;
+    H = width / 32; NH = L - 1; OQ = outDim <= 8 ? 1 : (outDim <= 16 ? 2 : 4);
+    return true;
+}
+
+template <int H, int NH, int OQ>
+hipError_t launchMlpWideShape(hipStream_t stream, const MlpArgs& a, int numCUs)
+{
+    // one workgroup per compute unit, as many waves as the weights leave registers for
+    // (16 waves: 128 registers each, 12: 168, 8: 256)
+    constexpr int WAVES = H == 1 ? 16 : (NH <= 2 ? 12 : 8);
+    const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
+    const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
+    noteKernel(false, "mlpWideKernel<e4m3-f16pipe,32x32x16,hidden=%dx%d,outputs<=%d>", NH, 32 * H, 8 * OQ);
+    hipLaunchKernelGGL((mlpWideKernel<H, NH, OQ, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+    return hipGetLastError();
+}
+
+inline hipError_t launchMlpWide(hipStream_t stream, const MlpArgs& a, int numCUs, int H, int NH, int OQ)
+{
+#define CV_W(h_, nh_, oq_) if (H == h_ && NH == nh_ && OQ == oq_) return launchMlpWideShape<h_, nh_, oq_>(stream, a, numCUs);
+    CV_W(2, 1, 1) CV_W(2, 2, 1) CV_W(2, 3, 1) CV_W(1, 1, 1) CV_W(1, 2, 1) CV_W(1, 3, 1)
+    CV_W(2, 1, 2) CV_W(2, 2, 2) CV_W(2, 3, 2) CV_W(2, 1, 4) CV_W(2, 2, 4) CV_W(2, 3, 4)
+#undef CV_W
+    return hipErrorInvalidValue;
+}
+
+} // namespace
+} // namespace cv

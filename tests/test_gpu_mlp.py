@@ -258,6 +258,60 @@ def test_e4m3_network_with_fp16_vectors(dims, B, flags):
     assert torch.equal(y_str.view(torch.int16), y_bytes.view(torch.int16))
 
 
+@pytest.mark.parametrize("dims,B", [([32, 64, 8], 4097), ([32, 64, 64, 8], 100003), ([32, 64, 64, 64, 8], 2048),
+                                    ([32, 32, 8], 33), ([32, 32, 32, 32, 4], 1000), ([32, 64, 64, 16], 777),
+                                    ([32, 64, 64, 32], 1501), ([32, 64, 12], 64), ([32, 64, 64, 8], 1), ([32, 64, 64, 8], 31)])
+@pytest.mark.parametrize("last_relu", [False, True])
+def test_e4m3_networks_on_32_sample_tiles(dims, B, last_relu):
+    # e4m3 networks with 32-byte input rows and ReLU hidden layers of 32 or 64 units run on 32-sample
+    # tiles (v_mfma_f32_32x32x16_f16, rows loaded straight in operand order, tiles drawn from a counter):
+    # same bits as the chain of single-layer operators for every depth, output width, layout and ragged batch
+    rng = np.random.default_rng(sum(dims) * 7 + B)
+    specs = make_net(rng, dims, CT.FloatE4M3, bias="none", init="half")
+    if last_relu:
+        specs[-1]["act"] = int(Activation.ReLU)
+    x = ob.encode_e4m3(rng.standard_normal((B, 32)) * 0.5)
+    xd = to_dev(x)
+    hid = []
+    yc = chain_of_single_layers(specs, xd, CT.FloatE4M3, hidden=hid)
+    for layout in (ML.RowMajor, ML.ColumnMajor, ML.InferencingOptimal):
+        y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, layout), xd, weightType=CT.FloatE4M3)
+        assert cv.lastKernelName().startswith("mlpWideKernel"), cv.lastKernelName()
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), layout
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, ob.E4M3, hid)
+    assert frac >= 0.99
+    # a padded output buffer: rows at a stride, nothing written between them
+    wide = torch.full((B, dims[-1] + 4), -7.0, dtype=torch.float16, device=DEV)
+    cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, ML.RowMajor), xd, weightType=CT.FloatE4M3, out=wide[:, :dims[-1]])
+    assert torch.equal(wide[:, :dims[-1]].contiguous().view(torch.int16), yc.view(torch.int16))
+    assert (wide[:, dims[-1]:] == -7.0).all()
+
+
+@pytest.mark.parametrize("B", [4096, 50])
+def test_e4m3_saturation_on_32_sample_tiles(B):
+    # ReLU networks (the 32-sample kernel): hidden sums beyond 448, also through an fp16 overflow, saturate
+    # to 448 when the carrier is re-quantised; an overflow of the network's own fp16 output stays inf
+    rng = np.random.default_rng(449)
+    specs = make_net(rng, [32, 64, 64, 8], CT.FloatE4M3, bias="none", init="half")
+    specs[0]["W"][:8] = ob.encode_e4m3(np.full((8, 32), 448.0))         # rows that overflow fp16
+    specs[0]["W"][16:24] = ob.encode_e4m3(np.full((8, 32), 2.0))        # beyond 448, within fp16
+    specs[1]["W"][:, :8] = ob.encode_e4m3(np.abs(rng.standard_normal((64, 8))) * 0.5)
+    specs[2]["W"][0] = ob.encode_e4m3(np.full(64, 448.0))               # output row that can overflow fp16
+    xf = rng.standard_normal((B, 32)) * 0.5
+    xf[::3] = 448.0
+    x = ob.encode_e4m3(xf)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, ML.InferencingOptimal), xd, weightType=CT.FloatE4M3)
+    assert cv.lastKernelName().startswith("mlpWideKernel"), cv.lastKernelName()
+    yc = chain_of_single_layers(specs, xd, CT.FloatE4M3)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    ref, acts = ob.ref_mlp_forward(specs, x, ob.E4M3, want_acts=True)
+    got = y.cpu().numpy()
+    assert np.isinf(ref).any() and np.isinf(acts[0]).any()              # the case is exercised
+    assert np.array_equal(np.isinf(got), np.isinf(ref))
+    assert np.array_equal(got[np.isinf(ref)], ref[np.isinf(ref)])
+
+
 def test_mlp_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_net(rng, [8, 16, 4], CT.Float16)
