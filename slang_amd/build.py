@@ -49,6 +49,23 @@ PER_FILE_FLAGS = {
 }
 
 
+# Kernels that must compile without register spills (a substring of the mangled name, per source file):
+# mlpWideKernel keeps loads in flight in registers the compiler does not know to be pending, so a spill or
+# reload of such a register would move stale data.  Checked from hipcc's kernel-resource-usage remarks.
+NO_SPILL_KERNELS = {"cv_mlp_fp8.hip": "mlpWideKernel"}
+
+
+def _check_no_spills(src: str, needle: str, remarks: str) -> None:
+    name = None
+    for line in remarks.splitlines():
+        if "remark: Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif name and needle in name:
+            for key in ("VGPRs Spill:", "SGPRs Spill:", "ScratchSize [bytes/lane]:"):
+                if key in line and int(line.split(key)[1].split()[0]) != 0:
+                    raise RuntimeError("%s: %s of %s is not zero (%s)" % (src, key.rstrip(":"), name, line.strip()))
+
+
 def _hipcc() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):
@@ -60,6 +77,9 @@ def _run(cmd: list[str]) -> None:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), proc.stdout))
+    src = os.path.basename(next((c for c in cmd if c.endswith(".hip")), ""))
+    if src in NO_SPILL_KERNELS:
+        _check_no_spills(src, NO_SPILL_KERNELS[src], proc.stdout)
 
 
 def build_library(jobs: int = 8, verbose: bool = False) -> str:
@@ -73,7 +93,8 @@ def build_library(jobs: int = 8, verbose: bool = False) -> str:
     for src in sources:
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmds.append([hipcc, *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src, []), "-I", os.path.join(REPO_DIR, "include"), "-c",
+        remarks = ["-Rpass-analysis=kernel-resource-usage"] if src in NO_SPILL_KERNELS else []
+        cmds.append([hipcc, *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src, []), *remarks, "-I", os.path.join(REPO_DIR, "include"), "-c",
                      os.path.join(CSRC, src), "-o", obj])
     with cf.ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         for cmd, _ in zip(cmds, pool.map(_run, cmds)):

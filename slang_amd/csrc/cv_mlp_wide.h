@@ -71,9 +71,12 @@ __device__ __forceinline__ void stageWideFragments(uint32_t* dst, const MlpLayer
 // rest with fewer and fewer waves (measured: wave 0 alive for 140 us of 311 us).  So one workgroup
 // fills a whole compute unit (WAVES waves) and its waves draw pairs of tiles from a counter in LDS;
 // all of them stay busy until the compute unit's share is used up.
-template <int H, int NH, int OQ, int WAVES>
+template <int H, int NH, int OQ, int WAVES, bool IN_HALF>
 __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
 {
+    constexpr uint32_t ROWB = IN_HALF ? 64u : 32u;       // bytes of an input row in memory
+    constexpr uint32_t TILEB = 32u * ROWB;               // bytes of a tile's input
+    constexpr int LOADS = IN_HALF ? 2 : 1;               // 16-byte loads per lane and tile
     constexpr int KS = 2 * H;                       // k-steps of a hidden vector
     constexpr int F0 = H * 2, FH = H * KS, FL = KS; // fragments of layer 0, of a hidden->hidden layer, of the last layer
     constexpr int TOTAL = F0 + (NH - 1) * FH + FL;
@@ -124,19 +127,20 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     };
     uint32_t pair = claim();
     if (pair >= numPairs) return;
-    const uint32_t inLane = (uint32_t)n * 32u + (uint32_t)h * 16u;
+    const uint32_t inLane = (uint32_t)n * ROWB + (uint32_t)h * (ROWB / 2u);
     const uint32_t outLane = (uint32_t)n * (uint32_t)a.outStride + (uint32_t)h * 8u;
-    const uint64_t totalBytes = (uint64_t)a.batch * 32u;
+    const uint64_t totalBytes = (uint64_t)a.batch * ROWB;
     const bool lastRelu = a.layers[NH].act == kActRelu;
     const int outDim = a.layers[NH].out;
     const halfx2 zero2 = {(half_t)0.f, (half_t)0.f};
 
-    // a tile's 1 KB of input, 16 bytes per lane, in one fully coalesced instruction.  Only the last
-    // tile can be partial; its lanes beyond the end of the input read the last 16 bytes instead.
+    // a tile's input, half a row per lane (16 bytes of e4m3, or 32 bytes of fp16 in two instructions), every
+    // instruction fully coalesced.  Only the last tile can be partial; its lanes beyond the end of the
+    // input read the last bytes instead.
     const uint32_t lastTile = numTiles - 1u;
     uint32_t tailLane = inLane;
     {
-        const uint64_t room = totalBytes - 16u - (uint64_t)lastTile * 1024u;    // rows are 32 bytes: never negative
+        const uint64_t room = totalBytes - ROWB / 2u - (uint64_t)lastTile * TILEB;    // a whole row is there: never negative
         if ((uint64_t)inLane > room) tailLane = (uint32_t)room;
     }
     // The input loads are issued and awaited by hand.  With the loads under its own control the compiler
@@ -149,24 +153,47 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     // such statements a slot is only passed along untouched: the kernel must compile without register
     // spills, and nothing may copy a slot while its load is on the way (both hold for every
     // instantiation below; the bit-exact tests at full batch would show a stale register).
-    auto issue = [&](u32x4& slot, uint32_t t) {
+    struct Slot { u32x4 v[LOADS]; };
+    auto issue = [&](Slot& slot, uint32_t t) {
         t = t < lastTile ? t : lastTile;
-        const uint8_t* base = a.in + (uint64_t)t * 1024u;
+        const uint8_t* base = a.in + (uint64_t)t * TILEB;
         const uint32_t voff = t < fullTiles ? inLane : tailLane;
-        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(slot) : "v"(voff), "s"(base) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=v"(slot.v[0]) : "v"(voff), "s"(base) : "memory");
+        if constexpr (IN_HALF)
+            asm volatile("global_load_dwordx4 %0, %1, %2 offset:16 nt" : "=v"(slot.v[1]) : "v"(voff), "s"(base) : "memory");
     };
-    // bytes [0,8) and [16,24) of a row go to half 0, [8,16) and [24,32) to half 1 (k-steps 0 and 1):
-    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
-    auto consume = [&](u32x4& slot, uint32_t t, uint32_t (&B0)[4], uint32_t (&B1)[4]) {
-        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(slot) : "n"(1) : "memory");
-        const u32x2 r0 = __builtin_amdgcn_permlane32_swap(slot.x, slot.z, false, false);
-        const u32x2 r1 = __builtin_amdgcn_permlane32_swap(slot.y, slot.w, false, false);
-        uint32_t lo[2] = {r0.x, r1.x}, hi[2] = {r0.y, r1.y};
+    // Half 0 of k-step 0 needs features 0..7 and of k-step 1 features 16..23, half 1 needs 8..15 and
+    // 24..31, while lane (n,0) has loaded features 0..15 and lane (n,1) features 16..31:
+    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second.
+    // RAW: per k-step the lane's eight features as they lie in memory (2 dwords of e4m3, 4 of fp16).
+    constexpr int RAW = IN_HALF ? 4 : 2;
+    auto consume = [&](Slot& slot, uint32_t t, uint32_t (&raw)[2][RAW], uint32_t (&Bj)[KS][4]) {
+        if constexpr (IN_HALF) {
+            asm volatile("s_waitcnt vmcnt(%2)" : "+v"(slot.v[0]), "+v"(slot.v[1]) : "n"(LOADS) : "memory");
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+                const u32x2 r = __builtin_amdgcn_permlane32_swap(slot.v[0][d], slot.v[1][d], false, false);
+                raw[0][d] = r.x; raw[1][d] = r.y;
+            }
+        } else {
+            asm volatile("s_waitcnt vmcnt(%1)" : "+v"(slot.v[0]) : "n"(LOADS) : "memory");
+            const u32x2 r0 = __builtin_amdgcn_permlane32_swap(slot.v[0].x, slot.v[0].z, false, false);
+            const u32x2 r1 = __builtin_amdgcn_permlane32_swap(slot.v[0].y, slot.v[0].w, false, false);
+            raw[0][0] = r0.x; raw[0][1] = r1.x; raw[1][0] = r0.y; raw[1][1] = r1.y;
+        }
         // the slot's registers are free from here on: the refill must not start before the rows are taken out
-        pinHere(lo[0]); pinHere(lo[1]); pinHere(hi[0]); pinHere(hi[1]);
+        // (e4m3 rows are decoded on the spot, which reads the slot's registers in place and saves the copies;
+        // fp16 rows must wait for the saturating mode)
+        if constexpr (!IN_HALF) {
+            Fp8AsF16Mma::decode(raw[0], Bj[0]);
+            Fp8AsF16Mma::decode(raw[1], Bj[1]);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { pinHere(Bj[0][i]); pinHere(Bj[1][i]); }
+        } else {
+#pragma unroll
+            for (int d = 0; d < RAW; ++d) { pinHere(raw[0][d]); pinHere(raw[1][d]); }
+        }
         issue(slot, t);
-        Fp8AsF16Mma::decode(lo, B0);
-        Fp8AsF16Mma::decode(hi, B1);
     };
 
     // Two tiles travel through the layers half a layer apart: while the vector ALU converts one tile's
@@ -235,26 +262,53 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
             }
         }
     };
-    auto pinOperands = [&]() {
+    uint32_t raw[2][2][RAW];
+    auto pinRaw = [&]() {      // whatever the first layer's operands are formed from, on both sides of the mode switch
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j) {
+            if constexpr (IN_HALF) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { pinHere(B[j][0][i]); pinHere(B[j][1][i]); }
+                for (int d = 0; d < RAW; ++d) { pinHere(raw[j][0][d]); pinHere(raw[j][1][d]); }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { pinHere(B[j][0][i]); pinHere(B[j][1][i]); }
+            }
+        }
+    };
+    // the first layer's operands from fp16 vectors: quantised to e4m3 (saturating by mode), decoded again
+    // (e4m3 rows were decoded when they were taken out of their slot)
+    auto firstOperands = [&](int j) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            if constexpr (IN_HALF) {
+                typedef short shortx2 __attribute__((ext_vector_type(2)));
+                uint32_t q[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const halfx2 p0 = __builtin_bit_cast(halfx2, raw[j][s][2 * i]), p1 = __builtin_bit_cast(halfx2, raw[j][s][2 * i + 1]);
+                    shortx2 r = __builtin_bit_cast(shortx2, p0);
+                    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, p0, 1.0f, false);
+                    r = __builtin_amdgcn_cvt_scalef32_pk_fp8_f16(r, p1, 1.0f, true);
+                    q[i] = __builtin_bit_cast(uint32_t, r);
+                }
+                Fp8AsF16Mma::decode(q, B[j][s]);
+            }
+        }
     };
 
-    u32x4 pf[2];
+    Slot pf[2];
     issue(pf[0], 2u * pair);
     issue(pf[1], 2u * pair + 1u);
     while (true) {
         const uint32_t next = claim();      // beyond the end: its loads are redirected to the last tile and never used
-        consume(pf[0], 2u * next, B[0][0], B[0][1]);
-        consume(pf[1], 2u * next + 1u, B[1][0], B[1][1]);
+        consume(pf[0], 2u * next, raw[0], B[0]);
+        consume(pf[1], 2u * next + 1u, raw[1], B[1]);
         // from here to the last layer's accumulators the conversions saturate by mode
-        pinOperands();
+        pinRaw();
         setFp16OverflowClamp<true>();
-        pinOperands();
-        firstLayer(0);
-        firstLayer(1);
+        pinRaw();
+        firstOperands(0); firstLayer(0);
+        firstOperands(1); firstLayer(1);
 #pragma unroll
         for (int l = 1; l < NH; ++l) {
             carrier(0); hiddenLayer(l, 0);
@@ -273,14 +327,15 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     }
 }
 
-// true when mlpWideKernel can take this call: e4m3 bytes in memory, 32 contiguous bytes per input
-// row, ReLU hidden layers of exactly 32 or 64 units without biases, at most 32 outputs in whole
+// true when mlpWideKernel can take this call: 32 inputs per sample in contiguous rows of e4m3 bytes or
+// (to be quantised on the way in) of fp16, ReLU hidden layers of exactly 32 or 64 units without biases, at most 32 outputs in whole
 // groups of four with 8-byte aligned rows
 inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
 {
     const int L = a.numLayers;
-    if (L < 2 || L > 4 || a.inHalfAsE4M3 || a.inEncoding != kEncodeNone) return false;
-    if (a.layers[0].in != 32 || a.inStride != 32u || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0) return false;
+    if (L < 2 || L > 4 || a.inEncoding != kEncodeNone) return false;
+    const uint64_t rowBytes = a.inHalfAsE4M3 ? 64u : 32u;
+    if (a.layers[0].in != 32 || a.inStride != rowBytes || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0) return false;
     const int width = a.layers[0].out;
     if (width != 32 && width != 64) return false;
     for (int l = 0; l < L; ++l) {
@@ -295,22 +350,24 @@ inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
     return true;
 }
 
-template <int H, int NH, int OQ>
+template <int H, int NH, int OQ, bool IN_HALF>
 hipError_t launchMlpWideShape(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     // one workgroup per compute unit, as many waves as the weights leave registers for
-    // (16 waves: 128 registers each, 12: 168, 8: 256)
-    constexpr int WAVES = H == 1 ? 16 : (NH <= 2 ? 12 : 8);
+    // (16 waves: 128 registers each, 12: 168, 8: 256); the build fails if an instantiation spills
+    constexpr int WAVES = H == 1 ? 16 : ((NH <= 2 && !(IN_HALF && OQ == 4)) ? 12 : 8);
     const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
     const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
-    noteKernel(false, "mlpWideKernel<e4m3-f16pipe,32x32x16,hidden=%dx%d,outputs<=%d>", NH, 32 * H, 8 * OQ);
-    hipLaunchKernelGGL((mlpWideKernel<H, NH, OQ, WAVES>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+    noteKernel(false, "mlpWideKernel<e4m3-f16pipe,32x32x16,hidden=%dx%d,outputs<=%d%s>", NH, 32 * H, 8 * OQ,
+               IN_HALF ? ",fp16-vectors" : "");
+    hipLaunchKernelGGL((mlpWideKernel<H, NH, OQ, WAVES, IN_HALF>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
     return hipGetLastError();
 }
 
 inline hipError_t launchMlpWide(hipStream_t stream, const MlpArgs& a, int numCUs, int H, int NH, int OQ)
 {
-#define CV_W(h_, nh_, oq_) if (H == h_ && NH == nh_ && OQ == oq_) return launchMlpWideShape<h_, nh_, oq_>(stream, a, numCUs);
+#define CV_W(h_, nh_, oq_) if (H == h_ && NH == nh_ && OQ == oq_) \
+        return a.inHalfAsE4M3 ? launchMlpWideShape<h_, nh_, oq_, true>(stream, a, numCUs) : launchMlpWideShape<h_, nh_, oq_, false>(stream, a, numCUs);
     CV_W(2, 1, 1) CV_W(2, 2, 1) CV_W(2, 3, 1) CV_W(1, 1, 1) CV_W(1, 2, 1) CV_W(1, 3, 1)
     CV_W(2, 1, 2) CV_W(2, 2, 2) CV_W(2, 3, 2) CV_W(2, 1, 4) CV_W(2, 2, 4) CV_W(2, 3, 4)
 #undef CV_W

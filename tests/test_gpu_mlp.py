@@ -287,6 +287,26 @@ def test_e4m3_networks_on_32_sample_tiles(dims, B, last_relu):
     assert (wide[:, dims[-1]:] == -7.0).all()
 
 
+@pytest.mark.parametrize("dims,B", [([32, 64, 64, 8], 5000), ([32, 64, 8], 33), ([32, 32, 32, 4], 1), ([32, 64, 64, 64, 8], 700),
+                                    ([32, 64, 64, 32], 257)])
+def test_fp16_vectors_on_32_sample_tiles(dims, B):
+    # CoopVec<half> + inputInterpretation FloatE4M3 on the 32-sample kernel: rows of 64 bytes, quantised
+    # (saturating, nearest even) after they are split between the lane halves; bit for bit the result of
+    # pre-quantised bytes, which in turn equals the chain of single-layer operators
+    rng = np.random.default_rng(sum(dims) + B)
+    specs = make_net(rng, dims, CT.FloatE4M3, bias="none", init="half")
+    xh = (rng.standard_normal((B, 32)) * 0.7).astype(np.float16)
+    xh[0, :8] = [1000.0, -1000.0, 464.0, -480.0, 2.0 ** -10, -0.0, 65504.0, np.inf]
+    xq = ob.encode_e4m3(np.clip(xh.astype(np.float32), -448.0, 448.0))
+    layers = gpu_layers(specs, CT.FloatE4M3, ML.InferencingOptimal)
+    y_bytes = cv.mlpForward(layers, to_dev(xq), weightType=CT.FloatE4M3)
+    y_half = cv.mlpForward(layers, to_dev(xh), weightType=CT.FloatE4M3)
+    assert cv.lastKernelName().startswith("mlpWideKernel") and "fp16-vectors" in cv.lastKernelName(), cv.lastKernelName()
+    assert torch.equal(y_half.view(torch.int16), y_bytes.view(torch.int16))
+    yc = chain_of_single_layers(specs, to_dev(xq), CT.FloatE4M3)
+    assert torch.equal(y_half.view(torch.int16), yc.view(torch.int16))
+
+
 @pytest.mark.parametrize("B", [4096, 50])
 def test_e4m3_saturation_on_32_sample_tiles(B):
     # ReLU networks (the 32-sample kernel): hidden sums beyond 448, also through an fp16 overflow, saturate
