@@ -71,7 +71,7 @@ __device__ __forceinline__ void stageWideFragments(uint32_t* dst, const MlpLayer
 // rest with fewer and fewer waves (measured: wave 0 alive for 140 us of 311 us).  So one workgroup
 // fills a whole compute unit (WAVES waves) and its waves draw pairs of tiles from a counter in LDS;
 // all of them stay busy until the compute unit's share is used up.
-template <int H, int NH, int OQ, int WAVES, bool IN_HALF>
+template <int H, int NH, int OQ, int WAVES, bool IN_HALF, bool HAS_BIAS>
 __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
 {
     constexpr uint32_t ROWB = IN_HALF ? 64u : 32u;       // bytes of an input row in memory
@@ -81,8 +81,23 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     constexpr int F0 = H * 2, FH = H * KS, FL = KS; // fragments of layer 0, of a hidden->hidden layer, of the last layer
     constexpr int TOTAL = F0 + (NH - 1) * FH + FL;
     __shared__ __attribute__((aligned(16))) uint32_t ldsW[TOTAL * 64 * 2];
+    // Biases enter as one more k-step in front of the others: A = the layer's biases in k-slot 0 (zeros
+    // elsewhere), B = 1.0 in k-slot 0, C = 0, which leaves exactly float(bias) in the accumulators, the
+    // value the 16-sample kernels start from.  One fragment per layer and 32-row tile, read from LDS at use.
+    constexpr int NBIAS = HAS_BIAS ? H * NH + 1 : 1;
+    __shared__ __attribute__((aligned(16))) uint32_t ldsBias[NBIAS * 64 * 4];
     __shared__ uint32_t nextClaim;
     if (threadIdx.x == 0) nextClaim = 0;
+    if constexpr (HAS_BIAS) {
+        for (int c = threadIdx.x; c < NBIAS * 64; c += blockDim.x) {
+            const int lane = c & 63, f = c >> 6, rho = lane & 31;
+            const int l = f < H * NH ? f / H : NH, T = f < H * NH ? f % H : 0;
+            const int unit = l < NH ? wideUnitOfRow(H, T, rho) : rho;
+            uint32_t v = 0;
+            if (lane < 32 && a.layers[l].bias && unit < a.layers[l].out) v = ((const uint16_t*)a.layers[l].bias)[unit];
+            ldsBias[4 * c] = v; ldsBias[4 * c + 1] = 0; ldsBias[4 * c + 2] = 0; ldsBias[4 * c + 3] = 0;
+        }
+    }
 
     // ---- weights into LDS in operand order ---------------------------------------------------
     stageWideFragments(ldsW, a.layers[0], H, 2,
@@ -201,10 +216,20 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     uint32_t B[2][KS][4];
     floatx16 acc[2][H];
+    const uint32_t onesB[4] = {h == 0 ? 0x3C00u : 0u, 0u, 0u, 0u};       // 1.0 in k-slot 0
+    auto seed = [&](int l, int T) -> floatx16 {       // float(bias) of layer l, tile T, or zeros
+        if constexpr (HAS_BIAS) {
+            const u32x4 bf = *(const u32x4*)&ldsBias[((l * H + T) * 64 + lane) * 4];
+            const uint32_t biasA[4] = {bf.x, bf.y, bf.z, bf.w};
+            return mfma32(biasA, onesB, zero16);
+        } else {
+            return zero16;
+        }
+    };
 
     auto firstLayer = [&](int j) {
 #pragma unroll
-        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][0], B[j][0], zero16);
+        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][0], B[j][0], seed(0, T));
 #pragma unroll
         for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][1], B[j][1], acc[j][T]);
     };
@@ -232,14 +257,14 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
     };
     auto hiddenLayer = [&](int l, int j) {
 #pragma unroll
-        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][0], B[j][0], zero16);
+        for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][0], B[j][0], seed(l, T));
 #pragma unroll
         for (int s = 1; s < KS; ++s)
 #pragma unroll
             for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][s], B[j][s], acc[j][T]);
     };
     auto lastLayer = [&](int j) {      // result in acc[j][0]
-        acc[j][0] = mfma32(WL[0], B[j][0], zero16);
+        acc[j][0] = mfma32(WL[0], B[j][0], seed(NH, 0));
 #pragma unroll
         for (int s = 1; s < KS; ++s) acc[j][0] = mfma32(WL[s], B[j][s], acc[j][0]);
     };
@@ -328,7 +353,7 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
 }
 
 // true when mlpWideKernel can take this call: 32 inputs per sample in contiguous rows of e4m3 bytes or
-// (to be quantised on the way in) of fp16, ReLU hidden layers of exactly 32 or 64 units without biases, at most 32 outputs in whole
+// (to be quantised on the way in) of fp16, ReLU hidden layers of exactly 32 or 64 units, at most 32 outputs in whole
 // groups of four with 8-byte aligned rows
 inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
 {
@@ -339,7 +364,6 @@ inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
     const int width = a.layers[0].out;
     if (width != 32 && width != 64) return false;
     for (int l = 0; l < L; ++l) {
-        if (a.layers[l].bias != nullptr) return false;
         if (l + 1 < L && (a.layers[l].out != width || a.layers[l].act != kActRelu)) return false;
         if (l > 0 && a.layers[l].in != width) return false;
     }
@@ -350,24 +374,33 @@ inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
     return true;
 }
 
-template <int H, int NH, int OQ, bool IN_HALF>
+template <int H, int NH, int OQ, bool IN_HALF, bool HAS_BIAS>
 hipError_t launchMlpWideShape(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     // one workgroup per compute unit, as many waves as the weights leave registers for
     // (16 waves: 128 registers each, 12: 168, 8: 256); the build fails if an instantiation spills
-    constexpr int WAVES = H == 1 ? 16 : ((NH <= 2 && !(IN_HALF && OQ == 4)) ? 12 : 8);
+    constexpr bool twelve = (NH == 1 && !(HAS_BIAS && (IN_HALF || OQ == 4))) || (NH == 2 && !HAS_BIAS && !(IN_HALF && OQ == 4));
+    constexpr int WAVES = H == 1 ? 16 : (twelve ? 12 : 8);
     const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
     const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
-    noteKernel(false, "mlpWideKernel<e4m3-f16pipe,32x32x16,hidden=%dx%d,outputs<=%d%s>", NH, 32 * H, 8 * OQ,
-               IN_HALF ? ",fp16-vectors" : "");
-    hipLaunchKernelGGL((mlpWideKernel<H, NH, OQ, WAVES, IN_HALF>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+    noteKernel(false, "mlpWideKernel<e4m3-f16pipe,32x32x16,hidden=%dx%d,outputs<=%d,%s%s>", NH, 32 * H, 8 * OQ,
+               HAS_BIAS ? "bias" : "nobias", IN_HALF ? ",fp16-vectors" : "");
+    hipLaunchKernelGGL((mlpWideKernel<H, NH, OQ, WAVES, IN_HALF, HAS_BIAS>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
     return hipGetLastError();
 }
 
 inline hipError_t launchMlpWide(hipStream_t stream, const MlpArgs& a, int numCUs, int H, int NH, int OQ)
 {
-#define CV_W(h_, nh_, oq_) if (H == h_ && NH == nh_ && OQ == oq_) \
-        return a.inHalfAsE4M3 ? launchMlpWideShape<h_, nh_, oq_, true>(stream, a, numCUs) : launchMlpWideShape<h_, nh_, oq_, false>(stream, a, numCUs);
+    bool hasBias = false;
+    for (int l = 0; l < a.numLayers; ++l) hasBias = hasBias || a.layers[l].bias != nullptr;
+    const int variant = (a.inHalfAsE4M3 ? 1 : 0) + (hasBias ? 2 : 0);
+#define CV_W(h_, nh_, oq_) if (H == h_ && NH == nh_ && OQ == oq_) { \
+        switch (variant) { \
+        case 0: return launchMlpWideShape<h_, nh_, oq_, false, false>(stream, a, numCUs); \
+        case 1: return launchMlpWideShape<h_, nh_, oq_, true, false>(stream, a, numCUs); \
+        case 2: return launchMlpWideShape<h_, nh_, oq_, false, true>(stream, a, numCUs); \
+        default: return launchMlpWideShape<h_, nh_, oq_, true, true>(stream, a, numCUs); \
+        } }
     CV_W(2, 1, 1) CV_W(2, 2, 1) CV_W(2, 3, 1) CV_W(1, 1, 1) CV_W(1, 2, 1) CV_W(1, 3, 1)
     CV_W(2, 1, 2) CV_W(2, 2, 2) CV_W(2, 3, 2) CV_W(2, 1, 4) CV_W(2, 2, 4) CV_W(2, 3, 4)
 #undef CV_W

@@ -307,6 +307,29 @@ def test_fp16_vectors_on_32_sample_tiles(dims, B):
     assert torch.equal(y_half.view(torch.int16), yc.view(torch.int16))
 
 
+@pytest.mark.parametrize("dims,B", [([32, 64, 64, 8], 3000), ([32, 64, 16], 65), ([32, 32, 32, 32, 8], 500), ([32, 64, 64, 64, 32], 129)])
+@pytest.mark.parametrize("fp16_vectors", [False, True])
+def test_biases_on_32_sample_tiles(dims, B, fp16_vectors):
+    # biases enter the 32-sample kernel as one more k-step (bias x 1.0 into zeroed accumulators), which
+    # leaves float(bias) where the 16-sample kernels seed their accumulators: same bits as the chain.
+    # One layer has no bias (a null pointer next to layers that have one).
+    rng = np.random.default_rng(sum(dims) + 3 * B)
+    specs = make_net(rng, dims, CT.FloatE4M3, bias="rand", init="half")
+    specs[1]["b"] = None
+    x = ob.encode_e4m3(rng.standard_normal((B, 32)) * 0.5)
+    xd = to_dev(x)
+    xin = to_dev(ob.decode_e4m3(x).astype(np.float16)) if fp16_vectors else xd
+    hid = []
+    yc = chain_of_single_layers(specs, xd, CT.FloatE4M3, hidden=hid)
+    for layout in (ML.RowMajor, ML.InferencingOptimal):
+        y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, layout), xin, weightType=CT.FloatE4M3)
+        name = cv.lastKernelName()
+        assert name.startswith("mlpWideKernel") and ",bias" in name and ("fp16-vectors" in name) == fp16_vectors, name
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), layout
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, ob.E4M3, hid)
+    assert frac >= 0.99
+
+
 @pytest.mark.parametrize("B", [4096, 50])
 def test_e4m3_saturation_on_32_sample_tiles(B):
     # ReLU networks (the 32-sample kernel): hidden sums beyond 448, also through an fp16 overflow, saturate
