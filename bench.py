@@ -10,9 +10,9 @@ metric is quoted on: a single fp16 coopVecMatMulAdd layer 64x64 (fp32 accumulate
 reported as `layout_conversion_us`).  Without --workload every other configuration is timed the same
 way in the same run (W warm-up steps, K timed steps, HIP events on the launch stream) and reported
 under "workloads": c1, c2b (c2 in bfloat16), c3, c4 (e4m3 decoded to the fp16 matrix pipeline), c4n
-(fp8 matrix pipeline), c5 (training step), op / rs (stand-alone outer-product / reduce-sum
+(fp8 matrix pipeline), c4h (c4 fed with fp16 vectors), c5 (training step), op / rs (stand-alone outer-product / reduce-sum
 accumulate).  With --workload only that one runs and becomes the headline (profiling runs; also
-c4h = c4 fed with fp16 vectors, c5g = c5 on the layer-by-layer step, copy = a plain device copy of
+c5g = c5 on the layer-by-layer step, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
 Before the W warm-up steps of a workload its step runs untimed for --clock-ramp-ms (default 100 ms,
@@ -44,17 +44,17 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 # HBM bytes per step (all kernels of the step) as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
 # scaled by a copy of known size): not measured by this script, quoted from the committed profile summaries.
 PROFILED_TRAFFIC = {
-    "c1": (717000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
-    "c2": (1084790000, "profiles/matmul_f16_64x64_batch4M.md"),
-    "c2b": (1084793000, "profiles/matmul_bf16_64x64_batch4M.md"),
-    "c3": (2684680000, "profiles/matmul_i8_128x128_batch4M.md"),
-    "c4": (805459000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c4n": (805467000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c4h": (1342320000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
+    "c1": (732000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
+    "c2": (1084765000, "profiles/matmul_f16_64x64_batch4M.md"),
+    "c2b": (1084788000, "profiles/matmul_bf16_64x64_batch4M.md"),
+    "c3": (2684654000, "profiles/matmul_i8_128x128_batch4M.md"),
+    "c4": (805499000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
+    "c4n": (820414000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
+    "c4h": (1342505000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c5": (47832000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
-    "op": (285453000, "profiles/outer_product_64x64_batch1M.md"),
-    "rs": (537966000, "profiles/reduce_sum_64_batch4M.md"),
-    "copy": (1073742000, "profiles/copy_calibration_512MiB.md"),
+    "op": (285455000, "profiles/outer_product_64x64_batch1M.md"),
+    "rs": (537964000, "profiles/reduce_sum_64_batch4M.md"),
+    "copy": (1073743000, "profiles/copy_calibration_512MiB.md"),
 }
 
 
@@ -461,7 +461,7 @@ WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2b": workload_c2b, "c3": wo
              "c4n": workload_c4n, "c5": workload_c5, "op": workload_op, "rs": workload_rs,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4n", "c5", "op", "rs")
+DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4h", "c4n", "c5", "op", "rs")
 HEADLINE = "c2"
 
 
