@@ -249,8 +249,13 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
     x = x_maker(torch, g, B, dims[0], dev)
     out = torch.empty(B, dims[-1], dtype=torch.float16, device=dev)
 
+    # the network description is marshalled once, as a C caller fills its CvMlpDesc once: a step is the
+    # C-ABI call with the vectors (for the small configuration the Python marshalling would otherwise
+    # cost more than the kernel)
+    plan = cv.MlpForwardPlan(layers, weightType=wtype, flags=flags)
+
     def step():
-        cv.mlpForward(layers, x, weightType=wtype, out=out, flags=flags)
+        plan(x, out)
 
     macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
     in_bytes = dims[0] * x.element_size()

@@ -577,6 +577,40 @@ def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
     return out
 
 
+class MlpForwardPlan:
+    """mlpForward with the network description marshalled once.
+
+    The example's host program fills its constant buffer of per-layer device addresses once and
+    dispatches many times (mlp-training-coopvec.cpp:146-161, :319-334); a C caller of cvMlpForward does
+    the same with one CvMlpDesc.  This is that pattern for the Python mirror: the descriptor is built
+    here, a call only passes the vectors.  The layers' buffers must stay alive and in place (the plan
+    keeps references), and a change of a FeedForwardLayer after the plan was made is not seen."""
+
+    def __init__(self, layers: Sequence[FeedForwardLayer], *, weightType: int = CoopVecComponentType.Float16,
+                 flags: int = 0, inputEncoding: int = 0):
+        self._layers = list(layers)
+        self._weightType = weightType
+        self._desc, self._keep = _mlp_desc(self._layers, weightType, CoopVecComponentType.Float32, flags, inputEncoding)
+        self._ref = ctypes.byref(self._desc)
+        self._fn = _lib.load().cvMlpForward
+        self._outputSize = self._layers[-1].outputSize
+        self._inCt = None
+
+    def __call__(self, input: torch.Tensor, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+        inCt, inStride = _vector_info(input, self._weightType, "input")
+        if inCt != self._inCt:
+            self._desc.inputType = int(inCt)
+            self._inCt = inCt
+        batch = input.shape[0]
+        if out is None:
+            out = torch.empty((batch, self._outputSize), dtype=torch.float16, device=input.device)
+        _, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
+        rc = self._fn(_stream_handle(stream), self._ref, input.data_ptr(), inStride, out.data_ptr(), outStride, batch)
+        if rc < 0:
+            _check(rc)
+        return out
+
+
 def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
                               gradType: int = CoopVecComponentType.Float32, flags: int = 0, inputEncoding: int = 0) -> int:
     d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, flags, inputEncoding)

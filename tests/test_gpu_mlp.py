@@ -355,6 +355,31 @@ def test_e4m3_saturation_on_32_sample_tiles(B):
     assert np.array_equal(got[np.isinf(ref)], ref[np.isinf(ref)])
 
 
+def test_forward_plan_equals_mlp_forward():
+    # the prepared call (descriptor marshalled once) is the same C-ABI call: same bits, same errors
+    rng = np.random.default_rng(21)
+    for wtype, dims in ((CT.Float16, [2, 16, 16, 16, 1]), (CT.FloatE4M3, [32, 64, 64, 8])):
+        specs = make_net(rng, dims, wtype, bias="rand" if wtype == CT.Float16 else "none", init="he" if wtype == CT.Float16 else "half")
+        layers = gpu_layers(specs, wtype, ML.RowMajor)
+        if wtype == CT.Float16:
+            xd = to_dev(rng.uniform(-1, 1, (1000, dims[0])).astype(np.float16))
+        else:
+            xd = to_dev(ob.encode_e4m3(rng.standard_normal((1000, dims[0])) * 0.5))
+        plan = cv.MlpForwardPlan(layers, weightType=wtype)
+        y0 = cv.mlpForward(layers, xd, weightType=wtype)
+        y1 = plan(xd)
+        out = torch.empty_like(y0)
+        y2 = plan(xd[:333], out=out[:333])
+        assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+        assert torch.equal(y0[:333].view(torch.int16), y2.view(torch.int16))
+        if wtype == CT.FloatE4M3:       # the same plan takes fp16 vectors (quantised on load)
+            xh = to_dev(ob.decode_e4m3(xd.cpu().numpy()).astype(np.float16))
+            assert torch.equal(plan(xh).view(torch.int16), y0.view(torch.int16))
+            assert torch.equal(plan(xd).view(torch.int16), y0.view(torch.int16))
+        with pytest.raises(cv.CoopVecError):
+            plan(xd[:, ::2])
+
+
 def test_mlp_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_net(rng, [8, 16, 4], CT.Float16)
