@@ -360,7 +360,7 @@ inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
     const int L = a.numLayers;
     if (L < 2 || L > 4 || a.inEncoding != kEncodeNone) return false;
     const uint64_t rowBytes = a.inHalfAsE4M3 ? 64u : 32u;
-    if (a.layers[0].in != 32 || a.inStride != rowBytes || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0) return false;
+    if (a.layers[0].in != 32 || a.inStride != rowBytes || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0 || a.batch > (1u << 31)) return false;
     const int width = a.layers[0].out;
     if (width != 32 && width != 64) return false;
     for (int l = 0; l < L; ++l) {
