@@ -330,6 +330,39 @@ def test_biases_on_32_sample_tiles(dims, B, fp16_vectors):
     assert frac >= 0.99
 
 
+def test_32_sample_tiles_keep_the_summation_order():
+    # The last layer's fp32 sums reach the fp16 output without any coarser rounding in between, so they
+    # show the order in which the 8-element chunks of k meet the accumulator: with hidden values and
+    # weights log-uniform over 2^-9 .. 2^4 the terms of one sum span far more than fp32 holds, most
+    # accumulations are inexact, and a different order moves the fp16 result in about one output of 10^4.
+    # The 32-sample kernel feeds the chunks in the order of the 16-sample operators: same bits on 6.4 million
+    # outputs.  (Layer 0 passes the inputs through: units 0..31 = relu(x), 32..63 = relu(-x), exact.)
+    rng = np.random.default_rng(1234)
+    B = 200000
+    mag = lambda shape: np.exp2(rng.uniform(-9, 4, shape)) * rng.choice([-1.0, 1.0], shape)
+    W0 = np.zeros((64, 32)); W0[np.arange(32), np.arange(32)] = 1.0; W0[32 + np.arange(32), np.arange(32)] = -1.0
+    W1 = ob.encode_e4m3(mag((32, 64)))
+    specs = [dict(W=ob.encode_e4m3(W0), b=None, act=int(Activation.ReLU), slope=0.0),
+             dict(W=W1, b=None, act=int(Activation.NoActivation), slope=0.0)]
+    x = ob.encode_e4m3(mag((B, 32)))
+    xd = to_dev(x)
+    yc = chain_of_single_layers(specs, xd, CT.FloatE4M3)
+    y = cv.mlpForward(gpu_layers(specs, CT.FloatE4M3, ML.RowMajor), xd, weightType=CT.FloatE4M3)
+    assert cv.lastKernelName().startswith("mlpWideKernel"), cv.lastKernelName()
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    # the case is exercised: summing the k axis in another order, in fp32, changes fp16 results
+    n = B
+    xf = ob.decode_e4m3(x[:n]).astype(np.float32)
+    hf = np.concatenate([np.maximum(xf, 0), np.maximum(-xf, 0)], axis=1)
+    wf = ob.decode_e4m3(W1).astype(np.float32)
+    fwd = np.zeros((n, 32), np.float32); bwd = np.zeros((n, 32), np.float32)
+    for k in range(64):
+        fwd += hf[:, k:k + 1] * wf[:, k][None, :]
+        bwd += hf[:, 63 - k:64 - k] * wf[:, 63 - k][None, :]
+    assert (fwd != bwd).mean() > 0.05
+    assert (fwd.astype(np.float16) != bwd.astype(np.float16)).sum() >= 5
+
+
 @pytest.mark.parametrize("B", [4096, 50])
 def test_e4m3_saturation_on_32_sample_tiles(B):
     # ReLU networks (the 32-sample kernel): hidden sums beyond 448, also through an fp16 overflow, saturate
