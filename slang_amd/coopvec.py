@@ -171,10 +171,13 @@ _TORCH_TO_CT = {
     torch.float32: CoopVecComponentType.Float32,
     torch.int8: CoopVecComponentType.SignedInt8,
     torch.uint8: CoopVecComponentType.UnsignedInt8,
+    torch.int16: CoopVecComponentType.SignedInt16,
     torch.int32: CoopVecComponentType.SignedInt32,
 }
 if hasattr(torch, "uint32"):
     _TORCH_TO_CT[torch.uint32] = CoopVecComponentType.UnsignedInt32
+if hasattr(torch, "uint16"):
+    _TORCH_TO_CT[torch.uint16] = CoopVecComponentType.UnsignedInt16
 if hasattr(torch, "float8_e4m3fn"):
     _TORCH_TO_CT[torch.float8_e4m3fn] = CoopVecComponentType.FloatE4M3
 if hasattr(torch, "float8_e5m2"):
@@ -304,8 +307,10 @@ def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpret
     batch = input.shape[0]
     if resultType is None:
         resultType = (CoopVecComponentType.SignedInt32 if inCt in (
-            CoopVecComponentType.SignedInt8, CoopVecComponentType.UnsignedInt8, CoopVecComponentType.SignedInt32,
+            CoopVecComponentType.SignedInt8, CoopVecComponentType.UnsignedInt8, CoopVecComponentType.SignedInt16,
+            CoopVecComponentType.UnsignedInt16, CoopVecComponentType.SignedInt32,
             CoopVecComponentType.UnsignedInt32) else
+            CoopVecComponentType.Float32 if inCt == CoopVecComponentType.Float32 else
             CoopVecComponentType.BFloat16 if inCt == CoopVecComponentType.BFloat16 else CoopVecComponentType.Float16)
     if out is None:
         if accumulate:

@@ -99,7 +99,8 @@ struct ComboKind {
     bool inUnsigned, matUnsigned;
 };
 
-bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
+// combinations served by a matrix instruction
+bool classifyMfmaCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
 {
     const bool noBias = biasInterp == CV_COMPONENT_NONE;
     ComboKind k{cv::MmaKind::F16, false, false};
@@ -145,6 +146,26 @@ bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t 
         return false;
     }
     if (out) *out = k;
+    return true;
+}
+
+// The scalar types the fallback's switch covers (hlsl.meta.slang:32866-32907) up to 32 bits.
+bool isPlainScalar(int32_t ct)
+{
+    return ct == CV_FLOAT16 || ct == CV_FLOAT32 || ct == CV_SINT8 || ct == CV_UINT8 || ct == CV_SINT16 || ct == CV_UINT16 ||
+           ct == CV_SINT32 || ct == CV_UINT32;
+}
+
+// Every combination of those types runs somewhere: on a matrix instruction where one exists, else as the
+// scalar definition (cv_matmul_scalar.hip): vectors stored as what they are interpreted as, results
+// half / float / int32 / uint32.
+bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
+{
+    if (classifyMfmaCombo(inType, inInterp, matInterp, biasInterp, resType, out)) return true;
+    const bool resOk = resType == CV_FLOAT16 || resType == CV_FLOAT32 || resType == CV_SINT32 || resType == CV_UINT32;
+    if (inType != inInterp || !isPlainScalar(inType) || !isPlainScalar(matInterp) || !resOk) return false;
+    if (biasInterp != CV_COMPONENT_NONE && !isPlainScalar(biasInterp)) return false;
+    if (out) *out = ComboKind{cv::MmaKind::Scalar, false, false};
     return true;
 }
 
@@ -406,6 +427,14 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     if (CV_FAILED(rc)) return rc;
     cv::MmaKind kind = combo.kind;
     if (kind == cv::MmaKind::Fp8AsF16 && (d->flags & CV_FLAG_FP8_MATRIX_PIPELINE)) kind = cv::MmaKind::Fp8Native;
+    if (kind == cv::MmaKind::Scalar) {
+        const bool floatRes = d->resultType == CV_FLOAT16 || d->resultType == CV_FLOAT32;
+        if (a.act > (floatRes ? CV_ACT_LEAKY_RELU : CV_ACT_RELU))
+            return fail(CV_E_NOT_AVAILABLE, "cvMatMul: activation %d with input %d, matrix %d, result %d (this combination takes NONE, RELU%s)",
+                        d->activation, d->inputType, d->matrixInterpretation, d->resultType, floatRes ? ", LEAKY_RELU" : "");
+        if (d->k > 12288)
+            return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d (limit 12288 for input %d, matrix %d)", d->k, d->inputType, d->matrixInterpretation);
+    }
     const hipError_t e = cv::launchMatMul((hipStream_t)stream, kind, a, cus);
     if (e == hipErrorInvalidValue)
         return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d is beyond what one 16-row block of the matrix can keep in LDS "

@@ -35,12 +35,15 @@ enum class MmaKind : int {
     Bf8AsF16 = 5,        // e5m2 vectors and matrix, decoded to fp16 operands
     F16VecAsE4M3 = 6,    // fp16 vectors quantised to e4m3 on load, e4m3 matrix (matMul only)
     I8AnySign = 7,       // signed/unsigned bytes on either side (matMul only)
-    F32 = 8              // fp32 vectors and matrix (matMul only)
+    F32 = 8,             // fp32 vectors and matrix (matMul only)
+    Scalar = 9           // combinations without a matrix instruction (16/32-bit integers, mixed forms): cv_matmul_scalar.hip
 };
 
 // Returns hipSuccess, or hipErrorInvalidValue when no kernel covers (m,k): k beyond what one
 // 16-row block of the matrix can hold in LDS.
 hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& args, int numCUs);
+// the scalar definition evaluated as written, for the combinations MmaKind::Scalar stands for
+hipError_t launchMatMulScalar(hipStream_t stream, const MatMulArgs& args, int numCUs);
 
 // ---- fused forward MLP --------------------------------------------------------------------
 constexpr int kMaxMlpLayers = 8;

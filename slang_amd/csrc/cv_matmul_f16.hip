@@ -27,6 +27,7 @@ hipError_t launchMatMul(hipStream_t stream, MmaKind kind, const MatMulArgs& a, i
     case MmaKind::I8: return launchMatMulI8(stream, a, numCUs);
     case MmaKind::I8AnySign: return launchMatMulI8AnySign(stream, a, numCUs);
     case MmaKind::F32: return launchMatMulF32(stream, a, numCUs);
+    case MmaKind::Scalar: return launchMatMulScalar(stream, a, numCUs);
     }
     return hipErrorInvalidValue;
 }

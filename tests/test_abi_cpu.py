@@ -123,6 +123,10 @@ def test_supported_combinations(lib):
     assert (ob.U32, ob.S8P, 4, ob.S8, ob.S32, ob.S32) in combos     # packed int8, as in
     # tools/slang-unit-test/unit-test-cooperative-type-metadata.cpp:667-701 (inputPackingFactor 4)
     assert (ob.E4M3, ob.E4M3, 1, ob.E4M3, ob.F16, ob.F16) in combos
+    # combinations without a matrix instruction run as the scalar definition
+    assert (ob.S16, ob.S16, 1, ob.S32, ob.S32, ob.S32) in combos
+    assert (ob.F32, ob.F32, 1, ob.S8, ob.F16, ob.F32) in combos
+    assert (ob.F64, ob.F64, 1, ob.F64, ob.F64, ob.F64) not in combos
 
 
 def _desc(**kw):
@@ -150,8 +154,13 @@ def test_matmul_argument_validation(lib):
     assert f(transpose=1) == E_INVALID                        # RowMajor + transpose, :32947
     assert f(accumulate=1, activation=1) == E_INVALID
     assert f(activation=9) == E_INVALID
-    assert f(inputType=ob.F32, inputInterpretation=ob.F32) == E_NOTAVAIL
-    assert f(matrixInterpretation=ob.U8) == E_NOTAVAIL
+    assert f(inputType=ob.F64, inputInterpretation=ob.F64, inputStride=512) == E_NOTAVAIL     # 64-bit types: not built
+    assert f(matrixInterpretation=ob.S64, matrixStride=512) == E_NOTAVAIL
+    assert f(inputType=ob.F16, inputInterpretation=ob.S16) == E_NOTAVAIL       # vectors reinterpreted as another plain type
+    assert f(matrixInterpretation=ob.E4M3, matrixStride=64, inputType=ob.F32, inputInterpretation=ob.F32,
+             inputStride=256) == E_NOTAVAIL                                    # 8-bit floats only with their own vectors
+    assert f(matrixInterpretation=ob.S16, layout=2) == E_NOTAVAIL              # no Optimal layout for 16-bit integers
+    assert f(matrixInterpretation=ob.S16, resultType=ob.S32, outputStride=256, activation=2) == E_NOTAVAIL   # leaky ReLU on integers
     assert f(inputType=ob.U32, inputInterpretation=ob.S8P, matrixInterpretation=ob.S8, resultType=ob.S32,
              k=6) == E_NOTAVAIL                               # packed needs k == 4*PackedK (:32846)
     assert f(input=0x1001) == E_INVALID                       # misaligned vector
