@@ -187,8 +187,8 @@ CV_API CvResult cvConvertMatrices(void* stream, void* dstBuffer, const CvMatrixD
  * W is M x k unless `transpose`, in which case memory holds k x M and is used transposed.
  * Float types accumulate in fp32, integer types in int32 (exact).
  * Type combinations: those with a matrix instruction (cvQuerySupportedCombinations lists all), and, for
- * the rest of the fallback's switch up to 32 bits (hlsl.meta.slang:32866-32907), every mix of SINT8/16/32,
- * UINT8/16/32, FLOAT16 and FLOAT32 for vector, matrix, bias and result (FLOAT16, FLOAT32, SINT32 or UINT32):
+ * the rest of the fallback's switch (hlsl.meta.slang:32866-32907), every mix of SINT8/16/32/64, UINT8/16/32/64,
+ * FLOAT16, FLOAT32 and FLOAT64 for vector, matrix, bias and result (FLOAT16/32/64, SINT32/64 or UINT32/64):
  * these run as the scalar definition, operands cast to the result type first, RowMajor / ColumnMajor only.
  * accumulate != 0 gives the member forms matMulAccum / matMulAddAccum
  * (hlsl.meta.slang:31476-31650): output += result (activation must be NONE).

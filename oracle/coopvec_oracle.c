@@ -211,13 +211,18 @@ static int elem_size(int ct)
 /* Slang CPU-target semantics                                                            */
 /* ===================================================================================== */
 
-/* A value of the CoopVec element type T.  T is one of FLOAT16 (bits in .h), FLOAT32,
- * SINT32, UINT32 -- the element types the reference's CPU tests and the example use. */
-typedef union { uint16_t h; float f; int32_t i; uint32_t u; } tval;
+/* A value of the CoopVec element type T.  T is one of FLOAT16 (bits in .h), FLOAT32, FLOAT64,
+ * SINT32, UINT32, SINT64, UINT64 (the integer pairs share their two's-complement bits). */
+typedef union { uint16_t h; float f; int32_t i; uint32_t u; double d; int64_t i64; uint64_t u64; } tval;
 
 static inline int t_supported(int T)
 {
-    return T == CVO_FLOAT16 || T == CVO_FLOAT32 || T == CVO_SINT32 || T == CVO_UINT32;
+    return T == CVO_FLOAT16 || T == CVO_FLOAT32 || T == CVO_SINT32 || T == CVO_UINT32 ||
+           T == CVO_FLOAT64 || T == CVO_SINT64 || T == CVO_UINT64;
+}
+static inline int t_size(int T)
+{
+    return T == CVO_FLOAT16 ? 2 : (T == CVO_FLOAT64 || T == CVO_SINT64 || T == CVO_UINT64) ? 8 : 4;
 }
 
 static inline uint16_t to_half(float f, int halfMode)
@@ -225,28 +230,36 @@ static inline uint16_t to_half(float f, int halfMode)
     return halfMode == CVO_HALF_SLANG_SOFT ? cvo_f32_to_f16_slang(f) : cvo_f32_to_f16_rne(f);
 }
 
-/* load<Wt>(p) then __arithmetic_cast<T>.  Wt is a scalar component type. */
+/* load<Wt>(p) then __arithmetic_cast<T>.  Wt is a scalar component type.  A source value is held as a
+ * double (every half / float / double exactly), as an int64, or as a uint64 (UINT64 sources). */
 static inline __attribute__((always_inline)) tval
 load_cast(const uint8_t* p, int Wt, int T, int halfMode, int* ok)
 {
-    tval r; r.u = 0;
-    int isFloatSrc = 0; float fs = 0.f; int64_t is = 0;
+    tval r; r.u64 = 0;
+    int kind = 0;   /* 0: signed integer in `is`, 1: unsigned 64-bit in `us`, 2: float in `fs` */
+    double fs = 0.0; int64_t is = 0; uint64_t us = 0;
     switch (Wt) {
-    case CVO_FLOAT16: { uint16_t h; memcpy(&h, p, 2); fs = cvo_f16_to_f32(h); isFloatSrc = 1; break; }
-    case CVO_FLOAT32: { memcpy(&fs, p, 4); isFloatSrc = 1; break; }
+    case CVO_FLOAT16: { uint16_t h; memcpy(&h, p, 2); fs = cvo_f16_to_f32(h); kind = 2; break; }
+    case CVO_FLOAT32: { float f; memcpy(&f, p, 4); fs = f; kind = 2; break; }
+    case CVO_FLOAT64: { memcpy(&fs, p, 8); kind = 2; break; }
     case CVO_SINT8: case CVO_SINT8_PACKED: { int8_t v; memcpy(&v, p, 1); is = v; break; }
     case CVO_UINT8: case CVO_UINT8_PACKED: { uint8_t v; memcpy(&v, p, 1); is = v; break; }
     case CVO_SINT16: { int16_t v; memcpy(&v, p, 2); is = v; break; }
     case CVO_UINT16: { uint16_t v; memcpy(&v, p, 2); is = v; break; }
     case CVO_SINT32: { int32_t v; memcpy(&v, p, 4); is = v; break; }
     case CVO_UINT32: { uint32_t v; memcpy(&v, p, 4); is = v; break; }
+    case CVO_SINT64: { memcpy(&is, p, 8); break; }
+    case CVO_UINT64: { memcpy(&us, p, 8); kind = 1; break; }
     default: *ok = 0; return r;
     }
     switch (T) {
-    case CVO_FLOAT16: r.h = to_half(isFloatSrc ? fs : (float)is, halfMode); break;
-    case CVO_FLOAT32: r.f = isFloatSrc ? fs : (float)is; break;
-    case CVO_SINT32:  r.i = isFloatSrc ? (int32_t)fs : (int32_t)is; break;
-    case CVO_UINT32:  r.u = isFloatSrc ? (uint32_t)fs : (uint32_t)is; break;
+    case CVO_FLOAT16: r.h = to_half(kind == 2 ? (float)fs : kind == 1 ? (float)us : (float)is, halfMode); break;
+    case CVO_FLOAT32: r.f = kind == 2 ? (float)fs : kind == 1 ? (float)us : (float)is; break;
+    case CVO_FLOAT64: r.d = kind == 2 ? fs : kind == 1 ? (double)us : (double)is; break;
+    case CVO_SINT32:  r.i = kind == 2 ? (int32_t)fs : kind == 1 ? (int32_t)us : (int32_t)is; break;
+    case CVO_UINT32:  r.u = kind == 2 ? (uint32_t)fs : kind == 1 ? (uint32_t)us : (uint32_t)is; break;
+    case CVO_SINT64:  r.i64 = kind == 2 ? (int64_t)fs : kind == 1 ? (int64_t)us : is; break;
+    case CVO_UINT64:  r.u64 = kind == 2 ? (uint64_t)fs : kind == 1 ? us : (uint64_t)is; break;
     default: *ok = 0;
     }
     return r;
@@ -254,10 +267,12 @@ load_cast(const uint8_t* p, int Wt, int T, int halfMode, int* ok)
 
 static inline __attribute__((always_inline)) tval t_mul(tval a, tval b, int T, int halfMode)
 {
-    tval r;
+    tval r; r.u64 = 0;
     switch (T) {
     case CVO_FLOAT16: r.h = to_half(cvo_f16_to_f32(a.h) * cvo_f16_to_f32(b.h), halfMode); break;
     case CVO_FLOAT32: r.f = a.f * b.f; break;
+    case CVO_FLOAT64: r.d = a.d * b.d; break;
+    case CVO_SINT64: case CVO_UINT64: r.u64 = a.u64 * b.u64; break;
     default:          r.u = a.u * b.u; break; /* two's complement wrap for both int types */
     }
     return r;
@@ -265,10 +280,12 @@ static inline __attribute__((always_inline)) tval t_mul(tval a, tval b, int T, i
 
 static inline __attribute__((always_inline)) tval t_add(tval a, tval b, int T, int halfMode)
 {
-    tval r;
+    tval r; r.u64 = 0;
     switch (T) {
     case CVO_FLOAT16: r.h = to_half(cvo_f16_to_f32(a.h) + cvo_f16_to_f32(b.h), halfMode); break;
     case CVO_FLOAT32: r.f = a.f + b.f; break;
+    case CVO_FLOAT64: r.d = a.d + b.d; break;
+    case CVO_SINT64: case CVO_UINT64: r.u64 = a.u64 + b.u64; break;
     default:          r.u = a.u + b.u; break;
     }
     return r;
@@ -276,14 +293,18 @@ static inline __attribute__((always_inline)) tval t_add(tval a, tval b, int T, i
 
 static inline void t_store(void* dst, int idx, tval v, int T)
 {
-    if (T == CVO_FLOAT16) memcpy((uint8_t*)dst + 2 * idx, &v.h, 2);
-    else                  memcpy((uint8_t*)dst + 4 * idx, &v.u, 4);
+    int sz = t_size(T);
+    if (sz == 2) memcpy((uint8_t*)dst + 2 * idx, &v.h, 2);
+    else if (sz == 8) memcpy((uint8_t*)dst + 8 * (size_t)idx, &v.u64, 8);
+    else memcpy((uint8_t*)dst + 4 * idx, &v.u, 4);
 }
 static inline tval t_load(const void* src, int idx, int T)
 {
-    tval v; v.u = 0;
-    if (T == CVO_FLOAT16) memcpy(&v.h, (const uint8_t*)src + 2 * idx, 2);
-    else                  memcpy(&v.u, (const uint8_t*)src + 4 * idx, 4);
+    tval v; v.u64 = 0;
+    int sz = t_size(T);
+    if (sz == 2) memcpy(&v.h, (const uint8_t*)src + 2 * idx, 2);
+    else if (sz == 8) memcpy(&v.u64, (const uint8_t*)src + 8 * (size_t)idx, 8);
+    else memcpy(&v.u, (const uint8_t*)src + 4 * idx, 4);
     return v;
 }
 
@@ -321,7 +342,7 @@ slang_matmul_impl(const void* input, int U, int packedK, int inInterp, int k,
     }
     int swap = (transpose != 0) ^ (layout == CVO_COLUMN_MAJOR);               /* :32862-32863 */
     for (int i = 0; i < M; ++i) {
-        tval r; r.u = 0;                                   /* CoopVec<T,M>(0): +0 in every T */
+        tval r; r.u64 = 0;                                 /* CoopVec<T,M>(0): +0 in every T */
         for (int j = 0; j < k; ++j) {
             int row = swap ? j : i;
             int col = swap ? i : j;

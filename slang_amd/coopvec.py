@@ -173,7 +173,11 @@ _TORCH_TO_CT = {
     torch.uint8: CoopVecComponentType.UnsignedInt8,
     torch.int16: CoopVecComponentType.SignedInt16,
     torch.int32: CoopVecComponentType.SignedInt32,
+    torch.int64: CoopVecComponentType.SignedInt64,
+    torch.float64: CoopVecComponentType.Float64,
 }
+if hasattr(torch, "uint64"):
+    _TORCH_TO_CT[torch.uint64] = CoopVecComponentType.UnsignedInt64
 if hasattr(torch, "uint32"):
     _TORCH_TO_CT[torch.uint32] = CoopVecComponentType.UnsignedInt32
 if hasattr(torch, "uint16"):
@@ -188,9 +192,13 @@ _CT_TO_TORCH = {
     CoopVecComponentType.BFloat16: torch.bfloat16,
     CoopVecComponentType.Float32: torch.float32,
     CoopVecComponentType.SignedInt32: torch.int32,
+    CoopVecComponentType.SignedInt64: torch.int64,
+    CoopVecComponentType.Float64: torch.float64,
 }
 if hasattr(torch, "uint32"):
     _CT_TO_TORCH[CoopVecComponentType.UnsignedInt32] = torch.uint32
+if hasattr(torch, "uint64"):
+    _CT_TO_TORCH[CoopVecComponentType.UnsignedInt64] = torch.uint64
 
 
 def lastKernelName() -> str:
@@ -310,6 +318,8 @@ def _matmul(input, inputInterpretation, k, matrix, matrixOffset, matrixInterpret
             CoopVecComponentType.SignedInt8, CoopVecComponentType.UnsignedInt8, CoopVecComponentType.SignedInt16,
             CoopVecComponentType.UnsignedInt16, CoopVecComponentType.SignedInt32,
             CoopVecComponentType.UnsignedInt32) else
+            CoopVecComponentType.SignedInt64 if inCt in (CoopVecComponentType.SignedInt64, CoopVecComponentType.UnsignedInt64) else
+            CoopVecComponentType.Float64 if inCt == CoopVecComponentType.Float64 else
             CoopVecComponentType.Float32 if inCt == CoopVecComponentType.Float32 else
             CoopVecComponentType.BFloat16 if inCt == CoopVecComponentType.BFloat16 else CoopVecComponentType.Float16)
     if out is None:

@@ -149,20 +149,21 @@ bool classifyMfmaCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int3
     return true;
 }
 
-// The scalar types the fallback's switch covers (hlsl.meta.slang:32866-32907) up to 32 bits.
+// The scalar types the fallback's switch covers (hlsl.meta.slang:32866-32907).
 bool isPlainScalar(int32_t ct)
 {
-    return ct == CV_FLOAT16 || ct == CV_FLOAT32 || ct == CV_SINT8 || ct == CV_UINT8 || ct == CV_SINT16 || ct == CV_UINT16 ||
-           ct == CV_SINT32 || ct == CV_UINT32;
+    return ct == CV_FLOAT16 || ct == CV_FLOAT32 || ct == CV_FLOAT64 || ct == CV_SINT8 || ct == CV_UINT8 || ct == CV_SINT16 ||
+           ct == CV_UINT16 || ct == CV_SINT32 || ct == CV_UINT32 || ct == CV_SINT64 || ct == CV_UINT64;
 }
 
 // Every combination of those types runs somewhere: on a matrix instruction where one exists, else as the
 // scalar definition (cv_matmul_scalar.hip): vectors stored as what they are interpreted as, results
-// half / float / int32 / uint32.
+// half / float / double / int32 / uint32 / int64 / uint64.
 bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
 {
     if (classifyMfmaCombo(inType, inInterp, matInterp, biasInterp, resType, out)) return true;
-    const bool resOk = resType == CV_FLOAT16 || resType == CV_FLOAT32 || resType == CV_SINT32 || resType == CV_UINT32;
+    const bool resOk = resType == CV_FLOAT16 || resType == CV_FLOAT32 || resType == CV_FLOAT64 || resType == CV_SINT32 ||
+                       resType == CV_UINT32 || resType == CV_SINT64 || resType == CV_UINT64;
     if (inType != inInterp || !isPlainScalar(inType) || !isPlainScalar(matInterp) || !resOk) return false;
     if (biasInterp != CV_COMPONENT_NONE && !isPlainScalar(biasInterp)) return false;
     if (out) *out = ComboKind{cv::MmaKind::Scalar, false, false};
@@ -428,12 +429,14 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     cv::MmaKind kind = combo.kind;
     if (kind == cv::MmaKind::Fp8AsF16 && (d->flags & CV_FLAG_FP8_MATRIX_PIPELINE)) kind = cv::MmaKind::Fp8Native;
     if (kind == cv::MmaKind::Scalar) {
-        const bool floatRes = d->resultType == CV_FLOAT16 || d->resultType == CV_FLOAT32;
+        const bool floatRes = d->resultType == CV_FLOAT16 || d->resultType == CV_FLOAT32 || d->resultType == CV_FLOAT64;
         if (a.act > (floatRes ? CV_ACT_LEAKY_RELU : CV_ACT_RELU))
             return fail(CV_E_NOT_AVAILABLE, "cvMatMul: activation %d with input %d, matrix %d, result %d (this combination takes NONE, RELU%s)",
                         d->activation, d->inputType, d->matrixInterpretation, d->resultType, floatRes ? ", LEAKY_RELU" : "");
-        if (d->k > 12288)
-            return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d (limit 12288 for input %d, matrix %d)", d->k, d->inputType, d->matrixInterpretation);
+        const int kLimit = cv::elemSize(d->resultType) == 8 ? 6144 : 12288;
+        if (d->k > kLimit)
+            return fail(CV_E_NOT_AVAILABLE, "cvMatMul: k=%d (limit %d for input %d, matrix %d, result %d)", d->k, kLimit, d->inputType,
+                        d->matrixInterpretation, d->resultType);
     }
     const hipError_t e = cv::launchMatMul((hipStream_t)stream, kind, a, cus);
     if (e == hipErrorInvalidValue)

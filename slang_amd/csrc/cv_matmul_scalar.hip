@@ -1,10 +1,10 @@
 // cv_matmul_scalar.hip -- coopVecMatMul[Add] for the type combinations that have no matrix instruction:
 // 16- and 32-bit integer matrices or vectors, and mixed forms such as fp32 vectors against an int8
 // matrix or fp16 vectors against an fp32 matrix.  The scalar definition (source/slang/hlsl.meta.slang:
-// 32835-32912, bias :33043-33103) is evaluated as it is written, one thread per sample:
+// 32835-32912, bias :33043-33103) is evaluated as it is written, one thread per sample (also for the 64-bit types):
 //     v[j] = cast<T>(input[j]);   r[i] = sum_j cast<T>(W[i][j]) * v[j]   (j ascending);   r[i] += cast<T>(bias[i])
-// with T = int32/uint32 in two's complement (exact, wraps like the reference), or T = float with every
-// product and sum rounded to fp32 in that order (no fused multiply-add), or T = half with the operands
+// with T = int32/uint32/int64/uint64 in two's complement (exact, wraps like the reference), or T = float / double
+// with every product and sum rounded to T in that order (no fused multiply-add), or T = half with the operands
 // cast to half, products and sums in fp32 and one rounding of the result (the rule of the matrix-pipeline
 // kernels).  The matrix block lives in LDS already cast to the accumulation type and is read as a broadcast.
 #include "cv_device.h"
@@ -12,41 +12,60 @@
 #include "cv_kernels.h"
 #include "cv_launch.h"
 
+#include <type_traits>
+
 namespace cv {
 namespace {
 
-// load<ct>(p) as an int32 bit pattern (8/16-bit sources sign- or zero-extended) or as a float
-__device__ __forceinline__ int32_t loadAsInt(const uint8_t* p, int ct)
+// The accumulation type per result type T: two's-complement integers of T's width (signed and unsigned share
+// their bits), float for half / float results, double for double.
+enum : int { kAccI32 = 0, kAccF32 = 1, kAccI64 = 2, kAccF64 = 3 };
+template <int ACC> struct AccOf;
+template <> struct AccOf<kAccI32> { typedef uint32_t type; };
+template <> struct AccOf<kAccF32> { typedef float type; };
+template <> struct AccOf<kAccI64> { typedef uint64_t type; };
+template <> struct AccOf<kAccF64> { typedef double type; };
+
+// load<ct>(p) followed by __arithmetic_cast to the accumulation type.  Integer targets: sign or zero extension /
+// truncation to the low bits, floats towards zero; `dstUnsigned` picks the unsigned float->integer conversion.
+// Float targets: nearest even; `viaHalf` (T = half) rounds the operand to half first.
+template <int ACC>
+__device__ __forceinline__ typename AccOf<ACC>::type loadCast(const uint8_t* p, int ct, bool dstUnsigned, bool viaHalf)
 {
-    switch (ct) {
-    case kS8: return (int32_t) * (const int8_t*)p;
-    case kU8: return (int32_t) * p;
-    case kS16: return (int32_t) * (const int16_t*)p;
-    case kU16: return (int32_t) * (const uint16_t*)p;
-    case kS32: case kU32: return *(const int32_t*)p;
-    case kF16: return (int32_t)(float)*(const half_t*)p;      // __arithmetic_cast<int>(half): towards zero
-    case kF32: return (int32_t) * (const float*)p;
+    typedef typename AccOf<ACC>::type A;
+    if constexpr (ACC == kAccI32 || ACC == kAccI64) {
+        typedef typename std::conditional<ACC == kAccI32, int32_t, int64_t>::type S;
+        switch (ct) {
+        case kS8: return (A)(S) * (const int8_t*)p;
+        case kU8: return (A) * p;
+        case kS16: return (A)(S) * (const int16_t*)p;
+        case kU16: return (A) * (const uint16_t*)p;
+        case kS32: return (A)(S) * (const int32_t*)p;
+        case kU32: return (A) * (const uint32_t*)p;
+        case kS64: case kU64: return (A) * (const uint64_t*)p;
+        case kF16: { const float f = (float)*(const half_t*)p; return dstUnsigned ? (A)f : (A)(S)f; }
+        case kF32: { const float f = *(const float*)p; return dstUnsigned ? (A)f : (A)(S)f; }
+        case kF64: { const double f = *(const double*)p; return dstUnsigned ? (A)f : (A)(S)f; }
+        }
+        return 0;
+    } else {
+        A f = 0;
+        switch (ct) {
+        case kF16: return (A)(float)*(const half_t*)p;
+        case kF32: f = (A) * (const float*)p; break;
+        case kF64: f = (A) * (const double*)p; break;
+        case kS8: f = (A) * (const int8_t*)p; break;
+        case kU8: f = (A) * p; break;
+        case kS16: f = (A) * (const int16_t*)p; break;
+        case kU16: f = (A) * (const uint16_t*)p; break;
+        case kS32: f = (A) * (const int32_t*)p; break;
+        case kU32: f = (A) * (const uint32_t*)p; break;
+        case kS64: f = (A) * (const int64_t*)p; break;
+        case kU64: f = (A) * (const uint64_t*)p; break;
+        }
+        if constexpr (ACC == kAccF32) return viaHalf ? (float)(half_t)f : f;       // T = half: cast<half>(x), nearest even
+        else return f;
     }
-    return 0;
-}
-__device__ __forceinline__ uint32_t loadAsUint(const uint8_t* p, int ct)
-{
-    switch (ct) {
-    case kF16: return (uint32_t)(float)*(const half_t*)p;
-    case kF32: return (uint32_t) * (const float*)p;
-    }
-    return (uint32_t)loadAsInt(p, ct);       // integers: the same bits modulo 2^32
-}
-__device__ __forceinline__ float loadAsFloat(const uint8_t* p, int ct, bool viaHalf)
-{
-    float f;
-    switch (ct) {
-    case kF16: return (float)*(const half_t*)p;
-    case kF32: f = *(const float*)p; break;
-    case kU32: f = (float)*(const uint32_t*)p; break;
-    default: f = (float)loadAsInt(p, ct); break;
-    }
-    return viaHalf ? (float)(half_t)f : f;       // T = half: cast<half>(x), nearest even
 }
 
 struct ScalarArgs {
@@ -54,16 +73,19 @@ struct ScalarArgs {
     uint32_t rowsPerBlock;      // matrix rows kept in LDS at once
 };
 
-constexpr int kScalarLdsElems = 12288;      // 48 KB of 4-byte elements
+constexpr int kScalarLdsBytes = 49152;      // of LDS for the matrix block
 constexpr int kRowChunk = 8;                // output rows accumulated in registers at once
 
-template <bool IS_FLOAT>
+template <int ACC>
 __global__ __launch_bounds__(256) void matmulScalarKernel(const ScalarArgs sa)
 {
+    typedef typename AccOf<ACC>::type A;
+    constexpr bool IS_FLOAT = ACC == kAccF32 || ACC == kAccF64;
     const MatMulArgs& a = sa.mm;
-    __shared__ uint32_t ldsW[kScalarLdsElems];
+    __shared__ __attribute__((aligned(8))) uint8_t ldsRaw[kScalarLdsBytes];
+    A* ldsW = (A*)ldsRaw;
     const int m = a.m, k = a.k;
-    const bool resHalf = a.outCt == kF16, resUnsigned = a.outCt == kU32;
+    const bool resHalf = a.outCt == kF16, resUnsigned = a.outCt == kU32 || a.outCt == kU64;
     const uint32_t inEsz = elemSize(a.inCt), outEsz = elemSize(a.outCt);
     const uint32_t biasEsz = a.bias ? elemSize(a.biasCt) : 0;
 
@@ -74,35 +96,23 @@ __global__ __launch_bounds__(256) void matmulScalarKernel(const ScalarArgs sa)
             const int i = e / k, j = e % k;
             const uint8_t* p = a.mat + (a.transpose ? elemOffset(a.shape, (uint32_t)j, (uint32_t)(r0 + i))
                                                     : elemOffset(a.shape, (uint32_t)(r0 + i), (uint32_t)j));
-            if constexpr (IS_FLOAT) ldsW[e] = __builtin_bit_cast(uint32_t, loadAsFloat(p, a.shape.ct, resHalf));
-            else ldsW[e] = resUnsigned ? loadAsUint(p, a.shape.ct) : (uint32_t)loadAsInt(p, a.shape.ct);
+            ldsW[e] = loadCast<ACC>(p, a.shape.ct, resUnsigned, resHalf);
         }
         __syncthreads();
         for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < a.batch; s += gridDim.x * 256u) {
             const uint8_t* x = a.in + (size_t)s * a.inStride;
             uint8_t* y = a.out + (size_t)s * a.outStride;
             for (int c0 = 0; c0 < rows; c0 += kRowChunk) {
-                float accF[kRowChunk];
-                uint32_t accI[kRowChunk];
+                A acc[kRowChunk];
 #pragma unroll
-                for (int r = 0; r < kRowChunk; ++r) { accF[r] = 0.f; accI[r] = 0u; }
+                for (int r = 0; r < kRowChunk; ++r) acc[r] = 0;
                 for (int j = 0; j < k; ++j) {
-                    const uint8_t* xp = x + (size_t)j * inEsz;
-                    if constexpr (IS_FLOAT) {
-                        const float v = loadAsFloat(xp, a.inCt, resHalf);
+                    const A v = loadCast<ACC>(x + (size_t)j * inEsz, a.inCt, resUnsigned, resHalf);
 #pragma unroll
-                        for (int r = 0; r < kRowChunk; ++r) {
-                            const int row = c0 + r < rows ? c0 + r : rows - 1;
-                            const float p = __builtin_bit_cast(float, ldsW[row * k + j]) * v;     // rounded product ...
-                            accF[r] = accF[r] + p;                                                 // ... then rounded sum
-                        }
-                    } else {
-                        const uint32_t v = resUnsigned ? loadAsUint(xp, a.inCt) : (uint32_t)loadAsInt(xp, a.inCt);
-#pragma unroll
-                        for (int r = 0; r < kRowChunk; ++r) {
-                            const int row = c0 + r < rows ? c0 + r : rows - 1;
-                            accI[r] += ldsW[row * k + j] * v;
-                        }
+                    for (int r = 0; r < kRowChunk; ++r) {
+                        const int row = c0 + r < rows ? c0 + r : rows - 1;
+                        const A p = ldsW[row * k + j] * v;      // floats: a rounded product ...
+                        acc[r] = acc[r] + p;                    // ... then a rounded sum (no contraction: -ffp-contract=off)
                     }
                 }
 #pragma unroll
@@ -110,29 +120,27 @@ __global__ __launch_bounds__(256) void matmulScalarKernel(const ScalarArgs sa)
                     const int i = r0 + c0 + r;
                     if (c0 + r >= rows) break;
                     uint8_t* o = y + (size_t)i * outEsz;
-                    if constexpr (IS_FLOAT) {
-                        float z = accF[r];
-                        if (a.bias) z = z + loadAsFloat(a.bias + (size_t)i * biasEsz, a.biasCt, resHalf);
+                    A z = acc[r];
+                    if (a.bias) z = z + loadCast<ACC>(a.bias + (size_t)i * biasEsz, a.biasCt, resUnsigned, resHalf);
+                    if constexpr (ACC == kAccF32) {
                         if (resHalf) {
                             half_t hz = (half_t)z;
                             if (a.act == kActRelu) hz = hz > (half_t)0.f ? hz : (half_t)0.f;
                             else if (a.act == kActLeakyRelu) { const half_t t = (half_t)(hz * (half_t)a.slope); hz = hz > t ? hz : t; }
                             if (a.accumulate) hz = (half_t)((float)*(const half_t*)o + (float)hz);
                             *(half_t*)o = hz;
-                        } else {
-                            if (a.act == kActRelu) z = z > 0.f ? z : 0.f;
-                            else if (a.act == kActLeakyRelu) { const float t = z * a.slope; z = z > t ? z : t; }
-                            if (a.accumulate) z = *(const float*)o + z;
-                            *(float*)o = z;
+                            continue;
                         }
-                    } else {
-                        uint32_t z = accI[r];
-                        if (a.bias) z += resUnsigned ? loadAsUint(a.bias + (size_t)i * biasEsz, a.biasCt)
-                                                     : (uint32_t)loadAsInt(a.bias + (size_t)i * biasEsz, a.biasCt);
-                        if (a.act == kActRelu && !resUnsigned) z = (int32_t)z > 0 ? z : 0u;
-                        if (a.accumulate) z += *(const uint32_t*)o;
-                        *(uint32_t*)o = z;
                     }
+                    if constexpr (IS_FLOAT) {
+                        if (a.act == kActRelu) z = z > (A)0 ? z : (A)0;
+                        else if (a.act == kActLeakyRelu) { const A t = z * (A)a.slope; z = z > t ? z : t; }
+                    } else {
+                        typedef typename std::conditional<ACC == kAccI32, int32_t, int64_t>::type S;
+                        if (a.act == kActRelu && !resUnsigned) z = (S)z > 0 ? z : (A)0;
+                    }
+                    if (a.accumulate) z = *(const A*)o + z;
+                    *(A*)o = z;
                 }
             }
         }
@@ -145,21 +153,27 @@ __global__ __launch_bounds__(256) void matmulScalarKernel(const ScalarArgs sa)
 hipError_t launchMatMulScalar(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
     if (a.batch == 0) return hipSuccess;
-    if (a.k > kScalarLdsElems) return hipErrorInvalidValue;
+    const int acc = a.outCt == kF16 || a.outCt == kF32 ? kAccF32 : a.outCt == kF64 ? kAccF64
+                  : (a.outCt == kS64 || a.outCt == kU64) ? kAccI64 : kAccI32;
+    const int capacity = kScalarLdsBytes / ((acc == kAccI64 || acc == kAccF64) ? 8 : 4);
+    if (a.k > capacity) return hipErrorInvalidValue;
     ScalarArgs sa;
     sa.mm = a;
-    uint32_t rpb = (uint32_t)(kScalarLdsElems / a.k);
+    uint32_t rpb = (uint32_t)(capacity / a.k);
     if (rpb > (uint32_t)a.m) rpb = (uint32_t)a.m;
     if (rpb > kRowChunk) rpb = rpb / kRowChunk * kRowChunk;
     sa.rowsPerBlock = rpb;
-    const bool isFloat = a.outCt == kF16 || a.outCt == kF32;
     const uint32_t needed = (a.batch + 255u) / 256u;
     const uint32_t maxBlocks = (uint32_t)numCUs * 8u;
     const uint32_t blocks = needed < maxBlocks ? needed : maxBlocks;
-    noteKernel(false, "matmulScalarKernel<%s,in=%d,matrix=%d,out=%d,rows/block=%u>", isFloat ? "fp32-accumulate" : "int32", a.inCt,
-               a.shape.ct, a.outCt, rpb);
-    if (isFloat) hipLaunchKernelGGL(matmulScalarKernel<true>, dim3(blocks), dim3(256), 0, stream, sa);
-    else hipLaunchKernelGGL(matmulScalarKernel<false>, dim3(blocks), dim3(256), 0, stream, sa);
+    static const char* const names[4] = {"int32", "fp32-accumulate", "int64", "fp64"};
+    noteKernel(false, "matmulScalarKernel<%s,in=%d,matrix=%d,out=%d,rows/block=%u>", names[acc], a.inCt, a.shape.ct, a.outCt, rpb);
+    switch (acc) {
+    case kAccI32: hipLaunchKernelGGL(matmulScalarKernel<kAccI32>, dim3(blocks), dim3(256), 0, stream, sa); break;
+    case kAccF32: hipLaunchKernelGGL(matmulScalarKernel<kAccF32>, dim3(blocks), dim3(256), 0, stream, sa); break;
+    case kAccI64: hipLaunchKernelGGL(matmulScalarKernel<kAccI64>, dim3(blocks), dim3(256), 0, stream, sa); break;
+    default:      hipLaunchKernelGGL(matmulScalarKernel<kAccF64>, dim3(blocks), dim3(256), 0, stream, sa); break;
+    }
     return hipGetLastError();
 }
 

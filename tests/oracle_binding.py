@@ -117,7 +117,8 @@ def slang_matmul(x: np.ndarray, x_ct: int, in_interp: int, k: int, result_ct: in
                  half_mode: int = HALF_RNE) -> np.ndarray:
     """The Slang fallback operator itself (cvo_slang_matmul), one call per row of x.  x holds the
     vectors as they lie in memory (packed forms: k/4 32-bit elements per row)."""
-    res_np = {F16: np.float16, F32: np.float32, S32: np.int32, U32: np.uint32}[result_ct]
+    res_np = {F16: np.float16, F32: np.float32, S32: np.int32, U32: np.uint32, F64: np.float64, S64: np.int64,
+              U64: np.uint64}[result_ct]
     B, packedK = x.shape
     out = np.zeros((B, M), res_np)
     for b in range(B):

@@ -126,7 +126,8 @@ def test_supported_combinations(lib):
     # combinations without a matrix instruction run as the scalar definition
     assert (ob.S16, ob.S16, 1, ob.S32, ob.S32, ob.S32) in combos
     assert (ob.F32, ob.F32, 1, ob.S8, ob.F16, ob.F32) in combos
-    assert (ob.F64, ob.F64, 1, ob.F64, ob.F64, ob.F64) not in combos
+    assert (ob.F64, ob.F64, 1, ob.S64, ob.U64, ob.F64) in combos
+    assert (ob.BF16, ob.BF16, 1, ob.F16, ob.F16, ob.F16) not in combos
 
 
 def _desc(**kw):
@@ -154,8 +155,8 @@ def test_matmul_argument_validation(lib):
     assert f(transpose=1) == E_INVALID                        # RowMajor + transpose, :32947
     assert f(accumulate=1, activation=1) == E_INVALID
     assert f(activation=9) == E_INVALID
-    assert f(inputType=ob.F64, inputInterpretation=ob.F64, inputStride=512) == E_NOTAVAIL     # 64-bit types: not built
-    assert f(matrixInterpretation=ob.S64, matrixStride=512) == E_NOTAVAIL
+    assert f(inputType=ob.BF16, inputInterpretation=ob.BF16) == E_NOTAVAIL     # bfloat16 only with a bfloat16 matrix
+    assert f(matrixInterpretation=ob.E5M2, matrixStride=64) == E_NOTAVAIL      # 8-bit floats only with their own vectors
     assert f(inputType=ob.F16, inputInterpretation=ob.S16) == E_NOTAVAIL       # vectors reinterpreted as another plain type
     assert f(matrixInterpretation=ob.E4M3, matrixStride=64, inputType=ob.F32, inputInterpretation=ob.F32,
              inputStride=256) == E_NOTAVAIL                                    # 8-bit floats only with their own vectors

@@ -16,23 +16,24 @@ from slang_amd.coopvec import Activation, CoopVecMatrixLayout as ML
 
 pytestmark = pytest.mark.gpu
 
-NP = {ob.F16: np.float16, ob.F32: np.float32, ob.S8: np.int8, ob.U8: np.uint8, ob.S16: np.int16, ob.U16: np.uint16,
-      ob.S32: np.int32, ob.U32: np.uint32}
+NP = {ob.F16: np.float16, ob.F32: np.float32, ob.F64: np.float64, ob.S8: np.int8, ob.U8: np.uint8, ob.S16: np.int16,
+      ob.U16: np.uint16, ob.S32: np.int32, ob.U32: np.uint32, ob.S64: np.int64, ob.U64: np.uint64}
 
 
 def values(rng, ct, shape, small=False):
-    if ct in (ob.F16, ob.F32):
+    if ct in (ob.F16, ob.F32, ob.F64):
         return (rng.standard_normal(shape) * (2.0 if small else 8.0)).astype(NP[ct])
     info = np.iinfo(NP[ct])
     lo, hi = (max(info.min, -6), min(info.max, 6)) if small else (info.min, info.max)
-    return rng.integers(lo, hi, shape, dtype=np.int64, endpoint=True).astype(NP[ct])
+    return rng.integers(lo, hi, shape, dtype=NP[ct], endpoint=True)
 
 
 def dev(a):
     t = torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(a.shape[0], -1)).to(DEV)
     dt = {np.dtype(np.float16): torch.float16, np.dtype(np.float32): torch.float32, np.dtype(np.int8): torch.int8,
           np.dtype(np.uint8): torch.uint8, np.dtype(np.int16): torch.int16, np.dtype(np.uint16): torch.uint16,
-          np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32}[a.dtype]
+          np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32, np.dtype(np.int64): torch.int64,
+          np.dtype(np.uint64): torch.uint64, np.dtype(np.float64): torch.float64}[a.dtype]
     return t.view(dt)
 
 
@@ -40,6 +41,9 @@ INT_CASES = [  # (input, matrix, bias, result)
     (ob.S16, ob.S16, ob.S32, ob.S32), (ob.U16, ob.S16, None, ob.S32), (ob.S32, ob.S32, ob.S32, ob.S32),
     (ob.U32, ob.U32, ob.U32, ob.U32), (ob.S8, ob.S16, ob.S16, ob.S32), (ob.S16, ob.U8, ob.S8, ob.U32),
     (ob.S32, ob.U16, None, ob.U32), (ob.U8, ob.S32, ob.U16, ob.S32),
+    # 64-bit arms of the switch (hlsl.meta.slang:32873-32903): 64-bit matrices, vectors and results
+    (ob.S64, ob.S64, ob.S64, ob.S64), (ob.U64, ob.U64, None, ob.U64), (ob.S16, ob.S64, ob.S32, ob.S64),
+    (ob.S64, ob.S8, ob.U64, ob.S32), (ob.U32, ob.U64, ob.S16, ob.U32), (ob.S32, ob.S32, ob.S64, ob.S64),
 ]
 
 
@@ -68,12 +72,14 @@ def test_integer_combinations_bit_exact(in_ct, w_ct, b_ct, r_ct, layout):
 FLOAT_CASES = [  # (input, matrix, bias, result)
     (ob.F32, ob.S8, ob.F32, ob.F32), (ob.F32, ob.F16, None, ob.F32), (ob.F16, ob.F32, ob.F16, ob.F32),
     (ob.S16, ob.F32, ob.F32, ob.F32), (ob.F32, ob.S16, ob.S8, ob.F32), (ob.U8, ob.F16, ob.F16, ob.F32),
+    (ob.F64, ob.F64, ob.F64, ob.F64), (ob.F32, ob.F64, None, ob.F64), (ob.S32, ob.F16, ob.F64, ob.F64),
+    (ob.F64, ob.S64, ob.F32, ob.F32), (ob.S64, ob.F32, ob.S64, ob.F64),
 ]
 
 
 @pytest.mark.parametrize("in_ct,w_ct,b_ct,r_ct", FLOAT_CASES)
-def test_fp32_results_equal_the_scalar_definition(in_ct, w_ct, b_ct, r_ct):
-    # T = float: every product and every sum rounded to fp32, j ascending, bias last: the same bits as the fallback
+def test_float_results_equal_the_scalar_definition(in_ct, w_ct, b_ct, r_ct):
+    # T = float / double: every product and every sum rounded to T, j ascending, bias last: the same bits as the fallback
     rng = np.random.default_rng(in_ct * 100 + w_ct * 10 + 7)
     B, k, M = 257, 45, 19
     x = values(rng, in_ct, (B, k), small=True); W = values(rng, w_ct, (M, k), small=True)
@@ -87,11 +93,12 @@ def test_fp32_results_equal_the_scalar_definition(in_ct, w_ct, b_ct, r_ct):
     else:
         y = cv.coopVecMatMulAdd(dev(x), in_ct, wd, 0, w_ct, as_bytes(to_dev(bias)), 0, b_ct, ML.RowMajor, False, stride, M=M, resultType=r_ct)
     assert cv.lastKernelName().startswith("matmulScalarKernel"), cv.lastKernelName()
-    assert np.array_equal(y.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    bits = np.uint64 if r_ct == ob.F64 else np.uint32
+    assert np.array_equal(y.cpu().numpy().view(bits), ref.view(bits))
     # and the definition itself: fp64 of the same operands agrees to fp32 accuracy
     z = x.astype(np.float64) @ W.astype(np.float64).T + (bias.astype(np.float64) if bias is not None else 0.0)
     terms = np.abs(x.astype(np.float64)) @ np.abs(W.astype(np.float64)).T + 1.0
-    assert (np.abs(ref.astype(np.float64) - z) <= 2.0 ** -20 * terms).all()
+    assert (np.abs(ref.astype(np.float64) - z) <= 2.0 ** (-48 if r_ct == ob.F64 and ob.F16 not in (in_ct, w_ct) else -20) * terms).all()
 
 
 @pytest.mark.parametrize("in_ct,w_ct", [(ob.F32, ob.F32), (ob.F16, ob.S16), (ob.S32, ob.F16), (ob.F32, ob.U8)])

@@ -319,3 +319,43 @@ def test_ref_max_tie_rule():
     assert dB[0].tolist() == [1.0] and dW[0].tolist() == [[1.0]]      # 0.5 * (2*1)
     dW, dB, _ = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=False)
     assert dB[0].tolist() == [0.0]
+
+
+def test_slang_matmul_with_64_bit_types_against_exact_arithmetic():
+    """The 64-bit arms of the fallback's switch (hlsl.meta.slang:32873-32903) in the oracle: int64 / uint64
+    results equal Python's exact integers modulo 2^64 (full-range operands, so the sums wrap), float64
+    results equal numpy's float64 products and sums taken in the same order, and casts between widths
+    follow C (sign extension, truncation to the low bits, nearest-even float conversions)."""
+    rng = np.random.default_rng(64)
+    B, k, M = 5, 13, 7
+    NPT = {ob.S8: np.int8, ob.U16: np.uint16, ob.S32: np.int32, ob.S64: np.int64, ob.U64: np.uint64, ob.F32: np.float32, ob.F64: np.float64}
+
+    def rand(ct, shape):
+        if ct in (ob.F32, ob.F64):
+            return rng.standard_normal(shape).astype(NPT[ct]) * 3
+        info = np.iinfo(NPT[ct])
+        return rng.integers(info.min, info.max, shape, dtype=NPT[ct], endpoint=True)
+
+    for in_ct, w_ct, b_ct, r_ct in ((ob.S64, ob.S64, ob.S64, ob.S64), (ob.U64, ob.S32, ob.U16, ob.U64), (ob.S8, ob.U64, ob.S64, ob.S64),
+                                    (ob.S64, ob.U64, ob.S32, ob.S32)):
+        x, W, bias = rand(in_ct, (B, k)), rand(w_ct, (M, k)), rand(b_ct, (M,))
+        got = ob.slang_matmul(x, in_ct, in_ct, k, r_ct, M, W.view(np.uint8).reshape(-1), w_ct, ob.ROW, k * W.itemsize, bias, b_ct)
+        bits = 32 if r_ct == ob.S32 else 64
+        mod = 1 << bits
+        for b in range(B):
+            for i in range(M):
+                # cast<T> of each operand first (the low bits), then exact arithmetic modulo 2^bits
+                acc = sum((int(W[i, j]) % mod) * (int(x[b, j]) % mod) for j in range(k)) + int(bias[i]) % mod
+                assert int(got[b, i]) % mod == acc % mod
+    for in_ct, w_ct, b_ct in ((ob.F64, ob.F64, ob.F64), (ob.F32, ob.F64, ob.S32), (ob.S32, ob.F64, ob.F32)):
+        x, W, bias = rand(in_ct, (B, k)), rand(w_ct, (M, k)), rand(b_ct, (M,))
+        got = ob.slang_matmul(x, in_ct, in_ct, k, ob.F64, M, W.view(np.uint8).reshape(-1), w_ct, ob.ROW, k * W.itemsize, bias, b_ct)
+        acc = np.zeros((B, M), np.float64)
+        for j in range(k):
+            acc = acc + x[:, j:j + 1].astype(np.float64) * W[:, j][None, :].astype(np.float64)
+        acc = acc + bias.astype(np.float64)[None, :]
+        assert np.array_equal(got.view(np.uint64), acc.view(np.uint64))
+    # a 64-bit matrix under a float result: cast<float>(int64) rounds to nearest even
+    W = np.array([[(1 << 53) + 1, -(1 << 40) - 1]], np.int64); x = np.array([[1.0, 1.0]], np.float32)
+    got = ob.slang_matmul(x, ob.F32, ob.F32, 2, ob.F32, 1, W.view(np.uint8).reshape(-1), ob.S64, ob.ROW, 16)
+    assert got[0, 0] == np.float32(np.float32(float((1 << 53) + 1)) + np.float32(float(-(1 << 40) - 1)))
