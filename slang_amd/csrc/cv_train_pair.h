@@ -22,9 +22,9 @@
 // LDS before either wave contracts over it) and once per round.  Only the pair meets, through a
 // sequence number each wave publishes in LDS (pairPublish, pairAwait), not the workgroup at s_barrier: the four
 // pairs of a workgroup drift apart, so that the two waves of a SIMD, which belong to different
-// pairs, are in different phases of the round and want different units.  Every wave runs the same
-// number of rounds (rounds past the end of the batch are run with all samples masked), so the
-// sequence numbers always match.  Partials and their second-stage reduction are those of the
+// pairs, are in different phases of the round and want different units.  The two waves of a pair run
+// the same rounds (a round past the end of the batch is run with all samples masked), so their
+// sequence numbers always match; the pairs of a workgroup take different numbers of rounds (below).  Partials and their second-stage reduction are those of the
 // one-wave kernel (mlpTrainReduceKernel): same layout, fixed order, no atomics.
 #pragma once
 #include "cv_train_impl.h"
@@ -186,8 +186,21 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int outDim = a.layers[L - 1].out;
     constexpr int OROWS = 4 * Net::MTL;
 
+    // Rounds blockIdx.x + j * gridDim.x belong to this workgroup; its four pairs share them unevenly.  A SIMD
+    // favours its older wave, and the waves of pairs 0 and 1 are the older ones on all four SIMDs: with equal
+    // shares they were done after 105 us and left pairs 2 and 3 to run alone, one wave per SIMD, for another
+    // 30 us.  With 37 : 27 the four pairs end together (146 -> 138 us for 8-64x4-1 at batch 2^20; 36 and 38 are
+    // within 1 %).  The split is a function of the pair's index, so results stay bitwise reproducible.
+#ifndef CV_TRAIN_PAIR_OLD_SHARE
+#define CV_TRAIN_PAIR_OLD_SHARE 37      // of 128: the share of each of the pairs 0 and 1 (pairs 2 and 3 get 64 minus that)
+#endif
     const uint32_t numRounds = (a.batch + 31u) / 32u;
-    const uint32_t roundsPerPair = (numRounds + gridDim.x * 4u - 1u) / (gridDim.x * 4u);   // the same for every wave
+    const uint32_t blockRounds = blockIdx.x < numRounds ? (numRounds - blockIdx.x + gridDim.x - 1u) / gridDim.x : 0u;
+    constexpr uint32_t kOld = CV_TRAIN_PAIR_OLD_SHARE, kYoung = 64u - kOld;
+    const uint32_t cumLo = pair == 0 ? 0u : pair == 1 ? kOld : pair == 2 ? 2u * kOld : 2u * kOld + kYoung;
+    const uint32_t cumHi = pair == 0 ? kOld : pair == 1 ? 2u * kOld : pair == 2 ? 2u * kOld + kYoung : 128u;
+    const uint32_t firstRound = blockRounds * cumLo / 128u, endRound = blockRounds * cumHi / 128u;
+    const uint32_t roundsPerPair = endRound - firstRound;     // the same for both waves of a pair
     const uint32_t lastSample = a.batch - 1;
     uint32_t* myX = ldsX + pair * (Net::totalXTiles * kPairTileDW);
     uint32_t* myDZ = ldsDZ + pair * (2 * Net::MTMAX * kPairTileDW);
@@ -445,10 +458,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // ---- main loop ---------------------------------------------------------------------------------
     {
         uint32_t cur[IN_DW], nxt[IN_DW];
-        uint32_t r = blockIdx.x * 4u + pair;
+        uint32_t r = blockIdx.x + firstRound * gridDim.x;
         loadTile(cur, r);
-        for (uint32_t k = 0; k < roundsPerPair; ++k, r += gridDim.x * 4u) {
-            loadTile(nxt, r + gridDim.x * 4u);
+        for (uint32_t k = 0; k < roundsPerPair; ++k, r += gridDim.x) {
+            loadTile(nxt, r + gridDim.x);
             asm volatile("" ::: "memory");        // the requests stay above the round ...
             round(cur, r);
 #pragma unroll
