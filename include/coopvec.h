@@ -190,6 +190,9 @@ CV_API CvResult cvConvertMatrices(void* stream, void* dstBuffer, const CvMatrixD
  * the rest of the fallback's switch (hlsl.meta.slang:32866-32907), every mix of SINT8/16/32/64, UINT8/16/32/64,
  * FLOAT16, FLOAT32 and FLOAT64 for vector, matrix, bias and result (FLOAT16/32/64, SINT32/64 or UINT32/64):
  * these run as the scalar definition, operands cast to the result type first, RowMajor / ColumnMajor only.
+ * There, as in the fallback (hlsl.meta.slang:32839-32856), a packed inputInterpretation (32-bit elements of four
+ * sign-extended bytes) goes with every matrix type, and a plain inputInterpretation other than the stored
+ * type is accepted and changes nothing: the stored elements are cast to the result type.
  * accumulate != 0 gives the member forms matMulAccum / matMulAddAccum
  * (hlsl.meta.slang:31476-31650): output += result (activation must be NONE).
  */

@@ -93,7 +93,8 @@ bool isOptimal(int layout) { return layout == CV_LAYOUT_INFERENCING_OPTIMAL || l
 // What the matMul kernels implement: the matrix-core flavour that serves a combination of
 // (type of the vectors in memory, inputInterpretation, matrixInterpretation, biasInterpretation or
 // CV_COMPONENT_NONE, resultType), or false.  The table of cvQuerySupportedCombinations is this
-// predicate evaluated over every combination, so the two cannot disagree.
+// predicate evaluated over every combination, so the two cannot disagree (one exception, stated where the
+// table is built: combinations that differ only by an interpretation the scalar definition ignores).
 struct ComboKind {
     cv::MmaKind kind;
     bool inUnsigned, matUnsigned;
@@ -157,14 +158,19 @@ bool isPlainScalar(int32_t ct)
 }
 
 // Every combination of those types runs somewhere: on a matrix instruction where one exists, else as the
-// scalar definition (cv_matmul_scalar.hip): vectors stored as what they are interpreted as, results
-// half / float / double / int32 / uint32 / int64 / uint64.
+// scalar definition (cv_matmul_scalar.hip), results half / float / double / int32 / uint32 / int64 / uint64.
+// The scalar definition casts the vector's elements, as they are stored, to the result type and never looks at
+// a plain inputInterpretation (hlsl.meta.slang:32839-32843), so a plain interpretation other than the stored
+// type changes nothing there; packed interpretations unpack four sign-extended bytes from each 32-bit element
+// (:32844-32856) and go with every plain matrix type.
 bool classifyCombo(int32_t inType, int32_t inInterp, int32_t matInterp, int32_t biasInterp, int32_t resType, ComboKind* out)
 {
     if (classifyMfmaCombo(inType, inInterp, matInterp, biasInterp, resType, out)) return true;
     const bool resOk = resType == CV_FLOAT16 || resType == CV_FLOAT32 || resType == CV_FLOAT64 || resType == CV_SINT32 ||
                        resType == CV_UINT32 || resType == CV_SINT64 || resType == CV_UINT64;
-    if (inType != inInterp || !isPlainScalar(inType) || !isPlainScalar(matInterp) || !resOk) return false;
+    const bool packedIn = inInterp == CV_SINT8_PACKED || inInterp == CV_UINT8_PACKED;
+    const bool inOk = packedIn ? (inType == CV_UINT32 || inType == CV_SINT32) : (isPlainScalar(inType) && isPlainScalar(inInterp));
+    if (!inOk || !isPlainScalar(matInterp) || !resOk) return false;
     if (biasInterp != CV_COMPONENT_NONE && !isPlainScalar(biasInterp)) return false;
     if (out) *out = ComboKind{cv::MmaKind::Scalar, false, false};
     return true;
@@ -183,7 +189,11 @@ const std::vector<CvCombination>& comboTable()
                 for (int32_t interp = 0; interp < kNumComponentTypes; ++interp)
                     for (int32_t bias = 0; bias < kNumComponentTypes; ++bias)
                         for (int32_t res = 0; res < kNumComponentTypes; ++res) {
-                            if (!classifyCombo(in, interp, mat, bias, res, nullptr)) continue;
+                            ComboKind kind;
+                            if (!classifyCombo(in, interp, mat, bias, res, &kind)) continue;
+                            // the scalar definition ignores a plain interpretation: the table lists each of
+                            // those combinations once, under the stored type
+                            if (kind.kind == cv::MmaKind::Scalar && interp != in && cvComponentPackingFactor(interp) == 1) continue;
                             CvCombination c;
                             c.inputType = in; c.inputInterpretation = interp;
                             c.inputPackingFactor = (uint32_t)cvComponentPackingFactor(interp);
@@ -429,6 +439,7 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     cv::MmaKind kind = combo.kind;
     if (kind == cv::MmaKind::Fp8AsF16 && (d->flags & CV_FLAG_FP8_MATRIX_PIPELINE)) kind = cv::MmaKind::Fp8Native;
     if (kind == cv::MmaKind::Scalar) {
+        if (packing != 1) a.inCt = CV_SINT8;      // the bytes of a packed vector, sign-extended for both packed kinds
         const bool floatRes = d->resultType == CV_FLOAT16 || d->resultType == CV_FLOAT32 || d->resultType == CV_FLOAT64;
         if (a.act > (floatRes ? CV_ACT_LEAKY_RELU : CV_ACT_RELU))
             return fail(CV_E_NOT_AVAILABLE, "cvMatMul: activation %d with input %d, matrix %d, result %d (this combination takes NONE, RELU%s)",

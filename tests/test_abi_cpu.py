@@ -128,6 +128,11 @@ def test_supported_combinations(lib):
     assert (ob.F32, ob.F32, 1, ob.S8, ob.F16, ob.F32) in combos
     assert (ob.F64, ob.F64, 1, ob.S64, ob.U64, ob.F64) in combos
     assert (ob.BF16, ob.BF16, 1, ob.F16, ob.F16, ob.F16) not in combos
+    # packed bytes against any plain matrix type; a plain interpretation the scalar definition ignores is
+    # accepted by cvMatMul and listed once, under the stored type
+    assert (ob.U32, ob.S8P, 4, ob.F16, ob.F16, ob.F32) in combos
+    assert (ob.S32, ob.U8P, 4, ob.S16, ob.S32, ob.S64) in combos
+    assert (ob.F32, ob.F16, 1, ob.S16, ob.F32, ob.F32) not in combos
 
 
 def _desc(**kw):
@@ -157,7 +162,10 @@ def test_matmul_argument_validation(lib):
     assert f(activation=9) == E_INVALID
     assert f(inputType=ob.BF16, inputInterpretation=ob.BF16) == E_NOTAVAIL     # bfloat16 only with a bfloat16 matrix
     assert f(matrixInterpretation=ob.E5M2, matrixStride=64) == E_NOTAVAIL      # 8-bit floats only with their own vectors
-    assert f(inputType=ob.F16, inputInterpretation=ob.S16) == E_NOTAVAIL       # vectors reinterpreted as another plain type
+    assert f(inputType=ob.F32, inputInterpretation=ob.S8P, inputStride=256) == E_NOTAVAIL   # packed bytes live in 32-bit integers
+    assert b"unsupported combination" in lib.cvGetLastErrorMessage()
+    assert f(inputType=ob.F16, inputInterpretation=ob.E5M2) == E_NOTAVAIL      # fp16 vectors quantise to e4m3 only
+    assert b"unsupported combination" in lib.cvGetLastErrorMessage()
     assert f(matrixInterpretation=ob.E4M3, matrixStride=64, inputType=ob.F32, inputInterpretation=ob.F32,
              inputStride=256) == E_NOTAVAIL                                    # 8-bit floats only with their own vectors
     assert f(matrixInterpretation=ob.S16, layout=2) == E_NOTAVAIL              # no Optimal layout for 16-bit integers

@@ -146,6 +146,60 @@ def test_accumulate_forms_strides_and_row_blocks():
     assert (got[:, M:] == 1000).all()
 
 
+PACKED_CASES = [  # (packed kind, element type of the vector, matrix, bias, result)
+    (ob.S8P, ob.U32, ob.S16, ob.S32, ob.S32), (ob.U8P, ob.S32, ob.U16, None, ob.U32), (ob.S8P, ob.S32, ob.S32, ob.S64, ob.S64),
+    (ob.U8P, ob.U32, ob.F16, ob.F32, ob.F32), (ob.S8P, ob.U32, ob.F32, None, ob.F32), (ob.S8P, ob.U32, ob.F64, ob.F64, ob.F64),
+    (ob.U8P, ob.U32, ob.S8, ob.S32, ob.S64), (ob.S8P, ob.S32, ob.U8, ob.F16, ob.F32),
+]
+
+
+@pytest.mark.parametrize("interp,in_ct,w_ct,b_ct,r_ct", PACKED_CASES)
+def test_packed_vectors_against_every_matrix_type(interp, in_ct, w_ct, b_ct, r_ct):
+    # coopVecMatMulPacked: four bytes per 32-bit element, sign-extended for both packed kinds
+    # (hlsl.meta.slang:32844-32856), then the scalar definition in the result type: the same bits as the fallback
+    rng = np.random.default_rng(interp * 1000 + w_ct * 10 + r_ct)
+    B, k, M = 260, 44, 17
+    x = rng.integers(0, 2 ** 32, (B, k // 4), dtype=np.uint64).astype(np.uint32).view(NP[in_ct])
+    W = values(rng, w_ct, (M, k), small=w_ct in (ob.F16, ob.F32, ob.F64))
+    bias = values(rng, b_ct, (M,), small=True) if b_ct is not None else None
+    stride = k * W.itemsize
+    ref = ob.slang_matmul(x, in_ct, interp, k, r_ct, M, W.view(np.uint8).reshape(-1), w_ct, ob.ROW, stride, bias,
+                          b_ct if b_ct is not None else -1)
+    wd = as_bytes(to_dev(W))
+    if bias is None:
+        y = cv.coopVecMatMulPacked(dev(x), interp, k, wd, 0, w_ct, ML.RowMajor, False, stride, M=M, resultType=r_ct)
+    else:
+        y = cv.coopVecMatMulAddPacked(dev(x), interp, k, wd, 0, w_ct, as_bytes(to_dev(bias)), 0, b_ct, ML.RowMajor, False,
+                                      stride, M=M, resultType=r_ct)
+    assert cv.lastKernelName().startswith("matmulScalarKernel"), cv.lastKernelName()
+    bits = {2: np.uint16, 4: np.uint32, 8: np.uint64}[ref.itemsize]
+    assert np.array_equal(y.cpu().numpy().view(bits), ref.view(bits))
+    # and the unpacking itself: byte j of the vector is (x[j / 4] >> 8 (j % 4)) as a signed byte
+    if r_ct in (ob.S32, ob.S64) and b_ct is None:
+        xb = x.view(np.int8).astype(np.int64)
+        assert np.array_equal(ref.astype(np.int64), (xb @ W.astype(np.int64).T).astype(NP[r_ct]).astype(np.int64))
+
+
+@pytest.mark.parametrize("in_ct,interp,w_ct,r_ct", [(ob.F32, ob.F16, ob.F16, ob.F32), (ob.S16, ob.S8, ob.S16, ob.S32),
+                                                    (ob.F16, ob.S16, ob.F32, ob.F32), (ob.U8, ob.F32, ob.S32, ob.S64)])
+def test_plain_interpretation_of_another_type_changes_nothing(in_ct, interp, w_ct, r_ct):
+    # the scalar definition casts the stored elements to the result type and never reads a plain
+    # inputInterpretation (hlsl.meta.slang:32839-32843)
+    rng = np.random.default_rng(in_ct * 100 + interp)
+    B, k, M = 140, 30, 12
+    x = values(rng, in_ct, (B, k), small=True); W = values(rng, w_ct, (M, k), small=True)
+    stride = k * W.itemsize
+    ref = ob.slang_matmul(x, in_ct, interp, k, r_ct, M, W.view(np.uint8).reshape(-1), w_ct, ob.ROW, stride)
+    wd = as_bytes(to_dev(W))
+    y = cv.coopVecMatMul(dev(x), interp, wd, 0, w_ct, ML.RowMajor, False, stride, M=M, resultType=r_ct)
+    assert cv.lastKernelName().startswith("matmulScalarKernel"), cv.lastKernelName()
+    same = cv.coopVecMatMul(dev(x), in_ct, wd, 0, w_ct, ML.RowMajor, False, stride, M=M, resultType=r_ct)
+    bits = {4: np.uint32, 8: np.uint64}[ref.itemsize]
+    assert np.array_equal(y.cpu().numpy().view(bits), ref.view(bits))
+    if cv.lastKernelName().startswith("matmulScalarKernel"):
+        assert torch.equal(y, same)
+
+
 def test_what_stays_unavailable():
     x = torch.zeros((4, 8), dtype=torch.int16, device=DEV)
     W = torch.zeros(64, dtype=torch.int16, device=DEV).view(torch.uint8)
