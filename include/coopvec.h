@@ -263,7 +263,10 @@ CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStrid
  * sin..fma :32231-32421) and the neural module's activations (activations.slang), over a batch:
  *   out[s][i] = op(a[s][i], b[s][i], c[s][i])
  * elementType is FLOAT16 or FLOAT32 (all operands and the result); FLOAT16 evaluates in fp32 and
- * rounds once.  Operands an operator does not take are ignored (may be NULL).  `param` is the
+ * rounds once.  The operators Slang declares on integer vectors -- ADD, SUB, MUL, DIV, NEG, MIN, MAX, CLAMP
+ * (hlsl.meta.slang:32115-32229) -- also take SINT8/16/32/64 and UINT8/16/32/64 (two's complement, wrapping; the
+ * quotients C leaves undefined are x / 0 = 0 and MIN / -1 = MIN) and FLOAT64, which takes STEP and FMA as well.
+ * Operands an operator does not take are ignored (may be NULL).  `param` is the
  * slope of CV_OP_LEAKY_RELU.  In-place use (out == a) is allowed. */
 typedef enum CvElementwiseOp {
     CV_OP_ADD = 0, CV_OP_SUB = 1, CV_OP_MUL = 2, CV_OP_DIV = 3, CV_OP_NEG = 4,
@@ -279,11 +282,19 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
                               const void* a, size_t aStride, const void* b, size_t bStride,
                               const void* c, size_t cStride, void* out, size_t outStride, float param);
 
+/* CoopVec<T,N>(CoopVec<U,N>) / CoopVec.copyFrom (hlsl.meta.slang:30683-30730) over a batch:
+ *   dst[s][i] = T(src[s][i])
+ * between any two of FLOAT16/32/64 and the 8/16/32/64-bit integers.  Integer -> integer keeps the low bits;
+ * to a float type: one rounding to nearest even; float -> integer: towards zero (what C leaves undefined is
+ * fixed as NaN -> 0 and out-of-range values saturated to 32 bits, 64 for 64-bit targets, then cut to the low bits). */
+CV_API CvResult cvVectorCast(void* stream, int32_t n, uint32_t batch, const void* src, size_t srcStride, int32_t srcType,
+                             void* dst, size_t dstStride, int32_t dstType);
+
 /* Reverse-mode derivative of the same operators, by Slang's rules (diff.meta.slang:1948-2470: the
  * larger operand of max / smaller of min takes dOut and a tie splits it in halves, clamp passes
  * dOut to x inside [min, max] including the bounds and to the bound it was clamped to otherwise):
  *   dA[s][i] = d op / d a * dOut[s][i], likewise dB, dC (overwritten, not accumulated).
- * Gradient outputs that are NULL, or that the operator has no operand for, are skipped. */
+ * Gradient outputs that are NULL, or that the operator has no operand for, are skipped.  FLOAT16 / FLOAT32 only. */
 CV_API CvResult cvElementwiseBackward(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
                                       const void* a, size_t aStride, const void* b, size_t bStride,
                                       const void* c, size_t cStride, const void* dOut, size_t dOutStride,

@@ -191,10 +191,15 @@ _CT_TO_TORCH = {
     CoopVecComponentType.Float16: torch.float16,
     CoopVecComponentType.BFloat16: torch.bfloat16,
     CoopVecComponentType.Float32: torch.float32,
+    CoopVecComponentType.SignedInt8: torch.int8,
+    CoopVecComponentType.UnsignedInt8: torch.uint8,
+    CoopVecComponentType.SignedInt16: torch.int16,
     CoopVecComponentType.SignedInt32: torch.int32,
     CoopVecComponentType.SignedInt64: torch.int64,
     CoopVecComponentType.Float64: torch.float64,
 }
+if hasattr(torch, "uint16"):
+    _CT_TO_TORCH[CoopVecComponentType.UnsignedInt16] = torch.uint16
 if hasattr(torch, "uint32"):
     _CT_TO_TORCH[CoopVecComponentType.UnsignedInt32] = torch.uint32
 if hasattr(torch, "uint64"):
@@ -420,7 +425,8 @@ def _ew_operand(t: Optional[torch.Tensor], like: torch.Tensor, what: str):
 
 def elementwise(op: int, a: torch.Tensor, b: Optional[torch.Tensor] = None, c: Optional[torch.Tensor] = None, *,
                 param: float = 0.0, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
-    """op(a, b, c) per component of every CoopVec of the batch (fp16 or fp32 tensors [batch, N]):
+    """op(a, b, c) per component of every CoopVec of the batch (fp16 or fp32 tensors [batch, N]; integer and
+    fp64 tensors for the arithmetic operators, min, max and clamp):
     e.g. elementwise(ElementwiseOp.Clamp, x, lo, hi) is Slang's clamp(x, lo, hi)."""
     ct = _TORCH_TO_CT.get(a.dtype)
     if out is None:
@@ -429,6 +435,23 @@ def elementwise(op: int, a: torch.Tensor, b: Optional[torch.Tensor] = None, c: O
     po, so = _ew_operand(out, a, "out")
     _check(_lib.load().cvElementwise(_stream_handle(stream), int(op), int(ct) if ct is not None else -1, a.shape[1],
                                      a.shape[0], pa, sa, pb, sb, pc, sc, po, so, float(param)))
+    return out
+
+
+def copyFrom(other: torch.Tensor, T: int, *, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
+    """CoopVec<T,N>(CoopVec<U,N>) / CoopVec.copyFrom (hlsl.meta.slang:30683-30730) for every vector of the batch:
+    the elements of `other` converted to component type T."""
+    src_ct, src_stride = _vector_info(other, -1, "other")
+    if out is None:
+        dt = _CT_TO_TORCH.get(CoopVecComponentType(T))
+        if dt is None:
+            raise CoopVecError(SLANG_E_NOT_AVAILABLE, "unsupported element type %s" % T)
+        out = torch.empty(other.shape, dtype=dt, device=other.device)
+    dst_ct, dst_stride = _vector_info(out, -1, "out")
+    if out.shape != other.shape or dst_ct != T:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "out must have the shape of `other` and element type T")
+    _check(_lib.load().cvVectorCast(_stream_handle(stream), other.shape[1], other.shape[0], other.data_ptr(), src_stride,
+                                    int(src_ct), out.data_ptr(), dst_stride, int(dst_ct)))
     return out
 
 

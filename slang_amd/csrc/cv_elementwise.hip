@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <type_traits>
 
 #include "cv_device.h"
 #include "cv_error.h"
@@ -165,6 +166,157 @@ __global__ __launch_bounds__(256) void elementwiseDenseKernel(const EwArgs e, ui
     }
 }
 
+// The operators Slang declares on integer vectors (arithmetic, min / max / clamp: hlsl.meta.slang:32115-32229) and,
+// for double, those and step / fma, evaluated in the element type itself.  Integers wrap in two's complement like
+// the reference's scalar code; the quotients C leaves undefined are given values here: x / 0 = 0, MIN / -1 = MIN.
+template <typename T>
+__device__ __forceinline__ T evalArith(int op, T a, T b, T c)
+{
+    if constexpr (std::is_integral<T>::value) {
+        typedef typename std::make_unsigned<T>::type U;
+        switch (op) {
+        case kOpAdd: return (T)((U)a + (U)b);
+        case kOpSub: return (T)((U)a - (U)b);
+        case kOpMul: return (T)((U)a * (U)b);
+        case kOpDiv:
+            if (b == 0) return 0;
+            if (std::is_signed<T>::value && b == (T)-1) return (T)((U)0 - (U)a);
+            return (T)(a / b);
+        case kOpNeg: return (T)((U)0 - (U)a);
+        case kOpMin: return a < b ? a : b;
+        case kOpMax: return a > b ? a : b;
+        case kOpClamp: { const T lo = a > b ? a : b; return lo < c ? lo : c; }
+        }
+        return a;
+    } else {
+        switch (op) {
+        case kOpAdd: return a + b;
+        case kOpSub: return a - b;
+        case kOpMul: return a * b;
+        case kOpDiv: return a / b;
+        case kOpNeg: return -a;
+        case kOpMin: return fmin(a, b);
+        case kOpMax: return fmax(a, b);
+        case kOpClamp: return fmin(fmax(a, b), c);
+        case kOpStep: return b >= a ? (T)1 : (T)0;
+        case kOpFma: return __builtin_fma(a, b, c);
+        }
+        return a;
+    }
+}
+
+bool arithOpFor(int32_t ct, int op)
+{
+    const bool common = op == kOpAdd || op == kOpSub || op == kOpMul || op == kOpDiv || op == kOpNeg || op == kOpMin ||
+                        op == kOpMax || op == kOpClamp;
+    return common || (ct == kF64 && (op == kOpStep || op == kOpFma));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void elementwiseArithKernel(const EwArgs e)
+{
+    const uint64_t total = (uint64_t)e.batch * (uint32_t)e.n;
+    const int nOps = operandCount(e.op);
+    for (uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256u) {
+        const uint64_t s = idx / (uint32_t)e.n;
+        const uint64_t off = (idx - s * (uint32_t)e.n) * sizeof(T);
+        const T a = *(const T*)(e.a + s * e.aStride + off);
+        const T b = nOps >= 2 ? *(const T*)(e.b + s * e.bStride + off) : (T)0;
+        const T c = nOps >= 3 ? *(const T*)(e.c + s * e.cStride + off) : (T)0;
+        *(T*)(e.out + s * e.outStride + off) = evalArith<T>(e.op, a, b, c);
+    }
+}
+
+// CoopVec<T,N>(CoopVec<U,N>) / copyFrom (hlsl.meta.slang:30683-30730): element-wise conversion between any two of the
+// plain types.  integer -> integer keeps the low bits (sign- or zero-extended from the source); integer -> float and
+// float -> float round to nearest even, in one rounding; float -> integer truncates towards zero, with the values C
+// leaves undefined fixed as: NaN -> 0, out of range -> saturated to 32 bits (64 for 64-bit targets), then the low
+// bits for narrower targets.
+struct CastArgs {
+    const uint8_t* src; uint8_t* dst;
+    uint64_t srcStride, dstStride;
+    int32_t srcCt, dstCt, n;
+    uint32_t batch;
+};
+
+// double -> half in one rounding: through a float that keeps a sticky last bit (round to odd)
+__device__ __forceinline__ half_t halfOfDouble(double d)
+{
+    float f = (float)d;
+    const double back = (double)f;
+    if (back != d) {
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        if (__builtin_fabs(back) > __builtin_fabs(d)) u -= 1u;      // towards zero
+        f = __builtin_bit_cast(float, u | 1u);
+    }
+    return (half_t)f;
+}
+
+__global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
+{
+    const uint64_t total = (uint64_t)e.batch * (uint32_t)e.n;
+    const uint32_t sEsz = elemSize(e.srcCt), dEsz = elemSize(e.dstCt);
+    const bool srcFloat = e.srcCt == kF16 || e.srcCt == kF32 || e.srcCt == kF64;
+    const bool srcUnsigned = e.srcCt == kU8 || e.srcCt == kU16 || e.srcCt == kU32 || e.srcCt == kU64;
+    for (uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256u) {
+        const uint64_t s = idx / (uint32_t)e.n, i = idx - s * (uint32_t)e.n;
+        const uint8_t* p = e.src + s * e.srcStride + i * sEsz;
+        uint8_t* q = e.dst + s * e.dstStride + i * dEsz;
+        double f = 0.0;          // a float source, exactly
+        uint64_t bits = 0;       // an integer source, extended to 64 bits
+        switch (e.srcCt) {
+        case kF16: f = (double)(float)*(const half_t*)p; break;
+        case kF32: f = (double)*(const float*)p; break;
+        case kF64: f = *(const double*)p; break;
+        case kS8: bits = (uint64_t)(int64_t) * (const int8_t*)p; break;
+        case kU8: bits = *p; break;
+        case kS16: bits = (uint64_t)(int64_t) * (const int16_t*)p; break;
+        case kU16: bits = *(const uint16_t*)p; break;
+        case kS32: bits = (uint64_t)(int64_t) * (const int32_t*)p; break;
+        case kU32: bits = *(const uint32_t*)p; break;
+        default: bits = *(const uint64_t*)p; break;
+        }
+        switch (e.dstCt) {
+        case kF16:
+            // integers below 2^53 are exact in double; larger ones are far beyond the half range either way
+            *(half_t*)q = srcFloat ? (e.srcCt == kF64 ? halfOfDouble(f) : (half_t)(float)f)
+                                   : halfOfDouble(srcUnsigned ? (double)bits : (double)(int64_t)bits);
+            break;
+        case kF32:
+            *(float*)q = srcFloat ? (float)f : (srcUnsigned ? (float)bits : (float)(int64_t)bits);
+            break;
+        case kF64:
+            *(double*)q = srcFloat ? f : (srcUnsigned ? (double)bits : (double)(int64_t)bits);
+            break;
+        case kS64:
+            *(int64_t*)q = srcFloat ? (f != f ? 0 : (f >= 9223372036854775808.0 ? INT64_MAX : (f <= -9223372036854775808.0 ? INT64_MIN : (int64_t)f)))
+                                    : (int64_t)bits;
+            break;
+        case kU64:
+            *(uint64_t*)q = srcFloat ? (f != f || f <= 0.0 ? 0u : (f >= 18446744073709551616.0 ? UINT64_MAX : (uint64_t)f)) : bits;
+            break;
+        default: {
+            const bool dstUnsigned = e.dstCt == kU8 || e.dstCt == kU16 || e.dstCt == kU32;
+            uint32_t v;
+            if (!srcFloat) v = (uint32_t)bits;
+            else if (f != f) v = 0u;
+            else if (dstUnsigned) v = f <= 0.0 ? 0u : (f >= 4294967296.0 ? UINT32_MAX : (uint32_t)f);
+            else v = (uint32_t)(f >= 2147483648.0 ? INT32_MAX : (f <= -2147483648.0 ? INT32_MIN : (int32_t)f));
+            if (dEsz == 1) *q = (uint8_t)v;
+            else if (dEsz == 2) *(uint16_t*)q = (uint16_t)v;
+            else *(uint32_t*)q = v;
+            break;
+        }
+        }
+    }
+}
+
+bool isPlainType(int32_t ct)
+{
+    return ct == kF16 || ct == kF32 || ct == kF64 || ct == kS8 || ct == kU8 || ct == kS16 || ct == kU16 || ct == kS32 ||
+           ct == kU32 || ct == kS64 || ct == kU64;
+}
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 int currentCUs()
@@ -179,7 +331,8 @@ CvResult checkCommon(const char* who, int32_t op, int32_t elementType, int32_t n
 {
     if (op < 0 || op >= kOpCount) return failWith(CV_E_INVALID_ARG, "%s: unknown operator %d", who, op);
     if (elementType != CV_FLOAT16 && elementType != CV_FLOAT32)
-        return failWith(CV_E_NOT_AVAILABLE, "%s: elementType %d (supported: FLOAT16, FLOAT32)", who, elementType);
+        return failWith(CV_E_NOT_AVAILABLE, "%s: elementType %d with operator %d (every operator: FLOAT16, FLOAT32; arithmetic, min, max, "
+                        "clamp: the integer types and FLOAT64, which also takes step and fma)", who, elementType, op);
     if (n <= 0) return failWith(CV_E_INVALID_ARG, "%s: n=%d", who, n);
     (void)esz;
     return CV_OK;
@@ -200,8 +353,11 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
                               const void* c, size_t cStride, void* out, size_t outStride, float param)
 {
     using namespace cv;
-    const uint32_t esz = elementType == CV_FLOAT32 ? 4u : 2u;
-    CvResult rc = checkCommon("cvElementwise", op, elementType, n, esz);
+    const bool arith = isPlainType(elementType) && elementType != CV_FLOAT16 && elementType != CV_FLOAT32 && op >= 0 &&
+                       op < kOpCount && arithOpFor(elementType, op);
+    const uint32_t esz = arith ? elemSize(elementType) : elementType == CV_FLOAT32 ? 4u : 2u;
+    CvResult rc = arith ? (n <= 0 ? failWith(CV_E_INVALID_ARG, "cvElementwise: n=%d", n) : CV_OK)
+                        : checkCommon("cvElementwise", op, elementType, n, esz);
     if (CV_FAILED(rc)) return rc;
     if (batch == 0) return CV_OK;
     const int nOps = operandCount(op);
@@ -219,7 +375,23 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
                        aligned16(a) && aligned16(out) && (nOps < 2 || aligned16(b)) && (nOps < 3 || aligned16(c)) &&
                        (total * esz) % 16 == 0;
     const uint32_t cap = (uint32_t)currentCUs() * 8u;
-    if (dense) {
+    if (arith) {
+        const uint32_t blocks = (uint32_t)((total + 255) / 256 < cap ? (total + 255) / 256 : cap);
+        noteKernel(false, "elementwiseArithKernel<type %d>", elementType);
+        const dim3 g(blocks), t(256);
+        hipStream_t st = (hipStream_t)stream;
+        switch (elementType) {
+        case CV_SINT8: hipLaunchKernelGGL(elementwiseArithKernel<int8_t>, g, t, 0, st, e); break;
+        case CV_UINT8: hipLaunchKernelGGL(elementwiseArithKernel<uint8_t>, g, t, 0, st, e); break;
+        case CV_SINT16: hipLaunchKernelGGL(elementwiseArithKernel<int16_t>, g, t, 0, st, e); break;
+        case CV_UINT16: hipLaunchKernelGGL(elementwiseArithKernel<uint16_t>, g, t, 0, st, e); break;
+        case CV_SINT32: hipLaunchKernelGGL(elementwiseArithKernel<int32_t>, g, t, 0, st, e); break;
+        case CV_UINT32: hipLaunchKernelGGL(elementwiseArithKernel<uint32_t>, g, t, 0, st, e); break;
+        case CV_SINT64: hipLaunchKernelGGL(elementwiseArithKernel<int64_t>, g, t, 0, st, e); break;
+        case CV_UINT64: hipLaunchKernelGGL(elementwiseArithKernel<uint64_t>, g, t, 0, st, e); break;
+        default: hipLaunchKernelGGL(elementwiseArithKernel<double>, g, t, 0, st, e); break;
+        }
+    } else if (dense) {
         const uint64_t pieces = total * esz / 16u;
         const uint32_t blocks = (uint32_t)((pieces + 255) / 256 < cap ? (pieces + 255) / 256 : cap);
         noteKernel(false, "elementwiseDenseKernel<%s>", esz == 2 ? "f16" : "f32");
@@ -233,6 +405,31 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
     }
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvElementwise launch: %s", hipGetErrorString(err));
+    return CV_OK;
+}
+
+CV_API CvResult cvVectorCast(void* stream, int32_t n, uint32_t batch, const void* src, size_t srcStride, int32_t srcType,
+                             void* dst, size_t dstStride, int32_t dstType)
+{
+    using namespace cv;
+    if (n <= 0) return failWith(CV_E_INVALID_ARG, "cvVectorCast: n=%d", n);
+    if (!isPlainType(srcType) || !isPlainType(dstType))
+        return failWith(CV_E_NOT_AVAILABLE, "cvVectorCast: from type %d to type %d (supported: FLOAT16/32/64 and the 8/16/32/64-bit integers)",
+                        srcType, dstType);
+    if (batch == 0) return CV_OK;
+    if (badOperand(src, srcStride, n, batch, elemSize(srcType)) || badOperand(dst, dstStride, n, batch, elemSize(dstType)))
+        return failWith(CV_E_INVALID_ARG, "cvVectorCast: null, misaligned or overlapping-row operand");
+    CastArgs e;
+    memset(&e, 0, sizeof(e));
+    e.src = (const uint8_t*)src; e.dst = (uint8_t*)dst; e.srcStride = srcStride; e.dstStride = dstStride;
+    e.srcCt = srcType; e.dstCt = dstType; e.n = n; e.batch = batch;
+    const uint64_t total = (uint64_t)batch * (uint32_t)n;
+    const uint32_t cap = (uint32_t)currentCUs() * 8u;
+    const uint32_t blocks = (uint32_t)((total + 255) / 256 < cap ? (total + 255) / 256 : cap);
+    noteKernel(false, "vectorCastKernel<%d -> %d>", srcType, dstType);
+    hipLaunchKernelGGL(vectorCastKernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, e);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvVectorCast launch: %s", hipGetErrorString(err));
     return CV_OK;
 }
 

@@ -121,7 +121,10 @@ def test_elementwise_argument_validation():
         cv.elementwise(T.ADD, x)             # binary operator without b
     assert e.value.result == cv.SLANG_E_INVALID_ARG
     with pytest.raises(cv.CoopVecError) as e:
-        cv.elementwise(T.NEG, x.to(torch.int32))
+        cv.elementwise(T.TANH, x.to(torch.int32))     # integer vectors: arithmetic, min, max, clamp only
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.elementwiseBackward(T.NEG, x.to(torch.float64), x.to(torch.float64))
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
     assert cv.elementwise(T.NEG, x[:0]).shape == (0, 8)
 
@@ -179,4 +182,149 @@ def test_mlp_with_smooth_activations_equals_layer_chain():
             L.biasesGrad = torch.zeros(L.outputSize * 4, dtype=torch.uint8, device=DEV)
             L.gradLayout = ML.RowMajor
         cv.mlpTrainStepWorkspaceSize(layers, B) and cv.mlpTrainStep(layers, x, None)
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+# ---------------------------------------------------------------------------------------------
+# integer and fp64 vectors; conversions between element types
+# ---------------------------------------------------------------------------------------------
+
+INT_TYPES = [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64]
+
+
+def _torch_dtype(np_dtype):
+    return {np.dtype(np.int8): torch.int8, np.dtype(np.uint8): torch.uint8, np.dtype(np.int16): torch.int16,
+            np.dtype(np.uint16): torch.uint16, np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32,
+            np.dtype(np.int64): torch.int64, np.dtype(np.uint64): torch.uint64, np.dtype(np.float16): torch.float16,
+            np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64}[np.dtype(np_dtype)]
+
+
+def _dev_typed(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(a.shape[0], -1)).to(DEV).view(_torch_dtype(a.dtype))
+
+
+def _wrap(v, dtype):
+    info = np.iinfo(dtype)
+    span = int(info.max) - int(info.min) + 1
+    return (v - int(info.min)) % span + int(info.min)
+
+
+def _int_ref(op, a, b, c, dtype):
+    """The operator on Python integers (unbounded), wrapped to the element type: independent of any machine arithmetic."""
+    info = np.iinfo(dtype)
+    out = np.empty(a.shape, dtype)
+    for idx in np.ndindex(a.shape):
+        x, y, z = int(a[idx]), int(b[idx]), int(c[idx])
+        if op == T.ADD: v = x + y
+        elif op == T.SUB: v = x - y
+        elif op == T.MUL: v = x * y
+        elif op == T.DIV:
+            # C's quotient (towards zero); x / 0 = 0 by this library's definition, MIN / -1 wraps to MIN
+            v = 0 if y == 0 else (abs(x) // abs(y)) * (1 if (x < 0) == (y < 0) else -1)
+        elif op == T.NEG: v = -x
+        elif op == T.MIN: v = min(x, y)
+        elif op == T.MAX: v = max(x, y)
+        elif op == T.CLAMP: v = min(max(x, y), z)
+        out[idx] = _wrap(v, dtype)
+    return out
+
+
+@pytest.mark.parametrize("dtype", INT_TYPES)
+def test_integer_vectors_bit_exact(dtype):
+    # Slang declares arithmetic, min, max and clamp on CoopVec<integer, N> (slang-ir-lower-coopvec.cpp:188-192,
+    # hlsl.meta.slang:32115-32229): two's complement, wrapping
+    rng = np.random.default_rng(np.dtype(dtype).itemsize * 2 + (np.dtype(dtype).kind == "u"))
+    info = np.iinfo(dtype)
+    B, N = 37, 11
+    def draw():
+        v = rng.integers(info.min, info.max, (B, N), dtype=dtype, endpoint=True)
+        small = rng.random((B, N)) < 0.3
+        v[small] = rng.integers(max(info.min, -3), 4, int(small.sum()), dtype=dtype)     # small values, zeros, -1
+        return v
+    a, b, c = draw(), draw(), draw()
+    a[0, :3] = info.min; b[0, 0] = dtype(-1) if info.min < 0 else dtype(1); b[0, 1] = 0
+    for op in (T.ADD, T.SUB, T.MUL, T.DIV, T.NEG, T.MIN, T.MAX, T.CLAMP):
+        lo, hi = (np.minimum(b, c), np.maximum(b, c)) if op == T.CLAMP else (b, c)
+        got = cv.elementwise(op, _dev_typed(a), _dev_typed(lo), _dev_typed(hi)).cpu().numpy().view(dtype)
+        assert cv.lastKernelName().startswith("elementwiseArithKernel"), cv.lastKernelName()
+        assert np.array_equal(got, _int_ref(op, a, lo, hi, dtype)), op
+
+
+def test_fp64_vectors():
+    rng = np.random.default_rng(64)
+    a, b, c = (rng.standard_normal((50, 9)) for _ in range(3))
+    b[0, 0] = a[0, 0]
+    lo, hi = np.minimum(b, c), np.maximum(b, c)
+    ops = {T.ADD: a + b, T.SUB: a - b, T.MUL: a * b, T.DIV: a / b, T.NEG: -a, T.MIN: np.minimum(a, b), T.MAX: np.maximum(a, b),
+           T.STEP: (b >= a).astype(np.float64)}
+    for op, want in ops.items():
+        got = cv.elementwise(op, _dev_typed(a), _dev_typed(b), _dev_typed(c)).cpu().numpy()
+        assert np.array_equal(got, want), op          # IEEE operations: the same bits
+    got = cv.elementwise(T.CLAMP, _dev_typed(a), _dev_typed(lo), _dev_typed(hi)).cpu().numpy()
+    assert np.array_equal(got, np.clip(a, lo, hi))
+    got = cv.elementwise(T.FMA, _dev_typed(a), _dev_typed(b), _dev_typed(c)).cpu().numpy()
+    import math
+    want = np.array([[math.fma(x, y, z) for x, y, z in zip(ra, rb, rc)] for ra, rb, rc in zip(a, b, c)]) if hasattr(math, "fma") else None
+    if want is not None:
+        assert np.array_equal(got, want)
+    else:             # one rounding: within half an ulp of the exact value, which a*b + c in long double brackets
+        exact = a.astype(np.longdouble) * b.astype(np.longdouble) + c.astype(np.longdouble)
+        assert (np.abs(got.astype(np.longdouble) - exact) <= np.spacing(np.abs(got)) * 0.5 + np.abs(exact) * 2.0 ** -63).all()
+
+
+ALL_TYPES = INT_TYPES + [np.float16, np.float32, np.float64]
+
+
+@pytest.mark.parametrize("src", ALL_TYPES)
+def test_copy_from_converts_between_all_plain_types(src):
+    # CoopVec<T,N>(CoopVec<U,N>) (hlsl.meta.slang:30683-30730): numpy's astype is C's conversion for values the
+    # target can hold (integers wrap, floats truncate towards zero, to float: one rounding to nearest even)
+    rng = np.random.default_rng(np.dtype(src).itemsize + 10 * (np.dtype(src).kind == "f"))
+    B, N = 61, 17
+    if np.dtype(src).kind == "f":
+        x = (rng.standard_normal((B, N)) * rng.choice([0.01, 1.0, 100.0], (B, N))).astype(src)
+        x[0, :4] = [0.5, -0.5, 2.5, -3.99]
+    else:
+        info = np.iinfo(src)
+        x = rng.integers(info.min, info.max, (B, N), dtype=src, endpoint=True)
+        small = rng.random((B, N)) < 0.5
+        x[small] = rng.integers(max(info.min, -100), 100, int(small.sum()), dtype=src)
+    for dst in ALL_TYPES:
+        xs = x
+        if np.dtype(src).kind == "f" and np.dtype(dst).kind != "f":
+            info = np.iinfo(dst)           # values the target holds; the rest is pinned by the next test
+            xs = np.clip(x, max(info.min, -100), min(info.max, 100)).astype(src)
+        with np.errstate(over="ignore"):
+            want = xs.astype(dst)
+        got = cv.copyFrom(_dev_typed(xs), {np.int8: CT.SignedInt8, np.uint8: CT.UnsignedInt8, np.int16: CT.SignedInt16,
+                                           np.uint16: CT.UnsignedInt16, np.int32: CT.SignedInt32, np.uint32: CT.UnsignedInt32,
+                                           np.int64: CT.SignedInt64, np.uint64: CT.UnsignedInt64, np.float16: CT.Float16,
+                                           np.float32: CT.Float32, np.float64: CT.Float64}[dst])
+        assert cv.lastKernelName().startswith("vectorCastKernel"), cv.lastKernelName()
+        bits = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[np.dtype(dst).itemsize]
+        assert np.array_equal(got.cpu().numpy().view(bits), want.view(bits)), (src, dst)
+
+
+def test_copy_from_single_rounding_and_the_values_c_leaves_open():
+    # double -> half in one rounding: 1 + 2^-11 + 2^-30 lies above the tie between 1 and 1 + 2^-10; rounding to
+    # float first would land on the tie and then on 1
+    x = np.array([[1.0 + 2.0 ** -11 + 2.0 ** -30, 1.0 + 2.0 ** -11, 65519.999, 65520.0, -1e300, 1e-8, 2.0 ** -25 * (1 + 1e-12)]], np.float64)
+    got = cv.copyFrom(_dev_typed(x), CT.Float16).cpu().numpy()
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got.view(np.uint16), x.astype(np.float16).view(np.uint16))
+    assert got[0, 0] == np.float16(1.0 + 2.0 ** -10) and got[0, 1] == np.float16(1.0)
+    # float -> integer outside the target: NaN -> 0, saturation at 32 bits (64 for 64-bit targets), then the low bits
+    f = np.array([[np.nan, 1e20, -1e20, 300.7, -129.9, 4294967295.5]], np.float64)
+    assert cv.copyFrom(_dev_typed(f), CT.SignedInt32).cpu().numpy().tolist() == [[0, 2 ** 31 - 1, -2 ** 31, 300, -129, 2 ** 31 - 1]]
+    assert cv.copyFrom(_dev_typed(f), CT.UnsignedInt32).cpu().numpy().view(np.uint32).tolist() == [[0, 2 ** 32 - 1, 0, 300, 0, 2 ** 32 - 1]]
+    assert cv.copyFrom(_dev_typed(f), CT.SignedInt8).cpu().numpy().tolist() == [[0, -1, 0, 44, 127, -1]]
+    assert cv.copyFrom(_dev_typed(f), CT.SignedInt64).cpu().numpy().tolist() == [[0, 2 ** 63 - 1, -2 ** 63, 300, -129, 4294967295]]
+    assert cv.copyFrom(_dev_typed(f), CT.UnsignedInt64).cpu().numpy().view(np.uint64).tolist() == [[0, 2 ** 64 - 1, 0, 300, 0, 4294967295]]
+    # strided rows, and nothing written past a row
+    src = torch.arange(5 * 12, dtype=torch.int32, device=DEV).reshape(5, 12)
+    out = torch.full((5, 16), -1.0, dtype=torch.float32, device=DEV)
+    cv.copyFrom(src[:, 2:9], CT.Float32, out=out[:, :7])
+    assert torch.equal(out[:, :7], src[:, 2:9].to(torch.float32)) and (out[:, 7:] == -1).all()
+    with pytest.raises(cv.CoopVecError) as e:
+        cv.copyFrom(torch.zeros(2, 4, dtype=torch.bfloat16, device=DEV), CT.Float32)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
