@@ -388,9 +388,10 @@ typedef struct CvMlpDesc {
     const CvMlpLayer* layers;   /* host array */
     int32_t  numLayers;
     int32_t  inputType;         /* element type of the input vectors in memory */
-    int32_t  weightType;        /* matrix interpretation of every layer: FLOAT16 or FLOAT_E4M3 */
-    int32_t  biasType;          /* FLOAT16 */
-    int32_t  outputType;        /* FLOAT16 */
+    int32_t  weightType;        /* matrix interpretation of every layer: FLOAT16 or FLOAT_E4M3; FLOAT32 or BFLOAT16 for
+                                   a network of that one type (vectors, biases and results too; forward only) */
+    int32_t  biasType;          /* FLOAT16 (weightType for FLOAT32 / BFLOAT16 networks) */
+    int32_t  outputType;        /* FLOAT16 (weightType for FLOAT32 / BFLOAT16 networks) */
     int32_t  gradType;          /* FLOAT16 or FLOAT32: element type of weightsGrad/biasesGrad */
     uint32_t flags;             /* CV_FLAG_* */
     int32_t  inputEncoding;     /* CvInputEncoding */
@@ -398,7 +399,8 @@ typedef struct CvMlpDesc {
 
 /* y = layer_{n-1}( ... layer_0(x) ): every layer is coopVecMatMulAdd + activation with
  * CoopVec<half> as the carrier between layers; with weightType FLOAT_E4M3 the carrier is
- * re-quantised to OCP e4m3 (saturating) in front of every layer.  Activations stay in
+ * re-quantised to OCP e4m3 (saturating) in front of every layer; with weightType FLOAT32 / BFLOAT16 the
+ * carrier is CoopVec<float> / bfloat16 (the FFLayer<float, ...> chain of the neural module).  Activations stay in
  * registers between layers. */
 CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp,
                              const void* input, size_t inputStride,
@@ -465,7 +467,8 @@ CV_API CvResult cvNeuralNetworkSize(const CvNeuralNetworkDesc* net, size_t* elem
 /* toOptimalLayout (:487-516) / toPortableLayout (:524-553) of the whole block in one launch. */
 CV_API CvResult cvNeuralToOptimalLayout(void* stream, const CvNeuralNetworkDesc* net, const void* portable, void* optimal);
 CV_API CvResult cvNeuralToPortableLayout(void* stream, const CvNeuralNetworkDesc* net, const void* optimal, void* portable);
-/* The FFLayer chain y = Activation_l(W_l x + b_l) (layers.slang:90-110) over a FLOAT16 parameter block,
+/* The FFLayer chain y = Activation_l(W_l x + b_l) (layers.slang:90-110) over a FLOAT16 or FLOAT32 parameter block
+ * (vectors and results have the block's element type),
  * in the portable (LinearLayout; optimalLayout = 0) or the optimal layout in NATIVE order
  * (optimalLayout = 1); layer l's bias sits WeightStorageSize elements behind its weights (:93-96).
  * activations / leakySlopes: one CvActivation / slope per layer (NULL: none).  Served by cvMlpForward. */

@@ -576,6 +576,12 @@ class InputEncoding(enum.IntEnum):
     XYSquares = 1
 
 
+def _mlp_carrier_type(weightType: int) -> CoopVecComponentType:
+    if weightType in (CoopVecComponentType.Float32, CoopVecComponentType.BFloat16):
+        return CoopVecComponentType(weightType)
+    return CoopVecComponentType.Float16
+
+
 def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int, flags: int,
               inputEncoding: int = 0):
     arr = (_lib.CvMlpLayer * len(layers))()
@@ -591,7 +597,8 @@ def _mlp_desc(layers: Sequence[FeedForwardLayer], weightType: int, gradType: int
     d = _lib.CvMlpDesc()
     d.layers = arr; d.numLayers = len(layers)
     d.inputType = int(weightType); d.weightType = int(weightType)
-    d.biasType = int(CoopVecComponentType.Float16); d.outputType = int(CoopVecComponentType.Float16)
+    carrier = _mlp_carrier_type(weightType)      # half, or T for networks of one type T = float / bfloat16
+    d.biasType = int(carrier); d.outputType = int(carrier)
     d.gradType = int(gradType); d.flags = int(flags); d.inputEncoding = int(inputEncoding)
     if inputEncoding:
         d.inputType = int(CoopVecComponentType.Float32)
@@ -602,12 +609,16 @@ def mlpForward(layers: Sequence[FeedForwardLayer], input: torch.Tensor, *,
                weightType: int = CoopVecComponentType.Float16, out: Optional[torch.Tensor] = None,
                flags: int = 0, inputEncoding: int = 0, stream=None) -> torch.Tensor:
     """network.eval over a batch: every layer is coopVecMatMulAdd + activation with CoopVec<half>
-    between layers (network.slang:41-47), fused into one kernel."""
+    between layers (network.slang:41-47), fused into one kernel.  weightType Float32 / BFloat16: a network
+    of that one type (vectors, biases, results), the neural module's FFLayer<float, ...> chain."""
     inCt, inStride = _vector_info(input, weightType, "input")
     batch = input.shape[0]
+    carrier = _mlp_carrier_type(weightType)
     if out is None:
-        out = torch.empty((batch, layers[-1].outputSize), dtype=torch.float16, device=input.device)
-    _, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
+        out = torch.empty((batch, layers[-1].outputSize), dtype=_CT_TO_TORCH[carrier], device=input.device)
+    outCt, outStride = _vector_info(out, carrier, "out")
+    if outCt != carrier:
+        raise CoopVecError(SLANG_E_INVALID_ARG, "out must have the network's result type")
     d, keep = _mlp_desc(layers, weightType, CoopVecComponentType.Float32, flags, inputEncoding)
     d.inputType = int(inCt)
     _check(_lib.load().cvMlpForward(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride,
@@ -632,6 +643,8 @@ class MlpForwardPlan:
         self._ref = ctypes.byref(self._desc)
         self._fn = _lib.load().cvMlpForward
         self._outputSize = self._layers[-1].outputSize
+        self._carrier = _mlp_carrier_type(weightType)
+        self._outDtype = _CT_TO_TORCH[self._carrier]
         self._inCt = None
 
     def __call__(self, input: torch.Tensor, out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
@@ -641,8 +654,10 @@ class MlpForwardPlan:
             self._inCt = inCt
         batch = input.shape[0]
         if out is None:
-            out = torch.empty((batch, self._outputSize), dtype=torch.float16, device=input.device)
-        _, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
+            out = torch.empty((batch, self._outputSize), dtype=self._outDtype, device=input.device)
+        outCt, outStride = _vector_info(out, self._carrier, "out")
+        if outCt != self._carrier:
+            raise CoopVecError(SLANG_E_INVALID_ARG, "out must have the network's result type")
         rc = self._fn(_stream_handle(stream), self._ref, input.data_ptr(), inStride, out.data_ptr(), outStride, batch)
         if rc < 0:
             _check(rc)
@@ -811,15 +826,17 @@ class NetworkParameterLayoutConverter:
 
     def eval(self, params: torch.Tensor, input: torch.Tensor, *, optimalLayout: bool, activations=None, leakySlopes=None,
              out: Optional[torch.Tensor] = None, stream=None) -> torch.Tensor:
-        """The FFLayer chain (layers.slang:90-110) over the block, fp16."""
-        _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+        """The FFLayer chain (layers.slang:90-110) over the block; vectors and results have the block's element type."""
+        _, inStride = _vector_info(input, self.desc.elementType, "input")
+        if input.dtype != self.dtype or (out is not None and out.dtype != self.dtype):
+            raise CoopVecError(SLANG_E_INVALID_ARG, "input and out must have the network's element type")
         if out is None:
-            out = torch.empty(input.shape[0], self.desc.dims[self.desc.layerCount], dtype=torch.float16, device=input.device)
+            out = torch.empty(input.shape[0], self.desc.dims[self.desc.layerCount], dtype=self.dtype, device=input.device)
         a, s = self._acts(activations, leakySlopes)
         count = self.ElementCountPhysical if optimalLayout else self.ElementCountLogical
         _check(_lib.load().cvNeuralMlpForward(_stream_handle(stream), ctypes.byref(self.desc), 1 if optimalLayout else 0,
                                               self._buf(params, count, "params"), a, s, input.data_ptr(), inStride,
-                                              out.data_ptr(), out.stride(0) * 2, input.shape[0]))
+                                              out.data_ptr(), out.stride(0) * out.element_size(), input.shape[0]))
         return out
 
     def trainStep(self, params: torch.Tensor, paramGrads: torch.Tensor, input: torch.Tensor, targets: Optional[torch.Tensor], *,

@@ -554,9 +554,16 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
     if (!mlp || !mlp->layers) return fail(CV_E_INVALID_ARG, "%s: mlp/layers is null", who);
     if (mlp->numLayers < 1 || mlp->numLayers > cv::kMaxMlpLayers)
         return fail(CV_E_INVALID_ARG, "%s: numLayers=%d (supported: 1..%d)", who, mlp->numLayers, cv::kMaxMlpLayers);
-    if (mlp->weightType != CV_FLOAT16 && mlp->weightType != CV_FLOAT_E4M3)
-        return fail(CV_E_NOT_AVAILABLE, "%s: weightType %d (supported: FLOAT16, FLOAT_E4M3)", who, mlp->weightType);
-    if (mlp->biasType != CV_FLOAT16 || mlp->outputType != CV_FLOAT16)
+    const bool uniformT = mlp->weightType == CV_FLOAT32 || mlp->weightType == CV_BFLOAT16;   // T = float / bfloat16 throughout
+    if (mlp->weightType != CV_FLOAT16 && mlp->weightType != CV_FLOAT_E4M3 && !uniformT)
+        return fail(CV_E_NOT_AVAILABLE, "%s: weightType %d (supported: FLOAT16, FLOAT_E4M3, and FLOAT32 / BFLOAT16 networks of one type)",
+                    who, mlp->weightType);
+    if (uniformT) {
+        if (mlp->inputType != mlp->weightType || mlp->biasType != mlp->weightType || mlp->outputType != mlp->weightType ||
+            mlp->inputEncoding != CV_ENCODE_NONE)
+            return fail(CV_E_NOT_AVAILABLE, "%s: a network with weightType %d takes vectors, biases and results of that type and no "
+                        "input encoding", who, mlp->weightType);
+    } else if (mlp->biasType != CV_FLOAT16 || mlp->outputType != CV_FLOAT16)
         return fail(CV_E_NOT_AVAILABLE, "%s: biasType/outputType must be FLOAT16", who);
     if (mlp->inputEncoding == CV_ENCODE_XY_SQUARES) {
         if (mlp->inputType != CV_FLOAT32 || mlp->weightType != CV_FLOAT16 || mlp->layers[0].inputSize != 4 || mlp->numLayers < 2)
@@ -589,7 +596,7 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
                                   isOptimal(L.weightLayout) ? 0 : (size_t)L.weightStride};
         if (cv::matrixSize(o.shape) == 0) return fail(CV_E_INVALID_ARG, "%s: layer %d: weightStride %u smaller than a row/column", who, l, L.weightStride);
         if ((uintptr_t)o.w % (isOptimal(L.weightLayout) ? 16u : wEsz) || (!isOptimal(L.weightLayout) && L.weightStride % wEsz) ||
-            (uintptr_t)o.bias % 2)
+            (uintptr_t)o.bias % cv::elemSize(mlp->biasType))
             return fail(CV_E_INVALID_ARG, "%s: layer %d: weights/bias misaligned", who, l);
         o.in = L.inputSize; o.out = L.outputSize; o.act = L.activation; o.slope = L.leakySlope;
     }
@@ -609,18 +616,19 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     const int L = mlp->numLayers;
     const bool encoded = mlp->inputEncoding == CV_ENCODE_XY_SQUARES;
     const size_t sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * inEsz;
-    if ((uintptr_t)input % inEsz || inputStride % inEsz || (uintptr_t)output % 2 || outputStride % 2)
+    const uint32_t outEsz = cv::elemSize(mlp->outputType);
+    if ((uintptr_t)input % inEsz || inputStride % inEsz || (uintptr_t)output % outEsz || outputStride % outEsz)
         return fail(CV_E_INVALID_ARG, "cvMlpForward: vector address/stride not aligned to the element size");
-    if (batch > 1 && (inputStride < sampleBytes || outputStride < (size_t)mlp->layers[L - 1].outputSize * 2))
+    if (batch > 1 && (inputStride < sampleBytes || outputStride < (size_t)mlp->layers[L - 1].outputSize * outEsz))
         return fail(CV_E_INVALID_ARG, "cvMlpForward: vector stride smaller than the vector");
     if (L == 1) {   // a single layer is the plain operator
         const CvMlpLayer& l0 = mlp->layers[0];
         CvMatMulDesc d;
         memset(&d, 0, sizeof(d));
         d.input = input; d.inputStride = inputStride; d.inputType = mlp->inputType; d.inputInterpretation = mlp->weightType;
-        d.k = l0.inputSize; d.output = output; d.outputStride = outputStride; d.resultType = CV_FLOAT16; d.m = l0.outputSize;
+        d.k = l0.inputSize; d.output = output; d.outputStride = outputStride; d.resultType = mlp->outputType; d.m = l0.outputSize;
         d.matrix = l0.weights; d.matrixInterpretation = mlp->weightType; d.layout = l0.weightLayout; d.matrixStride = l0.weightStride;
-        d.bias = l0.biases; d.biasInterpretation = CV_FLOAT16; d.activation = l0.activation; d.leakySlope = l0.leakySlope;
+        d.bias = l0.biases; d.biasInterpretation = mlp->biasType; d.activation = l0.activation; d.leakySlope = l0.leakySlope;
         d.batch = batch; d.flags = mlp->flags;
         return cvMatMul(stream, &d);
     }
@@ -632,10 +640,15 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     a.inHalfAsE4M3 = (mlp->inputType == CV_FLOAT16 && mlp->weightType == CV_FLOAT_E4M3) ? 1 : 0;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16
-                     : (mlp->flags & CV_FLAG_FP8_MATRIX_PIPELINE) ? cv::MmaKind::Fp8Native : cv::MmaKind::Fp8AsF16;
-    hipError_t e = cv::launchMlpForward((hipStream_t)stream, kind, a, cus);
-    if (e == hipErrorInvalidValue) e = cv::launchMlpGeneric((hipStream_t)stream, kind, a, cus);   // no built-in shape: general kernel
+    hipError_t e;
+    if (mlp->weightType == CV_FLOAT32 || mlp->weightType == CV_BFLOAT16) {
+        e = cv::launchMlpFloat((hipStream_t)stream, mlp->weightType == CV_FLOAT32 ? cv::MmaKind::F32 : cv::MmaKind::Bf16, a, cus);
+    } else {
+        cv::MmaKind kind = mlp->weightType == CV_FLOAT16 ? cv::MmaKind::F16
+                         : (mlp->flags & CV_FLAG_FP8_MATRIX_PIPELINE) ? cv::MmaKind::Fp8Native : cv::MmaKind::Fp8AsF16;
+        e = cv::launchMlpForward((hipStream_t)stream, kind, a, cus);
+        if (e == hipErrorInvalidValue) e = cv::launchMlpGeneric((hipStream_t)stream, kind, a, cus);   // no built-in shape: general kernel
+    }
     if (e == hipErrorInvalidValue)
         return fail(CV_E_NOT_AVAILABLE, "cvMlpForward: layer sizes beyond the fused kernels (every dimension must be <= 128 "
                     "and all weights must fit 144 KB of LDS); chain cvMatMul calls instead");

@@ -71,6 +71,9 @@ enum : int { kEncodeNone = 0, kEncodeXYSquares = 1 };
 hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 // any layer sizes up to 128 (weights read from LDS); hipErrorInvalidValue beyond that
 hipError_t launchMlpGeneric(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
+// networks of one type T = float (MmaKind::F32) or bfloat16 (MmaKind::Bf16): vectors, weights, biases, results;
+// same limits as launchMlpGeneric
+hipError_t launchMlpFloat(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 
 // ---- fused training step ------------------------------------------------------------------
 struct TrainLaunch {

@@ -166,7 +166,9 @@ CvResult layersFromBlock(const char* who, const CvNeuralNetworkDesc* n, int32_t 
 {
     CvResult rc = checkNet(who, n);
     if (CV_FAILED(rc)) return rc;
-    if (n->elementType != CV_FLOAT16) return failWith(CV_E_NOT_AVAILABLE, "%s: the fused kernels take FLOAT16 parameters (T = half)", who);
+    if (grads && n->elementType != CV_FLOAT16)
+        return failWith(CV_E_NOT_AVAILABLE, "%s: the fused training step takes FLOAT16 parameters (T = half)", who);
+    const size_t esz = n->elementType == CV_FLOAT32 ? 4u : 2u;
     if (optimal && n->order != CV_NEURAL_ORDER_NATIVE)
         return failWith(CV_E_NOT_AVAILABLE, "%s: an optimal-layout block must be in CV_NEURAL_ORDER_NATIVE order (convert it first)", who);
     if (n->layerCount > kMaxMlpLayers) return failWith(CV_E_NOT_AVAILABLE, "%s: at most %d layers", who, kMaxMlpLayers);
@@ -179,15 +181,15 @@ CvResult layersFromBlock(const char* who, const CvNeuralNetworkDesc* n, int32_t 
         const size_t bElems = optimal ? (size_t)align16(o) : (hasBias ? (size_t)o : 0);       // FFLayer::BiasStorageSize, :68-71
         CvMlpLayer& L = out[l];
         memset(&L, 0, sizeof(L));
-        L.weights = (const uint8_t*)params + off * 2;
-        L.biases = hasBias ? (const uint8_t*)params + (off + wElems) * 2 : nullptr;
+        L.weights = (const uint8_t*)params + off * esz;
+        L.biases = hasBias ? (const uint8_t*)params + (off + wElems) * esz : nullptr;
         if (grads) {
             L.weightsGrad = (uint8_t*)grads + off * 2;
             L.biasesGrad = hasBias ? (uint8_t*)grads + (off + wElems) * 2 : nullptr;
         }
         L.inputSize = in; L.outputSize = o;
         L.weightLayout = L.gradLayout = optimal ? CV_LAYOUT_TRAINING_OPTIMAL : CV_LAYOUT_ROW_MAJOR;
-        L.weightStride = L.gradStride = optimal ? 0u : (uint32_t)in * 2u;
+        L.weightStride = L.gradStride = optimal ? 0u : (uint32_t)(in * esz);
         L.activation = activations ? activations[l] : CV_ACT_NONE;
         L.leakySlope = leakySlopes ? leakySlopes[l] : 0.f;
         off += wElems + bElems;
@@ -229,7 +231,8 @@ CV_API CvResult cvNeuralMlpForward(void* stream, const CvNeuralNetworkDesc* net,
     CvMlpLayer layers[cv::kMaxMlpLayers];
     CvResult rc = cv::layersFromBlock("cvNeuralMlpForward", net, optimalLayout, params, nullptr, activations, leakySlopes, layers);
     if (CV_FAILED(rc)) return rc;
-    CvMlpDesc mlp = {layers, net->layerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_NONE};
+    const int32_t T = net->elementType;      // vectors, parameters and results share the network's element type
+    CvMlpDesc mlp = {layers, net->layerCount, T, T, T, T, CV_FLOAT16, 0, CV_ENCODE_NONE};
     return cvMlpForward(stream, &mlp, input, inputStride, output, outputStride, batch);
 }
 
@@ -256,6 +259,8 @@ CV_API CvResult cvNeuralMlpTrainStepWorkspaceSize(const CvNeuralNetworkDesc* net
 {
     CvMlpLayer layers[cv::kMaxMlpLayers];
     static const uint16_t dummy = 0;
+    if (net && net->elementType != CV_FLOAT16)
+        return cv::failWith(CV_E_NOT_AVAILABLE, "cvNeuralMlpTrainStepWorkspaceSize: the fused training step takes FLOAT16 parameters (T = half)");
     CvResult rc = cv::layersFromBlock("cvNeuralMlpTrainStepWorkspaceSize", net, 0, &dummy, nullptr, nullptr, nullptr, layers);
     if (CV_FAILED(rc)) return rc;
     CvMlpDesc mlp = {layers, net->layerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_NONE};
