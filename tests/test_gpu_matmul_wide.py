@@ -229,10 +229,12 @@ def test_float32_matrix_equals_the_slang_operator_on_exact_data():
     y = cv.coopVecMatMulAdd(to_dev(x), CT.Float32, to_dev(W.view(np.uint8).ravel()), 0, CT.Float32, as_bytes(to_dev(b)), 0,
                             CT.Float32, ML.RowMajor, False, 4 * K, M=M, resultType=CT.Float32)
     assert np.array_equal(y.cpu().numpy(), want)
-    # a Float32 matrix takes fp32 vectors only
-    with pytest.raises(cv.CoopVecError):
-        cv.coopVecMatMul(to_dev(x.astype(np.float16)), CT.Float16, to_dev(W.view(np.uint8).ravel()), 0, CT.Float32,
-                         ML.RowMajor, False, 4 * K, M=M)
+    # on the matrix pipeline a Float32 matrix takes fp32 vectors only; fp16 vectors against it run as the scalar
+    # definition (exact data: the same result)
+    y = cv.coopVecMatMul(to_dev(x.astype(np.float16)), CT.Float16, to_dev(W.view(np.uint8).ravel()), 0, CT.Float32,
+                         ML.RowMajor, False, 4 * K, M=M, resultType=CT.Float32)
+    assert cv.lastKernelName().startswith("matmulScalarKernel"), cv.lastKernelName()
+    assert np.array_equal(y.cpu().numpy(), x @ W.T)
 
 
 # ---- beyond 128 rows / 128 columns --------------------------------------------------------------
