@@ -349,6 +349,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 half_t gv[4];
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
+                    gv[rr] = (half_t)0;
+                    // rows 4t+rr and beyond of every lane group lie past the output (a one-output network uses one
+                    // of these four steps): a wave-uniform skip
+                    if (4 * t + rr >= outDim) continue;
                     const int row = g * OROWS + 4 * t + rr;
                     const bool on = live && row < outDim;
                     float tv = exampleLoss ? (float)gt[rr] : tgtAll;
