@@ -413,6 +413,34 @@ def test_forward_plan_equals_mlp_forward():
             plan(xd[:, ::2])
 
 
+def test_forward_in_a_hip_graph():
+    # a launch-bound loop of small forward passes recorded into one HIP graph: the library launches on the
+    # capturing stream and allocates nothing; every replay, with eager work in between, gives the eager result
+    rng = np.random.default_rng(41)
+    specs = make_net(rng, [2, 16, 16, 16, 1], CT.Float16, act=Activation.ReLU)
+    layers = gpu_layers(specs, CT.Float16, ML.RowMajor)
+    B = 4096
+    x = torch.zeros(B, 2, dtype=torch.float16, device=DEV)
+    outs = [torch.zeros(B, 1, dtype=torch.float16, device=DEV) for _ in range(3)]
+    plan = cv.MlpForwardPlan(layers)
+    plan(x, outs[0])                                   # first call outside the capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for o in outs:
+            plan(x, o)
+    for seed in range(4):
+        xn = to_dev(np.random.default_rng(seed).uniform(0, 1, (B, 2)).astype(np.float16))
+        want = cv.mlpForward(layers, xn)               # eager work between the replays
+        x.copy_(xn)
+        for o in outs:
+            o.fill_(-1)
+        g.replay()
+        torch.cuda.synchronize()
+        for o in outs:
+            assert torch.equal(o.view(torch.int16), want.view(torch.int16)), seed
+
+
 def test_mlp_argument_validation():
     rng = np.random.default_rng(0)
     specs = make_net(rng, [8, 16, 4], CT.Float16)
