@@ -154,9 +154,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         const MlpLayerArgs& ly = a.layers[l];
         const uint32_t gs = optGS((uint32_t)ly.in);
         uint32_t* base = ldsW + Net::fragBase(l) * 64 * RAW;
-        stageFragments<ESZ, EPL>(base, ly.w, ly.shape, false, MT, KT, gs, (uint32_t)ly.out, (uint32_t)ly.in);
+        stageFragments<ESZ, EPL>(base, ly.w, ly.shape, false, MT, KT, gs, (uint32_t)ly.out, (uint32_t)ly.in, 0, 0,
+                                 (uint32_t)(Net::fragBase(l) * 64) % 256u);
         // bias of tile t, lane group g, r: row g*ROWS + 4t + r  ->  ldsB[(biasBase + t)*16 + 4g + r]
-        for (int e = threadIdx.x; e < MT * 16; e += 256) {
+        // (each layer from another wave of the workgroup, like its weights: the loads of the layers overlap)
+        for (int e = (int)((threadIdx.x + 256u - 64u * (l % 4)) % 256u); e < MT * 16; e += 256) {
             const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
             const int row = g * ROWS + 4 * t + r;
             uint16_t v = 0;

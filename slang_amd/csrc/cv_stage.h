@@ -22,7 +22,8 @@ namespace cv {
 template <int ESZ, int EPL>
 __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* w, const MatrixShape& shape,
                                                bool transposed, int MT, int KT, uint32_t gs, uint32_t rows,
-                                               uint32_t cols, uint32_t rowOff = 0, uint32_t xorByte = 0)
+                                               uint32_t cols, uint32_t rowOff = 0, uint32_t xorByte = 0,
+                                               uint32_t firstThread = 0)
 {
     constexpr int CHUNK = ESZ * EPL;              // bytes of one lane-chunk: 8, 16 or 32
     static_assert(ESZ == 1 || ESZ == 2 || ESZ == 4, "element size");
@@ -40,7 +41,10 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
     const bool contiguous = (shape.layout == kRowMajor && !transposed) || (shape.layout == kColumnMajor && transposed);
     const uint32_t xorWord = xorByte * 0x01010101u;
     const int ROWS = 4 * MT;
-    for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    // firstThread: the thread that takes chunk 0.  A kernel that stages several small matrices gives each its own
+    // part of the workgroup, so that their round trips to memory overlap instead of following one another.
+    const uint32_t vt = threadIdx.x >= firstThread ? threadIdx.x - firstThread : threadIdx.x + blockDim.x - firstThread;
+    for (int c = (int)vt; c < chunks; c += blockDim.x) {
         const int lane = c & 63, f = c >> 6;
         const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
         const uint32_t row = (uint32_t)((i >> 2) * ROWS + 4 * t + (i & 3));
@@ -59,6 +63,30 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
             for (int i8 = 0; i8 < CHUNK / 8; ++i8) {
                 const u32x2 x = ((const u32x2*)p0)[i8];
                 ((u32x2*)d)[i8] = u32x2{x.x ^ xorWord, x.y ^ xorWord};
+            }
+        } else if (contiguous) {
+            // a ragged or unaligned run of elements that lie side by side: all loads first (always-valid
+            // addresses, masked afterwards), then the stores, so that the run costs one round trip to memory
+            // instead of one per element (small networks spend most of their few microseconds here)
+            uint32_t v[EPL];
+#pragma unroll
+            for (int s = 0; s < EPL; ++s) {
+                const uint8_t* p = s < nvalid ? p0 + s * ESZ : w;
+                if constexpr (ESZ == 4)      v[s] = *(const uint32_t*)p;
+                else if constexpr (ESZ == 2) v[s] = *(const uint16_t*)p;
+                else                         v[s] = (uint32_t)(*p ^ xorByte);
+            }
+#pragma unroll
+            for (int s = 0; s < EPL; ++s) v[s] = s < nvalid ? v[s] : 0u;
+            if constexpr (ESZ == 4) {
+#pragma unroll
+                for (int s = 0; s < EPL; ++s) d[s] = v[s];
+            } else if constexpr (ESZ == 2) {
+#pragma unroll
+                for (int s = 0; s < EPL; s += 2) d[s / 2] = v[s] | (v[s + 1] << 16);
+            } else {
+#pragma unroll
+                for (int s = 0; s < EPL; s += 4) d[s / 4] = v[s] | (v[s + 1] << 8) | (v[s + 2] << 16) | (v[s + 3] << 24);
             }
         } else {
             // element by element (kept as a loop: staging runs once per workgroup, and unrolled its code would be large)
