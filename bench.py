@@ -44,7 +44,7 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
 # HBM bytes per step (all kernels of the step) as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
 # scaled by a copy of known size): not measured by this script, quoted from the committed profile summaries.
 PROFILED_TRAFFIC = {
-    "c1": (732000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
+    "c1": (739000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
     "c2": (1084765000, "profiles/matmul_f16_64x64_batch4M.md"),
     "c2b": (1084788000, "profiles/matmul_bf16_64x64_batch4M.md"),
     "c3": (2684654000, "profiles/matmul_i8_128x128_batch4M.md"),
