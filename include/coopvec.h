@@ -232,8 +232,12 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* desc);
  *   Mat[i][j] += sum_s a[s][i] * b[s][j]
  * The per-sample atomics of the reference are replaced by an MFMA contraction over the batch,
  * per-workgroup fp32 partials in `workspace` and one fixed-order reduction, so the result is
- * bitwise reproducible.  a and b are FLOAT16 vectors; the matrix interpretation is FLOAT16
- * or FLOAT32; all four layouts are accepted for the destination. */
+ * bitwise reproducible.  That kernel takes FLOAT16 vectors and a FLOAT16 or FLOAT32 matrix in any of the four
+ * layouts.  Every other pair of the fallback's types (FLOAT16/32/64 and the 8/16/32/64-bit integers for the
+ * vectors and for the matrix, :33261-33315) runs as the scalar definition: the product in the vectors' type,
+ * cast to the matrix type, summed over the batch (integers modulo 2^width: bit-exact with the reference;
+ * floats in fp32, fp64 for a FLOAT64 matrix, in a fixed order), RowMajor / ColumnMajor (fp32 also the Optimal
+ * layouts). */
 CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t m, int32_t n, uint32_t batch,
                                                       size_t* outBytes);
 CV_API CvResult cvOuterProductAccumulate(void* stream,
@@ -246,8 +250,9 @@ CV_API CvResult cvOuterProductAccumulate(void* stream,
 
 /* coopVecReduceSumAccumulate over a batch (hlsl.meta.slang:33330-33353):
  *   buffer[i] += sum_s v[s][i]
- * v is FLOAT16; `bufferType` is FLOAT16 (the reference's rule: destination type = vector
- * type) or FLOAT32 (what "bias gradients into fp32 buffers" needs). Deterministic. */
+ * `bufferType` is the vectors' type (the reference's rule); FLOAT16 vectors also go into a FLOAT32 buffer
+ * (what "bias gradients into fp32 buffers" needs).  Vectors of FLOAT16/32/64 and of the 8/16/32/64-bit
+ * integers (these modulo 2^width, bit-exact with the reference).  Deterministic. */
 CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t n, uint32_t batch, size_t* outBytes);
 CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStride, int32_t n,
                                       int32_t elementType, uint32_t batch,

@@ -464,7 +464,8 @@ CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t m, int32_t n, uint
     CvResult rc;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    *outBytes = cv::outerWorkspaceBytes(m, n, batch ? batch : 1, cus);
+    const size_t fast = cv::outerWorkspaceBytes(m, n, batch ? batch : 1, cus), scalar = cv::accumScalarWorkspaceBytes(m, n, batch ? batch : 1);
+    *outBytes = fast > scalar ? fast : scalar;      // whichever kernel the element types select
     return CV_OK;
 }
 
@@ -475,13 +476,33 @@ CV_API CvResult cvOuterProductAccumulate(void* stream, const void* a, size_t aSt
                                          size_t workspaceBytes)
 {
     if (m <= 0 || n <= 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: m=%d n=%d", m, n);
-    if (elementType != CV_FLOAT16)
-        return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: vectors must be FLOAT16 (got %d)", elementType);
     if (cvComponentPackingFactor(matrixInterpretation) != 1)   // static_assert hlsl.meta.slang:33237
         return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: can't use packed component type in matrixInterpretation");
-    if (matrixInterpretation != CV_FLOAT16 && matrixInterpretation != CV_FLOAT32)
-        return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: matrixInterpretation %d (supported: FLOAT16, FLOAT32)", matrixInterpretation);
     if (layout < 0 || layout > 3) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: unknown layout %d", layout);
+    const bool onMatrixCores = elementType == CV_FLOAT16 && (matrixInterpretation == CV_FLOAT16 || matrixInterpretation == CV_FLOAT32);
+    if (!onMatrixCores) {
+        // every other pair of the fallback's types (hlsl.meta.slang:33261-33315): the scalar definition
+        if (!cv::isPlainComponent(elementType) || !cv::isPlainComponent(matrixInterpretation))
+            return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: vectors of type %d into a matrix of type %d (supported: FLOAT16/32/64 "
+                        "and the 8/16/32/64-bit integers on either side)", elementType, matrixInterpretation);
+        if (!cv::layoutSupports(matrixInterpretation, layout))
+            return fail(CV_E_NOT_AVAILABLE, "cvOuterProductAccumulate: component type %d has no layout %d", matrixInterpretation, layout);
+        if (batch == 0) return CV_OK;
+        if (!a || !b || !matrix || !workspace) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: null argument");
+        const uint32_t tsz = cv::elemSize(elementType), msz = cv::elemSize(matrixInterpretation);
+        if ((uintptr_t)a % tsz || aStride % tsz || (uintptr_t)b % tsz || bStride % tsz || (uintptr_t)workspace % 8)
+            return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: misaligned vectors/workspace");
+        if (batch > 1 && (aStride < (size_t)m * tsz || bStride < (size_t)n * tsz))
+            return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: vector stride smaller than the vector");
+        const cv::MatrixShape shape{(uint32_t)m, (uint32_t)n, matrixInterpretation, layout, isOptimal(layout) ? 0 : (size_t)matrixStride};
+        if (cv::matrixSize(shape) == 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrixStride %u smaller than a row/column", matrixStride);
+        uint8_t* dst = (uint8_t*)matrix + matrixOffset;
+        if ((uintptr_t)dst % msz || (!isOptimal(layout) && matrixStride % msz)) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrix misaligned");
+        const size_t need = cv::accumScalarWorkspaceBytes(m, n, batch);
+        if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvOuterProductAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+        return fromHip(cv::launchAccumScalar((hipStream_t)stream, (const uint8_t*)a, aStride, m, (const uint8_t*)b, bStride, n, elementType, batch,
+                                             dst, shape, workspace), "cvOuterProductAccumulate launch");
+    }
     if (batch == 0) return CV_OK;
     if (!a || !b || !matrix || !workspace) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: null argument");
     if ((uintptr_t)a % 2 || aStride % 2 || (uintptr_t)b % 2 || bStride % 2 || (uintptr_t)workspace % 16)
@@ -515,7 +536,8 @@ CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t n, uint32_t batch, si
     CvResult rc;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    *outBytes = cv::reduceSumWorkspaceBytes(batch ? batch : 1, cus);
+    const size_t fast = cv::reduceSumWorkspaceBytes(batch ? batch : 1, cus), scalar = cv::accumScalarWorkspaceBytes(n, 1, batch ? batch : 1);
+    *outBytes = fast > scalar ? fast : scalar;
     return CV_OK;
 }
 
@@ -524,8 +546,24 @@ CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStrid
                                       void* workspace, size_t workspaceBytes)
 {
     if (n <= 0) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: n=%d", n);
+    if (elementType != CV_FLOAT16) {
+        // the destination has the vectors' type (hlsl.meta.slang:33344-33352): the scalar definition for every plain type
+        if (!cv::isPlainComponent(elementType) || bufferType != elementType)
+            return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: vectors of type %d into a buffer of type %d (the buffer has the vectors' "
+                        "type; FLOAT16 vectors also go into FLOAT32)", elementType, bufferType);
+        if (batch == 0) return CV_OK;
+        if (!v || !buffer || !workspace) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: null argument");
+        const uint32_t tsz = cv::elemSize(elementType);
+        if ((uintptr_t)v % tsz || vStride % tsz || ((uintptr_t)buffer + offset) % tsz || (uintptr_t)workspace % 8)
+            return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: misaligned argument");
+        if (batch > 1 && vStride < (size_t)n * tsz) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: vector stride smaller than the vector");
+        const size_t need = cv::accumScalarWorkspaceBytes(n, 1, batch);
+        if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvReduceSumAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+        const cv::MatrixShape shape{(uint32_t)n, 1u, elementType, CV_LAYOUT_ROW_MAJOR, (size_t)tsz};
+        return fromHip(cv::launchAccumScalar((hipStream_t)stream, (const uint8_t*)v, vStride, n, nullptr, 0, 1, elementType, batch,
+                                             (uint8_t*)buffer + offset, shape, workspace), "cvReduceSumAccumulate launch");
+    }
     if (n > 256) return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: n=%d (limit 256)", n);
-    if (elementType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: vectors must be FLOAT16 (got %d)", elementType);
     if (bufferType != CV_FLOAT16 && bufferType != CV_FLOAT32)
         return fail(CV_E_NOT_AVAILABLE, "cvReduceSumAccumulate: bufferType %d (supported: FLOAT16, FLOAT32)", bufferType);
     if (batch == 0) return CV_OK;

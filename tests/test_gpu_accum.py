@@ -127,3 +127,159 @@ def test_accumulate_argument_validation():
         cv.coopVecOuterProductAccumulate(a, a, m, 0, 16, ML.RowMajor, CT.Float16, workspace=torch.zeros(16, dtype=torch.uint8, device=DEV))
     assert e.value.result == cv.SLANG_E_BUFFER_TOO_SMALL
     cv.coopVecReduceSumAccumulate(a[:0], m, 0)               # empty batch: nothing to do
+
+
+# ---------------------------------------------------------------------------------------------
+# every other plain element type: the scalar definition (hlsl.meta.slang:33261-33315, :33344-33352)
+# ---------------------------------------------------------------------------------------------
+
+NPT = {CT.Float16: np.float16, CT.Float32: np.float32, CT.Float64: np.float64, CT.SignedInt8: np.int8,
+       CT.UnsignedInt8: np.uint8, CT.SignedInt16: np.int16, CT.UnsignedInt16: np.uint16, CT.SignedInt32: np.int32,
+       CT.UnsignedInt32: np.uint32, CT.SignedInt64: np.int64, CT.UnsignedInt64: np.uint64}
+TORCHT = {np.dtype(np.float16): torch.float16, np.dtype(np.float32): torch.float32, np.dtype(np.float64): torch.float64,
+          np.dtype(np.int8): torch.int8, np.dtype(np.uint8): torch.uint8, np.dtype(np.int16): torch.int16,
+          np.dtype(np.uint16): torch.uint16, np.dtype(np.int32): torch.int32, np.dtype(np.uint32): torch.uint32,
+          np.dtype(np.int64): torch.int64, np.dtype(np.uint64): torch.uint64}
+
+
+def typed(a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.uint8).reshape(a.shape[0], -1)).to(DEV).view(TORCHT[a.dtype])
+
+
+def draw(rng, ct, shape, small=False):
+    dt = NPT[ct]
+    if np.dtype(dt).kind == "f":
+        return (rng.standard_normal(shape) * 2.0).astype(dt)
+    info = np.iinfo(dt)
+    lo, hi = (max(info.min, -9), min(info.max, 9)) if small else (info.min, info.max)
+    return rng.integers(lo, hi, shape, dtype=dt, endpoint=True)
+
+
+INT_PAIRS = [(CT.SignedInt8, CT.SignedInt32), (CT.UnsignedInt8, CT.UnsignedInt16), (CT.SignedInt16, CT.SignedInt64),
+             (CT.SignedInt32, CT.SignedInt8), (CT.UnsignedInt32, CT.UnsignedInt64), (CT.SignedInt64, CT.SignedInt64),
+             (CT.UnsignedInt16, CT.SignedInt32), (CT.UnsignedInt64, CT.UnsignedInt8), (CT.SignedInt32, CT.SignedInt32)]
+
+
+@pytest.mark.parametrize("t_ct,m_ct", INT_PAIRS)
+@pytest.mark.parametrize("layout", [ML.RowMajor, ML.ColumnMajor])
+def test_outer_product_integer_types_bit_exact(t_ct, m_ct, layout):
+    # product in T (wraps to T's width), cast to the matrix type (sign- or zero-extended, or cut), summed modulo the
+    # matrix type's width: numpy's same-type integer arithmetic is exactly that, and the order of the samples is free
+    rng = np.random.default_rng(int(t_ct) * 100 + int(m_ct))
+    B, M, N = 777, 7, 5
+    a = draw(rng, t_ct, (B, M)); b = draw(rng, t_ct, (B, N))
+    mt = NPT[m_ct]
+    before = draw(rng, m_ct, (M, N))
+    with np.errstate(over="ignore"):
+        prod = (a[:, :, None] * b[:, None, :]).astype(mt)             # [B, M, N], wrapped twice
+        want = before + prod.sum(axis=0, dtype=mt)
+    stored = np.ascontiguousarray(before if layout == ML.RowMajor else before.T)
+    d = as_bytes(to_dev(stored))
+    stride = stored.shape[1] * stored.itemsize
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, stride, layout, m_ct)
+    assert cv.lastKernelName().startswith("outerScalarKernel"), cv.lastKernelName()
+    got = d.cpu().numpy().view(mt).reshape(stored.shape)
+    got = got if layout == ML.RowMajor else got.T
+    assert np.array_equal(got, want)
+
+
+FLOAT_PAIRS = [(CT.Float32, CT.Float32), (CT.Float32, CT.Float64), (CT.Float64, CT.Float64), (CT.Float64, CT.Float32),
+               (CT.Float16, CT.Float64), (CT.Float32, CT.Float16), (CT.SignedInt16, CT.Float32), (CT.UnsignedInt8, CT.Float64)]
+
+
+@pytest.mark.parametrize("t_ct,m_ct", FLOAT_PAIRS)
+def test_outer_product_float_destinations(t_ct, m_ct):
+    # the products (rounded to T) summed over the batch: float64 of the same products, with the float bar of the
+    # destination type on the sum of magnitudes
+    rng = np.random.default_rng(int(t_ct) * 100 + int(m_ct) + 1)
+    B, M, N = 1500, 9, 6
+    a = draw(rng, t_ct, (B, M), small=True); b = draw(rng, t_ct, (B, N), small=True)
+    mt = NPT[m_ct]
+    before = rng.standard_normal((M, N)).astype(mt)
+    with np.errstate(over="ignore"):
+        prod = (a[:, :, None] * b[:, None, :]).astype(np.float64)      # the product in T, exactly representable in float64
+    want = before.astype(np.float64) + prod.sum(axis=0)
+    mag = np.abs(before.astype(np.float64)) + np.abs(prod).sum(axis=0)
+    d = as_bytes(to_dev(before))
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, N * before.itemsize, ML.RowMajor, m_ct)
+    assert cv.lastKernelName().startswith("outerScalarKernel"), cv.lastKernelName()
+    got = d.cpu().numpy().view(mt).reshape(M, N).astype(np.float64)
+    eps = {np.float16: 2.0 ** -10, np.float32: 2.0 ** -20, np.float64: 2.0 ** -48}[mt]
+    assert (np.abs(got - want) <= eps * mag).all()
+
+
+def test_outer_product_float_vectors_into_integers_and_optimal_layout():
+    rng = np.random.default_rng(99)
+    B, M, N = 300, 6, 4
+    a = (rng.standard_normal((B, M)) * 3).astype(np.float32); b = (rng.standard_normal((B, N)) * 3).astype(np.float32)
+    # cast<int>(product): towards zero, per product
+    want = np.trunc((a[:, :, None] * b[:, None, :]).astype(np.float32)).astype(np.int64).sum(axis=0).astype(np.int32)
+    d = torch.zeros(M * N, dtype=torch.int32, device=DEV)
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), as_bytes(d), 0, N * 4, ML.RowMajor, CT.SignedInt32)
+    assert np.array_equal(d.cpu().numpy().reshape(M, N), want)
+    # fp32 vectors into an fp32 TrainingOptimal matrix (the layout the reference asks for on hardware), read back by convert
+    size = cv.getCooperativeVectorMatrixSize(M, N, CT.Float32, ML.TrainingOptimal)
+    t = torch.zeros(size, dtype=torch.uint8, device=DEV)
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), t, 0, 0, ML.TrainingOptimal, CT.Float32)
+    row = torch.zeros(M * N * 4, dtype=torch.uint8, device=DEV)
+    D = cv.CooperativeVectorMatrixDesc
+    cv.convertCooperativeVectorMatrix(row, [D(M, N, CT.Float32, ML.RowMajor, M * N * 4, 0, N * 4)],
+                                      t, [D(M, N, CT.Float32, ML.TrainingOptimal, size, 0, 0)])
+    ref = a.astype(np.float64).T @ b.astype(np.float64)
+    assert np.allclose(row.view(torch.float32).cpu().numpy().reshape(M, N), ref, rtol=1e-5, atol=1e-4)
+
+
+def test_scalar_accumulate_equals_the_slang_operator_sample_by_sample():
+    # the fallback itself (oracle: cvo_slang_*), applied to one sample after the other: exact for integer
+    # destinations, and for a single sample also for fp32
+    rng = np.random.default_rng(5)
+    B, M, N = 40, 4, 6
+    for t_ct, m_ct, o_t, o_m in ((CT.SignedInt32, CT.SignedInt32, ob.S32, ob.S32), (CT.UnsignedInt32, CT.UnsignedInt8, ob.U32, ob.U8),
+                                 (CT.Float32, CT.SignedInt32, ob.F32, ob.S32), (CT.SignedInt32, CT.SignedInt8, ob.S32, ob.S8)):
+        a = draw(rng, t_ct, (B, M), small=True); b = draw(rng, t_ct, (B, N), small=True)
+        mat = draw(rng, m_ct, (M, N))
+        ref = mat.copy()
+        for s in range(B):
+            assert ob.lib().cvo_slang_outer_product_accumulate(ob.ptr(a[s]), M, ob.ptr(b[s]), N, o_t, ob.ptr(ref), 0, N * ref.itemsize,
+                                                               ob.ROW, o_m, ob.HALF_RNE) == 0
+        d = as_bytes(to_dev(mat))
+        cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, N * mat.itemsize, ML.RowMajor, m_ct)
+        assert np.array_equal(d.cpu().numpy().view(mat.dtype).reshape(M, N), ref), (t_ct, m_ct)
+    a = draw(rng, CT.Float32, (1, M)); b = draw(rng, CT.Float32, (1, N)); mat = draw(rng, CT.Float32, (M, N))
+    ref = mat.copy()
+    assert ob.lib().cvo_slang_outer_product_accumulate(ob.ptr(a[0]), M, ob.ptr(b[0]), N, ob.F32, ob.ptr(ref), 0, N * 4, ob.ROW, ob.F32, ob.HALF_RNE) == 0
+    d = as_bytes(to_dev(mat))
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, N * 4, ML.RowMajor, CT.Float32)
+    assert np.array_equal(d.cpu().numpy().view(np.uint32), ref.view(np.uint32).reshape(-1))
+    # reduce-sum: the destination has the vectors' type
+    for t_ct, o_t in ((CT.SignedInt32, ob.S32), (CT.UnsignedInt32, ob.U32)):
+        v = draw(rng, t_ct, (B, 9)); buf = draw(rng, t_ct, (9,))
+        ref = buf.copy()
+        for s in range(B):
+            assert ob.lib().cvo_slang_reduce_sum_accumulate(ob.ptr(v[s]), 9, o_t, ob.ptr(ref), 0, ob.HALF_RNE) == 0
+        d = as_bytes(to_dev(buf))
+        cv.coopVecReduceSumAccumulate(typed(v), d, 0)
+        assert cv.lastKernelName().startswith("outerScalarKernel"), cv.lastKernelName()
+        assert np.array_equal(d.cpu().numpy().view(buf.dtype), ref)
+
+
+@pytest.mark.parametrize("t_ct", [CT.SignedInt8, CT.UnsignedInt16, CT.SignedInt64, CT.UnsignedInt64, CT.Float32, CT.Float64])
+def test_reduce_sum_every_plain_type(t_ct):
+    rng = np.random.default_rng(int(t_ct) + 300)
+    B, N = 5000, 37
+    v = draw(rng, t_ct, (B, N)); buf = draw(rng, t_ct, (N,))
+    dt = NPT[t_ct]
+    d = as_bytes(to_dev(buf))
+    padded = torch.zeros((B, N + 3), dtype=TORCHT[np.dtype(dt)], device=DEV); padded[:, :N] = typed(v)     # strided rows
+    cv.coopVecReduceSumAccumulate(padded[:, :N], d, 0)
+    got = d.cpu().numpy().view(dt)
+    if np.dtype(dt).kind == "f":
+        want = buf.astype(np.float64) + v.astype(np.float64).sum(axis=0)
+        mag = np.abs(buf.astype(np.float64)) + np.abs(v.astype(np.float64)).sum(axis=0)
+        assert (np.abs(got.astype(np.float64) - want) <= (2.0 ** -20 if dt == np.float32 else 2.0 ** -48) * mag).all()
+    else:
+        with np.errstate(over="ignore"):
+            assert np.array_equal(got, buf + v.sum(axis=0, dtype=dt))      # modulo 2^width
+    with pytest.raises(cv.CoopVecError) as e:                              # the buffer has the vectors' type
+        cv.coopVecReduceSumAccumulate(typed(v), d, 0, bufferType=CT.Float16 if t_ct != CT.Float16 else CT.Float32)
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
