@@ -394,7 +394,8 @@ typedef struct CvMlpDesc {
     int32_t  numLayers;
     int32_t  inputType;         /* element type of the input vectors in memory */
     int32_t  weightType;        /* matrix interpretation of every layer: FLOAT16 or FLOAT_E4M3; FLOAT32 or BFLOAT16 for
-                                   a network of that one type (vectors, biases and results too; forward only) */
+                                   a network of that one type (vectors, biases, results and targets too; BFLOAT16 forward
+                                   only, FLOAT32 also trains: layer by layer, FLOAT32 gradients) */
     int32_t  biasType;          /* FLOAT16 (weightType for FLOAT32 / BFLOAT16 networks) */
     int32_t  outputType;        /* FLOAT16 (weightType for FLOAT32 / BFLOAT16 networks) */
     int32_t  gradType;          /* FLOAT16 or FLOAT32: element type of weightsGrad/biasesGrad */
@@ -481,8 +482,8 @@ CV_API CvResult cvNeuralMlpForward(void* stream, const CvNeuralNetworkDesc* net,
                                    const int32_t* activations, const float* leakySlopes,
                                    const void* input, size_t inputStride, void* output, size_t outputStride, uint32_t batch);
 /* bwd_diff through the chain with a gradient block laid out like the parameter block (the
- * DifferentialPtrPair of layers.slang:21-25): gradients are accumulated in FLOAT16 at the same element
- * offsets.  Served by cvMlpTrainStep (same loss, targets, workspace rules). */
+ * DifferentialPtrPair of layers.slang:21-25): gradients are accumulated in the block's element type (FLOAT16 or
+ * FLOAT32) at the same element offsets.  Served by cvMlpTrainStep (same loss, targets, workspace rules). */
 CV_API CvResult cvNeuralMlpTrainStepWorkspaceSize(const CvNeuralNetworkDesc* net, uint32_t batch, size_t* outBytes);
 CV_API CvResult cvNeuralMlpTrainStep(void* stream, const CvNeuralNetworkDesc* net, int32_t optimalLayout, const void* params,
                                      void* paramGrads, const int32_t* activations, const float* leakySlopes,

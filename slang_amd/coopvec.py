@@ -665,8 +665,9 @@ class MlpForwardPlan:
 
 
 def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
-                              gradType: int = CoopVecComponentType.Float32, flags: int = 0, inputEncoding: int = 0) -> int:
-    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, flags, inputEncoding)
+                              gradType: int = CoopVecComponentType.Float32, flags: int = 0, inputEncoding: int = 0,
+                              weightType: int = CoopVecComponentType.Float16) -> int:
+    d, keep = _mlp_desc(layers, weightType, gradType, flags, inputEncoding)
     out = ctypes.c_size_t(0)
     _check(_lib.load().cvMlpTrainStepWorkspaceSize(ctypes.byref(d), batch, ctypes.byref(out)))
     return out.value
@@ -675,14 +676,15 @@ def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
 def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor] = None, *,
                  lossScale: float = 1.0, gradType: int = CoopVecComponentType.Float32,
                  workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None,
-                 inputEncoding: int = 0, flags: int = 0, stream=None):
+                 inputEncoding: int = 0, flags: int = 0, weightType: int = CoopVecComponentType.Float16, stream=None):
     """learnGradient over a batch (kernels.slang:9-27): forward, bwd_diff of the squared-error loss,
     weight gradients accumulated into every layer's weightsGrad (coopVecOuterProductAccumulate,
     fflayer.slang:35-41) and bias gradients into biasesGrad (coopVecReduceSumAccumulate, :44),
-    deterministically.  Returns (workspace, lossSum) so that both can be reused."""
-    _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+    deterministically.  Returns (workspace, lossSum) so that both can be reused.  weightType Float32: a network
+    of float (vectors, targets, parameters), stepped layer by layer with Float32 gradients."""
+    _, inStride = _vector_info(input, weightType, "input")
     batch = input.shape[0]
-    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, flags, inputEncoding)
+    d, keep = _mlp_desc(layers, weightType, gradType, flags, inputEncoding)
     lib = _lib.load()
     if workspace is None:
         need = ctypes.c_size_t(0)
@@ -692,7 +694,7 @@ def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, target
         lossSum = torch.zeros(1, dtype=torch.float32, device=input.device)
     tptr, tstride = None, 0
     if targets is not None:
-        _, tstride = _vector_info(targets, CoopVecComponentType.Float16, "targets")
+        _, tstride = _vector_info(targets, weightType, "targets")
         tptr = targets.data_ptr()
     _check(lib.cvMlpTrainStep(_stream_handle(stream), ctypes.byref(d), input.data_ptr(), inStride, tptr, tstride,
                               float(lossScale), batch, lossSum.data_ptr(), workspace.data_ptr(),
@@ -841,8 +843,11 @@ class NetworkParameterLayoutConverter:
 
     def trainStep(self, params: torch.Tensor, paramGrads: torch.Tensor, input: torch.Tensor, targets: Optional[torch.Tensor], *,
                   optimalLayout: bool, activations=None, leakySlopes=None, lossScale: float = 1.0, stream=None) -> torch.Tensor:
-        """bwd_diff through the chain; gradients accumulate in `paramGrads`, laid out like `params`."""
-        _, inStride = _vector_info(input, CoopVecComponentType.Float16, "input")
+        """bwd_diff through the chain; gradients accumulate in `paramGrads`, laid out like `params`; vectors and
+        targets have the block's element type."""
+        _, inStride = _vector_info(input, self.desc.elementType, "input")
+        if input.dtype != self.dtype or (targets is not None and targets.dtype != self.dtype):
+            raise CoopVecError(SLANG_E_INVALID_ARG, "input and targets must have the network's element type")
         a, s = self._acts(activations, leakySlopes)
         count = self.ElementCountPhysical if optimalLayout else self.ElementCountLogical
         need = ctypes.c_size_t(0)
@@ -852,7 +857,7 @@ class NetworkParameterLayoutConverter:
         loss = torch.zeros(1, dtype=torch.float32, device=input.device)
         tptr, tstride = None, 0
         if targets is not None:
-            _, tstride = _vector_info(targets, CoopVecComponentType.Float16, "targets")
+            _, tstride = _vector_info(targets, self.desc.elementType, "targets")
             tptr = targets.data_ptr()
         _check(lib.cvNeuralMlpTrainStep(_stream_handle(stream), ctypes.byref(self.desc), 1 if optimalLayout else 0,
                                         self._buf(params, count, "params"), self._buf(paramGrads, count, "paramGrads"), a, s,

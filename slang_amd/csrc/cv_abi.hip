@@ -701,15 +701,17 @@ CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch
     memset(&a, 0, sizeof(a));
     CvResult rc = fillMlpLayers("cvMlpTrainStepWorkspaceSize", mlp, a.layers);
     if (CV_FAILED(rc)) return rc;
-    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights");
+    const bool f32net = mlp->weightType == CV_FLOAT32;      // a network of float: layer by layer
+    if (mlp->weightType != CV_FLOAT16 && !f32net)
+        return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: training needs FLOAT16 weights (or a FLOAT32 network)");
     if (mlp->numLayers < 2) return fail(CV_E_NOT_AVAILABLE, "cvMlpTrainStep: needs at least two layers");
     a.numLayers = mlp->numLayers;
     a.batch = batch;
     a.inEncoding = mlp->inputEncoding == CV_ENCODE_XY_SQUARES ? cv::kEncodeXYSquares : cv::kEncodeNone;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    size_t n = (mlp->flags & CV_FLAG_LAYERWISE_TRAINING) ? 0 : cv::trainWorkspaceBytes(a, cus);
-    if (!n) n = cv::trainGeneralWorkspaceBytes(a, cus);   // no fused shape: the layer-by-layer step
+    size_t n = ((mlp->flags & CV_FLAG_LAYERWISE_TRAINING) || f32net) ? 0 : cv::trainWorkspaceBytes(a, cus);
+    if (!n) n = cv::trainGeneralWorkspaceBytes(a, cus, f32net ? CV_FLOAT32 : CV_FLOAT16);   // no fused shape: the layer-by-layer step
     *outBytes = n;
     return CV_OK;
 }
@@ -724,22 +726,27 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     memset(&t, 0, sizeof(t));
     CvResult rc = fillMlpLayers(who, mlp, t.mlp.layers);
     if (CV_FAILED(rc)) return rc;
-    if (mlp->weightType != CV_FLOAT16) return fail(CV_E_NOT_AVAILABLE, "%s: training needs FLOAT16 weights", who);
+    const bool f32net = mlp->weightType == CV_FLOAT32;      // a network of float: layer by layer, fp32 gradients
+    if (mlp->weightType != CV_FLOAT16 && !f32net)
+        return fail(CV_E_NOT_AVAILABLE, "%s: training needs FLOAT16 weights (or a FLOAT32 network)", who);
     if (mlp->gradType != CV_FLOAT16 && mlp->gradType != CV_FLOAT32)
         return fail(CV_E_NOT_AVAILABLE, "%s: gradType %d (supported: FLOAT16, FLOAT32)", who, mlp->gradType);
+    if (f32net && mlp->gradType != CV_FLOAT32)
+        return fail(CV_E_NOT_AVAILABLE, "%s: a FLOAT32 network accumulates FLOAT32 gradients", who);
+    const size_t vEsz = f32net ? 4 : 2;                     // element size of vectors and targets
     const int L = mlp->numLayers;
     if (L < 2) return fail(CV_E_NOT_AVAILABLE, "%s: needs at least two layers", who);
     if (batch == 0) return CV_OK;
     if (!input || !workspace) return fail(CV_E_INVALID_ARG, "%s: null input/workspace", who);
     const bool encoded = mlp->inputEncoding == CV_ENCODE_XY_SQUARES;
-    const size_t inAlignTo = encoded ? 4 : 2, sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * 2;
-    if ((uintptr_t)input % inAlignTo || inputStride % inAlignTo || (uintptr_t)targets % 2 || targetStride % 2 ||
+    const size_t inAlignTo = encoded ? 4 : vEsz, sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * vEsz;
+    if ((uintptr_t)input % inAlignTo || inputStride % inAlignTo || (uintptr_t)targets % vEsz || targetStride % vEsz ||
         (uintptr_t)workspace % 16 || (uintptr_t)lossSum % 4)
         return fail(CV_E_INVALID_ARG, "%s: misaligned input/targets/workspace/lossSum", who);
     if (encoded && !targets && mlp->layers[L - 1].outputSize != 4)
         return fail(CV_E_INVALID_ARG, "%s: the example's loss (targets == NULL with CV_ENCODE_XY_SQUARES) needs 4 outputs", who);
     if (batch > 1 && (inputStride < sampleBytes ||
-                      (targets && targetStride < (size_t)mlp->layers[L - 1].outputSize * 2)))
+                      (targets && targetStride < (size_t)mlp->layers[L - 1].outputSize * vEsz)))
         return fail(CV_E_INVALID_ARG, "%s: vector stride smaller than the vector", who);
     const uint32_t gEsz = cv::elemSize(mlp->gradType);
     for (int l = 0; l < L; ++l) {
@@ -771,13 +778,14 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     t.targetStride = targetStride;
     t.lossScale = lossScale;
     t.gradCt = mlp->gradType;
+    t.carrierCt = f32net ? CV_FLOAT32 : CV_FLOAT16;
     t.lossSum = lossSum;
     t.workspace = (float*)workspace;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
-    size_t need = (mlp->flags & CV_FLAG_LAYERWISE_TRAINING) ? 0 : cv::trainWorkspaceBytes(t.mlp, cus);
+    size_t need = ((mlp->flags & CV_FLAG_LAYERWISE_TRAINING) || f32net) ? 0 : cv::trainWorkspaceBytes(t.mlp, cus);
     const bool fused = need != 0;
-    if (!fused) need = cv::trainGeneralWorkspaceBytes(t.mlp, cus);   // layer by layer, any layer sizes
+    if (!fused) need = cv::trainGeneralWorkspaceBytes(t.mlp, cus, t.carrierCt);   // layer by layer, any layer sizes
     if (workspaceBytes < need) {
         if (ownScratch)
             return fail(CV_E_NOT_AVAILABLE, "%s: this network needs %zu bytes of scratch, the built-in array holds %zu; "

@@ -86,6 +86,7 @@ struct TrainLaunch {
     uint8_t* bGrad[kMaxMlpLayers];
     MatrixShape gradShape[kMaxMlpLayers];
     int32_t gradCt;
+    int32_t carrierCt;           // kF16, or kF32 for a network of float (layer-by-layer step only)
     float* lossSum;
     float* workspace;            // partials
 };
@@ -95,7 +96,7 @@ size_t trainWorkspaceBytes(const MlpArgs& shapes, int numCUs);
 hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCUs);
 // The same step layer by layer through the batched kernels, for any layer sizes: per-layer vectors
 // of the whole batch are parked in the workspace, whose size therefore grows with mlp.batch.
-size_t trainGeneralWorkspaceBytes(const MlpArgs& shapesAndBatch, int numCUs);
+size_t trainGeneralWorkspaceBytes(const MlpArgs& shapesAndBatch, int numCUs, int carrierCt);
 hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& args, int numCUs);
 
 // ---- batched outer-product / reduce-sum accumulate ---------------------------------------

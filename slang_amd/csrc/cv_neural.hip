@@ -166,8 +166,6 @@ CvResult layersFromBlock(const char* who, const CvNeuralNetworkDesc* n, int32_t 
 {
     CvResult rc = checkNet(who, n);
     if (CV_FAILED(rc)) return rc;
-    if (grads && n->elementType != CV_FLOAT16)
-        return failWith(CV_E_NOT_AVAILABLE, "%s: the fused training step takes FLOAT16 parameters (T = half)", who);
     const size_t esz = n->elementType == CV_FLOAT32 ? 4u : 2u;
     if (optimal && n->order != CV_NEURAL_ORDER_NATIVE)
         return failWith(CV_E_NOT_AVAILABLE, "%s: an optimal-layout block must be in CV_NEURAL_ORDER_NATIVE order (convert it first)", who);
@@ -184,8 +182,8 @@ CvResult layersFromBlock(const char* who, const CvNeuralNetworkDesc* n, int32_t 
         L.weights = (const uint8_t*)params + off * esz;
         L.biases = hasBias ? (const uint8_t*)params + (off + wElems) * esz : nullptr;
         if (grads) {
-            L.weightsGrad = (uint8_t*)grads + off * 2;
-            L.biasesGrad = hasBias ? (uint8_t*)grads + (off + wElems) * 2 : nullptr;
+            L.weightsGrad = (uint8_t*)grads + off * esz;
+            L.biasesGrad = hasBias ? (uint8_t*)grads + (off + wElems) * esz : nullptr;
         }
         L.inputSize = in; L.outputSize = o;
         L.weightLayout = L.gradLayout = optimal ? CV_LAYOUT_TRAINING_OPTIMAL : CV_LAYOUT_ROW_MAJOR;
@@ -245,7 +243,8 @@ CV_API CvResult cvNeuralMlpTrainStep(void* stream, const CvNeuralNetworkDesc* ne
     if (!paramGrads) return cv::failWith(CV_E_INVALID_ARG, "cvNeuralMlpTrainStep: paramGrads is null");
     CvResult rc = cv::layersFromBlock("cvNeuralMlpTrainStep", net, optimalLayout, params, paramGrads, activations, leakySlopes, layers);
     if (CV_FAILED(rc)) return rc;
-    CvMlpDesc mlp = {layers, net->layerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_NONE};
+    const int32_t T = net->elementType;      // the gradient block has the parameters' type and layout
+    CvMlpDesc mlp = {layers, net->layerCount, T, T, T, T, T, 0, CV_ENCODE_NONE};
     if (!workspace) {       // size query
         size_t need = 0;
         rc = cvMlpTrainStepWorkspaceSize(&mlp, batch, &need);
@@ -258,12 +257,11 @@ CV_API CvResult cvNeuralMlpTrainStep(void* stream, const CvNeuralNetworkDesc* ne
 CV_API CvResult cvNeuralMlpTrainStepWorkspaceSize(const CvNeuralNetworkDesc* net, uint32_t batch, size_t* outBytes)
 {
     CvMlpLayer layers[cv::kMaxMlpLayers];
-    static const uint16_t dummy = 0;
-    if (net && net->elementType != CV_FLOAT16)
-        return cv::failWith(CV_E_NOT_AVAILABLE, "cvNeuralMlpTrainStepWorkspaceSize: the fused training step takes FLOAT16 parameters (T = half)");
-    CvResult rc = cv::layersFromBlock("cvNeuralMlpTrainStepWorkspaceSize", net, 0, &dummy, nullptr, nullptr, nullptr, layers);
+    alignas(16) static const uint8_t dummy[16] = {};      // stands for a parameter block: only its alignment is looked at
+    CvResult rc = cv::layersFromBlock("cvNeuralMlpTrainStepWorkspaceSize", net, 0, dummy, nullptr, nullptr, nullptr, layers);
     if (CV_FAILED(rc)) return rc;
-    CvMlpDesc mlp = {layers, net->layerCount, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_NONE};
+    const int32_t T = net->elementType;
+    CvMlpDesc mlp = {layers, net->layerCount, T, T, T, T, T, 0, CV_ENCODE_NONE};
     return cvMlpTrainStepWorkspaceSize(&mlp, batch, outBytes);
 }
 

@@ -15,6 +15,10 @@
 //
 // Every rounding point is the fused kernel's (and the oracle's); all reductions run in a fixed
 // order, so the result is bitwise reproducible.  Any layer sizes the matMul kernels serve.
+//
+// Networks of T = float (the neural module's FFLayer<float, ...>) run the same steps with every "half" above
+// read as float: fp32 matMul kernels, element-wise steps in float, gradients summed by the scalar accumulate
+// kernels into fp32 destinations.
 #include <cstring>
 
 #include "cv_device.h"
@@ -42,23 +46,26 @@ struct GeneralPlan {
 
 constexpr uint32_t kLossSamplesPerBlock = 1024;
 
-GeneralPlan makePlan(const MlpArgs& a, int numCUs)
+GeneralPlan makePlan(const MlpArgs& a, int numCUs, int carrierCt)
 {
+    const size_t esz = elemSize(carrierCt);
     GeneralPlan p{};
     const int L = a.numLayers;
     const size_t batch = a.batch ? a.batch : 1;
     size_t off = 0;
     int widest = a.layers[0].in;
     p.x0 = off;
-    if (a.inEncoding != kEncodeNone) off += alignUp(batch * 4 * 2);
+    if (a.inEncoding != kEncodeNone) off += alignUp(batch * 4 * 2);      // (fp16 networks only)
     for (int l = 0; l < L; ++l) {
-        const size_t bytes = alignUp(batch * (size_t)a.layers[l].out * 2);
+        const size_t bytes = alignUp(batch * (size_t)a.layers[l].out * esz);
         p.z[l] = off; off += bytes;
-        if (a.layers[l].act == kActNone) p.act[l] = p.z[l];
-        else { p.act[l] = off; off += bytes; }
+        // (room for the activations is reserved whether or not the layer has one: the size then depends on the
+        // layer sizes and the batch alone, which is all a size query knows)
+        p.act[l] = a.layers[l].act == kActNone ? p.z[l] : off;
+        off += bytes;
         if (a.layers[l].out > widest) widest = a.layers[l].out;
     }
-    const size_t gBytes = alignUp(batch * (size_t)widest * 2);
+    const size_t gBytes = alignUp(batch * (size_t)widest * esz);
     p.gA = off; off += gBytes;
     p.gB = off; off += gBytes;
     p.lossBlocks = (uint32_t)((batch + kLossSamplesPerBlock - 1) / kLossSamplesPerBlock);
@@ -67,6 +74,10 @@ GeneralPlan makePlan(const MlpArgs& a, int numCUs)
     for (int l = 0; l < L; ++l) {
         const size_t o = outerWorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch, numCUs);
         if (o > part) part = o;
+        if (carrierCt != kF16) {
+            const size_t sc = accumScalarWorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch);
+            if (sc > part) part = sc;
+        }
     }
     p.partials = off; off += alignUp(part);
     p.total = off;
@@ -85,56 +96,73 @@ __global__ __launch_bounds__(256) void encodeXYKernel(const uint8_t* in, uint64_
     x0[2 * s] = xy; x0[2 * s + 1] = sq;
 }
 
-// eight halves per thread and step where the arrays allow it (16-byte accesses), the rest one by one
-__global__ __launch_bounds__(256) void activationKernel(const half_t* z, half_t* out, size_t count, int act, float slope)
+// activation and its derivative rule in the carrier type T
+template <typename T> __device__ __forceinline__ T activateT(T z, int act, float slope);
+template <> __device__ __forceinline__ half_t activateT<half_t>(half_t z, int act, float slope) { return activateHalf(z, act, slope); }
+template <> __device__ __forceinline__ float activateT<float>(float z, int act, float slope)
 {
-    const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x, nthreads = (size_t)gridDim.x * 256u;
-    const size_t chunks = count / 8;
-    for (size_t c = tid; c < chunks; c += nthreads) {
-        const halfx8 v = ((const halfx8*)z)[c];
-        halfx8 r;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = activateHalf(v[i], act, slope);
-        ((halfx8*)out)[c] = r;
-    }
-    for (size_t i = chunks * 8 + tid; i < count; i += nthreads) out[i] = activateHalf(z[i], act, slope);
+    if (act == kActRelu) return z > 0.f ? z : 0.f;
+    if (act == kActLeakyRelu) return fmaxf(z, z * slope);      // as the fp32 matMul kernels apply it
+    return z;
 }
 
-// dz = g * act'(z), every product and sum rounded to half
-__device__ __forceinline__ half_t activationGrad(half_t g, half_t z, int act, float slope)
+// dz = g * act'(z), every product and sum rounded to T
+template <typename T>
+__device__ __forceinline__ T activationGrad(T g, T z, int act, float slope)
 {
-    const half_t halfG = (half_t)(0.5f * (float)g);
-    if (act == kActRelu) return z > (half_t)0 ? g : (z == (half_t)0 ? halfG : (half_t)0);
+    const T halfG = (T)(0.5f * (float)g);
+    if (act == kActRelu) return z > (T)0 ? g : (z == (T)0 ? halfG : (T)0);
     if (act == kActLeakyRelu) {
-        const half_t zs = (half_t)((float)z * slope);
-        half_t da, db;
-        if (z > zs) { da = g; db = (half_t)0; }
-        else if (z < zs) { da = (half_t)0; db = g; }
+        const T zs = (T)((float)z * slope);
+        T da, db;
+        if (z > zs) { da = g; db = (T)0; }
+        else if (z < zs) { da = (T)0; db = g; }
         else { da = halfG; db = halfG; }
-        const half_t dbs = (half_t)((float)db * slope);
-        return (half_t)((float)da + (float)dbs);
+        const T dbs = (T)((float)db * slope);
+        return (T)((float)da + (float)dbs);
     }
     return g;
 }
 
-__global__ __launch_bounds__(256) void activationGradKernel(const half_t* g, const half_t* z, half_t* dz, size_t count, int act, float slope)
+// 16 bytes per thread and step where the arrays allow it, the rest one by one
+template <typename T>
+__global__ __launch_bounds__(256) void activationKernel(const T* z, T* out, size_t count, int act, float slope)
 {
+    constexpr int PER = 16 / sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(PER)));
     const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x, nthreads = (size_t)gridDim.x * 256u;
-    const size_t chunks = count / 8;
+    const size_t chunks = count / PER;
     for (size_t c = tid; c < chunks; c += nthreads) {
-        const halfx8 gv = ((const halfx8*)g)[c], zv = ((const halfx8*)z)[c];
-        halfx8 r;
+        const Vec v = ((const Vec*)z)[c];
+        Vec r;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = activationGrad(gv[i], zv[i], act, slope);
-        ((halfx8*)dz)[c] = r;
+        for (int i = 0; i < PER; ++i) r[i] = activateT<T>(v[i], act, slope);
+        ((Vec*)out)[c] = r;
     }
-    for (size_t i = chunks * 8 + tid; i < count; i += nthreads) dz[i] = activationGrad(g[i], z[i], act, slope);
+    for (size_t i = chunks * PER + tid; i < count; i += nthreads) out[i] = activateT<T>(z[i], act, slope);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void activationGradKernel(const T* g, const T* z, T* dz, size_t count, int act, float slope)
+{
+    constexpr int PER = 16 / sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(PER)));
+    const size_t tid = (size_t)blockIdx.x * 256u + threadIdx.x, nthreads = (size_t)gridDim.x * 256u;
+    const size_t chunks = count / PER;
+    for (size_t c = tid; c < chunks; c += nthreads) {
+        const Vec gv = ((const Vec*)g)[c], zv = ((const Vec*)z)[c];
+        Vec r;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) r[i] = activationGrad<T>(gv[i], zv[i], act, slope);
+        ((Vec*)dz)[c] = r;
+    }
+    for (size_t i = chunks * PER + tid; i < count; i += nthreads) dz[i] = activationGrad<T>(g[i], z[i], act, slope);
 }
 
 struct LossArgs {
-    const half_t* y;            // network output, [batch][outDim]
-    const half_t* z;            // last layer's pre-activation
-    half_t* dz;                 // gradient at the last layer's pre-activation
+    const void* y;              // network output, [batch][outDim] of the carrier type
+    const void* z;              // last layer's pre-activation
+    void* dz;                   // gradient at the last layer's pre-activation
     const uint8_t* targets; uint64_t targetStride;
     const uint8_t* in; uint64_t inStride;   // network input as the caller passed it
     int32_t inDim, outDim, inEncoding;
@@ -145,8 +173,10 @@ struct LossArgs {
 };
 
 // One thread per sample; a workgroup's squared errors are summed in a fixed order.
+template <typename T>
 __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
 {
+    const T* const y = (const T*)a.y; const T* const z = (const T*)a.z; T* const dzOut = (T*)a.dz;
     __shared__ float red[256];
     float loss = 0.f;
     const uint32_t first = blockIdx.x * kLossSamplesPerBlock;
@@ -164,19 +194,19 @@ __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
             for (int g = 0; g < 4; ++g)
                 for (int q = 0; q < gs; ++q) {
                     const int j = g * gs + q;
-                    if (j < a.inDim) part[g] += (float)((const half_t*)xin)[j];
+                    if (j < a.inDim) part[g] += (float)((const T*)xin)[j];
                 }
             // lane group g adds the partner groups in the order g^1, then the pair sums: (p0+p1)+(p2+p3)
-            tgtAll = (float)(half_t)sinf((part[0] + part[1]) + (part[2] + part[3]));
+            tgtAll = (float)(T)sinf((part[0] + part[1]) + (part[2] + part[3]));
         }
         for (int i = 0; i < a.outDim; ++i) {
             const size_t e = (size_t)s * a.outDim + i;
-            const float tv = a.targets ? (float)*(const half_t*)(a.targets + (size_t)s * a.targetStride + 2 * i)
+            const float tv = a.targets ? (float)*(const T*)(a.targets + (size_t)s * a.targetStride + sizeof(T) * i)
                                        : (exampleLoss ? (float)gt[i & 3] : tgtAll);
-            const half_t diff = (half_t)((float)a.y[e] - tv);
+            const T diff = (T)((float)y[e] - tv);
             loss += (float)diff * (float)diff;
-            const half_t g = (half_t)(2.0f * (float)diff * a.lossScale);
-            a.dz[e] = activationGrad(g, a.z[e], a.act, a.slope);
+            const T g = (T)(2.0f * (float)diff * a.lossScale);
+            dzOut[e] = activationGrad<T>(g, z[e], a.act, a.slope);
         }
     }
     red[threadIdx.x] = loss;
@@ -217,10 +247,10 @@ uint32_t alignOfPtr(const void* p, uint64_t stride)
 
 } // namespace
 
-size_t trainGeneralWorkspaceBytes(const MlpArgs& a, int numCUs)
+size_t trainGeneralWorkspaceBytes(const MlpArgs& a, int numCUs, int carrierCt)
 {
     if (a.numLayers < 2) return 0;
-    return makePlan(a, numCUs).total;
+    return makePlan(a, numCUs, carrierCt).total;
 }
 
 hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int numCUs)
@@ -230,7 +260,11 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
     if (batch == 0) return hipSuccess;
     const int L = a.numLayers;
     if (L < 2) return hipErrorInvalidValue;
-    const GeneralPlan p = makePlan(a, numCUs);
+    const int ct = t.carrierCt;                 // kF16 or kF32: vectors, weights, biases
+    const bool f32 = ct == kF32;
+    const uint64_t esz = elemSize(ct);
+    const MmaKind mma = f32 ? MmaKind::F32 : MmaKind::F16;
+    const GeneralPlan p = makePlan(a, numCUs, ct);
     uint8_t* ws = (uint8_t*)t.workspace;
     hipError_t e;
 
@@ -252,33 +286,36 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
         MatMulArgs m;
         memset(&m, 0, sizeof(m));
         m.in = x; m.inStride = xStride;
-        m.out = ws + p.z[l]; m.outStride = (uint64_t)ly.out * 2;
-        m.mat = ly.w; m.bias = ly.bias; m.biasCt = kF16;
+        m.out = ws + p.z[l]; m.outStride = (uint64_t)ly.out * esz;
+        m.mat = ly.w; m.bias = ly.bias; m.biasCt = ct;
         m.shape = ly.shape; m.transpose = 0; m.m = ly.out; m.k = ly.in;
-        m.inCt = kF16; m.outCt = kF16; m.act = kActNone; m.batch = batch;
+        m.inCt = ct; m.outCt = ct; m.act = kActNone; m.batch = batch;
         m.inAlign = alignOfPtr(m.in, m.inStride); m.outAlign = alignOfPtr(m.out, m.outStride);
-        if ((e = launchMatMul(stream, MmaKind::F16, m, numCUs)) != hipSuccess) return e;
+        if ((e = launchMatMul(stream, mma, m, numCUs)) != hipSuccess) return e;
         if (ly.act != kActNone) {
             const size_t count = (size_t)batch * ly.out;
-            hipLaunchKernelGGL(activationKernel, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
-                               (const half_t*)(ws + p.z[l]), (half_t*)(ws + p.act[l]), count, ly.act, ly.slope);
+            if (f32) hipLaunchKernelGGL(activationKernel<float>, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                                        (const float*)(ws + p.z[l]), (float*)(ws + p.act[l]), count, ly.act, ly.slope);
+            else hipLaunchKernelGGL(activationKernel<half_t>, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                                    (const half_t*)(ws + p.z[l]), (half_t*)(ws + p.act[l]), count, ly.act, ly.slope);
             if ((e = hipGetLastError()) != hipSuccess) return e;
         }
-        x = ws + p.act[l]; xStride = (uint64_t)ly.out * 2;
+        x = ws + p.act[l]; xStride = (uint64_t)ly.out * esz;
     }
 
     // ---- loss and the gradient at the last pre-activation -----------------------------------------
     {
         const MlpLayerArgs& ly = a.layers[L - 1];
         LossArgs la;
-        la.y = (const half_t*)(ws + p.act[L - 1]); la.z = (const half_t*)(ws + p.z[L - 1]);
-        la.dz = (half_t*)(ws + p.gA);
+        la.y = ws + p.act[L - 1]; la.z = ws + p.z[L - 1];
+        la.dz = ws + p.gA;
         la.targets = t.targets; la.targetStride = t.targetStride;
         la.in = a.in; la.inStride = a.inStride;
         la.inDim = a.layers[0].in; la.outDim = ly.out; la.inEncoding = a.inEncoding;
         la.act = ly.act; la.slope = ly.slope; la.lossScale = t.lossScale; la.batch = batch;
         la.partials = (float*)(ws + p.lossPartials);
-        hipLaunchKernelGGL(lossGradKernel, dim3(p.lossBlocks), dim3(256), 0, stream, la);
+        if (f32) hipLaunchKernelGGL(lossGradKernel<float>, dim3(p.lossBlocks), dim3(256), 0, stream, la);
+        else hipLaunchKernelGGL(lossGradKernel<half_t>, dim3(p.lossBlocks), dim3(256), 0, stream, la);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if (t.lossSum) {
             hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(64), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum);
@@ -291,8 +328,19 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
     for (int l = L - 1; l >= 0; --l) {
         const MlpLayerArgs& ly = a.layers[l];
         const uint8_t* dz = ws + dzOff;
-        const uint64_t dzStride = (uint64_t)ly.out * 2;
-        if (t.bGrad[l]) {
+        const uint64_t dzStride = (uint64_t)ly.out * esz;
+        if (f32) {
+            // fp32 vectors: the scalar accumulate kernels (db: the reduce-sum form, b == 1)
+            if (t.bGrad[l]) {
+                const MatrixShape bs{(uint32_t)ly.out, 1u, t.gradCt, kRowMajor, (size_t)elemSize(t.gradCt)};
+                if ((e = launchAccumScalar(stream, dz, dzStride, ly.out, nullptr, 0, 1, ct, batch, t.bGrad[l], bs, ws + p.partials)) != hipSuccess) return e;
+            }
+            if (t.wGrad[l]) {
+                if ((e = launchAccumScalar(stream, dz, dzStride, ly.out, xl[l], xlStride[l], ly.in, ct, batch, t.wGrad[l], t.gradShape[l],
+                                           ws + p.partials)) != hipSuccess) return e;
+            }
+        }
+        if (!f32 && t.bGrad[l]) {
             for (int c0 = 0; c0 < ly.out; c0 += 256) {      // the reduce kernel takes up to 256 columns
                 const int n = ly.out - c0 < 256 ? ly.out - c0 : 256;
                 ReduceSumArgs r;
@@ -304,7 +352,7 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
                 if ((e = launchReduceSum(stream, r, numCUs)) != hipSuccess) return e;
             }
         }
-        if (t.wGrad[l]) {
+        if (!f32 && t.wGrad[l]) {
             OuterArgs o;
             memset(&o, 0, sizeof(o));
             o.a = dz; o.aStride = dzStride; o.aAlign = alignOfPtr(o.a, o.aStride);
@@ -321,17 +369,20 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
         MatMulArgs m;
         memset(&m, 0, sizeof(m));
         m.in = dz; m.inStride = dzStride;
-        m.out = ws + otherOff; m.outStride = (uint64_t)ly.in * 2;
+        m.out = ws + otherOff; m.outStride = (uint64_t)ly.in * esz;
         m.mat = ly.w; m.shape = ly.shape; m.transpose = 1; m.m = ly.in; m.k = ly.out;
-        m.inCt = kF16; m.outCt = kF16; m.act = kActNone; m.batch = batch;
+        m.inCt = ct; m.outCt = ct; m.act = kActNone; m.batch = batch;
         m.inAlign = alignOfPtr(m.in, m.inStride); m.outAlign = alignOfPtr(m.out, m.outStride);
-        if ((e = launchMatMul(stream, MmaKind::F16, m, numCUs)) != hipSuccess) return e;
+        if ((e = launchMatMul(stream, mma, m, numCUs)) != hipSuccess) return e;
         if (prevAct) {
             // in place: element i of dz depends on element i of g only
             const size_t count = (size_t)batch * ly.in;
-            hipLaunchKernelGGL(activationGradKernel, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
-                               (const half_t*)(ws + otherOff), (const half_t*)(ws + p.z[l - 1]), (half_t*)(ws + otherOff),
-                               count, prev.act, prev.slope);
+            if (f32) hipLaunchKernelGGL(activationGradKernel<float>, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                                        (const float*)(ws + otherOff), (const float*)(ws + p.z[l - 1]), (float*)(ws + otherOff),
+                                        count, prev.act, prev.slope);
+            else hipLaunchKernelGGL(activationGradKernel<half_t>, dim3(gridFor(count, numCUs)), dim3(256), 0, stream,
+                                    (const half_t*)(ws + otherOff), (const half_t*)(ws + p.z[l - 1]), (half_t*)(ws + otherOff),
+                                    count, prev.act, prev.slope);
             if ((e = hipGetLastError()) != hipSuccess) return e;
         }
         const size_t tmp = dzOff; dzOff = otherOff; otherOff = tmp;

@@ -146,6 +146,100 @@ def test_fp32_parameter_block_of_the_neural_module():
             z = z + portable[off:off + fo].astype(np.float64); off += fo
         h = act64(z, acts[k], 0.0)
     assert np.allclose(y_lin.cpu().numpy(), h, rtol=1e-5, atol=1e-5)
-    with pytest.raises(cv.CoopVecError) as e:
-        conv.trainStep(pd, torch.zeros_like(pd), x, None, optimalLayout=False)
-    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+    # bwd_diff through the block: the gradients land at the parameters' offsets, the same from both layouts
+    t = to_dev(rng.standard_normal((B, dims[-1])).astype(np.float32))
+    g_lin = torch.zeros_like(pd); g_opt = torch.zeros_like(opt)
+    acts_t = [Activation.ReLU, Activation.LeakyReLU, Activation.NoActivation]
+    l1 = conv.trainStep(pd, g_lin, x, t, optimalLayout=False, activations=acts_t, leakySlopes=[0, 0.125, 0])
+    l2 = conv.trainStep(opt, g_opt, x, t, optimalLayout=True, activations=acts_t, leakySlopes=[0, 0.125, 0])
+    assert torch.equal(l1, l2)
+    assert torch.equal(conv.toPortableLayout(g_opt).view(torch.int32), g_lin.view(torch.int32))
+    want_loss, want_g = backprop64(portable, dims, mask, acts_t, 0.125, x.cpu().numpy(), t.cpu().numpy(), 1.0)
+    assert abs(float(l1) - want_loss) <= 1e-5 * want_loss
+    got = g_lin.cpu().numpy().astype(np.float64)
+    assert np.linalg.norm(got - want_g) <= 1e-5 * np.linalg.norm(want_g)
+
+
+def backprop64(portable, dims, mask, acts, slope, x, t, loss_scale):
+    """The step in float64 on a portable parameter block: (loss sum, gradient block of the same layout)."""
+    L = len(dims) - 1
+    Ws, bs, off = [], [], 0
+    for k in range(L):
+        fi, fo = dims[k], dims[k + 1]
+        Ws.append(portable[off:off + fi * fo].reshape(fo, fi).astype(np.float64)); off += fi * fo
+        if (mask >> k) & 1:
+            bs.append(portable[off:off + fo].astype(np.float64)); off += fo
+        else:
+            bs.append(None)
+    hs, zs = [x.astype(np.float64)], []
+    for k in range(L):
+        z = hs[-1] @ Ws[k].T + (bs[k] if bs[k] is not None else 0.0)
+        zs.append(z); hs.append(act64(z, acts[k], slope))
+    diff = hs[-1] - t.astype(np.float64)
+    loss = float((diff ** 2).sum())
+    g = 2.0 * diff * loss_scale
+    out = np.zeros(portable.shape, np.float64)
+    grads = []
+    for k in range(L - 1, -1, -1):
+        z = zs[k]
+        if acts[k] == Activation.ReLU: d = np.where(z > 0, 1.0, np.where(z == 0, 0.5, 0.0))
+        elif acts[k] == Activation.LeakyReLU: d = np.where(z > 0, 1.0, np.where(z == 0, 0.5 + 0.5 * slope, slope))
+        else: d = 1.0
+        dz = g * d
+        grads.append((dz.T @ hs[k], dz.sum(axis=0)))
+        g = dz @ Ws[k]
+    grads.reverse()
+    off = 0
+    for k in range(L):
+        fi, fo = dims[k], dims[k + 1]
+        out[off:off + fi * fo] = grads[k][0].reshape(-1); off += fi * fo
+        if (mask >> k) & 1:
+            out[off:off + fo] = grads[k][1]; off += fo
+    return loss, out
+
+
+@pytest.mark.parametrize("grad_layout", [ML.RowMajor, ML.TrainingOptimal])
+def test_fp32_training_step_against_float64(grad_layout):
+    # learnGradient for a network of float (layer by layer): loss and every gradient against float64 backpropagation
+    # on the same fp32 parameters; "+=" into pre-filled destinations; bitwise reproducible
+    rng = np.random.default_rng(17)
+    dims, mask = [6, 20, 13, 3], 0b111
+    acts = [Activation.ReLU, Activation.LeakyReLU, Activation.NoActivation]
+    n_par = sum(dims[k] * dims[k + 1] + dims[k + 1] for k in range(3))
+    portable = (rng.standard_normal(n_par) * 0.5).astype(np.float32)
+    B = 3000
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float32); t = rng.standard_normal((B, dims[-1])).astype(np.float32)
+    want_loss, want_g = backprop64(portable, dims, mask, acts, 0.125, x, t, 0.5)
+
+    def run():
+        layers, views, off = [], [], 0
+        for k in range(3):
+            fi, fo = dims[k], dims[k + 1]
+            W = portable[off:off + fi * fo]; off += fi * fo
+            b = portable[off:off + fo]; off += fo
+            gsize = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float32, grad_layout, fi * 4)
+            wg = torch.zeros(gsize, dtype=torch.uint8, device=DEV)
+            bg = torch.full((fo,), 1.0, dtype=torch.float32, device=DEV)          # pre-filled: the step adds
+            layers.append(FeedForwardLayer(fi, fo, as_bytes(to_dev(W)), as_bytes(to_dev(b)), ML.RowMajor, fi * 4, acts[k], 0.125,
+                                           wg, as_bytes(bg), grad_layout, fi * 4 if grad_layout == ML.RowMajor else 0))
+            views.append((wg, bg, gsize))
+        _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=0.5, weightType=CT.Float32)
+        assert "layer-by-layer" in cv.lastKernelName()
+        out = []
+        for k, (wg, bg, gsize) in enumerate(views):
+            fi, fo = dims[k], dims[k + 1]
+            if grad_layout != ML.RowMajor:
+                row = torch.zeros(fo * fi * 4, dtype=torch.uint8, device=DEV)
+                D = cv.CooperativeVectorMatrixDesc
+                cv.convertCooperativeVectorMatrix(row, [D(fo, fi, CT.Float32, ML.RowMajor, fo * fi * 4, 0, fi * 4)],
+                                                  wg, [D(fo, fi, CT.Float32, grad_layout, gsize, 0, 0)])
+                wg = row
+            out.append(wg.view(torch.float32).cpu().numpy().copy()); out.append(bg.cpu().numpy().copy() - 1.0)
+        return float(loss), np.concatenate(out)
+
+    loss1, g1 = run()
+    loss2, g2 = run()
+    assert loss1 == loss2 and np.array_equal(g1.view(np.uint32), g2.view(np.uint32))
+    assert abs(loss1 - want_loss) <= 1e-5 * want_loss
+    assert np.linalg.norm(g1.astype(np.float64) - want_g) <= 2e-5 * np.linalg.norm(want_g)
+    assert (np.abs(g1.astype(np.float64) - want_g) <= 1e-4 * (np.abs(want_g) + np.abs(want_g).mean())).all()
