@@ -289,8 +289,9 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
 
 /* CoopVec<T,N>(CoopVec<U,N>) / CoopVec.copyFrom (hlsl.meta.slang:30683-30730) over a batch:
  *   dst[s][i] = T(src[s][i])
- * between any two of FLOAT16/32/64 and the 8/16/32/64-bit integers.  Integer -> integer keeps the low bits;
- * to a float type: one rounding to nearest even; float -> integer: towards zero (what C leaves undefined is
+ * between any two of FLOAT16/32/64, BFLOAT16 and the 8/16/32/64-bit integers.  Integer -> integer keeps the low bits;
+ * to a float type: one rounding to nearest even of the exact source value (also from fp64 and from 64-bit
+ * integers to FLOAT16 / BFLOAT16); float -> integer: towards zero (what C leaves undefined is
  * fixed as NaN -> 0 and out-of-range values saturated to 32 bits, 64 for 64-bit targets, then cut to the low bits). */
 CV_API CvResult cvVectorCast(void* stream, int32_t n, uint32_t batch, const void* src, size_t srcStride, int32_t srcType,
                              void* dst, size_t dstStride, int32_t dstType);

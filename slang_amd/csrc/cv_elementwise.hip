@@ -239,6 +239,23 @@ struct CastArgs {
     uint32_t batch;
 };
 
+// A 64-bit integer as a double that rounds like the integer itself in any later rounding to fewer bits: exact up to
+// 2^53, beyond that the top 53 bits with the last one set if anything was cut off (sticky).
+__device__ __forceinline__ double stickyDoubleOfInt(uint64_t bits, bool isUnsigned)
+{
+    const bool neg = !isUnsigned && (int64_t)bits < 0;
+    const uint64_t mag = neg ? (uint64_t)0 - bits : bits;
+    double d;
+    if (mag < (1ull << 53)) {
+        d = (double)mag;
+    } else {
+        const int sh = 64 - __builtin_clzll(mag) - 53;
+        const uint64_t top = (mag >> sh) | ((mag & ((1ull << sh) - 1ull)) ? 1ull : 0ull);
+        d = __builtin_ldexp((double)top, sh);
+    }
+    return neg ? -d : d;
+}
+
 // double -> half in one rounding: through a float that keeps a sticky last bit (round to odd)
 __device__ __forceinline__ half_t halfOfDouble(double d)
 {
@@ -256,7 +273,7 @@ __global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
 {
     const uint64_t total = (uint64_t)e.batch * (uint32_t)e.n;
     const uint32_t sEsz = elemSize(e.srcCt), dEsz = elemSize(e.dstCt);
-    const bool srcFloat = e.srcCt == kF16 || e.srcCt == kF32 || e.srcCt == kF64;
+    const bool srcFloat = e.srcCt == kF16 || e.srcCt == kF32 || e.srcCt == kF64 || e.srcCt == kBF16;
     const bool srcUnsigned = e.srcCt == kU8 || e.srcCt == kU16 || e.srcCt == kU32 || e.srcCt == kU64;
     for (uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x; idx < total; idx += (uint64_t)gridDim.x * 256u) {
         const uint64_t s = idx / (uint32_t)e.n, i = idx - s * (uint32_t)e.n;
@@ -266,6 +283,7 @@ __global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
         uint64_t bits = 0;       // an integer source, extended to 64 bits
         switch (e.srcCt) {
         case kF16: f = (double)(float)*(const half_t*)p; break;
+        case kBF16: f = (double)__builtin_bit_cast(float, (uint32_t)*(const uint16_t*)p << 16); break;
         case kF32: f = (double)*(const float*)p; break;
         case kF64: f = *(const double*)p; break;
         case kS8: bits = (uint64_t)(int64_t) * (const int8_t*)p; break;
@@ -278,13 +296,25 @@ __global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
         }
         switch (e.dstCt) {
         case kF16:
-            // integers below 2^53 are exact in double; larger ones are far beyond the half range either way
             *(half_t*)q = srcFloat ? (e.srcCt == kF64 ? halfOfDouble(f) : (half_t)(float)f)
-                                   : halfOfDouble(srcUnsigned ? (double)bits : (double)(int64_t)bits);
+                                   : halfOfDouble(stickyDoubleOfInt(bits, srcUnsigned));
             break;
         case kF32:
             *(float*)q = srcFloat ? (float)f : (srcUnsigned ? (float)bits : (float)(int64_t)bits);
             break;
+        case kBF16: {
+            // one rounding to the 8 significant bits of bfloat16: through a float with a sticky last bit where the
+            // source holds more than a float does (fp64, integers beyond 2^24)
+            const double d = srcFloat ? f : stickyDoubleOfInt(bits, srcUnsigned);
+            float x = (float)d;
+            const double back = (double)x;
+            if (back != d) {
+                uint32_t u = __builtin_bit_cast(uint32_t, x);
+                if (__builtin_fabs(back) > __builtin_fabs(d)) u -= 1u;
+                x = __builtin_bit_cast(float, u | 1u);
+            }
+            *(bf16_t*)q = (bf16_t)x;
+            break; }
         case kF64:
             *(double*)q = srcFloat ? f : (srcUnsigned ? (double)bits : (double)(int64_t)bits);
             break;
@@ -311,11 +341,14 @@ __global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
     }
 }
 
+bool isCastType(int32_t ct);
 bool isPlainType(int32_t ct)
 {
     return ct == kF16 || ct == kF32 || ct == kF64 || ct == kS8 || ct == kU8 || ct == kS16 || ct == kU16 || ct == kS32 ||
            ct == kU32 || ct == kS64 || ct == kU64;
 }
+
+bool isCastType(int32_t ct) { return isPlainType(ct) || ct == kBF16; }      // conversions also serve bfloat16
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
@@ -413,8 +446,8 @@ CV_API CvResult cvVectorCast(void* stream, int32_t n, uint32_t batch, const void
 {
     using namespace cv;
     if (n <= 0) return failWith(CV_E_INVALID_ARG, "cvVectorCast: n=%d", n);
-    if (!isPlainType(srcType) || !isPlainType(dstType))
-        return failWith(CV_E_NOT_AVAILABLE, "cvVectorCast: from type %d to type %d (supported: FLOAT16/32/64 and the 8/16/32/64-bit integers)",
+    if (!isCastType(srcType) || !isCastType(dstType))
+        return failWith(CV_E_NOT_AVAILABLE, "cvVectorCast: from type %d to type %d (supported: FLOAT16/32/64, BFLOAT16 and the 8/16/32/64-bit integers)",
                         srcType, dstType);
     if (batch == 0) return CV_OK;
     if (badOperand(src, srcStride, n, batch, elemSize(srcType)) || badOperand(dst, dstStride, n, batch, elemSize(dstType)))

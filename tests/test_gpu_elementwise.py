@@ -326,5 +326,30 @@ def test_copy_from_single_rounding_and_the_values_c_leaves_open():
     cv.copyFrom(src[:, 2:9], CT.Float32, out=out[:, :7])
     assert torch.equal(out[:, :7], src[:, 2:9].to(torch.float32)) and (out[:, 7:] == -1).all()
     with pytest.raises(cv.CoopVecError) as e:
-        cv.copyFrom(torch.zeros(2, 4, dtype=torch.bfloat16, device=DEV), CT.Float32)
+        cv.copyFrom(torch.zeros(2, 4, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn), CT.Float32)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+def test_copy_from_bfloat16():
+    # bfloat16 is the high half of binary32: to it, one rounding to nearest even of the exact source value; from it, exact
+    rng = np.random.default_rng(16)
+    x32 = (rng.standard_normal((50, 33)) * rng.choice([1e-3, 1.0, 1e4], (50, 33))).astype(np.float32)
+    x32[0, :3] = [1.0 + 2.0 ** -8, 1.0 + 2.0 ** -8 + 2.0 ** -20, 3.3895314e38]           # a tie, just above it, near the top
+    got = cv.copyFrom(to_dev(x32), CT.BFloat16)
+    assert got.dtype == torch.bfloat16
+    assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), ob.bf16_bits(x32))
+    back = cv.copyFrom(got, CT.Float32).cpu().numpy()
+    assert np.array_equal(back.view(np.uint32), ob.bf16_bits(x32).astype(np.uint32) << 16)
+    # double -> bfloat16 in one rounding: above the tie by less than float resolves
+    d = np.array([[1.0 + 2.0 ** -8 + 2.0 ** -40, 1.0 + 2.0 ** -8, -(1.0 + 3 * 2.0 ** -8 + 2.0 ** -45)]], np.float64)
+    got = cv.copyFrom(_dev_typed(d), CT.BFloat16).float().cpu().numpy()
+    assert got.tolist() == [[1.0 + 2.0 ** -7, 1.0, -(1.0 + 2.0 ** -6)]]
+    # 64-bit integers beyond 2^53: (2^8 + 1) 2^55 is a tie of the 8 significant bits (-> 2^63, the even one), one more
+    # rounds up -- a conversion through double alone would land on the tie
+    big = np.array([[257 << 55, (257 << 55) + 1, 3 << 56]], np.uint64)
+    got = cv.copyFrom(_dev_typed(big), CT.BFloat16).float().cpu().numpy().astype(np.float64)
+    assert got.tolist() == [[float(1 << 63), float(129 << 56), float(3 << 56)]]
+    ints = rng.integers(-70000, 70000, (20, 9), dtype=np.int32)
+    got = cv.copyFrom(_dev_typed(ints), CT.BFloat16)
+    assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16), ob.bf16_bits(ints.astype(np.float32)))
+    assert cv.copyFrom(got, CT.SignedInt32).cpu().numpy().tolist() == ob.bf16_to_f32(ob.bf16_bits(ints.astype(np.float32))).astype(np.int32).tolist()
