@@ -39,7 +39,7 @@ sys.path.insert(0, os.path.join(REPO, "tests"))
 
 METRIC = "CoopVec MLP samples/sec (fp16/fp8/int8 fwd, fp16 train step); % MFMA peak"
 HBM_PEAK_GBS = 8000.0
-MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0}
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
 
 # HBM bytes per step (all kernels of the step) as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
 # scaled by a copy of known size): not measured by this script, quoted from the committed profile summaries.
@@ -328,6 +328,50 @@ def workload_c4h(torch, cv, steps, warmup):
                          lambda fi: 0.5, with_bias=False)
 
 
+def workload_f32(torch, cv, steps, warmup):
+    """Forward pass of a network of float (the neural module's FFLayer<float> chain), 32->64->64->8, batch 2^22."""
+    import numpy as np
+    from slang_amd.coopvec import Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML, FeedForwardLayer
+    dev = "cuda"
+    dims = [32, 64, 64, 8]
+    B = 1 << 22
+    g = torch.Generator(device=dev); g.manual_seed(20259)
+    layers, host = [], []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = torch.randn(fo, fi, device=dev, generator=g) * (2.0 / fi) ** 0.5
+        bias = torch.randn(fo, device=dev, generator=g) * 0.1
+        last = i == len(dims) - 2
+        layers.append(FeedForwardLayer(fi, fo, W.contiguous().view(torch.uint8).flatten(), bias.view(torch.uint8), ML.RowMajor, fi * 4,
+                                       Activation.NoActivation if last else Activation.ReLU, 0.0))
+        host.append((W, bias))
+    x = torch.rand(B, dims[0], device=dev, generator=g) * 2 - 1
+    out = torch.empty(B, dims[-1], dtype=torch.float32, device=dev)
+    plan = cv.MlpForwardPlan(layers, weightType=CT.Float32)
+
+    def step():
+        plan(x, out)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+
+    def cpu_baseline():
+        n = 1 << 17
+        h = x[:n].cpu().numpy()
+        t0 = time.perf_counter()
+        for i, (W, b) in enumerate(host):
+            h = h @ W.cpu().numpy().T + b.cpu().numpy()
+            if i < len(host) - 1:
+                h = np.maximum(h, 0)
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vectors; numpy fp32 (the fallback's arithmetic for T = float is plain fp32 products and sums)" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * (dims[0] + dims[-1]) * 4, alg_flops=B * 2 * macs, bound="hbm", mfma="f32",
+                dtype="f32", config={"workload": "f32: fp32 MLP 32->64->64->8, ReLU, fp32 in and out, batch 2^22, fused forward "
+                                                 "(v_mfma_f32_16x16x4_f32)", "batch": B, "layers": dims},
+                cpu_baseline=cpu_baseline, key="f32")
+
+
 def workload_c5(torch, cv, steps, warmup, flags=0):
     """fp16 training step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, fp32 TrainingOptimal grads."""
     import numpy as np
@@ -467,7 +511,7 @@ def workload_rs(torch, cv, steps, warmup):
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2b": workload_c2b, "c3": workload_c3, "c4": workload_c4,
              "c4n": workload_c4n, "c5": workload_c5, "op": workload_op, "rs": workload_rs,
              # only with --workload: variants and the counter-calibration copy
-             "c4h": workload_c4h, "c5g": workload_c5g, "copy": workload_copy}
+             "c4h": workload_c4h, "c5g": workload_c5g, "f32": workload_f32, "copy": workload_copy}
 DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4h", "c4n", "c5", "op", "rs")
 HEADLINE = "c2"
 
