@@ -54,7 +54,7 @@ PROFILED_TRAFFIC = {
     "c5": (47843000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
     "op": (285455000, "profiles/outer_product_64x64_batch1M.md"),
     "rs": (537964000, "profiles/reduce_sum_64_batch4M.md"),
-    "f32": (672078000, "profiles/mlp_forward_f32_32-64-64-8_batch4M.md"),
+    "f32": (671764000, "profiles/mlp_forward_f32_32-64-64-8_batch4M.md"),
     "copy": (1073743000, "profiles/copy_calibration_512MiB.md"),
 }
 

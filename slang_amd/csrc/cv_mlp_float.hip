@@ -17,8 +17,7 @@ namespace cv {
 
 namespace {
 
-constexpr int kFltMaxTiles = 8;                     // 128 rows / columns
-constexpr int kFltMaxKT = kFltMaxTiles / 2;         // B fragments of a 128-wide vector
+constexpr int kFltTileLimit = 8;                    // 128 rows / columns
 constexpr uint32_t kFltLdsDwords = 36 * 1024;       // 144 KB for all layers' fragments and biases
 
 struct FltLayer {
@@ -40,9 +39,12 @@ __device__ __forceinline__ float activateFloat(float x, int act, float slope)
     return x;
 }
 
-template <class Mma>
+// MAXT: the unrolled bound on a layer's 16-row tiles (4 for networks up to 64 wide, which then need half the
+// registers and run more waves per SIMD; 8 up to 128)
+template <class Mma, int MAXT>
 __global__ __launch_bounds__(256) void mlpFloatKernel(const FltArgs ga)
 {
+    constexpr int kFltMaxTiles = MAXT, kFltMaxKT = MAXT / 2;
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     constexpr bool F32 = ESZ == 4;
     static_assert(EPL == 8, "the layer chain needs 8 k-slots per lane per fragment");
@@ -161,33 +163,41 @@ __global__ __launch_bounds__(256) void mlpFloatKernel(const FltArgs ga)
     }
 }
 
+template <class Mma, int MAXT>
+hipError_t launchFloatSized(hipStream_t stream, const FltArgs& ga, size_t ldsBytes, int numCUs)
+{
+    const hipError_t ea = allowDynamicLds<mlpFloatKernel<Mma, MAXT>>((int)(kFltLdsDwords * 4));
+    if (ea != hipSuccess) return ea;
+    int perCU = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpFloatKernel<Mma, MAXT>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
+    const uint32_t numTiles = (ga.mlp.batch + 15) / 16, need = (numTiles + 3) / 4;
+    const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
+    noteKernel(false, "mlpFloatKernel<%s,up to %d rows>", Mma::kName, 16 * MAXT);
+    hipLaunchKernelGGL((mlpFloatKernel<Mma, MAXT>), dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
+    return hipGetLastError();
+}
+
 template <class Mma>
 hipError_t launchFloat(hipStream_t stream, const MlpArgs& a, int ct, int numCUs)
 {
     FltArgs ga;
     ga.mlp = a;
     ga.ct = ct;
-    uint32_t frag = 0, bias = 0;
+    uint32_t frag = 0, bias = 0, widest = 0;
     for (int l = 0; l < a.numLayers; ++l) {
         const uint32_t mt = optMT((uint32_t)a.layers[l].out), kt = optKT((uint32_t)a.layers[l].in, Mma::kEpl);
-        if (mt > (uint32_t)kFltMaxTiles || kt > (uint32_t)kFltMaxKT) return hipErrorInvalidValue;
+        if (mt > (uint32_t)kFltTileLimit || kt > (uint32_t)kFltTileLimit / 2) return hipErrorInvalidValue;
         ga.gl[l].mt = (int32_t)mt; ga.gl[l].kt = (int32_t)kt;
         ga.gl[l].fragBase = frag; ga.gl[l].biasBase = bias;
         frag += mt * kt; bias += mt * 16;
+        if (mt > widest) widest = mt;
+        if (2 * kt > widest) widest = 2 * kt;
     }
     ga.biasDwordBase = frag * 64 * Mma::kRawDW;
     const uint32_t dwords = ga.biasDwordBase + bias;
     if (dwords > kFltLdsDwords) return hipErrorInvalidValue;
     const size_t ldsBytes = (size_t)dwords * 4;
-    const hipError_t ea = allowDynamicLds<mlpFloatKernel<Mma>>((int)(kFltLdsDwords * 4));
-    if (ea != hipSuccess) return ea;
-    int perCU = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpFloatKernel<Mma>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
-    const uint32_t numTiles = (a.batch + 15) / 16, need = (numTiles + 3) / 4;
-    const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
-    noteKernel(false, "mlpFloatKernel<%s>", Mma::kName);
-    hipLaunchKernelGGL(mlpFloatKernel<Mma>, dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
-    return hipGetLastError();
+    return widest <= 4 ? launchFloatSized<Mma, 4>(stream, ga, ldsBytes, numCUs) : launchFloatSized<Mma, 8>(stream, ga, ldsBytes, numCUs);
 }
 
 } // namespace

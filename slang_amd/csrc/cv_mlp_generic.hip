@@ -15,8 +15,7 @@ namespace cv {
 
 namespace {
 
-constexpr int kGenMaxTiles = 8;                     // 128 rows / columns
-constexpr int kGenMaxKT = kGenMaxTiles / 2;         // B fragments of a 128-wide vector
+constexpr int kGenTileLimit = 8;                    // 128 rows / columns
 constexpr uint32_t kGenLdsDwords = 36 * 1024;       // 144 KB for all layers' fragments
 
 struct GenLayer {
@@ -30,9 +29,12 @@ struct GenArgs {
     uint32_t biasDwordBase;  // biases follow the fragments in LDS
 };
 
-template <class Mma>
+// MAXT: the unrolled bound on a layer's 16-row tiles (4 for networks up to 64 wide, which then need half the
+// registers and run more waves per SIMD; 8 up to 128)
+template <class Mma, int MAXT>
 __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
 {
+    constexpr int kGenMaxTiles = MAXT, kGenMaxKT = MAXT / 2;
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
     const MlpArgs& a = ga.mlp;
     const int L = a.numLayers;
@@ -151,32 +153,40 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
     }
 }
 
+template <class Mma, int MAXT>
+hipError_t launchGenericSized(hipStream_t stream, const GenArgs& ga, size_t ldsBytes, int numCUs)
+{
+    const hipError_t ea = allowDynamicLds<mlpGenericKernel<Mma, MAXT>>((int)(kGenLdsDwords * 4));
+    if (ea != hipSuccess) return ea;
+    int perCU = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpGenericKernel<Mma, MAXT>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
+    const uint32_t numTiles = (ga.mlp.batch + 15) / 16, need = (numTiles + 3) / 4;
+    const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
+    noteKernel(false, "mlpGenericKernel<%s,up to %d rows>", Mma::kName, 16 * MAXT);
+    hipLaunchKernelGGL((mlpGenericKernel<Mma, MAXT>), dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
+    return hipGetLastError();
+}
+
 template <class Mma>
 hipError_t launchGeneric(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     GenArgs ga;
     ga.mlp = a;
-    uint32_t frag = 0, bias = 0;
+    uint32_t frag = 0, bias = 0, widest = 0;
     for (int l = 0; l < a.numLayers; ++l) {
         const uint32_t mt = optMT((uint32_t)a.layers[l].out), kt = optKT((uint32_t)a.layers[l].in, Mma::kEpl);
-        if (mt > (uint32_t)kGenMaxTiles || kt > (uint32_t)kGenMaxKT) return hipErrorInvalidValue;
+        if (mt > (uint32_t)kGenTileLimit || kt > (uint32_t)kGenTileLimit / 2) return hipErrorInvalidValue;
         ga.gl[l].mt = (int32_t)mt; ga.gl[l].kt = (int32_t)kt;
         ga.gl[l].fragBase = frag; ga.gl[l].biasBase = bias;
         frag += mt * kt; bias += mt * 16;
+        if (mt > widest) widest = mt;
+        if (2 * kt > widest) widest = 2 * kt;
     }
     ga.biasDwordBase = frag * 64 * Mma::kRawDW;
     const uint32_t dwords = ga.biasDwordBase + bias;
     if (dwords > kGenLdsDwords) return hipErrorInvalidValue;
     const size_t ldsBytes = (size_t)dwords * 4;
-    const hipError_t ea = allowDynamicLds<mlpGenericKernel<Mma>>((int)(kGenLdsDwords * 4));
-    if (ea != hipSuccess) return ea;
-    int perCU = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpGenericKernel<Mma>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
-    const uint32_t numTiles = (a.batch + 15) / 16, need = (numTiles + 3) / 4;
-    const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
-    noteKernel(false, "mlpGenericKernel<%s>", Mma::kName);
-    hipLaunchKernelGGL(mlpGenericKernel<Mma>, dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
-    return hipGetLastError();
+    return widest <= 4 ? launchGenericSized<Mma, 4>(stream, ga, ldsBytes, numCUs) : launchGenericSized<Mma, 8>(stream, ga, ldsBytes, numCUs);
 }
 
 } // namespace
