@@ -56,6 +56,18 @@ struct PairSplit {
         return b;
     }
     static constexpr int totalLocDb = locDbBase(L);
+    static constexpr int layerOfLoc(int q)          // the layer a wave's q-th dW tile belongs to
+    {
+        int l = 0;
+        while (l + 1 < L && locBase(l + 1) <= q) ++l;
+        return l;
+    }
+    static constexpr int layerOfLocDb(int q)
+    {
+        int l = 0;
+        while (l + 1 < L && locDbBase(l + 1) <= q) ++l;
+        return l;
+    }
 };
 
 // LDS tile of one 16-feature group over the 32 samples of a round, 1 KB, in 8-byte chunks of four
@@ -131,7 +143,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int B_DW = Net::totalBiasTiles * 16;
     constexpr int X_DW = 4 * Net::totalXTiles * kPairTileDW;          // per pair: every layer's input of the round
     constexpr int DZ_DW = 4 * 2 * Net::MTMAX * kPairTileDW;           // per pair: two alternating slots for dZ
-    static_assert(X_DW >= 8 * 256, "the final reduction reuses the X tiles");
     constexpr int FLAG_DW = 8;                                        // per wave: the number of its last meeting
     static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
     __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW];
@@ -144,24 +155,32 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (threadIdx.x < FLAG_DW) ldsFlag[threadIdx.x] = 0u;
 
     // ---- stage W, W^T and biases ----------------------------------------------------------------
+    // All loads of all layers first, then all stores: one round trip to memory for the whole staging (layer after
+    // layer, each matrix and each bias vector waiting for its own loads, it took 14 us of a 131 us kernel).
+    constexpr int kStageIters = (Net::MTMAX * Net::KTMAX * 64 + 511) / 512 > (Net::MTMAX * Net::KOMAX * 64 + 511) / 512
+                                    ? (Net::MTMAX * Net::KTMAX * 64 + 511) / 512 : (Net::MTMAX * Net::KOMAX * 64 + 511) / 512;
+    FragmentStage<2, EPL, kStageIters, 512> stW[L], stWT[L];
+    float stB[L];
     staticFor<0, L>([&](auto lc) {
         constexpr int l = decltype(lc)::value;
         constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
+        static_assert(MT * 16 <= 512, "one bias value per thread and layer");
         const MlpLayerArgs& ly = a.layers[l];
-        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, optGS((uint32_t)ly.in),
-                               (uint32_t)ly.out, (uint32_t)ly.in);
+        stW[l].load(ly.w, ly.shape, false, MT, KT, optGS((uint32_t)ly.in), (uint32_t)ly.out, (uint32_t)ly.in);
         if constexpr (l > 0) {
             constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
-            stageFragments<2, EPL>(ldsWT + Net::tFragBase(l) * 64 * RAW, ly.w, ly.shape, true, MTI, KTO, 4u * MT,
-                                   (uint32_t)ly.in, (uint32_t)ly.out);
+            stWT[l].load(ly.w, ly.shape, true, MTI, KTO, 4u * MT, (uint32_t)ly.in, (uint32_t)ly.out);
         }
-        for (int e = threadIdx.x; e < MT * 16; e += blockDim.x) {
-            const int t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
-            const int row = gg * ROWS + 4 * t + r;
-            float v = 0.f;
-            if (ly.bias && row < ly.out) v = (float)((const half_t*)ly.bias)[row];
-            ldsB[(Net::biasBase(l) + t) * 16 + 4 * gg + r] = v;
-        }
+        const int e = threadIdx.x, t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
+        const int row = gg * ROWS + 4 * t + r;
+        stB[l] = (e < MT * 16 && ly.bias && row < ly.out) ? (float)((const half_t*)ly.bias)[row] : 0.f;
+    });
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l);
+        stW[l].store(ldsW + Net::fragBase(l) * 64 * RAW, MT, KT);
+        if constexpr (l > 0) stWT[l].store(ldsWT + Net::tFragBase(l) * 64 * RAW, Net::mt(l - 1), Net::ktOut(l));
+        if ((int)threadIdx.x < MT * 16) ldsB[Net::biasBase(l) * 16 + threadIdx.x] = stB[l];
     });
     __syncthreads();
 
@@ -475,38 +494,61 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
     if (timeouts) lossAcc = __builtin_nanf("");       // a meeting timed out: the step's result is void, and the loss says so
-    __syncthreads();                              // every pair has left its last round: the X tiles are free
-    float* ldsRed = (float*)ldsX;                 // 8 waves x 256 floats
+    __syncthreads();                              // every pair has left its last round: the X and dZ tiles are free
+    // The eight waves put up to ten of their dW tiles at a time into the tile area (X and dZ tiles lie back to back), and all
+    // 512 threads sum them: a few rounds of two barriers instead of two barriers per tile (which took 15 us of a 135 us
+    // step).  The order of every sum is what it was: waves 0, 2, 4, 6 of a parity, left to right.
+    constexpr int kRoomForTiles = (X_DW + DZ_DW - 8 * Split::totalLocDb * 64 - 512) / (8 * 256);
+    constexpr int kTilesPerPhase = kRoomForTiles < 10 ? kRoomForTiles : 10;
+    constexpr int kRedTileFloats = 8 * kTilesPerPhase * 256;
+    static_assert(kTilesPerPhase >= 1, "the final reduction reuses the tile area");
+    float* ldsRed = (float*)ldsX;                 // [8 waves][kTilesPerPhase][256], then [8 waves][totalLocDb][64], then 512 for the loss
+    float* ldsRedB = ldsRed + kRedTileFloats;
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
     const int rpar = threadIdx.x >> 8, ridx = threadIdx.x & 255;      // the parity / element this thread sums
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l), NI = Net::nIt(l);
+    constexpr int kPhases = (Split::totalLoc + kTilesPerPhase - 1) / kTilesPerPhase;
+    staticFor<0, kPhases>([&](auto pc) {
+        constexpr int q0 = decltype(pc)::value * kTilesPerPhase;
+        constexpr int q1 = q0 + kTilesPerPhase < Split::totalLoc ? q0 + kTilesPerPhase : Split::totalLoc;
+        if constexpr (q0 > 0) __syncthreads();    // the sums of the phase before have been read
+        staticFor<q0, q1>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            *(floatx4*)&ldsRed[(wave * kTilesPerPhase + (q - q0)) * 256 + lane * 4] = accW[q];
+        });
+        if constexpr (q0 == 0) {
 #pragma unroll
-        for (int j = 0; j < OO * OI; ++j) {
-            *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[Split::locBase(l) + j];
-            __syncthreads();
-            const float s = ((ldsRed[(0 + rpar) * 256 + ridx] + ldsRed[(2 + rpar) * 256 + ridx]) + ldsRed[(4 + rpar) * 256 + ridx]) +
-                            ldsRed[(6 + rpar) * 256 + ridx];
-            const int eo = (Split::byOut(l) ? rpar * OO : 0) + j / OI, ei = (Split::byIn(l) ? rpar * OI : 0) + j % OI;
-            if (!Split::single(l) || rpar == 0) part[(Net::gradTileBase(l) + eo * NI + ei) * 256 + ridx] = s;
-            __syncthreads();
+            for (int j = 0; j < Split::totalLocDb; ++j) ldsRedB[(wave * Split::totalLocDb + j) * 64 + lane] = accB[j];
         }
-#pragma unroll
-        for (int j = 0; j < OO; ++j) {
-            ldsRed[wave * 64 + lane] = accB[Split::locDbBase(l) + j];
-            __syncthreads();
-            if (threadIdx.x < 32) {
-                const int p2 = threadIdx.x >> 4, q = threadIdx.x & 15;
-                float s = 0.f;
+        __syncthreads();
+        staticFor<q0, q1>([&](auto qc) {
+            constexpr int q = decltype(qc)::value;
+            constexpr int l = Split::layerOfLoc(q), j = q - Split::locBase(l);
+            constexpr int OO = Split::ownedOut(l), OI = Split::ownedIn(l), NI = Net::nIt(l);
+            const float* r = ldsRed + (q - q0) * 256 + ridx;
+            constexpr int W = kTilesPerPhase * 256;      // floats from one wave's tiles to the next wave's
+            const float sum = ((r[(0 + rpar) * W] + r[(2 + rpar) * W]) + r[(4 + rpar) * W]) + r[(6 + rpar) * W];
+            const int eo = (Split::byOut(l) ? rpar * OO : 0) + j / OI, ei = (Split::byIn(l) ? rpar * OI : 0) + j % OI;
+            if (!Split::single(l) || rpar == 0) part[(Net::gradTileBase(l) + eo * NI + ei) * 256 + ridx] = sum;
+        });
+        if constexpr (q0 == 0) {
+            // bias gradients: 16 values per output row (four waves of a parity x four lane groups), summed by one thread
+            if (threadIdx.x < 32 * Split::totalLocDb) {
+                const int j = threadIdx.x >> 5, p2 = (threadIdx.x >> 4) & 1, q = threadIdx.x & 15;
+                float sum = 0.f;
                 for (int w = 0; w < 4; ++w)
-                    for (int gg = 0; gg < 4; ++gg) s += ldsRed[(2 * w + p2) * 64 + gg * 16 + q];
-                const int eo = (Split::byOut(l) ? p2 * OO : 0) + j;
-                if (Split::byOut(l) || p2 == 0) part[Net::totalGradTiles * 256 + (Net::dbTileBase(l) + eo) * 16 + q] = s;
+                    for (int gg = 0; gg < 4; ++gg) sum += ldsRedB[((2 * w + p2) * Split::totalLocDb + j) * 64 + gg * 16 + q];
+                staticFor<0, Split::totalLocDb>([&](auto jc) {
+                    constexpr int jj = decltype(jc)::value;
+                    constexpr int l = Split::layerOfLocDb(jj), jl = jj - Split::locDbBase(l), OO = Split::ownedOut(l);
+                    if (j == jj) {
+                        const int eo = (Split::byOut(l) ? p2 * OO : 0) + jl;
+                        if (Split::byOut(l) || p2 == 0) part[Net::totalGradTiles * 256 + (Net::dbTileBase(l) + eo) * 16 + q] = sum;
+                    }
+                });
             }
-            __syncthreads();
         }
     });
+    ldsRed = ldsRedB + 8 * Split::totalLocDb * 64;      // the loss: one value per thread, behind the bias values
     ldsRed[threadIdx.x] = lossAcc;
     __syncthreads();
     if (threadIdx.x == 0) {
