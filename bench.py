@@ -51,7 +51,7 @@ PROFILED_TRAFFIC = {
     "c4": (805499000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4n": (820414000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
     "c4h": (1342505000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c5": (47843000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
+    "c5": (47728000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
     "op": (285455000, "profiles/outer_product_64x64_batch1M.md"),
     "rs": (537964000, "profiles/reduce_sum_64_batch4M.md"),
     "f32": (671764000, "profiles/mlp_forward_f32_32-64-64-8_batch4M.md"),
