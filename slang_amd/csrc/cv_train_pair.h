@@ -504,6 +504,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     static_assert(kTilesPerPhase >= 1, "the final reduction reuses the tile area");
     float* ldsRed = (float*)ldsX;                 // [8 waves][kTilesPerPhase][256], then [8 waves][totalLocDb][64], then 512 for the loss
     float* ldsRedB = ldsRed + kRedTileFloats;
+    float* ldsLoss = ldsRedB + 8 * Split::totalLocDb * 64;      // one value per thread, behind the bias values
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
     const int rpar = threadIdx.x >> 8, ridx = threadIdx.x & 255;      // the parity / element this thread sums
     constexpr int kPhases = (Split::totalLoc + kTilesPerPhase - 1) / kTilesPerPhase;
@@ -518,6 +519,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (q0 == 0) {
 #pragma unroll
             for (int j = 0; j < Split::totalLocDb; ++j) ldsRedB[(wave * Split::totalLocDb + j) * 64 + lane] = accB[j];
+            ldsLoss[threadIdx.x] = lossAcc;
         }
         __syncthreads();
         staticFor<q0, q1>([&](auto qc) {
@@ -548,13 +550,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         }
     });
-    ldsRed = ldsRedB + 8 * Split::totalLocDb * 64;      // the loss: one value per thread, behind the bias values
-    ldsRed[threadIdx.x] = lossAcc;
-    __syncthreads();
-    if (threadIdx.x == 0) {
+    // The loss (its 512 values were put up with the bias values): the last wave sums them in a fixed order, eight
+    // neighbours per lane, then lanes 32, 16, 8, 4, 2, 1 places apart.
+    if (threadIdx.x >= 448) {
         float s = 0.f;
-        for (int i = 0; i < 512; ++i) s += ldsRed[i];
-        part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s += ldsLoss[lane * 8 + i];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+        if (lane == 0) part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
     }
 }
 
