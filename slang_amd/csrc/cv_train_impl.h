@@ -615,10 +615,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     ldsRed[threadIdx.x] = lossAcc;
     __syncthreads();
-    if (threadIdx.x == 0) {
+    // the loss: one wave sums the 256 values in a fixed order, four neighbours per lane, then lanes 32 ... 1 places apart
+    if (wave == 0) {
         float s = 0.f;
-        for (int i = 0; i < 256; ++i) s += ldsRed[i];
-        part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s += ldsRed[lane * 4 + i];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+        if (lane == 0) part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
     }
 }
 
