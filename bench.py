@@ -224,7 +224,8 @@ def workload_c3(torch, cv, steps, warmup):
                 cpu_baseline=cpu_baseline, key="c3")
 
 
-def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std, with_bias=True):
+def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std, with_bias=True, row_major=False,
+                  bias_range=0.0, bound="hbm"):
     import numpy as np
     from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
                                    CooperativeVectorMatrixDesc as D, FeedForwardLayer)
@@ -238,13 +239,17 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
         Wt = Wf.half() if wtype == CT.Float16 else Wf.clamp(-448, 448).to(torch.float8_e4m3fn)
         esz = Wt.element_size()
         wrow = Wt.contiguous().view(torch.uint8).flatten()
-        size = cv.getCooperativeVectorMatrixSize(fo, fi, wtype, ML.InferencingOptimal)
-        wopt = torch.empty(size, dtype=torch.uint8, device=dev)
-        cv.convertCooperativeVectorMatrix(wopt, [D(fo, fi, wtype, ML.InferencingOptimal, size, 0, 0)],
-                                          wrow, [D(fo, fi, wtype, ML.RowMajor, fo * fi * esz, 0, fi * esz)])
-        bias = torch.zeros(fo, dtype=torch.float16, device=dev)      # the configurations have zero / no biases
+        if row_major:
+            wmem, wlayout, wstride = wrow, ML.RowMajor, fi * esz
+        else:
+            size = cv.getCooperativeVectorMatrixSize(fo, fi, wtype, ML.InferencingOptimal)
+            wmem, wlayout, wstride = torch.empty(size, dtype=torch.uint8, device=dev), ML.InferencingOptimal, 0
+            cv.convertCooperativeVectorMatrix(wmem, [D(fo, fi, wtype, ML.InferencingOptimal, size, 0, 0)],
+                                              wrow, [D(fo, fi, wtype, ML.RowMajor, fo * fi * esz, 0, fi * esz)])
+        # the configurations have zero / no biases unless a range is given
+        bias = ((torch.rand(fo, device=dev, generator=g) * 2 - 1) * bias_range).half()
         last = i == len(dims) - 2
-        layers.append(FeedForwardLayer(fi, fo, wopt, bias.view(torch.uint8) if with_bias else None, ML.InferencingOptimal, 0,
+        layers.append(FeedForwardLayer(fi, fo, wmem, bias.view(torch.uint8) if with_bias else None, wlayout, wstride,
                                        Activation.NoActivation if last else Activation.ReLU, 0.0))
         host.append((Wt, bias))
     x = x_maker(torch, g, B, dims[0], dev)
@@ -293,7 +298,7 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
                           "layer (fp16 accumulate, software half), -O2" % n}
 
     return dict(step=step, samples=B, alg_bytes=B * (in_bytes + dims[-1] * 2), alg_flops=B * 2 * macs,
-                bound="hbm", mfma="fp8" if flags else "f16", dtype=wtype_name,
+                bound=bound, mfma="fp8" if flags == 1 else "f16", dtype=wtype_name,
                 config={"workload": desc, "batch": B, "layers": dims}, cpu_baseline=cpu_baseline, key=key)
 
 
@@ -305,6 +310,20 @@ def workload_c1(torch, cv, steps, warmup):
                       lambda fi: (1.0 / fi) ** 0.5)
     w["graph"] = True       # a few microseconds of kernel per step: launch-bound
     return w
+
+
+def workload_c5f(torch, cv, steps, warmup, flags=0):
+    """Forward pass of config 5's network: fp16 8->64->64->64->64->1, ReLU, biases, RowMajor weights, batch 2^22.
+    25 728 flop against 18 bytes per sample: the fp16 inference workload that the matrix pipeline bounds."""
+    return _mlp_workload(torch, cv, [8, 64, 64, 64, 64, 1], 1 << 22, "f16", flags, "c5f" if not flags else "c5f16",
+                         "c5f: fp16 MLP 8->64->64->64->64->1 forward, ReLU, biases, RowMajor weights, batch 2^22, fused forward"
+                         + (", kernels on 16-sample tiles" if flags else ""),
+                         lambda torch, g, B, k, dev: (torch.rand(B, k, device=dev, generator=g) * 2 - 1).half(),
+                         lambda fi: (2.0 / fi) ** 0.5, row_major=True, bias_range=0.1, bound="mfma")
+
+
+def workload_c5f16(torch, cv, steps, warmup):
+    return workload_c5f(torch, cv, steps, warmup, flags=cv.FLAG_FORWARD_TILE16)
 
 
 def workload_c4(torch, cv, steps, warmup, flags=0):
@@ -510,10 +529,10 @@ def workload_rs(torch, cv, steps, warmup):
 
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2b": workload_c2b, "c3": workload_c3, "c4": workload_c4,
-             "c4n": workload_c4n, "c5": workload_c5, "op": workload_op, "rs": workload_rs,
+             "c4n": workload_c4n, "c5": workload_c5, "c5f": workload_c5f, "op": workload_op, "rs": workload_rs,
              # only with --workload: variants and the counter-calibration copy
-             "c4h": workload_c4h, "c5g": workload_c5g, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4h", "c4n", "c5", "op", "rs")
+             "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
+DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4h", "c4n", "c5f", "c5", "op", "rs")
 HEADLINE = "c2"
 
 

@@ -106,6 +106,8 @@ typedef enum CvActivation {
 /* cvMlpTrainStep[WorkspaceSize]: take the layer-by-layer step (the one that serves any layer sizes)
  * also where a fused kernel exists.  Same rounding points; for cross-checking the two. */
 #define CV_FLAG_LAYERWISE_TRAINING 2u
+/* cvMlpForward: keep to the kernels that work on 16-sample tiles (cross-checks of the 32-sample-tile kernels) */
+#define CV_FLAG_FORWARD_TILE16 4u
 
 /* Mirrors the fields the example fills in rhi::CooperativeVectorMatrixDesc
  * (mlp-training-coopvec.cpp:204-225).  `offset` is in bytes from the buffer handed to

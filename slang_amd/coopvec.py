@@ -90,6 +90,7 @@ def componentTypeToRhi(componentType: int) -> RhiCooperativeVectorComponentType:
 
 FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.h
 FLAG_LAYERWISE_TRAINING = 2    # CV_FLAG_LAYERWISE_TRAINING
+FLAG_FORWARD_TILE16 = 4         # CV_FLAG_FORWARD_TILE16: keep cvMlpForward to the kernels on 16-sample tiles
 
 
 class Activation(enum.IntEnum):

@@ -676,6 +676,7 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     a.inAlign = alignOf(input, inputStride); a.outAlign = alignOf(output, outputStride);
     a.inEncoding = encoded ? cv::kEncodeXYSquares : cv::kEncodeNone;
     a.inHalfAsE4M3 = (mlp->inputType == CV_FLOAT16 && mlp->weightType == CV_FLOAT_E4M3) ? 1 : 0;
+    a.noWideTiles = (mlp->flags & CV_FLAG_FORWARD_TILE16) ? 1 : 0;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     hipError_t e;

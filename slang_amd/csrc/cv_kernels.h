@@ -65,6 +65,7 @@ struct MlpArgs {
     uint32_t inAlign, outAlign;
     int32_t inEncoding;     // kEncodeNone, or kEncodeXYSquares: a sample is a float2, layer 0 sees (x, y, x*x, y*y)
     int32_t inHalfAsE4M3;   // e4m3 networks: the vectors in memory are fp16 and are quantised to e4m3 as they are loaded
+    int32_t noWideTiles;    // keep to the kernels on 16-sample tiles (cross-checks)
 };
 enum : int { kEncodeNone = 0, kEncodeXYSquares = 1 };
 // hipErrorInvalidValue when no built-in specialisation covers the layer shapes

@@ -21,28 +21,10 @@
 // order as in the 16-sample kernels: chunk (kt, g) there is chunk (s, h) = (2*kt + g/2, g%2) here.
 #pragma once
 #include "cv_mlp_impl.h"
+#include "cv_wide_tiles.h"
 
 namespace cv {
 namespace {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-// hidden unit computed by MFMA row rho of 32-row tile T (H = hidden width / 32)
-__host__ __device__ constexpr int wideUnitOfRow(int H, int T, int rho)
-{
-    return (2 * (rho / 16) + (rho % 8) / 4) * (8 * H) + 8 * T + 4 * ((rho % 16) / 8) + rho % 4;
-}
-// hidden unit consumed by element e of half h in k-step s
-__host__ __device__ constexpr int wideUnitOfSlot(int H, int s, int h, int e)
-{
-    return (2 * (s % 2) + h) * (8 * H) + 8 * (s / 2) + e;
-}
-
-__device__ __forceinline__ floatx16 mfma32(const uint32_t* a, const uint32_t* b, floatx16 c)
-{
-    const u32x4 av = {a[0], a[1], a[2], a[3]}, bv = {b[0], b[1], b[2], b[3]};
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, av), __builtin_bit_cast(halfx8, bv), c, 0, 0, 0);
-}
 
 // One fragment = 64 lanes x 8 e4m3 bytes: lane (rho, h) holds W[rowOf(T, rho)][colOf(s, h, e)], e < 8, where the
 // eight columns of a lane are neighbours: colOf(s, h, e) = colOf(s, h, 0) + e.  In a linear layout they lie at a fixed
@@ -393,7 +375,7 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
 inline bool mlpWideEligible(const MlpArgs& a, int& H, int& NH, int& OQ)
 {
     const int L = a.numLayers;
-    if (L < 2 || L > 4 || a.inEncoding != kEncodeNone) return false;
+    if (L < 2 || L > 4 || a.inEncoding != kEncodeNone || a.noWideTiles) return false;
     const uint64_t rowBytes = a.inHalfAsE4M3 ? 64u : 32u;
     if (a.layers[0].in != 32 || a.inStride != rowBytes || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0 || a.batch > (1u << 31)) return false;
     const int width = a.layers[0].out;

@@ -1,0 +1,352 @@
+// cv_mlp_wide16.h -- fused forward MLP on 32-sample tiles (v_mfma_f32_32x32x16_f16) for fp16
+// networks: the chain FeedForwardLayer.eval builds (examples/mlp-training-coopvec/fflayer.slang:60-66,
+// network.slang:41-47) for hidden layers of 32 or 64 units.
+//
+// An fp16 network has a short carrier chain between layers (fp32 -> fp16, ReLU: one v_cvt_pk_f16_f32
+// and one v_pk_max_f16 per pair of hidden values), so what can bind it is the matrix pipeline itself.
+// v_mfma_f32_32x32x16_f16 does twice the multiply-adds of v_mfma_f32_16x16x32_f16 for a lower issue
+// cost (7.3 against 8.7 cycles of the vector-ALU port), all weights stay in registers as A operands
+// (nothing is re-read from LDS per tile), and a tile's input is loaded straight in operand order.
+// Geometry, row order of the hidden layers and the order in which the 8-element chunks of k meet the
+// accumulator are those of cv_mlp_wide.h: every layer computes bit for bit what the single-layer
+// operator computes.
+//
+// Biases.  The single-layer operator starts its fp32 accumulators from float(bias).  Here the first
+// matrix instruction of a layer takes its C operand from sixteen registers that were filled from LDS
+// (one 64-byte line per layer, 32-row tile and lane half, read as a broadcast) while the other tile of
+// the pair was in the matrix pipeline; a network without biases uses the constant 0 instead.
+#pragma once
+#include "cv_mlp_impl.h"
+#include "cv_wide_tiles.h"
+
+namespace cv {
+namespace {
+
+// One fragment = 64 lanes x 8 halves (16 bytes): lane (rho, h) holds W[rowOf(T, rho)][colOf(s, h, 0) + e], e < chunkElems
+// (4 or 8), zeros behind them.
+template <class RowFn, class ColFn>
+__device__ __forceinline__ void stageWideFragments16(uint32_t* dst, const MlpLayerArgs& ly, int tiles, int steps, int chunkElems, RowFn rowOf, ColFn colOf)
+{
+    const MatrixShape& shape = ly.shape;
+    const bool linear = shape.layout == kRowMajor || shape.layout == kColumnMajor;
+    const size_t line = shape.stride ? shape.stride : (size_t)(shape.layout == kRowMajor ? shape.cols : shape.rows) * 2u;
+    const size_t sr = shape.layout == kRowMajor ? line : (size_t)2, sc = shape.layout == kRowMajor ? (size_t)2 : line;
+    for (int c = threadIdx.x; c < tiles * steps * 64; c += blockDim.x) {
+        const int lane = c & 63, f = c >> 6, s = f % steps, T = f / steps, rho = lane & 31, h = lane >> 5;
+        const int row = rowOf(T, rho), col0 = colOf(s, h, 0);
+        int nvalid = row < ly.out ? ly.in - col0 : 0;
+        nvalid = nvalid < 0 ? 0 : (nvalid > chunkElems ? chunkElems : nvalid);
+        u32x4 out = {0u, 0u, 0u, 0u};
+        const uint8_t* p0 = ly.w;
+        bool whole = false;
+        size_t step = 0;
+        if (linear) {
+            if (nvalid > 0) p0 = ly.w + (size_t)row * sr + (size_t)col0 * sc;
+            step = sc;
+            whole = sc == 2 && nvalid == 8;
+        } else if (nvalid > 0) {
+            // An Optimal layout: eight neighbouring columns that start at a multiple of eight are one lane-chunk of the
+            // 16-sample fragments when the two ends of the run say so; anything else goes through the index map.
+            const size_t off0 = elemOffset(shape, (uint32_t)row, (uint32_t)col0);
+            p0 = ly.w + off0;
+            whole = nvalid == 8 && elemOffset(shape, (uint32_t)row, (uint32_t)(col0 + 7)) == off0 + 14;
+        }
+        if (whole && ((uintptr_t)p0 & 15) == 0) {
+            out = *(const u32x4*)p0;
+        } else if (whole && ((uintptr_t)p0 & 3) == 0) {
+            out = u32x4{((const uint32_t*)p0)[0], ((const uint32_t*)p0)[1], ((const uint32_t*)p0)[2], ((const uint32_t*)p0)[3]};
+        } else if (linear) {
+            uint32_t v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = *(const uint16_t*)(e < nvalid ? p0 + (size_t)e * step : ly.w);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = e < nvalid ? v[e] : 0u;
+            out = u32x4{v[0] | (v[1] << 16), v[2] | (v[3] << 16), v[4] | (v[5] << 16), v[6] | (v[7] << 16)};
+        } else {
+            uint32_t v[4] = {0u, 0u, 0u, 0u};
+#pragma nounroll
+            for (int e = 0; e < nvalid; ++e) {
+                const uint32_t x = *(const uint16_t*)(ly.w + elemOffset(shape, (uint32_t)row, (uint32_t)(col0 + e)));
+                v[e >> 1] |= x << (16 * (e & 1));
+            }
+            out = u32x4{v[0], v[1], v[2], v[3]};
+        }
+        *(u32x4*)&dst[4 * c] = out;
+    }
+}
+
+// H: hidden width / 32 (1 or 2); NH: hidden layers (1..4); K0: inputs per sample (8, 16 or 32 halves in contiguous
+// rows).  Up to 32 outputs.  Hidden layers are ReLU; the last layer's activation (none or ReLU)
+// is read from the arguments.  Work distribution as in mlpWideKernel: one workgroup per compute unit, whose waves
+// draw pairs of tiles from a counter in LDS.
+template <int H, int NH, int K0, int WAVES, bool HAS_BIAS>
+__global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
+{
+    constexpr int KS = 2 * H;                          // k-steps of a hidden vector
+    // k-steps of the input vector, and the inputs per lane and k-step.  The result of a matrix instruction depends on
+    // which products share a lane's eight k-slots, so the inputs are dealt out as the single-layer operator deals them
+    // (cv_layout.h: a lane group owns 4*ceil(K/16) inputs): four per lane for 8 and 16 inputs (the other four k-slots
+    // zero), eight per lane for 32.  Same chunks, same bits.
+    constexpr int S0 = K0 == 8 ? 1 : 2;
+    constexpr int CE0 = K0 == 32 ? 8 : 4;
+    constexpr int F0 = H * S0, FH = H * KS, FL = KS;   // fragments of layer 0, of a hidden->hidden layer, of the last layer
+    constexpr int TOTAL = F0 + (NH - 1) * FH + FL;
+    __shared__ __attribute__((aligned(16))) uint32_t ldsW[TOTAL * 64 * 4];
+    // float(bias) in accumulator order: [layer * H + T][h][r] = bias of row 8*(r/4) + 4*h + r%4 of tile T
+    constexpr int NSEED = HAS_BIAS ? H * NH + 1 : 1;
+    __shared__ __attribute__((aligned(16))) float ldsSeed[NSEED * 32];
+    __shared__ uint32_t nextClaim;
+    if (threadIdx.x == 0) nextClaim = 0;
+    if constexpr (HAS_BIAS) {
+        for (int c = threadIdx.x; c < NSEED * 32; c += blockDim.x) {
+            const int f = c >> 5, hh = (c >> 4) & 1, r = c & 15, rho = 8 * (r / 4) + 4 * hh + r % 4;
+            const int l = f < H * NH ? f / H : NH, T = f < H * NH ? f % H : 0;
+            const int unit = l < NH ? wideUnitOfRow(H, T, rho) : rho;
+            float v = 0.f;
+            if (a.layers[l].bias && unit < a.layers[l].out) v = (float)((const half_t*)a.layers[l].bias)[unit];
+            ldsSeed[c] = v;
+        }
+    }
+
+    // ---- weights into LDS in operand order ---------------------------------------------------
+    stageWideFragments16(ldsW, a.layers[0], H, S0, CE0,
+                         [](int T, int rho) { return wideUnitOfRow(H, T, rho); },
+                         [](int s, int h, int e) { return 2 * CE0 * s + CE0 * h + e; });
+#pragma unroll
+    for (int l = 1; l < NH; ++l)
+        stageWideFragments16(ldsW + (F0 + (l - 1) * FH) * 256, a.layers[l], H, KS, 8,
+                             [](int T, int rho) { return wideUnitOfRow(H, T, rho); },
+                             [](int s, int h, int e) { return wideUnitOfSlot(H, s, h, e); });
+    stageWideFragments16(ldsW + (F0 + (NH - 1) * FH) * 256, a.layers[NH], 1, KS, 8,
+                         [](int, int rho) { return rho; },
+                         [](int s, int h, int e) { return wideUnitOfSlot(H, s, h, e); });
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int n = lane & 31, h = lane >> 5;
+
+    uint32_t W0[H][S0][4], WH[NH > 1 ? NH - 1 : 1][H][KS][4], WL[KS][4];
+    auto loadFrag = [&](int frag, uint32_t* dst) {
+        const u32x4 v = *(const u32x4*)&ldsW[(frag * 64 + lane) * 4];
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+    };
+#pragma unroll
+    for (int T = 0; T < H; ++T)
+#pragma unroll
+        for (int s = 0; s < S0; ++s) loadFrag(T * S0 + s, W0[T][s]);
+#pragma unroll
+    for (int l = 1; l < NH; ++l)
+#pragma unroll
+        for (int T = 0; T < H; ++T)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) loadFrag(F0 + (l - 1) * FH + T * KS + s, WH[l - 1][T][s]);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) loadFrag(F0 + (NH - 1) * FH + s, WL[s]);
+
+    const uint32_t numTiles = (a.batch + 31u) / 32u;
+    const uint32_t numPairs = (numTiles + 1u) / 2u;
+    const uint32_t numGroups = (uint32_t)__builtin_amdgcn_readfirstlane((int)gridDim.x);
+    // the c-th claim of this workgroup is pair c * numGroups + blockIdx.x (tiles 2*pair, 2*pair + 1)
+    auto claim = [&]() -> uint32_t {
+        uint32_t c = 0;
+        if (lane == 0) c = __hip_atomic_fetch_add(&nextClaim, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)c) * numGroups + blockIdx.x;
+    };
+    uint32_t pair = claim();
+    if (pair >= numPairs) return;
+    const uint32_t lastSample = a.batch - 1u;
+    const bool lastRelu = a.layers[NH].act == kActRelu;
+    const int outDim = a.layers[NH].out;
+    const bool storeQuads = outDim % 4 == 0 && a.outAlign >= 8u;
+    const halfx2 zero2 = {(half_t)0.f, (half_t)0.f};
+
+    // A pair's input, per tile and lane.  Rows beyond the end of the batch read the last row instead (their results
+    // are not stored).
+    //   K0 == 8 : 8 bytes: inputs 4h .. 4h+3 of sample n, the lane's operand of the one k-step as they are;
+    //   K0 == 16: 16 bytes: inputs 8h .. 8h+7;  K0 == 32: 32 bytes: inputs 16h .. 16h+15.
+    constexpr int NDW = K0 / 4;     // dwords per lane and tile
+    struct Input { uint32_t v[2][NDW]; };
+    auto loadPair = [&](uint32_t p) -> Input {
+        Input in;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint32_t s = (2u * p + (uint32_t)j) * 32u + (uint32_t)n;
+            s = s < lastSample ? s : lastSample;
+            const uint8_t* row = a.in + (uint64_t)s * (2u * K0) + (uint32_t)h * (uint32_t)K0;
+            if constexpr (K0 == 8) {
+                const u32x2 x = *(const u32x2*)row;
+                in.v[j][0] = x.x; in.v[j][1] = x.y;
+            } else {
+#pragma unroll
+                for (int i = 0; i < NDW / 4; ++i) {
+                    const u32x4 x = *(const u32x4*)(row + 16 * i);
+                    in.v[j][4 * i] = x.x; in.v[j][4 * i + 1] = x.y; in.v[j][4 * i + 2] = x.z; in.v[j][4 * i + 3] = x.w;
+                }
+            }
+        }
+        return in;
+    };
+
+    uint32_t B[2][KS > S0 ? KS : S0][4];
+    floatx16 acc[2][H];
+    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
+    auto firstOperands = [&](const Input& in) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if constexpr (K0 == 8) {
+                B[j][0][0] = in.v[j][0]; B[j][0][1] = in.v[j][1]; B[j][0][2] = 0u; B[j][0][3] = 0u;
+            } else if constexpr (K0 == 16) {
+                // lane (n,0) holds inputs 0..7, lane (n,1) inputs 8..15; k-step s wants 8s + 4h .. 8s + 4h + 3
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+                    const u32x2 r = __builtin_amdgcn_permlane32_swap(in.v[j][d], in.v[j][2 + d], false, false);
+                    B[j][0][d] = r.x; B[j][1][d] = r.y;
+                    B[j][0][2 + d] = 0u; B[j][1][2 + d] = 0u;
+                }
+            } else {
+                // lane (n,0) holds inputs 0..15, lane (n,1) inputs 16..31; k-step s wants 16s + 8h .. 16s + 8h + 7
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const u32x2 r = __builtin_amdgcn_permlane32_swap(in.v[j][d], in.v[j][4 + d], false, false);
+                    B[j][0][d] = r.x; B[j][1][d] = r.y;
+                }
+            }
+        }
+    };
+
+    const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // (the address passes through an empty asm statement inside the loop: the lines are the same for every tile, and
+    // the optimiser would otherwise keep all of them in registers, which the weights need)
+    const uint32_t seedLane = (uint32_t)h * 16u;
+    auto seed = [&](int l, int T) -> floatx16 {       // float(bias) of layer l, tile T, or zeros
+        if constexpr (HAS_BIAS) {
+            uint32_t off = seedLane;
+            asm volatile("" : "+v"(off));
+            const floatx4* p = (const floatx4*)&ldsSeed[(l * H + T) * 32 + off];
+            const floatx4 s0 = p[0], s1 = p[1], s2 = p[2], s3 = p[3];
+            return floatx16{s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3], s2[0], s2[1], s2[2], s2[3], s3[0], s3[1], s3[2], s3[3]};
+        } else {
+            return zero16;
+        }
+    };
+    // the accumulators of tile j start from the biases of layer l
+    auto seedLayer = [&](int l, int j) {
+#pragma unroll
+        for (int T = 0; T < (l < NH ? H : 1); ++T) acc[j][T] = seed(l, T);
+    };
+    auto firstLayer = [&](int j) {
+#pragma unroll
+        for (int T = 0; T < H; ++T)
+#pragma unroll
+            for (int s = 0; s < S0; ++s) acc[j][T] = mfma32(W0[T][s], B[j][s], acc[j][T]);
+    };
+    // accumulators -> fp16 -> ReLU = operands of the next layer, in place
+    auto carrier = [&](int j) {
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const int T = s / 2, r0 = 8 * (s % 2);
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const halfx2 p = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[j][T][r0 + 2 * i], acc[j][T][r0 + 2 * i + 1]}, halfx2), zero2);
+                B[j][s][i] = __builtin_bit_cast(uint32_t, p);
+            }
+        }
+    };
+    auto hiddenLayer = [&](int l, int j) {
+#pragma unroll
+        for (int T = 0; T < H; ++T)
+#pragma unroll
+            for (int s = 0; s < KS; ++s) acc[j][T] = mfma32(WH[l - 1][T][s], B[j][s], acc[j][T]);
+    };
+    auto lastLayer = [&](int j) {      // result in acc[j][0]
+#pragma unroll
+        for (int s = 0; s < KS; ++s) acc[j][0] = mfma32(WL[s], B[j][s], acc[j][0]);
+    };
+    auto storeTile = [&](int j, uint32_t t) {
+        const floatx16 o = acc[j][0];
+        const uint32_t sample = t * 32u + (uint32_t)n;
+        if (sample >= a.batch) return;
+        uint8_t* orow = a.out + (uint64_t)sample * a.outStride;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            typedef float floatx2 __attribute__((ext_vector_type(2)));
+            const int row0 = 8 * q + 4 * h;
+            if (row0 >= outDim) continue;
+            halfx2 p0 = __builtin_convertvector(floatx2{o[4 * q], o[4 * q + 1]}, halfx2);
+            halfx2 p1 = __builtin_convertvector(floatx2{o[4 * q + 2], o[4 * q + 3]}, halfx2);
+            if (lastRelu) {
+                p0 = __builtin_elementwise_max(p0, zero2);
+                p1 = __builtin_elementwise_max(p1, zero2);
+            }
+            if (storeQuads) {
+                const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
+                *(u32x2*)(orow + 2 * row0) = v;
+            } else {
+                half_t* o16 = (half_t*)(orow + 2 * row0);
+                o16[0] = p0.x;
+                if (row0 + 1 < outDim) o16[1] = p0.y;
+                if (row0 + 2 < outDim) o16[2] = p1.x;
+                if (row0 + 3 < outDim) o16[3] = p1.y;
+            }
+        }
+    };
+
+    // Two tiles travel through the layers half a layer apart: while the vector ALU turns one tile's accumulators into
+    // the next layer's operands (and its next biases arrive from LDS), the matrix pipeline works on the other tile.
+    Input in = loadPair(pair);
+    seedLayer(0, 0);
+    seedLayer(0, 1);
+    while (true) {
+        const uint32_t next = claim();
+        firstOperands(in);
+        in = loadPair(next < numPairs ? next : numPairs - 1u);      // beyond the end: loaded again, never used
+        firstLayer(0);
+        firstLayer(1);
+#pragma unroll
+        for (int l = 1; l < NH; ++l) {
+            carrier(0); seedLayer(l, 0); hiddenLayer(l, 0);
+            carrier(1); seedLayer(l, 1); hiddenLayer(l, 1);
+        }
+        carrier(0); seedLayer(NH, 0); lastLayer(0);
+        carrier(1); seedLayer(NH, 1); lastLayer(1);
+        storeTile(0, 2u * pair); seedLayer(0, 0);
+        storeTile(1, 2u * pair + 1u); seedLayer(0, 1);
+        if (next >= numPairs) return;
+        pair = next;
+    }
+}
+
+// Shapes: fp16 vectors of 8, 16 or 32 elements in contiguous rows at a 16-byte aligned address, ReLU hidden layers of
+// exactly 32 or 64 units (one to four of them), at most 32 outputs (checked by the dispatcher in cv_mlp_f16.hip).
+template <int H, int NH, int K0, bool HAS_BIAS>
+hipError_t launchMlpWide16Shape(hipStream_t stream, const MlpArgs& a, int numCUs)
+{
+    // one workgroup per compute unit, as many waves as the weights leave registers for
+    // (16 waves: 128 registers each, 12: 168, 8: 256); the build fails if an instantiation spills
+    constexpr int KS = 2 * H, S0 = K0 == 8 ? 1 : 2;
+    constexpr int WREGS = 4 * (H * S0 + (NH - 1) * H * KS + KS);
+    constexpr int WAVES = (WREGS + 48 * H + 32 <= 128) ? 16 : ((WREGS + 48 * H + 32 <= 168) ? 12 : 8);
+    const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
+    const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
+    noteKernel(false, "mlpWide16Kernel<f16,32x32x16,inputs=%d,hidden=%dx%d,%s,waves=%d>", K0, NH, 32 * H,
+               HAS_BIAS ? "bias" : "nobias", WAVES);
+    hipLaunchKernelGGL((mlpWide16Kernel<H, NH, K0, WAVES, HAS_BIAS>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+    return hipGetLastError();
+}
+
+// all shapes of one input width (one translation unit each, compiled in parallel)
+template <int K0>
+hipError_t launchMlpWide16K(hipStream_t stream, const MlpArgs& a, int numCUs, int H, int NH)
+{
+    bool hasBias = false;
+    for (int l = 0; l < a.numLayers; ++l) hasBias = hasBias || a.layers[l].bias != nullptr;
+#define CV_W16(h_, nh_) if (H == h_ && NH == nh_) \
+        return hasBias ? launchMlpWide16Shape<h_, nh_, K0, true>(stream, a, numCUs) : launchMlpWide16Shape<h_, nh_, K0, false>(stream, a, numCUs);
+    CV_W16(1, 1) CV_W16(1, 2) CV_W16(1, 3) CV_W16(1, 4) CV_W16(2, 1) CV_W16(2, 2) CV_W16(2, 3) CV_W16(2, 4)
+#undef CV_W16
+    return hipErrorInvalidValue;
+}
+
+} // namespace
+} // namespace cv

@@ -330,6 +330,61 @@ def test_biases_on_32_sample_tiles(dims, B, fp16_vectors):
     assert frac >= 0.99
 
 
+@pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 100003), ([8, 64, 64, 64, 64, 1], 1), ([8, 64, 1], 63), ([8, 32, 32, 3], 65),
+                                    ([16, 64, 64, 8], 4097), ([16, 32, 32, 32, 32, 20], 1000), ([16, 64, 32], 31),
+                                    ([32, 64, 64, 8], 5000), ([32, 64, 64, 64, 16], 129), ([32, 32, 7], 33), ([32, 64, 64, 64, 64, 4], 2049)])
+@pytest.mark.parametrize("bias", ["rand", "none"])
+def test_fp16_networks_on_32_sample_tiles(dims, B, bias):
+    # fp16 networks with 8, 16 or 32 inputs in contiguous rows and ReLU hidden layers of 32 or 64 units run on
+    # 32-sample tiles (v_mfma_f32_32x32x16_f16, all weights in registers, biases as the C operand of a layer's first
+    # matrix instruction): same bits as the chain of single-layer operators and as the kernels on 16-sample tiles, for
+    # every depth, output width, weight layout and ragged batch; one layer without a bias next to layers that have one
+    rng = np.random.default_rng(sum(dims) * 11 + B)
+    specs = make_net(rng, dims, CT.Float16, bias=bias, init="he")
+    if bias == "rand" and len(specs) > 2:
+        specs[1]["b"] = None
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    xd = to_dev(x)
+    hid = []
+    yc = chain_of_single_layers(specs, xd, CT.Float16, hidden=hid)
+    for layout in (ML.RowMajor, ML.ColumnMajor, ML.InferencingOptimal):
+        y = cv.mlpForward(gpu_layers(specs, CT.Float16, layout), xd)
+        name = cv.lastKernelName()
+        assert name.startswith("mlpWide16Kernel") and ((",bias" in name) == (bias == "rand")), name
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), layout
+    y16 = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), xd, flags=cv.FLAG_FORWARD_TILE16)
+    assert not cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+    assert torch.equal(y16.view(torch.int16), yc.view(torch.int16))
+    frac, _ = end_to_end_ok(y.cpu().numpy(), specs, x, ob.F16, hid)      # (every outlier is checked to be a boundary case)
+    assert frac >= 0.99
+    # a ReLU behind the last layer, and a padded output buffer: rows at a stride, nothing written between them
+    specs[-1]["act"] = int(Activation.ReLU)
+    wide = torch.full((B, dims[-1] + 3), -7.0, dtype=torch.float16, device=DEV)
+    cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), xd, out=wide[:, :dims[-1]])
+    assert cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+    assert torch.equal(wide[:, :dims[-1]].contiguous().view(torch.int16), torch.clamp_min(yc, 0).view(torch.int16))
+    assert (wide[:, dims[-1]:] == -7.0).all()
+
+
+def test_fp16_32_sample_tiles_fall_back():
+    # leaky ReLU, rows at a stride and other widths stay on the 16-sample kernels (same results either way)
+    rng = np.random.default_rng(99)
+    dims, B = [8, 64, 64, 1], 500
+    x = rng.uniform(-1, 1, (B, 8)).astype(np.float16)
+    specs = make_net(rng, dims, CT.Float16, act=Activation.LeakyReLU, slope=0.01, bias="rand", init="he")
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), to_dev(x))
+    assert not cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+    assert torch.equal(y.view(torch.int16), chain_of_single_layers(specs, to_dev(x), CT.Float16).view(torch.int16))
+    specs = make_net(rng, dims, CT.Float16, bias="rand", init="he")
+    strided = torch.zeros((B, 12), dtype=torch.float16, device=DEV)
+    strided[:, :8] = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), strided[:, :8])
+    assert not cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+    y2 = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), to_dev(x))
+    assert cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
 def test_32_sample_tiles_keep_the_summation_order():
     # The last layer's fp32 sums reach the fp16 output without any coarser rounding in between, so they
     # show the order in which the 8-element chunks of k meet the accumulator: with hidden values and
