@@ -75,6 +75,26 @@ __device__ __forceinline__ void stageWideFragments16(uint32_t* dst, const MlpLay
     }
 }
 
+// Order of one scheduling region for the instruction scheduler: NM matrix instructions; the NV vector-ALU instructions
+// spread evenly behind all but the last two of them; the NL LDS reads in two halves, each as soon as the vector-ALU
+// instructions that free its destination registers are through, so that the second half has two matrix instructions of
+// time left before the next phase asks for it.
+template <int NM, int NV, int NL>
+__device__ __forceinline__ void interleavePhase()
+{
+    constexpr int NS = NM > 3 ? NM - 2 : NM;      // matrix instructions that have vector-ALU work behind them
+    staticFor<0, NM>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                       // one MFMA
+        if constexpr (i < NS) {
+            constexpr int nv = NV * (i + 1) / NS - NV * i / NS;
+            if constexpr (nv > 0) __builtin_amdgcn_sched_group_barrier(0x002, nv, 0);            // VALU
+            if constexpr (NL > 0 && i == (NS - 1) / 2) __builtin_amdgcn_sched_group_barrier(0x100, NL / 2, 0);    // DS reads
+            if constexpr (NL > 0 && i == NS - 1) __builtin_amdgcn_sched_group_barrier(0x100, NL - NL / 2, 0);
+        }
+    });
+}
+
 // H: hidden width / 32 (1 or 2); NH: hidden layers (1..4); K0: inputs per sample (8, 16 or 32 halves in contiguous
 // rows).  Up to 32 outputs.  Hidden layers are ReLU; the last layer's activation (none or ReLU)
 // is read from the arguments.  Work distribution as in mlpWideKernel: one workgroup per compute unit, whose waves
@@ -215,14 +235,13 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     };
 
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    // (the address passes through an empty asm statement inside the loop: the lines are the same for every tile, and
-    // the optimiser would otherwise keep all of them in registers, which the weights need)
-    const uint32_t seedLane = (uint32_t)h * 16u;
-    auto seed = [&](int l, int T) -> floatx16 {       // float(bias) of layer l, tile T, or zeros
+    // (the lane's offset passes through an empty asm statement once per round of the loop: the lines are the same for
+    // every tile, and the optimiser would otherwise keep all of them in registers, which the weights need)
+    // (one offset per tile of the pair, or the two tiles would share one read and hold its result in extra registers)
+    uint32_t seedOff[2] = {(uint32_t)h * 16u, (uint32_t)h * 16u};
+    auto seed = [&](int l, int T, int j) -> floatx16 {       // float(bias) of layer l, tile T, or zeros
         if constexpr (HAS_BIAS) {
-            uint32_t off = seedLane;
-            asm volatile("" : "+v"(off));
-            const floatx4* p = (const floatx4*)&ldsSeed[(l * H + T) * 32 + off];
+            const floatx4* p = (const floatx4*)&ldsSeed[(l * H + T) * 32 + seedOff[j]];
             const floatx4 s0 = p[0], s1 = p[1], s2 = p[2], s3 = p[3];
             return floatx16{s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3], s2[0], s2[1], s2[2], s2[3], s3[0], s3[1], s3[2], s3[3]};
         } else {
@@ -232,13 +251,14 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     // the accumulators of tile j start from the biases of layer l
     auto seedLayer = [&](int l, int j) {
 #pragma unroll
-        for (int T = 0; T < (l < NH ? H : 1); ++T) acc[j][T] = seed(l, T);
+        for (int T = 0; T < (l < NH ? H : 1); ++T) acc[j][T] = seed(l, T, j);
     };
+    // (k-step outer, 32-row tile inner: no two dependent matrix instructions follow one another)
     auto firstLayer = [&](int j) {
 #pragma unroll
-        for (int T = 0; T < H; ++T)
+        for (int s = 0; s < S0; ++s)
 #pragma unroll
-            for (int s = 0; s < S0; ++s) acc[j][T] = mfma32(W0[T][s], B[j][s], acc[j][T]);
+            for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][s], B[j][s], acc[j][T]);
     };
     // accumulators -> fp16 -> ReLU = operands of the next layer, in place
     auto carrier = [&](int j) {
@@ -255,9 +275,9 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     };
     auto hiddenLayer = [&](int l, int j) {
 #pragma unroll
-        for (int T = 0; T < H; ++T)
+        for (int s = 0; s < KS; ++s)
 #pragma unroll
-            for (int s = 0; s < KS; ++s) acc[j][T] = mfma32(WH[l - 1][T][s], B[j][s], acc[j][T]);
+            for (int T = 0; T < H; ++T) acc[j][T] = mfma32(WH[l - 1][T][s], B[j][s], acc[j][T]);
     };
     auto lastLayer = [&](int j) {      // result in acc[j][0]
 #pragma unroll
@@ -292,25 +312,38 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
         }
     };
 
-    // Two tiles travel through the layers half a layer apart: while the vector ALU turns one tile's accumulators into
-    // the next layer's operands (and its next biases arrive from LDS), the matrix pipeline works on the other tile.
+    // Two tiles travel through the layers half a layer apart.  A phase = the matrix instructions of one layer for one
+    // tile, and between them the vector-ALU work of the other tile: its accumulators of the layer before become operands
+    // (two instructions per pair of values), then the biases of its next layer are requested from LDS into the
+    // accumulators just freed, a whole phase before the matrix instruction that takes them as C operand.  The order
+    // within a phase is given to the scheduler explicitly (left alone it requests the biases right in front of their
+    // use and the wave sits out the LDS latency once per layer and tile); nothing moves across a phase boundary.
+    constexpr int NV = 16 * H;      // vector-ALU instructions of one tile's carrier
+    constexpr int NL = HAS_BIAS ? 4 * H : 0;
+    auto endPhase = []() { __builtin_amdgcn_sched_barrier(0); };
     Input in = loadPair(pair);
     seedLayer(0, 0);
     seedLayer(0, 1);
     while (true) {
         const uint32_t next = claim();
+        if constexpr (HAS_BIAS) asm volatile("" : "+v"(seedOff[0]), "+v"(seedOff[1]));
         firstOperands(in);
         in = loadPair(next < numPairs ? next : numPairs - 1u);      // beyond the end: loaded again, never used
         firstLayer(0);
-        firstLayer(1);
+        endPhase();
+        firstLayer(1); carrier(0); seedLayer(1, 0);
+        interleavePhase<H * S0, NV, NL>(); endPhase();
 #pragma unroll
         for (int l = 1; l < NH; ++l) {
-            carrier(0); seedLayer(l, 0); hiddenLayer(l, 0);
-            carrier(1); seedLayer(l, 1); hiddenLayer(l, 1);
+            hiddenLayer(l, 0); carrier(1); seedLayer(l, 1);
+            interleavePhase<H * KS, NV, NL>(); endPhase();
+            hiddenLayer(l, 1); carrier(0); seedLayer(l + 1, 0);
+            interleavePhase<H * KS, NV, NL>(); endPhase();
         }
-        carrier(0); seedLayer(NH, 0); lastLayer(0);
-        carrier(1); seedLayer(NH, 1); lastLayer(1);
-        storeTile(0, 2u * pair); seedLayer(0, 0);
+        lastLayer(0); carrier(1); seedLayer(NH, 1);
+        interleavePhase<KS, NV, HAS_BIAS ? 4 : 0>(); endPhase();
+        lastLayer(1); storeTile(0, 2u * pair); seedLayer(0, 0);
+        endPhase();
         storeTile(1, 2u * pair + 1u); seedLayer(0, 1);
         if (next >= numPairs) return;
         pair = next;

@@ -332,7 +332,8 @@ def test_biases_on_32_sample_tiles(dims, B, fp16_vectors):
 
 @pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 100003), ([8, 64, 64, 64, 64, 1], 1), ([8, 64, 1], 63), ([8, 32, 32, 3], 65),
                                     ([16, 64, 64, 8], 4097), ([16, 32, 32, 32, 32, 20], 1000), ([16, 64, 32], 31),
-                                    ([32, 64, 64, 8], 5000), ([32, 64, 64, 64, 16], 129), ([32, 32, 7], 33), ([32, 64, 64, 64, 64, 4], 2049)])
+                                    ([32, 64, 64, 64, 8], 5000), ([32, 64, 64, 64, 16], 129), ([32, 32, 32, 32, 7], 33), ([32, 64, 64, 64, 64, 4], 2049),
+                                    ([16, 64, 64, 64, 2], 70001)])
 @pytest.mark.parametrize("bias", ["rand", "none"])
 def test_fp16_networks_on_32_sample_tiles(dims, B, bias):
     # fp16 networks with 8, 16 or 32 inputs in contiguous rows and ReLU hidden layers of 32 or 64 units run on
