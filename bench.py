@@ -9,9 +9,11 @@ metric is quoted on: a single fp16 coopVecMatMulAdd layer 64x64 (fp32 accumulate
 2^22 vectors, weights in InferencingOptimal layout (the layout conversion is timed separately and
 reported as `layout_conversion_us`).  Without --workload every other configuration is timed the same
 way in the same run (W warm-up steps, K timed steps, HIP events on the launch stream) and reported
-under "workloads": c1, c2b (c2 in bfloat16), c3, c4 (e4m3 decoded to the fp16 matrix pipeline), c4n
-(fp8 matrix pipeline), c4h (c4 fed with fp16 vectors), c5 (training step), op / rs (stand-alone outer-product / reduce-sum
-accumulate).  With --workload only that one runs and becomes the headline (profiling runs; also
+under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (c2 with RowMajor weights), c2b (c2 in
+bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
+c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
+matrix pipeline bounds), c5 (training step), ex (one whole iteration of the example at its own shape: training step +
+Adam update, three kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate).  With --workload only that one runs and becomes the headline (profiling runs; also
 c5g = c5 on the layer-by-layer step, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
@@ -41,22 +43,18 @@ METRIC = "CoopVec MLP samples/sec (fp16/fp8/int8 fwd, fp16 train step); % MFMA p
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "fp8": 5000.0, "int8": 5000.0, "f32": 157.3}
 
-# HBM bytes per step (all kernels of the step) as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE,
-# scaled by a copy of known size): not measured by this script, quoted from the committed profile summaries.
-PROFILED_TRAFFIC = {
-    "c1": (739000, "profiles/mlp_forward_f16_2-16x3-1_batch64K.md"),
-    "c2": (1084765000, "profiles/matmul_f16_64x64_batch4M.md"),
-    "c2b": (1084788000, "profiles/matmul_bf16_64x64_batch4M.md"),
-    "c3": (2684654000, "profiles/matmul_i8_128x128_batch4M.md"),
-    "c4": (805499000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c4n": (820414000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c4h": (1342505000, "profiles/mlp_forward_e4m3_32-64-64-8_batch16M.md"),
-    "c5": (47728000, "profiles/mlp_train_8-64x4-1_batch1M.md"),
-    "op": (285455000, "profiles/outer_product_64x64_batch1M.md"),
-    "rs": (537964000, "profiles/reduce_sum_64_batch4M.md"),
-    "f32": (671764000, "profiles/mlp_forward_f32_32-64-64-8_batch4M.md"),
-    "copy": (1073743000, "profiles/copy_calibration_512MiB.md"),
-}
+def profiled_traffic():
+    """HBM bytes per step (all kernels of the step) as measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a
+    copy of known size): not measured by this script, read from the committed profile summaries, whose lines
+    `traffic[<workload>] = <bytes> B per step` carry them.  {workload: (bytes, file)}"""
+    import glob
+    import re
+    found = {}
+    for path in sorted(glob.glob(os.path.join(REPO, "profiles", "*.md"))):
+        with open(path) as f:
+            for m in re.finditer(r"^traffic\[(\w+)\] = (\d+) B per step", f.read(), re.M):
+                found[m.group(1)] = (int(m.group(2)), "profiles/" + os.path.basename(path))
+    return found
 
 
 def ensure_built():
@@ -67,8 +65,8 @@ def ensure_built():
     return _lib.load()
 
 
-def workload_c2(torch, cv, steps, warmup, bf16=False):
-    """fp16 (or bfloat16) 64x64 matMulAdd, batch 2^22, InferencingOptimal weights."""
+def workload_c2(torch, cv, steps, warmup, bf16=False, row_major=False):
+    """fp16 (or bfloat16) 64x64 matMulAdd, batch 2^22, InferencingOptimal (or RowMajor) weights."""
     import numpy as np
     from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML, CooperativeVectorMatrixDesc as D
     dev = "cuda"
@@ -95,7 +93,10 @@ def workload_c2(torch, cv, steps, warmup, bf16=False):
     out = torch.empty(B, M, dtype=tdt, device=dev)
 
     def step():
-        cv.coopVecMatMulAdd(x, ct, wopt, 0, ct, bb, 0, ct, ML.InferencingOptimal, False, 0, M=M, out=out)
+        if row_major:
+            cv.coopVecMatMulAdd(x, ct, wrow, 0, ct, bb, 0, ct, ML.RowMajor, False, K * 2, M=M, out=out)
+        else:
+            cv.coopVecMatMulAdd(x, ct, wopt, 0, ct, bb, 0, ct, ML.InferencingOptimal, False, 0, M=M, out=out)
 
     def cpu_baseline_bf16():
         import oracle_binding as ob
@@ -142,17 +143,23 @@ def workload_c2(torch, cv, steps, warmup, bf16=False):
                           "fallback (fp16 accumulate, software half as gcc<12 selects), -O2" % (n, per_core)}
 
     name = "bf16" if bf16 else "fp16"
+    key = "c2b" if bf16 else ("c2r" if row_major else "c2")
+    layout = "RowMajor" if row_major else "InferencingOptimal"
     return dict(step=step, samples=B, alg_bytes=B * (K * 2 + M * 2), alg_flops=B * 2 * M * K,
                 bound="hbm", mfma="f16", dtype="bf16" if bf16 else "f16",
-                config={"workload": "%s: %s coopVecMatMulAdd 64x64, batch 2^22, InferencingOptimal weights, "
-                                    "fp32 accumulate, %s out" % ("c2b" if bf16 else "c2", name, name), "batch": B, "m": M, "k": K,
-                        "layout": "InferencingOptimal"},
-                extra={"layout_conversion_us": conv_us}, cpu_baseline=cpu_baseline_bf16 if bf16 else cpu_baseline,
-                key="c2b" if bf16 else "c2")
+                config={"workload": "%s: %s coopVecMatMulAdd 64x64, batch 2^22, %s weights, "
+                                    "fp32 accumulate, %s out" % (key, name, layout, name), "batch": B, "m": M, "k": K,
+                        "layout": layout},
+                extra={} if row_major else {"layout_conversion_us": conv_us},
+                cpu_baseline=cpu_baseline_bf16 if bf16 else cpu_baseline, key=key)
 
 
 def workload_c2b(torch, cv, steps, warmup):
     return workload_c2(torch, cv, steps, warmup, bf16=True)
+
+
+def workload_c2r(torch, cv, steps, warmup):
+    return workload_c2(torch, cv, steps, warmup, row_major=True)
 
 
 def workload_copy(torch, cv, steps, warmup):
@@ -170,8 +177,8 @@ def workload_copy(torch, cv, steps, warmup):
                 cpu_baseline=lambda: None, key="copy", kernel="torch copy kernel")
 
 
-def workload_c3(torch, cv, steps, warmup):
-    """int8 128x128 -> int32 + int32 bias, batch 2^22, InferencingOptimal weights (bit-exact path)."""
+def workload_c3(torch, cv, steps, warmup, column_major=False):
+    """int8 128x128 -> int32 + int32 bias, batch 2^22, InferencingOptimal (or ColumnMajor) weights (bit-exact path)."""
     import numpy as np
     from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML, CooperativeVectorMatrixDesc as D
     dev = "cuda"
@@ -183,14 +190,25 @@ def workload_c3(torch, cv, steps, warmup):
     wcol = W.t().contiguous().view(torch.uint8).flatten()          # ColumnMajor storage of the M x K matrix
     size = cv.getCooperativeVectorMatrixSize(M, K, CT.SignedInt8, ML.InferencingOptimal)
     wopt = torch.empty(size, dtype=torch.uint8, device=dev)
-    cv.convertCooperativeVectorMatrix(wopt, [D(M, K, CT.SignedInt8, ML.InferencingOptimal, size, 0, 0)],
-                                      wcol, [D(M, K, CT.SignedInt8, ML.ColumnMajor, M * K, 0, M)])
+    dst, src = [D(M, K, CT.SignedInt8, ML.InferencingOptimal, size, 0, 0)], [D(M, K, CT.SignedInt8, ML.ColumnMajor, M * K, 0, M)]
+    cv.convertCooperativeVectorMatrix(wopt, dst, wcol, src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        cv.convertCooperativeVectorMatrix(wopt, dst, wcol, src)
+    e1.record(); torch.cuda.synchronize()
+    conv_us = e0.elapsed_time(e1) / 20 * 1e3
     bb = b.view(torch.uint8)
     out = torch.empty(B, M, dtype=torch.int32, device=dev)
 
     def step():
-        cv.coopVecMatMulAdd(x, CT.SignedInt8, wopt, 0, CT.SignedInt8, bb, 0, CT.SignedInt32, ML.InferencingOptimal,
-                            False, 0, M=M, out=out)
+        if column_major:
+            cv.coopVecMatMulAdd(x, CT.SignedInt8, wcol, 0, CT.SignedInt8, bb, 0, CT.SignedInt32, ML.ColumnMajor,
+                                False, M, M=M, out=out)
+        else:
+            cv.coopVecMatMulAdd(x, CT.SignedInt8, wopt, 0, CT.SignedInt8, bb, 0, CT.SignedInt32, ML.InferencingOptimal,
+                                False, 0, M=M, out=out)
 
     def cpu_baseline():
         import concurrent.futures as cf
@@ -218,10 +236,16 @@ def workload_c3(torch, cv, steps, warmup):
                 "sample": "first %d of the 2^22 vectors; C restatement of the Slang CPU-target fallback "
                           "(packed int8, ColumnMajor, int32 accumulate), -O2" % n}
 
+    layout = "ColumnMajor" if column_major else "InferencingOptimal"
     return dict(step=step, samples=B, alg_bytes=B * (K + M * 4), alg_flops=B * 2 * M * K, bound="hbm", mfma="int8", dtype="int8",
-                config={"workload": "c3: int8 coopVecMatMulAdd 128x128 -> int32 + int32 bias, batch 2^22, "
-                                    "InferencingOptimal weights", "batch": B, "m": M, "k": K},
-                cpu_baseline=cpu_baseline, key="c3")
+                config={"workload": "%s: int8 coopVecMatMulAdd 128x128 -> int32 + int32 bias, batch 2^22, "
+                                    "%s weights" % ("c3c" if column_major else "c3", layout), "batch": B, "m": M, "k": K, "layout": layout},
+                extra={} if column_major else {"layout_conversion_us": conv_us},
+                cpu_baseline=cpu_baseline, key="c3c" if column_major else "c3")
+
+
+def workload_c3c(torch, cv, steps, warmup):
+    return workload_c3(torch, cv, steps, warmup, column_major=True)
 
 
 def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, init_std, with_bias=True, row_major=False,
@@ -305,9 +329,9 @@ def _mlp_workload(torch, cv, dims, B, wtype_name, flags, key, desc, x_maker, ini
 def workload_c1(torch, cv, steps, warmup):
     """fp16 2->16->16->16->1 ReLU MLP, batch 65536 (the CPU-runnable configuration)."""
     w = _mlp_workload(torch, cv, [2, 16, 16, 16, 1], 65536, "f16", 0, "c1",
-                      "c1: fp16 MLP 2->16->16->16->1, ReLU, batch 65536, fused forward",
+                      "c1: fp16 MLP 2->16->16->16->1, ReLU, zero biases, RowMajor weights, batch 65536, fused forward",
                       lambda torch, g, B, k, dev: torch.rand(B, k, device=dev, generator=g).half(),
-                      lambda fi: (1.0 / fi) ** 0.5)
+                      lambda fi: (1.0 / fi) ** 0.5, row_major=True)
     w["graph"] = True       # a few microseconds of kernel per step: launch-bound
     return w
 
@@ -328,11 +352,19 @@ def workload_c5f16(torch, cv, steps, warmup):
 
 def workload_c4(torch, cv, steps, warmup, flags=0):
     """e4m3 32->64->64->8 decoder MLP, batch 2^24."""
-    return _mlp_workload(torch, cv, [32, 64, 64, 8], 1 << 24, "fp8", flags, "c4" if not flags else "c4n",
+    w = _mlp_workload(torch, cv, [32, 64, 64, 8], 1 << 24, "fp8", flags, "c4" if not flags else "c4n",
                          "c4: e4m3 MLP 32->64->64->8, ReLU, fp16 out, batch 2^24, fused forward, "
                          + ("fp8 matrix pipeline" if flags else "e4m3 decoded to the fp16 matrix pipeline"),
                          lambda torch, g, B, k, dev: (torch.randn(B, k, device=dev, generator=g) * 0.5).to(torch.float8_e4m3fn),
                          lambda fi: 0.5, with_bias=False)
+    if not flags:
+        # What bounds this kernel is issue on the vector-ALU port, not HBM or the matrix pipeline: per 32-sample tile
+        # 32 conversions to e4m3 (8.3 cycles each), 16 matrix instructions (7.3) and 127 other vector instructions (4.3),
+        # 512 tiles per SIMD, at the 1.945 GHz the shader clock settles at under this load.
+        w["issue_bound"] = {"ms": 929 * 512 / 1.945e9 * 1e3,
+                            "model": "929 vector-ALU port cycles per 32-sample tile (32 x 8.3 + 16 x 7.3 + 127 x 4.3), "
+                                     "512 tiles per SIMD, 1.945 GHz"}
+    return w
 
 
 def workload_c4n(torch, cv, steps, warmup):
@@ -449,6 +481,71 @@ def workload_c5g(torch, cv, steps, warmup):
     return workload_c5(torch, cv, steps, warmup, flags=cv.FLAG_LAYERWISE_TRAINING)
 
 
+def workload_ex(torch, cv, steps, warmup):
+    """One whole iteration of examples/mlp-training-coopvec at its own shape (mlp-training-coopvec.cpp:164-250):
+    4 -> 16 -> 4, leaky ReLU, 16 float2 samples encoded (x, y, x^2, y^2), fp16 TrainingOptimal gradients; learnGradient
+    (cvMlpTrainStep: two kernels) + the parameter update read straight from those gradients (cvMlpAdamStep: one
+    kernel, which also leaves them cleared).  Launch-bound: the figure to hold it against is the cost of three graph
+    nodes."""
+    import numpy as np
+    from slang_amd.coopvec import Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML, FeedForwardLayer
+    dev = "cuda"
+    dims = [4, 16, 4]
+    n = 16
+    g = torch.Generator(device=dev); g.manual_seed(1072)
+    layers, wst, bst, host = [], [], [], []
+    slope = float(np.float16(0.001))
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = (torch.rand(fo, fi, device=dev, generator=g) * 2 - 1).half()
+        b = (torch.rand(fo, device=dev, generator=g) * 2 - 1).half()
+        gsize = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float16, ML.TrainingOptimal)
+        wg = torch.zeros(gsize, dtype=torch.uint8, device=dev)
+        bg = torch.zeros(fo, dtype=torch.float16, device=dev)
+        layers.append(FeedForwardLayer(fi, fo, W.view(torch.uint8).flatten(), b.view(torch.uint8), ML.RowMajor, fi * 2,
+                                       Activation.LeakyReLU, slope, wg, bg.view(torch.uint8), ML.TrainingOptimal, 0))
+        wst.append(torch.zeros(fo * fi * 8, dtype=torch.uint8, device=dev))
+        bst.append(torch.zeros(fo * 8, dtype=torch.uint8, device=dev))
+        host.append((W.clone(), b.clone()))
+    xy = torch.rand(n, 2, device=dev, generator=g)
+    ws = torch.empty(cv.mlpTrainStepWorkspaceSize(layers, n, gradType=CT.Float16, inputEncoding=1), dtype=torch.uint8, device=dev)
+    loss = torch.zeros(1, dtype=torch.float32, device=dev)
+    lmax = torch.zeros(1, dtype=torch.float32, device=dev)
+
+    def step():
+        cv.mlpTrainStep(layers, xy, None, gradType=CT.Float16, workspace=ws, lossSum=loss, lossMax=lmax, inputEncoding=1)
+        cv.mlpAdjustParameters(layers, wst, bst, gradType=CT.Float16)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+    nparams = sum(dims[i] * dims[i + 1] + dims[i + 1] for i in range(len(dims) - 1))
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        specs = [dict(W=W.cpu().numpy(), b=b.cpu().numpy(), act=2, slope=slope) for W, b in host]
+        xs = xy.cpu().numpy().astype(np.float16)
+        enc = np.concatenate([xs, (xs.astype(np.float32) ** 2).astype(np.float16)], axis=1)
+        tgt = np.zeros((n, 4), np.float16)
+        p = np.zeros(nparams, np.float16); st = np.zeros(nparams, ob.ADAM_STATE_DTYPE); gr = np.zeros(nparams, np.float16)
+        reps = 200
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            ob.ref_mlp_train(specs, enc, tgt, 1.0, True)
+            ob.slang_adam_step(st, p, gr)
+        t1 = time.perf_counter()
+        return {"value": reps * n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "%d iterations of 16 samples, one core; the parity oracle's training step plus the C restatement "
+                          "of AdamOptimizer::step, called from Python" % reps}
+
+    w = dict(step=step, samples=n, alg_bytes=n * 8 + nparams * 12, alg_flops=n * 2 * (3 * macs), bound="hbm", mfma="f16",
+             dtype="f16", cpu_baseline=cpu_baseline, key="ex",
+             config={"workload": "ex: one iteration of the example (4->16->4, leaky ReLU, 16 float2 samples, fp16 TrainingOptimal "
+                                 "gradients): learnGradient + Adam update read from those gradients, three kernels", "batch": n,
+                     "layers": dims, "launches_per_step": 3})
+    w["graph"] = True
+    w["launch_floor_us"] = 3 * 1.6      # three graph nodes; an empty kernel costs 1.6 us per node of a HIP graph on MI355X
+    return w
+
+
 def workload_op(torch, cv, steps, warmup):
     """stand-alone coopVecOuterProductAccumulate 64x64 over 2^20 vector pairs, fp32 TrainingOptimal destination."""
     from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML
@@ -528,11 +625,11 @@ def workload_rs(torch, cv, steps, warmup):
                         "batch": B, "n": N}, cpu_baseline=cpu_baseline, key="rs")
 
 
-WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2b": workload_c2b, "c3": workload_c3, "c4": workload_c4,
-             "c4n": workload_c4n, "c5": workload_c5, "c5f": workload_c5f, "op": workload_op, "rs": workload_rs,
+WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": workload_c2b, "c3": workload_c3, "c3c": workload_c3c, "c4": workload_c4,
+             "c4n": workload_c4n, "c5": workload_c5, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2b", "c3", "c4", "c4h", "c4n", "c5f", "c5", "op", "rs")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "ex", "op", "rs")
 HEADLINE = "c2"
 
 
@@ -597,7 +694,7 @@ def measure(torch, w, steps, warmup, with_cpu, ramp_ms=0.0):
         achieved, peak, unit = hbm, HBM_PEAK_GBS, "GB/s"
     else:
         achieved, peak, unit = tflops, mfma_peak, "TFLOP/s"
-    traffic = PROFILED_TRAFFIC.get(w["key"])
+    traffic = profiled_traffic().get(w["key"])
     roofline = {"bound": w["bound"], "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak,
                 "traffic": traffic[0] if traffic else None,
                 "traffic_source": (traffic[1] + " (rocprofv3 --pmc, not measured by this run)") if traffic else None,
@@ -605,6 +702,14 @@ def measure(torch, w, steps, warmup, with_cpu, ramp_ms=0.0):
                 "alg_bytes_per_launch": w["alg_bytes"], "alg_flops_per_launch": w["alg_flops"],
                 "hbm_GBps": hbm, "hbm_frac": hbm / HBM_PEAK_GBS,
                 "mfma_TFLOPs": tflops, "mfma_peak_TFLOPs": mfma_peak, "mfma_frac": tflops / mfma_peak}
+    if w.get("launch_floor_us"):
+        # launch-bound workloads: the time of a step against what its graph nodes cost when they are empty kernels
+        roofline["launch_floor_us"] = w["launch_floor_us"]
+        roofline["launch_floor_frac"] = w["launch_floor_us"] / (kern_ms * 1e3)
+    if w.get("issue_bound"):
+        roofline["issue_bound_ms"] = w["issue_bound"]["ms"]
+        roofline["issue_bound_model"] = w["issue_bound"]["model"]
+        roofline["issue_bound_frac"] = w["issue_bound"]["ms"] / kern_ms
     return {"value": w["samples"] / (wall_ms * 1e-3), "unit": "samples/s", "ms_per_step": wall_ms, "dtype": w["dtype"],
             "config": w["config"], "roofline": roofline,
             "cpu_baseline": w["cpu_baseline"]() if with_cpu else None, "extra": extra}

@@ -86,7 +86,9 @@ typedef enum CvRhiComponentType {
 } CvRhiComponentType;
 
 /* Activation fused behind a matMulAdd.  RELU is max(z, 0) as the neural module defines it
- * (source/standard-modules/neural/activations.slang:25-42); LEAKY_RELU is the example's
+ * (source/standard-modules/neural/activations.slang:25-42); the kernels evaluate it with the packed fp16
+ * maximum, which returns 0 for a NaN z (the scalar definition keeps the NaN): NaN results of a fused RELU,
+ * in cvMatMul and in the fused networks alike, are outside the parity claim; LEAKY_RELU is the example's
  * max(z, z * slope) evaluated in half (examples/mlp-training-coopvec/fflayer.slang:64-65). */
 typedef enum CvActivation {
     CV_ACT_NONE = 0, CV_ACT_RELU = 1, CV_ACT_LEAKY_RELU = 2,
@@ -274,7 +276,8 @@ CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStrid
  * (hlsl.meta.slang:32115-32229) -- also take SINT8/16/32/64 and UINT8/16/32/64 (two's complement, wrapping; the
  * quotients C leaves undefined are x / 0 = 0 and MIN / -1 = MIN) and FLOAT64, which takes STEP and FMA as well.
  * Operands an operator does not take are ignored (may be NULL).  `param` is the
- * slope of CV_OP_LEAKY_RELU.  In-place use (out == a) is allowed. */
+ * slope of CV_OP_LEAKY_RELU and the scalar of CV_OP_SCALE (converted to the element type first).  FLOAT16 fma is
+ * rounded once from the exact a*b + c.  In-place use (out == a) is allowed. */
 typedef enum CvElementwiseOp {
     CV_OP_ADD = 0, CV_OP_SUB = 1, CV_OP_MUL = 2, CV_OP_DIV = 3, CV_OP_NEG = 4,
     CV_OP_MIN = 5, CV_OP_MAX = 6, CV_OP_CLAMP = 7 /* clamp(a, b, c) */, CV_OP_STEP = 8 /* step(edge = a, x = b) */,
@@ -282,7 +285,8 @@ typedef enum CvElementwiseOp {
     CV_OP_TANH = 15, CV_OP_ATAN = 16, CV_OP_FMA = 17 /* a*b + c */,
     CV_OP_RELU = 18, CV_OP_LEAKY_RELU = 19 /* a < 0 ? param*a : a */, CV_OP_SIGMOID = 20, CV_OP_SILU = 21,
     CV_OP_QUICK_GELU = 22,
-    CV_OP_COUNT = 23
+    CV_OP_SCALE = 23 /* a * T(param): vector times scalar, hlsl.meta.slang:32004, :32038 */,
+    CV_OP_COUNT = 24
 } CvElementwiseOp;
 
 CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int32_t n, uint32_t batch,
@@ -404,6 +408,9 @@ typedef struct CvMlpDesc {
     int32_t  gradType;          /* FLOAT16 or FLOAT32: element type of weightsGrad/biasesGrad */
     uint32_t flags;             /* CV_FLAG_* */
     int32_t  inputEncoding;     /* CvInputEncoding */
+    float*   lossMax;           /* device, optional (NULL: not wanted): cvMlpTrainStep overwrites it with max_s loss_s, the
+                                   figure the example's learnGradient leaves in its loss buffer (WaveActiveMax + atomic max
+                                   over a cleared buffer, kernels.slang:21-26) */
 } CvMlpDesc;
 
 /* y = layer_{n-1}( ... layer_0(x) ): every layer is coopVecMatMulAdd + activation with
@@ -420,7 +427,11 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp,
  * sum_s dY (x) X into every layer's weightsGrad and sum_s dY into biasesGrad ("+=").
  * targets == NULL selects target = sin(sum of the sample's inputs) for every output (with
  * inputEncoding CV_ENCODE_XY_SQUARES: the example's groundtruth(x, y)).
- * lossSum (device, optional, one float) is overwritten with sum_s loss_s. */
+ * lossSum (device, optional, one float) is overwritten with sum_s loss_s; mlp->lossMax, if set, with max_s loss_s.
+ * The fused kernel for 64-wide networks runs pairs of waves that wait for each other with a bounded spin; should such a
+ * wait ever time out (only a defect of the kernel could cause that), the step is void: lossSum, lossMax and every
+ * gradient sum the step adds are NaN, whether or not the loss outputs are requested.  A NaN loss for any other reason
+ * (NaN samples) has the same effect. */
 CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes);
 CV_API CvResult cvMlpTrainStep(void* stream, const CvMlpDesc* mlp,
                                const void* input, size_t inputStride,
@@ -505,6 +516,17 @@ CV_API CvResult cvNeuralMlpTrainStep(void* stream, const CvNeuralNetworkDesc* ne
  * The example's constants: beta1 0.9, beta2 0.999, epsilon 1e-7, learningRate 0.01. */
 CV_API CvResult cvAdamStep(void* stream, void* states, void* params, void* gradients, uint32_t count,
                            float beta1, float beta2, float epsilon, float learningRate);
+
+/* The same update for every parameter of a network in one launch, read straight from the gradient buffers
+ * cvMlpTrainStep fills: it replaces convertCooperativeVectorMatrix (TrainingOptimal -> RowMajor,
+ * mlp-training-coopvec.cpp:203-236) + adjustParameters (:238-250) of the example's iteration, and the clear of the
+ * gradient segment at the top of the next one (:183-188), since every gradient element it reads is left at zero.
+ * Layer l: `weights` (FLOAT16, any layout, updated in place), `weightsGrad` (gradType FLOAT16 or FLOAT32, any layout; an
+ * FLOAT32 sum is rounded to half first), `biases` / `biasesGrad` (or both NULL).  weightStates[l] holds one AdamState per
+ * weight in row-major order [outputSize][inputSize], biasStates[l] one per bias.  Results equal
+ * cvConvertMatrices + cvAdamStep bit for bit. */
+CV_API CvResult cvMlpAdamStep(void* stream, const CvMlpDesc* mlp, void* const* weightStates, void* const* biasStates,
+                              float beta1, float beta2, float epsilon, float learningRate);
 
 #ifdef __cplusplus
 }

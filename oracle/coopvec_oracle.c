@@ -940,10 +940,25 @@ static double ew_load(const void* p, int ct, size_t i)
     return (double)cvo_f16_to_f32(((const uint16_t*)p)[i]);
 }
 
+/* double -> half in one rounding: a float that is truncated towards zero with its last bit set whenever anything
+ * was cut off (round to odd) carries enough to round to the 11 bits of a half exactly once */
+static uint16_t ew_f64_to_f16(double v)
+{
+    float f = (float)v;
+    if ((double)f != v && f == f && f - f == 0.0f) {
+        uint32_t u;
+        memcpy(&u, &f, 4);
+        if (fabs((double)f) > fabs(v)) u -= 1u;
+        u |= 1u;
+        memcpy(&f, &u, 4);
+    }
+    return cvo_f32_to_f16_rne(f);
+}
+
 static void ew_store(void* p, int ct, size_t i, double v)
 {
     if (ct == CVO_FLOAT32) ((float*)p)[i] = (float)v;
-    else ((uint16_t*)p)[i] = cvo_f32_to_f16_rne((float)v);
+    else ((uint16_t*)p)[i] = ew_f64_to_f16(v);
 }
 
 static double ew_sigmoid(double x)
@@ -995,6 +1010,8 @@ int cvo_elementwise(int op, int ct, size_t count, const void* a, const void* b, 
         case CVO_OP_SIGMOID: r = ew_sigmoid(x); break;
         case CVO_OP_SILU: r = x * ew_sigmoid(x); break;                 /* :186-193 */
         case CVO_OP_QUICK_GELU: r = x * ew_sigmoid(1.702 * x); break;   /* :215-223 */
+        case CVO_OP_SCALE:                                              /* hlsl.meta.slang:32004: vector * T(scalar) */
+            r = x * (ct == CVO_FLOAT16 ? (double)cvo_f16_to_f32(cvo_f32_to_f16_rne(param)) : (double)param); break;
         }
         ew_store(out, ct, i, r);
     }
@@ -1044,6 +1061,7 @@ int cvo_elementwise_backward(int op, int ct, size_t count, const void* a, const 
         case CVO_OP_SIGMOID: { const double sg = ew_sigmoid(x); dx = sg * (1 - sg) * g; break; }
         case CVO_OP_SILU: { const double sg = ew_sigmoid(x); dx = (sg + x * sg * (1 - sg)) * g; break; }
         case CVO_OP_QUICK_GELU: { const double sg = ew_sigmoid(1.702 * x); dx = (sg + 1.702 * x * sg * (1 - sg)) * g; break; }
+        case CVO_OP_SCALE: dx = (ct == CVO_FLOAT16 ? (double)cvo_f16_to_f32(cvo_f32_to_f16_rne(param)) : (double)param) * g; break;
         }
         if (dA) ew_store(dA, ct, i, dx);
         if (dB && n >= 2) ew_store(dB, ct, i, dy);

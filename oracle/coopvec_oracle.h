@@ -184,7 +184,7 @@ void cvo_slang_adam_step_nudged(CvoAdamState* states, uint16_t* params, uint16_t
 enum {
     CVO_OP_ADD = 0, CVO_OP_SUB, CVO_OP_MUL, CVO_OP_DIV, CVO_OP_NEG, CVO_OP_MIN, CVO_OP_MAX, CVO_OP_CLAMP, CVO_OP_STEP,
     CVO_OP_SIN, CVO_OP_COS, CVO_OP_EXP, CVO_OP_LOG, CVO_OP_LOG2, CVO_OP_EXP2, CVO_OP_TANH, CVO_OP_ATAN, CVO_OP_FMA,
-    CVO_OP_RELU, CVO_OP_LEAKY_RELU, CVO_OP_SIGMOID, CVO_OP_SILU, CVO_OP_QUICK_GELU, CVO_OP_COUNT
+    CVO_OP_RELU, CVO_OP_LEAKY_RELU, CVO_OP_SIGMOID, CVO_OP_SILU, CVO_OP_QUICK_GELU, CVO_OP_SCALE, CVO_OP_COUNT
 };
 /* out[i] = op(a[i], b[i], c[i]) over `count` elements of type ct (FLOAT16 or FLOAT32), evaluated in
  * double and rounded once: the per-component functions of CoopVec<T,N> (hlsl.meta.slang:32043-32421)

@@ -75,7 +75,8 @@ class CvMlpDesc(ctypes.Structure):
     _fields_ = [("layers", ctypes.POINTER(CvMlpLayer)), ("numLayers", ctypes.c_int32),
                 ("inputType", ctypes.c_int32), ("weightType", ctypes.c_int32),
                 ("biasType", ctypes.c_int32), ("outputType", ctypes.c_int32),
-                ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32), ("inputEncoding", ctypes.c_int32)]
+                ("gradType", ctypes.c_int32), ("flags", ctypes.c_uint32), ("inputEncoding", ctypes.c_int32),
+                ("lossMax", ctypes.c_void_p)]
 
 
 PERMUTO_MAX_DIMS, PERMUTO_MAX_LEVELS = 8, 16
@@ -173,6 +174,9 @@ SIGNATURES = {
                                                ctypes.c_uint32, ctypes.c_void_p]),
     "cvAdamStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint32,
                                     ctypes.c_float, ctypes.c_float, ctypes.c_float, ctypes.c_float]),
+    "cvMlpAdamStep": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.POINTER(ctypes.c_void_p),
+                                       ctypes.POINTER(ctypes.c_void_p), ctypes.c_float, ctypes.c_float, ctypes.c_float,
+                                       ctypes.c_float]),
 }
 
 

@@ -133,6 +133,7 @@ class ElementwiseOp(enum.IntEnum):
     Sigmoid = 20
     SiLU = 21
     QuickGELU = 22
+    Scale = 23      # vector * scalar (hlsl.meta.slang:32004): a * T(param)
 
 
 # SlangResult values (include/slang.h:1400-1464)
@@ -677,15 +678,22 @@ def mlpTrainStepWorkspaceSize(layers: Sequence[FeedForwardLayer], batch: int,
 def mlpTrainStep(layers: Sequence[FeedForwardLayer], input: torch.Tensor, targets: Optional[torch.Tensor] = None, *,
                  lossScale: float = 1.0, gradType: int = CoopVecComponentType.Float32,
                  workspace: Optional[torch.Tensor] = None, lossSum: Optional[torch.Tensor] = None,
-                 inputEncoding: int = 0, flags: int = 0, weightType: int = CoopVecComponentType.Float16, stream=None):
+                 inputEncoding: int = 0, flags: int = 0, weightType: int = CoopVecComponentType.Float16,
+                 lossMax: Optional[torch.Tensor] = None, stream=None):
     """learnGradient over a batch (kernels.slang:9-27): forward, bwd_diff of the squared-error loss,
     weight gradients accumulated into every layer's weightsGrad (coopVecOuterProductAccumulate,
     fflayer.slang:35-41) and bias gradients into biasesGrad (coopVecReduceSumAccumulate, :44),
     deterministically.  Returns (workspace, lossSum) so that both can be reused.  weightType Float32: a network
-    of float (vectors, targets, parameters), stepped layer by layer with Float32 gradients."""
+    of float (vectors, targets, parameters), stepped layer by layer with Float32 gradients.  lossMax (one float32 on
+    the device) receives the largest per-sample loss, the figure learnGradient leaves in its loss buffer
+    (kernels.slang:21-26)."""
     _, inStride = _vector_info(input, weightType, "input")
     batch = input.shape[0]
     d, keep = _mlp_desc(layers, weightType, gradType, flags, inputEncoding)
+    if lossMax is not None:
+        if lossMax.dtype != torch.float32 or lossMax.numel() < 1:
+            raise CoopVecError(SLANG_E_INVALID_ARG, "lossMax must be a float32 tensor")
+        d.lossMax = lossMax.data_ptr()
     lib = _lib.load()
     if workspace is None:
         need = ctypes.c_size_t(0)
@@ -889,3 +897,19 @@ def adjustParameters(adamStates: torch.Tensor, params: torch.Tensor, gradients: 
     _check(_lib.load().cvAdamStep(_stream_handle(stream), _buffer_ptr(adamStates, "adamStates"),
                                   _buffer_ptr(params, "params"), _buffer_ptr(gradients, "gradients"), int(count),
                                   beta1, beta2, epsilon, learningRate))
+
+
+def mlpAdjustParameters(layers: Sequence[FeedForwardLayer], weightStates: Sequence[torch.Tensor],
+                        biasStates: Optional[Sequence[Optional[torch.Tensor]]] = None, *,
+                        gradType: int = CoopVecComponentType.Float16, beta1: float = 0.9, beta2: float = 0.999,
+                        epsilon: float = 1e-7, learningRate: float = 0.01, stream=None) -> None:
+    """adjustParameters for a whole network in one launch, straight from the gradient buffers mlpTrainStep fills (any
+    layout, TrainingOptimal included): what the example does with convertCooperativeVectorMatrix + adjustParameters
+    (mlp-training-coopvec.cpp:203-250).  Every gradient element read is left at zero.  weightStates[l] / biasStates[l]:
+    raw bytes, 8 per parameter, weights in row-major order."""
+    d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, gradType, 0)
+    n = len(layers)
+    ws = (ctypes.c_void_p * n)(*[_buffer_ptr(t, "weightStates") for t in weightStates])
+    bs = (ctypes.c_void_p * n)(*[(_buffer_ptr(t, "biasStates") if t is not None else None)
+                                 for t in (biasStates if biasStates is not None else [None] * n)])
+    _check(_lib.load().cvMlpAdamStep(_stream_handle(stream), ctypes.byref(d), ws, bs, beta1, beta2, epsilon, learningRate))

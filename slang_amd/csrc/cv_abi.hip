@@ -742,8 +742,8 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     const bool encoded = mlp->inputEncoding == CV_ENCODE_XY_SQUARES;
     const size_t inAlignTo = encoded ? 4 : vEsz, sampleBytes = encoded ? 2 * sizeof(float) : (size_t)mlp->layers[0].inputSize * vEsz;
     if ((uintptr_t)input % inAlignTo || inputStride % inAlignTo || (uintptr_t)targets % vEsz || targetStride % vEsz ||
-        (uintptr_t)workspace % 16 || (uintptr_t)lossSum % 4)
-        return fail(CV_E_INVALID_ARG, "%s: misaligned input/targets/workspace/lossSum", who);
+        (uintptr_t)workspace % 16 || (uintptr_t)lossSum % 4 || (uintptr_t)mlp->lossMax % 4)
+        return fail(CV_E_INVALID_ARG, "%s: misaligned input/targets/workspace/lossSum/lossMax", who);
     if (encoded && !targets && mlp->layers[L - 1].outputSize != 4)
         return fail(CV_E_INVALID_ARG, "%s: the example's loss (targets == NULL with CV_ENCODE_XY_SQUARES) needs 4 outputs", who);
     if (batch > 1 && (inputStride < sampleBytes ||
@@ -781,6 +781,7 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     t.gradCt = mlp->gradType;
     t.carrierCt = f32net ? CV_FLOAT32 : CV_FLOAT16;
     t.lossSum = lossSum;
+    t.lossMax = mlp->lossMax;
     t.workspace = (float*)workspace;
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;

@@ -8,6 +8,9 @@
 // Pure streaming: 12 bytes read and written per parameter.
 #include <hip/hip_runtime.h>
 
+#include <string.h>
+
+#include "coopvec.h"
 #include "cv_device.h"
 #include "cv_error.h"
 
@@ -18,15 +21,14 @@ struct AdamState { half_t mean, variance; int32_t iteration; };   // adam.slang:
 
 __device__ __forceinline__ half_t H(float x) { return (half_t)x; }
 
-__global__ __launch_bounds__(256) void adamKernel(AdamState* states, half_t* params, half_t* grads, uint32_t count,
-                                                  float beta1f, float beta2f, float epsf, float lrf)
+struct AdamConstants { float beta1, beta2, eps, lr; };
+
+// AdamOptimizer::step (adam.slang:20-36) behind the guards of adjustParameters (kernels.slang:39-43) for one
+// parameter; returns false when the gradient is NaN (the update is skipped; the caller clears the gradient either way)
+__device__ __forceinline__ bool adamUpdate(AdamState& st, half_t& param, float g, const AdamConstants& k)
 {
-    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
-    if (tid >= count) return;
-    float g = (float)grads[tid];
-    if (g != g) { grads[tid] = (half_t)0; return; }
-    const float beta1 = (float)H(beta1f), beta2 = (float)H(beta2f), eps = (float)H(epsf), lr = (float)H(lrf);
-    AdamState st = states[tid];
+    if (g != g) return false;
+    const float beta1 = (float)H(k.beta1), beta2 = (float)H(k.beta2), eps = (float)H(k.eps), lr = (float)H(k.lr);
     st.iteration++;
     if (__builtin_isinf(g)) g = g > 0 ? (float)H(10000.0f) : (float)H(-10000.0f);
     float mean = (float)st.mean, var = (float)st.variance;
@@ -37,11 +39,77 @@ __global__ __launch_bounds__(256) void adamKernel(AdamState* states, half_t* par
     const float meanHat = (float)H(mean / (float)H(1.0f - (float)H(powf(beta1, it))));
     const float varHat = (float)H(var / (float)H(1.0f - (float)H(powf(beta2, it))));
     const float denom = (float)H(sqrtf((float)H(fmaxf(0.0f, varHat) + eps)));
-    params[tid] = H((float)params[tid] - (float)H((float)H(lr * meanHat) / denom));
+    param = H((float)param - (float)H((float)H(lr * meanHat) / denom));
     st.mean = H(mean);
     st.variance = H(var);
-    states[tid] = st;
+    return true;
+}
+
+__global__ __launch_bounds__(256) void adamKernel(AdamState* states, half_t* params, half_t* grads, uint32_t count,
+                                                  AdamConstants k)
+{
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    if (tid >= count) return;
+    AdamState st = states[tid];
+    half_t p = params[tid];
+    if (adamUpdate(st, p, (float)grads[tid], k)) {
+        params[tid] = p;
+        states[tid] = st;
+    }
     grads[tid] = (half_t)0;
+}
+
+// The same update for a whole network, read straight from the gradient buffers the training step fills: the example
+// first copies every weight gradient from its TrainingOptimal buffer to a row-major one
+// (mlp-training-coopvec.cpp:203-236) and clears the TrainingOptimal segment at the top of the next iteration
+// (:183-188); here a thread finds its gradient element through the layout's index map and leaves a zero behind.
+struct AdamLayer {
+    uint8_t* weights; uint8_t* wGrad; AdamState* wStates;
+    half_t* biases; uint8_t* bGrad; AdamState* bStates;
+    MatrixShape wShape, gShape;
+    uint32_t first;          // index of the layer's first element among all threads' elements
+    uint32_t weightCount, biasCount;
+};
+constexpr int kMaxAdamLayers = 8;
+struct AdamLayersArgs {
+    AdamLayer layers[kMaxAdamLayers];
+    int32_t numLayers;
+    int32_t gradCt;          // kF16 or kF32
+    uint32_t total;
+    AdamConstants k;
+};
+
+__global__ __launch_bounds__(256) void adamLayersKernel(const AdamLayersArgs a)
+{
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    if (tid >= a.total) return;
+    int l = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxAdamLayers; ++i)
+        if (i < a.numLayers && tid >= a.layers[i].first) l = i;
+    const AdamLayer& ly = a.layers[l];
+    const uint32_t e = tid - ly.first;
+    half_t* param; uint8_t* grad; AdamState* state;
+    if (e < ly.weightCount) {
+        const uint32_t o = e / ly.wShape.cols, i = e - o * ly.wShape.cols;
+        param = (half_t*)(ly.weights + elemOffset(ly.wShape, o, i));
+        grad = ly.wGrad + elemOffset(ly.gShape, o, i);
+        state = ly.wStates + e;
+    } else {
+        const uint32_t o = e - ly.weightCount;
+        param = ly.biases + o;
+        grad = ly.bGrad + (size_t)o * (a.gradCt == kF32 ? 4u : 2u);
+        state = ly.bStates + o;
+    }
+    // an fp32 gradient buffer holds the sum the half buffer of the example would have held unrounded: rounded here
+    const float g = a.gradCt == kF32 ? (float)H(*(const float*)grad) : (float)*(const half_t*)grad;
+    AdamState st = *state;
+    half_t p = *param;
+    if (adamUpdate(st, p, g, a.k)) {
+        *param = p;
+        *state = st;
+    }
+    if (a.gradCt == kF32) *(float*)grad = 0.f; else *(half_t*)grad = (half_t)0;
 }
 
 } // namespace
@@ -56,9 +124,62 @@ extern "C" CV_API CvResult cvAdamStep(void* stream, void* states, void* params, 
         return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: misaligned argument");
     cv::noteKernel(false, "adamKernel");
     hipLaunchKernelGGL(cv::adamKernel, dim3((count + 255) / 256), dim3(256), 0, (hipStream_t)stream,
-                       (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count, beta1, beta2,
-                       epsilon, learningRate);
+                       (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count,
+                       cv::AdamConstants{beta1, beta2, epsilon, learningRate});
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return cv::failWith(CV_E_INTERNAL_FAIL, "cvAdamStep launch: %s", hipGetErrorString(e));
+    return CV_OK;
+}
+
+extern "C" CV_API CvResult cvMlpAdamStep(void* stream, const CvMlpDesc* mlp, void* const* weightStates, void* const* biasStates,
+                                         float beta1, float beta2, float epsilon, float learningRate)
+{
+    using namespace cv;
+    const char* who = "cvMlpAdamStep";
+    if (!mlp || !mlp->layers || !weightStates) return failWith(CV_E_INVALID_ARG, "%s: null argument", who);
+    if (mlp->numLayers < 1 || mlp->numLayers > kMaxAdamLayers)
+        return failWith(CV_E_INVALID_ARG, "%s: numLayers=%d (1..%d)", who, mlp->numLayers, kMaxAdamLayers);
+    if (mlp->weightType != CV_FLOAT16 || mlp->biasType != CV_FLOAT16)
+        return failWith(CV_E_NOT_AVAILABLE, "%s: the optimizer's arithmetic is half (adam.slang:3): FLOAT16 parameters only", who);
+    if (mlp->gradType != CV_FLOAT16 && mlp->gradType != CV_FLOAT32)
+        return failWith(CV_E_NOT_AVAILABLE, "%s: gradType %d (FLOAT16 or FLOAT32)", who, mlp->gradType);
+    AdamLayersArgs a;
+    memset(&a, 0, sizeof(a));
+    a.numLayers = mlp->numLayers; a.gradCt = mlp->gradType;
+    a.k = AdamConstants{beta1, beta2, epsilon, learningRate};
+    const uint32_t gEsz = elemSize(mlp->gradType);
+    uint64_t total = 0;
+    for (int l = 0; l < mlp->numLayers; ++l) {
+        const CvMlpLayer& L = mlp->layers[l];
+        if (L.inputSize <= 0 || L.outputSize <= 0) return failWith(CV_E_INVALID_ARG, "%s: layer %d is %dx%d", who, l, L.outputSize, L.inputSize);
+        if (!L.weights || !L.weightsGrad || !weightStates[l])
+            return failWith(CV_E_INVALID_ARG, "%s: layer %d: weights, weightsGrad and weightStates are needed", who, l);
+        if ((L.biases != nullptr) != (L.biasesGrad != nullptr) || (L.biases && (!biasStates || !biasStates[l])))
+            return failWith(CV_E_INVALID_ARG, "%s: layer %d: biases, biasesGrad and biasStates go together", who, l);
+        AdamLayer& o = a.layers[l];
+        const bool wOpt = L.weightLayout == CV_LAYOUT_INFERENCING_OPTIMAL || L.weightLayout == CV_LAYOUT_TRAINING_OPTIMAL;
+        const bool gOpt = L.gradLayout == CV_LAYOUT_INFERENCING_OPTIMAL || L.gradLayout == CV_LAYOUT_TRAINING_OPTIMAL;
+        o.wShape = MatrixShape{(uint32_t)L.outputSize, (uint32_t)L.inputSize, CV_FLOAT16, L.weightLayout, wOpt ? 0 : (size_t)L.weightStride};
+        o.gShape = MatrixShape{(uint32_t)L.outputSize, (uint32_t)L.inputSize, mlp->gradType, L.gradLayout, gOpt ? 0 : (size_t)L.gradStride};
+        if (L.weightLayout < 0 || L.weightLayout > 3 || L.gradLayout < 0 || L.gradLayout > 3 || matrixSize(o.wShape) == 0 || matrixSize(o.gShape) == 0)
+            return failWith(CV_E_INVALID_ARG, "%s: layer %d: layout/stride of the weights or of their gradient", who, l);
+        if ((uintptr_t)L.weights % 2 || (uintptr_t)L.weightsGrad % gEsz || (uintptr_t)weightStates[l] % 4 ||
+            (!wOpt && L.weightStride % 2) || (!gOpt && L.gradStride % gEsz) || (uintptr_t)L.biases % 2 || (uintptr_t)L.biasesGrad % gEsz ||
+            (L.biases && (uintptr_t)biasStates[l] % 4))
+            return failWith(CV_E_INVALID_ARG, "%s: layer %d: misaligned argument", who, l);
+        o.weights = (uint8_t*)const_cast<void*>(L.weights); o.wGrad = (uint8_t*)L.weightsGrad; o.wStates = (AdamState*)weightStates[l];
+        o.biases = (half_t*)const_cast<void*>(L.biases); o.bGrad = (uint8_t*)L.biasesGrad;
+        o.bStates = L.biases ? (AdamState*)biasStates[l] : nullptr;
+        o.first = (uint32_t)total;
+        o.weightCount = (uint32_t)L.outputSize * (uint32_t)L.inputSize;
+        o.biasCount = L.biases ? (uint32_t)L.outputSize : 0u;
+        total += (uint64_t)o.weightCount + o.biasCount;
+        if (total > 0xffffffffull) return failWith(CV_E_NOT_AVAILABLE, "%s: more than 2^32 parameters", who);
+    }
+    a.total = (uint32_t)total;
+    noteKernel(false, "adamLayersKernel<%d layers>", mlp->numLayers);
+    hipLaunchKernelGGL(adamLayersKernel, dim3((a.total + 255) / 256), dim3(256), 0, (hipStream_t)stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "%s launch: %s", who, hipGetErrorString(e));
     return CV_OK;
 }

@@ -29,7 +29,7 @@ struct EwArgs {
 
 enum : int {
     kOpAdd = 0, kOpSub, kOpMul, kOpDiv, kOpNeg, kOpMin, kOpMax, kOpClamp, kOpStep, kOpSin, kOpCos, kOpExp, kOpLog,
-    kOpLog2, kOpExp2, kOpTanh, kOpAtan, kOpFma, kOpRelu, kOpLeakyRelu, kOpSigmoid, kOpSilu, kOpQuickGelu, kOpCount
+    kOpLog2, kOpExp2, kOpTanh, kOpAtan, kOpFma, kOpRelu, kOpLeakyRelu, kOpSigmoid, kOpSilu, kOpQuickGelu, kOpScale, kOpCount
 };
 
 __host__ __device__ inline int operandCount(int op)
@@ -39,6 +39,19 @@ __host__ __device__ inline int operandCount(int op)
     case kOpClamp: case kOpFma: return 3;
     }
     return 1;
+}
+
+// double -> half in one rounding: through a float that keeps a sticky last bit (round to odd)
+__device__ __forceinline__ half_t halfOfDouble(double d)
+{
+    float f = (float)d;
+    const double back = (double)f;
+    if (back != d) {
+        uint32_t u = __builtin_bit_cast(uint32_t, f);
+        if (__builtin_fabs(back) > __builtin_fabs(d)) u -= 1u;      // towards zero
+        f = __builtin_bit_cast(float, u | 1u);
+    }
+    return (half_t)f;
 }
 
 __device__ __forceinline__ float evalOp(int op, float a, float b, float c, float param)
@@ -67,8 +80,22 @@ __device__ __forceinline__ float evalOp(int op, float a, float b, float c, float
     case kOpSigmoid: return smoothActivation(a, kActSigmoid);
     case kOpSilu: return smoothActivation(a, kActSilu);
     case kOpQuickGelu: return smoothActivation(a, kActQuickGelu);
+    case kOpScale: return a * param;                    // vector * scalar, hlsl.meta.slang:32004 (param already of type T)
     }
     return a;
+}
+
+// The result as an element of type T.  A half vector is evaluated in float and rounded once, which is the correctly
+// rounded half result for + - * / (a float holds more than twice the bits of a half plus two); fma is not of that kind
+// (a float result can land on a half tie that the exact value misses), so it is summed exactly in double (exact for
+// half operands whenever the result is finite) and rounded to half once.
+template <typename T>
+__device__ __forceinline__ T evalOpAs(int op, float a, float b, float c, float param)
+{
+    if constexpr (std::is_same<T, half_t>::value) {
+        if (op == kOpFma) return halfOfDouble((double)a * (double)b + (double)c);
+    }
+    return (T)evalOp(op, a, b, c, param);
 }
 
 // d(sigmoid(k x) * x)/dx for k = 1 (SiLU) or 1.702 (QuickGELU): s + k x s (1 - s)
@@ -116,6 +143,7 @@ __device__ __forceinline__ void gradOp(int op, float a, float b, float c, float 
     case kOpSigmoid: { const float s = smoothActivation(a, kActSigmoid); da = s * (1.f - s) * g; break; }
     case kOpSilu: da = gatedSigmoidGrad(a, 1.f) * g; break;
     case kOpQuickGelu: da = gatedSigmoidGrad(a, 1.702f) * g; break;
+    case kOpScale: da = param * g; break;
     }
 }
 
@@ -135,7 +163,7 @@ __global__ __launch_bounds__(256) void elementwiseKernel(const EwArgs e)
         const float b = nOps >= 2 ? ld<T>(e.b + s * e.bStride + off) : 0.f;
         const float c = nOps >= 3 ? ld<T>(e.c + s * e.cStride + off) : 0.f;
         if constexpr (!BACKWARD) {
-            st<T>(e.out + s * e.outStride + off, evalOp(e.op, a, b, c, e.param));
+            *(T*)(e.out + s * e.outStride + off) = evalOpAs<T>(e.op, a, b, c, e.param);
         } else {
             const float g = ld<T>(e.dOut + s * e.dOutStride + off);
             float da, db, dc;
@@ -161,7 +189,7 @@ __global__ __launch_bounds__(256) void elementwiseDenseKernel(const EwArgs e, ui
         if (nOps >= 3) *(u32x4*)vc = *(const u32x4*)(e.c + p * 16u);
 #pragma unroll
         for (int i = 0; i < PER; ++i)
-            vo[i] = (T)evalOp(e.op, (float)va[i], nOps >= 2 ? (float)vb[i] : 0.f, nOps >= 3 ? (float)vc[i] : 0.f, e.param);
+            vo[i] = evalOpAs<T>(e.op, (float)va[i], nOps >= 2 ? (float)vb[i] : 0.f, nOps >= 3 ? (float)vc[i] : 0.f, e.param);
         *(u32x4*)(e.out + p * 16u) = *(const u32x4*)vo;
     }
 }
@@ -254,19 +282,6 @@ __device__ __forceinline__ double stickyDoubleOfInt(uint64_t bits, bool isUnsign
         d = __builtin_ldexp((double)top, sh);
     }
     return neg ? -d : d;
-}
-
-// double -> half in one rounding: through a float that keeps a sticky last bit (round to odd)
-__device__ __forceinline__ half_t halfOfDouble(double d)
-{
-    float f = (float)d;
-    const double back = (double)f;
-    if (back != d) {
-        uint32_t u = __builtin_bit_cast(uint32_t, f);
-        if (__builtin_fabs(back) > __builtin_fabs(d)) u -= 1u;      // towards zero
-        f = __builtin_bit_cast(float, u | 1u);
-    }
-    return (half_t)f;
 }
 
 __global__ __launch_bounds__(256) void vectorCastKernel(const CastArgs e)
@@ -401,7 +416,8 @@ CV_API CvResult cvElementwise(void* stream, int32_t op, int32_t elementType, int
     memset(&e, 0, sizeof(e));
     e.a = (const uint8_t*)a; e.b = (const uint8_t*)b; e.c = (const uint8_t*)c; e.out = (uint8_t*)out;
     e.aStride = aStride; e.bStride = bStride; e.cStride = cStride; e.outStride = outStride;
-    e.op = op; e.n = n; e.batch = batch; e.param = param;
+    e.op = op; e.n = n; e.batch = batch;
+    e.param = (op == kOpScale && elementType == CV_FLOAT16) ? (float)(_Float16)param : param;      // the scalar is of the element type
     const uint64_t total = (uint64_t)batch * (uint32_t)n;
     const size_t row = (size_t)n * esz;
     const bool dense = aStride == row && outStride == row && (nOps < 2 || bStride == row) && (nOps < 3 || cStride == row) &&
@@ -489,7 +505,8 @@ CV_API CvResult cvElementwiseBackward(void* stream, int32_t op, int32_t elementT
     e.dA = (uint8_t*)dA; e.dB = (uint8_t*)dB; e.dC = (uint8_t*)dC;
     e.aStride = aStride; e.bStride = bStride; e.cStride = cStride; e.dOutStride = dOutStride;
     e.dAStride = dAStride; e.dBStride = dBStride; e.dCStride = dCStride;
-    e.op = op; e.n = n; e.batch = batch; e.param = param;
+    e.op = op; e.n = n; e.batch = batch;
+    e.param = (op == kOpScale && elementType == CV_FLOAT16) ? (float)(_Float16)param : param;      // the scalar is of the element type
     const uint64_t total = (uint64_t)batch * (uint32_t)n;
     const uint32_t cap = (uint32_t)currentCUs() * 8u;
     const uint32_t blocks = (uint32_t)((total + 255) / 256 < cap ? (total + 255) / 256 : cap);

@@ -89,6 +89,7 @@ struct TrainLaunch {
     int32_t gradCt;
     int32_t carrierCt;           // kF16, or kF32 for a network of float (layer-by-layer step only)
     float* lossSum;
+    float* lossMax;              // optional: max over the samples of the per-sample loss
     float* workspace;            // partials
 };
 // Bytes of workspace the training step needs for this network on a device with numCUs compute

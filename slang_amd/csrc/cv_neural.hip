@@ -122,6 +122,12 @@ CvResult checkNet(const char* who, const CvNeuralNetworkDesc* n)
     if (n->elementType != CV_FLOAT32 && n->elementType != CV_FLOAT16)
         return failWith(CV_E_NOT_AVAILABLE, "%s: elementType %d (supported: FLOAT32, FLOAT16)", who, n->elementType);
     if (n->order < CV_NEURAL_ORDER_NATIVE || n->order > CV_NEURAL_ORDER_CUDA_MATRIX_B) return failWith(CV_E_INVALID_ARG, "%s: unknown order %d", who, n->order);
+    // the kernels index a layer's elements with 32-bit integers: a layer of 2^31 padded elements or more is refused
+    for (int l = 0; l < n->layerCount; ++l) {
+        const uint64_t pin = ((uint64_t)n->dims[l] + 15u) / 16u * 16u, pout = ((uint64_t)n->dims[l + 1] + 15u) / 16u * 16u;
+        if (pin * pout + pout >= (1ull << 31))
+            return failWith(CV_E_NOT_AVAILABLE, "%s: layer %d (%d -> %d) has 2^31 padded elements or more", who, l, n->dims[l], n->dims[l + 1]);
+    }
     return CV_OK;
 }
 

@@ -39,6 +39,7 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ta.targetStride = t.targetStride;
     ta.lossScale = t.lossScale;
     ta.partials = t.workspace;
+    ta.wantLossMax = t.lossMax ? 1 : 0;
     const uint32_t blocks = (uint32_t)numCUs;      // one resident workgroup per compute unit
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
@@ -78,6 +79,7 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ra.partials = t.workspace;
     ra.numPartials = blocks;
     ra.lossSum = t.lossSum;
+    ra.lossMax = t.lossMax;
     constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
     hipLaunchKernelGGL((mlpTrainReduceKernel<Net>), dim3((total + 63) / 64), dim3(64 * kReduceWaves), 0, stream, ra);
     return hipGetLastError();

@@ -69,7 +69,7 @@ GeneralPlan makePlan(const MlpArgs& a, int numCUs, int carrierCt)
     p.gA = off; off += gBytes;
     p.gB = off; off += gBytes;
     p.lossBlocks = (uint32_t)((batch + kLossSamplesPerBlock - 1) / kLossSamplesPerBlock);
-    p.lossPartials = off; off += alignUp((size_t)p.lossBlocks * sizeof(float));
+    p.lossPartials = off; off += alignUp((size_t)p.lossBlocks * 2 * sizeof(float));      // sums, then maxima
     size_t part = reduceSumWorkspaceBytes((uint32_t)batch, numCUs);
     for (int l = 0; l < L; ++l) {
         const size_t o = outerWorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch, numCUs);
@@ -169,7 +169,8 @@ struct LossArgs {
     int32_t act; float slope;
     float lossScale;
     uint32_t batch;
-    float* partials;
+    float* partials;            // per workgroup: the sum of its samples' losses, and behind all sums the largest one
+    uint32_t numBlocks;
 };
 
 // One thread per sample; a workgroup's squared errors are summed in a fixed order.
@@ -178,7 +179,10 @@ __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
 {
     const T* const y = (const T*)a.y; const T* const z = (const T*)a.z; T* const dzOut = (T*)a.dz;
     __shared__ float red[256];
-    float loss = 0.f;
+    __shared__ uint32_t maxBits;        // the largest per-sample loss as bits (non-negative floats order like integers)
+    if (threadIdx.x == 0) maxBits = 0u;
+    __syncthreads();
+    float loss = 0.f, lossMax = 0.f;
     const uint32_t first = blockIdx.x * kLossSamplesPerBlock;
     for (uint32_t s = first + threadIdx.x; s < min(first + kLossSamplesPerBlock, a.batch); s += 256u) {
         const uint8_t* xin = a.in + (size_t)s * a.inStride;
@@ -199,36 +203,50 @@ __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
             // lane group g adds the partner groups in the order g^1, then the pair sums: (p0+p1)+(p2+p3)
             tgtAll = (float)(T)sinf((part[0] + part[1]) + (part[2] + part[3]));
         }
+        float sampleLoss = 0.f;
         for (int i = 0; i < a.outDim; ++i) {
             const size_t e = (size_t)s * a.outDim + i;
             const float tv = a.targets ? (float)*(const T*)(a.targets + (size_t)s * a.targetStride + sizeof(T) * i)
                                        : (exampleLoss ? (float)gt[i & 3] : tgtAll);
             const T diff = (T)((float)y[e] - tv);
             loss += (float)diff * (float)diff;
+            sampleLoss += (float)diff * (float)diff;
             const T g = (T)(2.0f * (float)diff * a.lossScale);
             dzOut[e] = activationGrad<T>(g, z[e], a.act, a.slope);
         }
+        lossMax = (sampleLoss > lossMax || sampleLoss != sampleLoss) ? sampleLoss : lossMax;
     }
     red[threadIdx.x] = loss;
+    atomicMax(&maxBits, __builtin_bit_cast(uint32_t, lossMax));
     __syncthreads();
     for (int w = 128; w > 0; w >>= 1) {
         if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
         __syncthreads();
     }
-    if (threadIdx.x == 0) a.partials[blockIdx.x] = red[0];
+    if (threadIdx.x == 0) {
+        a.partials[blockIdx.x] = red[0];
+        a.partials[a.numBlocks + blockIdx.x] = __builtin_bit_cast(float, maxBits);
+    }
 }
 
-__global__ __launch_bounds__(64) void lossFinalKernel(const float* partials, uint32_t n, float* lossSum)
+__global__ __launch_bounds__(64) void lossFinalKernel(const float* partials, uint32_t n, float* lossSum, float* lossMax)
 {
     __shared__ float red[64];
+    __shared__ uint32_t maxBits;
+    if (threadIdx.x == 0) maxBits = 0u;
+    __syncthreads();
     float c = 0.f;
-    for (uint32_t i = threadIdx.x; i < n; i += 64u) c += partials[i];
+    for (uint32_t i = threadIdx.x; i < n; i += 64u) {
+        c += partials[i];
+        atomicMax(&maxBits, __builtin_bit_cast(uint32_t, partials[n + i]));
+    }
     red[threadIdx.x] = c;
     __syncthreads();
     if (threadIdx.x == 0) {
         float s = 0.f;
         for (int i = 0; i < 64; ++i) s += red[i];
-        *lossSum = s;
+        if (lossSum) *lossSum = s;
+        if (lossMax) *lossMax = __builtin_bit_cast(float, maxBits);
     }
 }
 
@@ -314,11 +332,12 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
         la.inDim = a.layers[0].in; la.outDim = ly.out; la.inEncoding = a.inEncoding;
         la.act = ly.act; la.slope = ly.slope; la.lossScale = t.lossScale; la.batch = batch;
         la.partials = (float*)(ws + p.lossPartials);
+        la.numBlocks = p.lossBlocks;
         if (f32) hipLaunchKernelGGL(lossGradKernel<float>, dim3(p.lossBlocks), dim3(256), 0, stream, la);
         else hipLaunchKernelGGL(lossGradKernel<half_t>, dim3(p.lossBlocks), dim3(256), 0, stream, la);
         if ((e = hipGetLastError()) != hipSuccess) return e;
-        if (t.lossSum) {
-            hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(64), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum);
+        if (t.lossSum || t.lossMax) {
+            hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(64), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum, t.lossMax);
             if ((e = hipGetLastError()) != hipSuccess) return e;
         }
     }

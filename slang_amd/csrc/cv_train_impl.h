@@ -74,6 +74,7 @@ struct TrainArgs {
     uint64_t targetStride;
     float lossScale;
     float* partials;             // [gridDim.x][partialFloats]
+    int32_t wantLossMax;         // also track the largest per-sample loss (slot 1 behind the loss sum of a partial)
 };
 
 struct TrainReduceArgs {
@@ -87,7 +88,22 @@ struct TrainReduceArgs {
     const float* partials;
     uint32_t numPartials;
     float* lossSum;              // optional
+    float* lossMax;              // optional
 };
+
+// The largest per-sample loss of a workgroup, kept as the bits of a non-negative float (whose order is that of the
+// integers; a NaN compares above everything, so it wins).  A maximum does not depend on the order of its operands: the
+// LDS atomic keeps the result reproducible.
+__device__ __forceinline__ void noteLossMax(uint32_t* ldsMaxBits, float waveLaneMax)
+{
+    float m = waveLaneMax;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const float o = __shfl_xor(m, d, 64);
+        m = (o > m || o != o) ? o : m;
+    }
+    if ((threadIdx.x & 63u) == 0) atomicMax(ldsMaxBits, __builtin_bit_cast(uint32_t, m));
+}
 
 // Gradient multiplier of max(z, zs) with respect to its first operand, per element of a packed
 // fp16 pair: 1 where z wins, 0 where zs wins, 0.5 at a tie (diff.meta.slang:2258-2277).  For the
@@ -166,6 +182,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __shared__ __attribute__((aligned(16))) uint32_t ldsWT[(Net::totalTFrags > 0 ? Net::totalTFrags : 1) * 64 * RAW];
     __shared__ __attribute__((aligned(16))) float ldsB[Net::totalBiasTiles * 16];   // biases as fp32
     __shared__ __attribute__((aligned(16))) float ldsRed[4 * 256];
+    __shared__ uint32_t ldsLossMax;               // the workgroup's largest per-sample loss, as bits
+    if (threadIdx.x == 0) ldsLossMax = 0u;
     // per-wave parking space for the F-orientation copies of every layer's input
     __shared__ __attribute__((aligned(16))) uint32_t ldsXF[4 * Net::totalXTiles * 256];
 
@@ -218,7 +236,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int i = 0; i < Net::totalGradTiles; ++i) accW[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < Net::totalDbTiles; ++i) accB[i] = 0.f;
-    float lossAcc = 0.f;
+    float lossAcc = 0.f, lossMaxAcc = 0.f;
 
     // ---- per-lane constants ----------------------------------------------------------------
     const int in0 = a.layers[0].in;
@@ -482,6 +500,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     tgtAll = (float)(half_t)sinf(sumOverGroups(part));
                 }
                 halfx2 dz[Net::MTL][2];
+                float sampleLoss = 0.f;         // this lane's rows of the sample's loss
 #pragma unroll
                 for (int t = 0; t < Net::MTL; ++t) {
                     const half_t yv[4] = {yS[j][t][0].x, yS[j][t][0].y, yS[j][t][1].x, yS[j][t][1].y};
@@ -496,6 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                                 : (exampleLoss ? (float)gt[row & 3] : tgtAll);
                             const half_t diff = (half_t)((float)yv[r] - tv);
                             lossAcc += (float)diff * (float)diff;
+                            sampleLoss += (float)diff * (float)diff;
                             gv[r] = (half_t)(2.0f * (float)diff * ta.lossScale);
                         }
                     }
@@ -505,6 +525,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     dz[t][1] = applyActGrad<LEAKY>(halfx2{gv[2], gv[3]}, m23, actl, slope2);
                 }
                 packS(dz, Net::MTL, Net::ktOut(L - 1), bS[j]);
+                if (ta.wantLossMax) {       // the sample's rows lie in the four lane groups
+                    const float whole = sumOverGroups(sampleLoss);
+                    lossMaxAcc = (whole > lossMaxAcc || whole != whole) ? whole : lossMaxAcc;
+                }
             }
         }
 
@@ -614,6 +638,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         __syncthreads();
     }
     ldsRed[threadIdx.x] = lossAcc;
+    if (ta.wantLossMax) noteLossMax(&ldsLossMax, lossMaxAcc);
     __syncthreads();
     // the loss: one wave sums the 256 values in a fixed order, four neighbours per lane, then lanes 32 ... 1 places apart
     if (wave == 0) {
@@ -622,7 +647,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int i = 0; i < 4; ++i) s += ldsRed[lane * 4 + i];
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
-        if (lane == 0) part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+        if (lane == 0) {
+            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1] = __builtin_bit_cast(float, ldsLossMax);
+        }
     }
 }
 
@@ -636,8 +664,26 @@ __global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const 
     const uint32_t p = blockIdx.x * 64u + (threadIdx.x & 63u);
     constexpr uint32_t nW = Net::totalGradTiles * 256, nB = Net::totalDbTiles * 16;
     const bool inRange = p < nW + nB + 1;
+    // A workgroup whose loss partial is NaN declares its whole partial void: a wave of the paired kernel that gave up
+    // waiting for its partner has worked on stale tiles and says so there (so does a NaN that came in with the samples).
+    // Then every sum of the step is NaN, whether or not the caller reads the loss.
+    __shared__ uint32_t maxBits;
+    const bool ownsLoss = blockIdx.x == (nW + nB) / 64u;      // the workgroup whose values include the loss
+    if (threadIdx.x == 0) maxBits = 0u;
+    __syncthreads();
+    bool voidStep = false;
+    for (uint32_t b = threadIdx.x; b < ra.numPartials; b += 64u * kReduceWaves) {
+        const float* lossOf = ra.partials + (size_t)b * Net::partialFloats + nW + nB;
+        const float lp = lossOf[0];
+        voidStep = voidStep || lp != lp;
+        if (ra.lossMax && ownsLoss) atomicMax(&maxBits, __builtin_bit_cast(uint32_t, lossOf[1]));
+    }
+    voidStep = __syncthreads_or(voidStep) != 0;
+    if (ra.lossMax && ownsLoss && threadIdx.x == 0)
+        *ra.lossMax = voidStep ? __builtin_nanf("") : __builtin_bit_cast(float, maxBits);
     float s;
     if (!sumPartials(ra.partials + p, Net::partialFloats, ra.numPartials, inRange, red, s) || !inRange) return;
+    if (voidStep) s = __builtin_nanf("");
     if (p == nW + nB) {
         if (ra.lossSum) *ra.lossSum = s;
         return;

@@ -144,15 +144,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int X_DW = 4 * Net::totalXTiles * kPairTileDW;          // per pair: every layer's input of the round
     constexpr int DZ_DW = 4 * 2 * Net::MTMAX * kPairTileDW;           // per pair: two alternating slots for dZ
     constexpr int FLAG_DW = 8;                                        // per wave: the number of its last meeting
-    static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
-    __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW];
+    constexpr int MAX_DW = 4;                                         // the workgroup's largest per-sample loss (one word used)
+    static_assert((W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW + MAX_DW) * 4 <= 160 * 1024, "LDS of one compute unit");
+    __shared__ __attribute__((aligned(16))) uint32_t lds[W_DW + WT_DW + B_DW + X_DW + DZ_DW + FLAG_DW + MAX_DW];
     uint32_t* const ldsW = lds;
     uint32_t* const ldsWT = lds + W_DW;
     float* const ldsB = (float*)(lds + W_DW + WT_DW);
     uint32_t* const ldsX = lds + W_DW + WT_DW + B_DW;
     uint32_t* const ldsDZ = ldsX + X_DW;
     uint32_t* const ldsFlag = ldsDZ + DZ_DW;
-    if (threadIdx.x < FLAG_DW) ldsFlag[threadIdx.x] = 0u;
+    uint32_t* const ldsLossMax = ldsFlag + FLAG_DW;
+    if (threadIdx.x < FLAG_DW + MAX_DW) ldsFlag[threadIdx.x] = 0u;
 
     // ---- stage W, W^T and biases ----------------------------------------------------------------
     // All loads of all layers first, then all stores: one round trip to memory for the whole staging (layer after
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int i = 0; i < Split::totalLoc; ++i) accW[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < Split::totalLocDb; ++i) accB[i] = 0.f;
-    float lossAcc = 0.f;
+    float lossAcc = 0.f, lossMaxAcc = 0.f;
 
     // ---- per-lane constants ----------------------------------------------------------------------
     const int in0 = a.layers[0].in;
@@ -362,6 +364,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         uint32_t bS[Net::KOMAX][FD];                // S fragments of dZ of the current layer
         {
             halfx2 dz[Net::MTL][2];
+            float sampleLoss = 0.f;             // this lane's rows of the sample's loss
 #pragma unroll
             for (int t = 0; t < Net::MTL; ++t) {
                 const half_t yv[4] = {yS[t][0].x, yS[t][0].y, yS[t][1].x, yS[t][1].y};
@@ -380,10 +383,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     // straight-line: rows past the output and samples past the batch compute, then count for nothing
                     const half_t diff = (half_t)((float)yv[rr] - tv);
                     lossAcc += on ? (float)diff * (float)diff : 0.f;
+                    sampleLoss += on ? (float)diff * (float)diff : 0.f;
                     gv[rr] = on ? (half_t)(2.0f * (float)diff * ta.lossScale) : (half_t)0;
                 }
                 dz[t][0] = halfx2{gv[0], gv[1]};       // the last layer has no activation
                 dz[t][1] = halfx2{gv[2], gv[3]};
+            }
+            if (ta.wantLossMax) {       // the sample's rows lie in the four lane groups
+                const float whole = sumOverGroups(sampleLoss);
+                lossMaxAcc = (whole > lossMaxAcc || whole != whole) ? whole : lossMaxAcc;
             }
             packS(dz, Net::MTL, Net::ktOut(L - 1), bS);
         }
@@ -493,7 +501,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 
     // ---- workgroup partial: the four waves of each parity hold the same tiles; summed in a fixed order
-    if (timeouts) lossAcc = __builtin_nanf("");       // a meeting timed out: the step's result is void, and the loss says so
+    // a meeting timed out: the step's result is void; the NaN in the workgroup's loss partial makes the reduction
+    // kernel turn the loss and every gradient sum of the step into NaN
+    if (timeouts) lossAcc = __builtin_nanf("");
+    if (ta.wantLossMax) noteLossMax(ldsLossMax, lossMaxAcc);
     __syncthreads();                              // every pair has left its last round: the X and dZ tiles are free
     // The eight waves put up to ten of their dW tiles at a time into the tile area (X and dZ tiles lie back to back), and all
     // 512 threads sum them: a few rounds of two barriers instead of two barriers per tile (which took 15 us of a 135 us
@@ -558,7 +569,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int i = 0; i < 8; ++i) s += ldsLoss[lane * 8 + i];
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
-        if (lane == 0) part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+        if (lane == 0) {
+            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
+            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1] = __builtin_bit_cast(float, *ldsLossMax);
+        }
     }
 }
 

@@ -9,9 +9,17 @@
 //   RowMajor -> adjustParameters (Adam) -> every 10 iterations read back the loss.
 // What the Slang kernels do per thread is done here by cvMlpTrainStep / cvConvertMatrices /
 // cvAdamStep.  The input encoding (x, y, x^2, y^2) (network.slang:35-38) and the ground truth
-// (network.slang:67-75) are evaluated on the host in half, as the shader would.
+// (network.slang:67-75) are evaluated by the training kernel in half, as the shader would.
 //
-//   mlp_training_host [iterations=1000]
+// Two forms of the iteration, same parameters bit for bit:
+//   --unfused : the example's five steps as listed above (memset, 2 kernels, convert, Adam);
+//   default   : cvMlpTrainStep + cvMlpAdamStep, which reads the TrainingOptimal gradients where they lie and leaves
+//               them at zero, so the convert and the clear go away; the three kernels are recorded once into a HIP
+//               graph and an iteration is one graph launch.
+// The loss printed is the one the example prints: the largest per-sample loss of the iteration (learnGradient's
+// WaveActiveMax + atomic max, kernels.slang:21-26), followed by the mean.
+//
+//   mlp_training_host [iterations=1000] [--unfused] [--time]
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -70,7 +78,13 @@ static uint16_t referenceFloatToHalf(float value)
 
 int main(int argc, char** argv)
 {
-    const int iterations = argc > 1 ? atoi(argv[1]) : 1000;
+    int iterations = 1000;
+    bool unfused = false, timeIt = false;
+    for (int i = 1; i < argc; i++) {
+        if (!strcmp(argv[i], "--unfused")) unfused = true;
+        else if (!strcmp(argv[i], "--time")) timeIt = true;
+        else iterations = atoi(argv[i]);
+    }
 
     // ---- buffer plan: | weights_i bias_i ... | row-major grads ... | training-optimal weight grads |
     std::vector<LayerAllocation> layers(kLayerCount);
@@ -111,7 +125,7 @@ int main(int argc, char** argv)
     // training step converts them to half2, encodes (x, y, x*x, y*y) and evaluates groundtruth(x, y) itself
     uint8_t* params = nullptr;
     void *adamStates = nullptr, *dInputs = nullptr, *workspace = nullptr;
-    float* dLoss = nullptr;
+    float* dLoss = nullptr;      // [0] sum, [1] max of the per-sample losses
     const size_t paramCount = bufferSize / sizeof(NFloat);
     HIP_OK(hipMalloc((void**)&params, bufferSize));
     HIP_OK(hipMemcpy(params, initParams.data(), bufferSize, hipMemcpyHostToDevice));
@@ -119,7 +133,7 @@ int main(int argc, char** argv)
     HIP_OK(hipMemset(adamStates, 0, paramCount * 8));
     HIP_OK(hipMalloc(&dInputs, inputData.size() * sizeof(float)));
     HIP_OK(hipMemcpy(dInputs, inputData.data(), inputData.size() * sizeof(float), hipMemcpyHostToDevice));
-    HIP_OK(hipMalloc((void**)&dLoss, sizeof(float)));
+    HIP_OK(hipMalloc((void**)&dLoss, 2 * sizeof(float)));
     // the gradient segments start from zero (the reference's random fill there would be noise)
     HIP_OK(hipMemset(params + gradientOffset, 0, bufferSize - gradientOffset));
 
@@ -146,13 +160,21 @@ int main(int argc, char** argv)
                                    CV_LAYOUT_ROW_MAJOR, layers[i].weightsSize, layers[i].weightsGradOffset,
                                    (size_t)kLayerSizes[i] * sizeof(NFloat)};
     }
-    CvMlpDesc mlp = {net, kLayerCount, CV_FLOAT32, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_XY_SQUARES};
+    CvMlpDesc mlp = {net, kLayerCount, CV_FLOAT32, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, CV_FLOAT16, 0, CV_ENCODE_XY_SQUARES, dLoss + 1};
     size_t workspaceBytes = 0;
     CV_OK_OR_FAIL(cvMlpTrainStepWorkspaceSize(&mlp, sampleCount, &workspaceBytes));
     HIP_OK(hipMalloc(&workspace, workspaceBytes));
+    // Adam states: one record per element of the parameter buffer, at the element's own index (adjustParameters'
+    // states[tid]); a layer's weights and biases find theirs at their offsets
+    void *weightStates[kLayerCount], *biasStates[kLayerCount];
+    for (int i = 0; i < kLayerCount; i++) {
+        weightStates[i] = (uint8_t*)adamStates + layers[i].weightsOffset / sizeof(NFloat) * 8;
+        biasStates[i] = (uint8_t*)adamStates + layers[i].biasOffset / sizeof(NFloat) * 8;
+    }
 
     hipStream_t stream = nullptr;
-    for (int k = 0; k < iterations; k++) {
+    HIP_OK(hipStreamCreate(&stream));
+    auto unfusedIteration = [&]() -> int {
         HIP_OK(hipMemsetAsync(params + gradientTrainingOffset, 0, bufferSize - gradientTrainingOffset, stream));
         CV_OK_OR_FAIL(cvMlpTrainStep(stream, &mlp, dInputs, 2 * sizeof(float), nullptr, 0, 1.0f, sampleCount, dLoss,
                                      workspace, workspaceBytes));
@@ -160,13 +182,58 @@ int main(int argc, char** argv)
         CV_OK_OR_FAIL(cvAdamStep(stream, adamStates, params, params + gradientOffset,
                                  (uint32_t)((gradientTrainingOffset - gradientOffset) / sizeof(NFloat)), 0.9f, 0.999f,
                                  1e-7f, 0.01f));
-        if ((k + 1) % 10 == 0) {
-            float loss = 0.f;
+        return 0;
+    };
+    auto fusedIteration = [&]() -> int {
+        CV_OK_OR_FAIL(cvMlpTrainStep(stream, &mlp, dInputs, 2 * sizeof(float), nullptr, 0, 1.0f, sampleCount, dLoss,
+                                     workspace, workspaceBytes));
+        CV_OK_OR_FAIL(cvMlpAdamStep(stream, &mlp, weightStates, biasStates, 0.9f, 0.999f, 1e-7f, 0.01f));
+        return 0;
+    };
+    hipGraphExec_t graphExec = nullptr;
+    hipEvent_t t0, t1;
+    HIP_OK(hipEventCreate(&t0));
+    HIP_OK(hipEventCreate(&t1));
+    HIP_OK(hipEventRecord(t0, stream));
+    for (int k = 0; k < iterations; k++) {
+        if (unfused) {
+            if (unfusedIteration()) return 1;
+        } else if (k == 0) {
+            // the first iteration runs as plain launches (the library looks up its kernels' residency once per
+            // device), then the same three kernels are recorded for all later ones
+            if (fusedIteration()) return 1;
+            hipGraph_t graph = nullptr;
+            HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal));
+            if (fusedIteration()) return 1;
+            HIP_OK(hipStreamEndCapture(stream, &graph));
+            HIP_OK(hipGraphInstantiate(&graphExec, graph, nullptr, nullptr, 0));
+            HIP_OK(hipGraphDestroy(graph));
+        } else {
+            HIP_OK(hipGraphLaunch(graphExec, stream));
+        }
+        if ((k + 1) % 10 == 0 && !timeIt) {
+            float loss[2] = {0.f, 0.f};
             HIP_OK(hipStreamSynchronize(stream));
-            HIP_OK(hipMemcpy(&loss, dLoss, sizeof(float), hipMemcpyDeviceToHost));
-            printf("Loss after %d iterations: %f\n", k + 1, loss / sampleCount);
+            HIP_OK(hipMemcpy(loss, dLoss, sizeof(loss), hipMemcpyDeviceToHost));
+            printf("Loss after %d iterations: %f (mean %f)\n", k + 1, loss[1], loss[0] / sampleCount);
         }
     }
+    HIP_OK(hipEventRecord(t1, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    if (timeIt) {
+        float ms = 0.f;
+        HIP_OK(hipEventElapsedTime(&ms, t0, t1));
+        printf("%s iteration: %.2f us (%d iterations)\n", unfused ? "unfused" : "fused, one graph launch per", ms * 1e3f / iterations, iterations);
+    }
+    // a digest of the parameters, so that two runs can be compared bit for bit
+    std::vector<uint16_t> finalParams(gradientOffset / sizeof(NFloat));
+    HIP_OK(hipMemcpy(finalParams.data(), params, gradientOffset, hipMemcpyDeviceToHost));
+    uint64_t digest = 1469598103934665603ull;
+    for (int i = 0; i < kLayerCount; i++) {
+        for (size_t e = 0; e < layers[i].weightsSize / 2; e++) digest = (digest ^ finalParams[layers[i].weightsOffset / 2 + e]) * 1099511628211ull;
+        for (size_t e = 0; e < layers[i].biasSize / 2; e++) digest = (digest ^ finalParams[layers[i].biasOffset / 2 + e]) * 1099511628211ull;
+    }
+    printf("Parameter digest: %016llx\n", (unsigned long long)digest);
     HIP_OK(hipDeviceSynchronize());
     return 0;
 }

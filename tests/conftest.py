@@ -29,17 +29,35 @@ def pytest_collection_modifyitems(config, items):
             item.add_marker(skip)
 
 
-def pytest_sessionfinish(session, exitstatus):
-    """Writes the float-parity statistics of the session (how many compared elements passed only through the
-    summation-order term of the tolerance) to the file COOPVEC_PARITY_STATS_FILE names, if it is set."""
-    path = os.environ.get("COOPVEC_PARITY_STATS_FILE")
-    if not path:
-        return
+def pytest_terminal_summary(terminalreporter, exitstatus, config):
+    """Prints the float-parity statistics of the session: elements compared against the oracle under the bar
+    max(2 ulp, 1e-3 relative, 2^-18 sum|terms|), how many of them passed only through the third (summation-order)
+    term, and per test the outputs of multi-layer networks that lay outside the bar (each one checked to be a
+    rounding-boundary case of a hidden unit).  COOPVEC_PARITY_STATS_FILE, if set, also receives them as JSON."""
     try:
         import json
         import oracle_binding as ob
-        if ob.PARITY_STATS["elements"]:
-            with open(path, "w") as f:
-                json.dump(ob.PARITY_STATS, f)
     except Exception:
-        pass
+        return
+    st = ob.PARITY_STATS
+    if not st["elements"]:
+        return
+    tr = terminalreporter
+    tr.write_sep("-", "float parity statistics")
+    tr.write_line("elements compared with the oracle: %d; inside the bar only through the 2^-18 sum|terms| term: %d"
+                  % (st["elements"], st["passed_only_by_floor_term"]))
+    e2e = st["end_to_end"]
+    if e2e:
+        tr.write_line("multi-layer outputs outside the bar (every one a checked rounding-boundary case), per test:")
+        for name in sorted(e2e):
+            o, t = e2e[name]
+            if o:
+                tr.write_line("  %s: %d of %d" % (name, o, t))
+        tr.write_line("  total: %d of %d" % (sum(o for o, _ in e2e.values()), sum(t for _, t in e2e.values())))
+    path = os.environ.get("COOPVEC_PARITY_STATS_FILE")
+    if path:
+        try:
+            with open(path, "w") as f:
+                json.dump(st, f)
+        except OSError:
+            pass

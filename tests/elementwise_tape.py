@@ -5,7 +5,7 @@ backward(op, dOut, a, b, c, param) on arrays of one element type."""
 from __future__ import annotations
 
 ADD, SUB, MUL, DIV, NEG, MIN, MAX, CLAMP, STEP, SIN, COS, EXP, LOG, LOG2, EXP2, TANH, ATAN, FMA = range(18)
-RELU, LEAKY_RELU, SIGMOID, SILU, QUICK_GELU = range(18, 23)
+RELU, LEAKY_RELU, SIGMOID, SILU, QUICK_GELU, SCALE = range(18, 24)
 N_OPERANDS = {ADD: 2, SUB: 2, MUL: 2, DIV: 2, MIN: 2, MAX: 2, STEP: 2, CLAMP: 3, FMA: 3}
 
 

@@ -227,7 +227,16 @@ def f16_ulp(ref: np.ndarray) -> np.ndarray:
 
 # Elements judged by float_parity_violations in this process: how many, and how many of those were
 # inside the bar only through its third (summation-order) term.  conftest.py writes the totals out.
-PARITY_STATS = {"elements": 0, "passed_only_by_floor_term": 0}
+PARITY_STATS = {"elements": 0, "passed_only_by_floor_term": 0, "end_to_end": {}}
+
+
+def note_end_to_end(outside: int, total: int) -> None:
+    """Records, under the running test's name, how many outputs of a multi-layer network lay outside the bar (each of
+    them shown by the caller to be a rounding-boundary case of a hidden unit)."""
+    import os
+    name = os.environ.get("PYTEST_CURRENT_TEST", "?").split(" ")[0].split("::")[-1]
+    o, t = PARITY_STATS["end_to_end"].get(name, (0, 0))
+    PARITY_STATS["end_to_end"][name] = (o + int(outside), t + int(total))
 
 
 def float_parity_violations(got_f16: np.ndarray, ref_f32: np.ndarray, abs_terms: np.ndarray | None = None,

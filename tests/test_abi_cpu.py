@@ -228,3 +228,20 @@ def test_rhi_component_type_numbering(lib):
     assert lib.cvGetMatrixSize(16, 4, lib.cvComponentTypeFromRhi(0), 0, 0, ctypes.byref(fp16)) == OK
     assert lib.cvGetMatrixSize(16, 4, 0, 0, 0, ctypes.byref(raw0)) == OK
     assert fp16.value == 16 * 4 * 2 and raw0.value == 16 * 4
+
+
+def test_bench_traffic_figures_come_from_the_profile_summaries():
+    # bench.py quotes `roofline.traffic` from lines `traffic[<workload>] = <bytes> B per step` of profiles/*.md:
+    # every workload of the default run that has a summary must be found there, with a plausible figure
+    import importlib.util
+    import os
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_module", os.path.join(repo, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    traffic = bench.profiled_traffic()
+    for key in ("c1", "c2", "c2b", "c3", "c4", "c4h", "c4n", "c5", "op", "rs", "copy"):
+        assert key in traffic, "no traffic[%s] line in profiles/" % key
+        nbytes, path = traffic[key]
+        assert nbytes > 100000 and os.path.exists(os.path.join(repo, path))
+    assert set(bench.DEFAULT_RUN) <= set(bench.WORKLOADS) and bench.HEADLINE in bench.WORKLOADS

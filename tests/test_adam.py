@@ -118,3 +118,58 @@ def test_gpu_adam_matches_oracle():
         # continue from the GPU's state so that differences do not accumulate in the comparison
         p = got.copy(); st = stg.copy()
     assert pow_cases <= n // 100
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("grad_type", ["f16", "f32"])
+def test_network_adam_step_equals_convert_plus_adam(grad_type):
+    # cvMlpAdamStep reads every layer's gradient where the training step left it (TrainingOptimal here) and updates
+    # weights and biases in one launch: same bits as the example's convert (TrainingOptimal -> RowMajor) followed by
+    # adjustParameters over the row-major gradients, over several steps (the states carry over), NaN / inf
+    # gradients included; and it leaves the gradient buffers at zero
+    import torch
+    from slang_amd import coopvec as cv
+    from slang_amd.coopvec import Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML, FeedForwardLayer
+    from slang_amd.coopvec import CooperativeVectorMatrixDesc as D
+    rng = np.random.default_rng(17)
+    dims = [4, 16, 20, 3]
+    gct, gdt, gnp = (CT.Float16, torch.float16, np.float16) if grad_type == "f16" else (CT.Float32, torch.float32, np.float32)
+    dev = "cuda"
+    W = [torch.from_numpy(rng.uniform(-1, 1, (dims[i + 1], dims[i])).astype(np.float16)).to(dev) for i in range(3)]
+    Bv = [torch.from_numpy(rng.uniform(-1, 1, dims[i + 1]).astype(np.float16)).to(dev) for i in range(3)]
+    Bv[1] = None                                   # a layer without biases
+    Wref = [w.clone() for w in W]; Bref = [b.clone() if b is not None else None for b in Bv]
+    wst = [torch.zeros(w.numel() * 8, dtype=torch.uint8, device=dev) for w in W]
+    bst = [torch.zeros(b.numel() * 8, dtype=torch.uint8, device=dev) if b is not None else None for b in Bv]
+    wst_ref = [t.clone() for t in wst]; bst_ref = [t.clone() if t is not None else None for t in bst]
+    sizes = [cv.getCooperativeVectorMatrixSize(dims[i + 1], dims[i], gct, ML.TrainingOptimal) for i in range(3)]
+    for step in range(4):
+        layers, gref = [], []
+        for i in range(3):
+            fo, fi = dims[i + 1], dims[i]
+            g = (rng.standard_normal((fo, fi)) * 10.0 ** rng.integers(-3, 2, (fo, fi))).astype(gnp)
+            g[0, 0] = np.nan; g[1 % fo, 1] = np.inf
+            grow = torch.from_numpy(g).to(dev)
+            gopt = torch.zeros(sizes[i], dtype=torch.uint8, device=dev)
+            esz = grow.element_size()
+            cv.convertCooperativeVectorMatrix(gopt, [D(fo, fi, gct, ML.TrainingOptimal, sizes[i], 0, 0)],
+                                              grow.contiguous().view(torch.uint8).flatten(), [D(fo, fi, gct, ML.RowMajor, fo * fi * esz, 0, fi * esz)])
+            bg = torch.from_numpy((rng.standard_normal(fo) * 0.1).astype(gnp)).to(dev) if Bv[i] is not None else None
+            layers.append(FeedForwardLayer(fi, fo, W[i].view(torch.uint8).flatten(), Bv[i].view(torch.uint8) if Bv[i] is not None else None,
+                                           ML.RowMajor, fi * 2, Activation.ReLU, 0.0, gopt,
+                                           bg.view(torch.uint8) if bg is not None else None, ML.TrainingOptimal, 0))
+            gref.append((grow.to(torch.float16).clone(), bg.to(torch.float16).clone() if bg is not None else None))
+        cv.mlpAdjustParameters(layers, wst, bst, gradType=gct)
+        assert cv.lastKernelName().startswith("adamLayersKernel")
+        for i in range(3):
+            cv.adjustParameters(wst_ref[i], Wref[i].view(-1), gref[i][0].contiguous().view(-1))
+            if Bref[i] is not None:
+                cv.adjustParameters(bst_ref[i], Bref[i], gref[i][1])
+            assert torch.equal(W[i].view(torch.int16), Wref[i].view(torch.int16)), (step, i)
+            assert torch.equal(wst[i], wst_ref[i]), (step, i)
+            if Bv[i] is not None:
+                assert torch.equal(Bv[i].view(torch.int16), Bref[i].view(torch.int16)) and torch.equal(bst[i], bst_ref[i])
+                assert (layers[i].biasesGrad == 0).all()
+            assert (layers[i].weightsGrad == 0).all()
+    with pytest.raises(cv.CoopVecError):
+        cv.mlpAdjustParameters(layers, wst[:2] + [None], bst, gradType=gct)

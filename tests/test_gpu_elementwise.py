@@ -77,7 +77,7 @@ def _close(got, want, dtype):
 def test_every_operator_against_oracle(dtype, shape):
     rng = np.random.default_rng(11 + shape[1])
     B, N = shape
-    for op in range(23):
+    for op in range(24):
         a, b, c = _operands(rng, op, B, N, dtype)
         da, db, dc = [to_dev(v) if v is not None else None for v in (a, b, c)]
         got = cv.elementwise(op, da, db, dc, param=0.1).cpu().numpy()
@@ -95,6 +95,31 @@ def test_every_operator_against_oracle(dtype, shape):
             if dtype == np.float16:      # a product of two rounded factors: one more ulp
                 ok |= np.abs(gg.cpu().numpy().astype(np.float64) - ww.astype(np.float64)) <= 3.0 * ob.f16_ulp(ww.astype(np.float32))
             assert ok.all(), (op, k, dtype)
+
+
+def test_half_fma_is_rounded_once_and_scale_takes_a_scalar_of_the_element_type():
+    # fma on half vectors: a*b = 1.5 + 1.5 ulp exactly (a tie of the half grid), c = -2^-24 pulls the exact sum below the
+    # tie, so the correctly rounded result is the lower neighbour 0x3E01; a float fma lands on the tie (its own tie, to
+    # even) and a second rounding to half would give 0x3E02
+    a = np.full((3, 8), 1.0009765625, np.float16); b = np.full((3, 8), 1.5, np.float16)
+    c = np.full((3, 8), -2.0 ** -24, np.float16)
+    got = cv.elementwise(T.FMA, to_dev(a), to_dev(b), to_dev(c)).cpu().numpy()
+    assert (got.view(np.uint16) == 0x3E01).all(), hex(int(got.view(np.uint16)[0, 0]))
+    assert (ob.elementwise(T.FMA, a, b, c, 0.0).view(np.uint16) == 0x3E01).all()
+    wide = cv.elementwise(T.FMA, to_dev(a[:, :5]), to_dev(b[:, :5]), to_dev(c[:, :5])).cpu().numpy()      # the strided kernel
+    assert (wide.view(np.uint16) == 0x3E01).all()
+    # vector * scalar (hlsl.meta.slang:32004): the scalar is converted to the element type first
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-4, 4, (100, 16)).astype(np.float16)
+    k = 0.3                                   # not a half: half(0.3) = 0.300048828125
+    got = cv.elementwise(T.SCALE, to_dev(x), param=k).cpu().numpy()
+    want = (x.astype(np.float32) * np.float32(np.float16(k))).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    g = rng.uniform(-1, 1, x.shape).astype(np.float16)
+    da, _, _ = cv.elementwiseBackward(T.SCALE, to_dev(g), to_dev(x), param=k)
+    assert np.array_equal(da.cpu().numpy().view(np.uint16), (g.astype(np.float32) * np.float32(np.float16(k))).astype(np.float16).view(np.uint16))
+    xf = x.astype(np.float32)
+    assert np.array_equal(cv.elementwise(T.SCALE, to_dev(xf), param=k).cpu().numpy(), xf * np.float32(k))
 
 
 def test_strided_rows_and_in_place():

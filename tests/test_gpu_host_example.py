@@ -25,4 +25,10 @@ def test_example_training_loop_converges():
     assert last < 0.25 * first, (first, last)
     # bitwise reproducible: the deterministic gradient reduction makes the whole run repeat exactly
     out2 = subprocess.run([BIN, "200"], capture_output=True, text=True, timeout=120)
-    assert out2.stdout.splitlines() == out.stdout.splitlines()[:20]
+    assert out2.stdout.splitlines()[:20] == out.stdout.splitlines()[:20]
+    # the example's five steps per iteration (clear, learnGradient, convert, adjustParameters) arrive at the same
+    # parameters, bit for bit, as the fused iteration replayed from a HIP graph
+    out3 = subprocess.run([BIN, "200", "--unfused"], capture_output=True, text=True, timeout=120)
+    assert out3.returncode == 0, out3.stderr
+    assert out3.stdout.splitlines() == out2.stdout.splitlines()
+    assert out2.stdout.splitlines()[-1].startswith("Parameter digest:")

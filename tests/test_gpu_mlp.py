@@ -115,6 +115,7 @@ def end_to_end_ok(y, specs, x, x_ct, gpu_hidden, floor=2.0 ** -18):
         # and the two sides are neighbours in fp16
         d = np.abs(gpu_hidden[first][s][units].astype(np.float32) - acts[first][s][units].astype(np.float32))
         assert (d <= ob.f16_ulp(acts[first][s][units].astype(np.float32)) * (1.0 if floor <= 2.0 ** -17 else 64.0)).all()
+    ob.note_end_to_end(bad.sum(), bad.size)
     return 1.0 - bad.mean(), bad
 
 

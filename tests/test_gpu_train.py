@@ -126,6 +126,105 @@ def test_train_step_sin_target_in_kernel():
     assert abs(loss.item() - rloss) <= 1e-3 * rloss
 
 
+def gradient_term_sums(specs, x, t):
+    """sum over the batch of |dZ_l[s][i] * X_l[s][j]| (and of |dZ_l[s][i]| for the biases) of a ReLU network with an MSE
+    loss, carriers rounded to half like the kernels': the scale against which an element of a gradient is
+    cancellation-dominated or not."""
+    a = [x.astype(np.float32)]
+    zs = []
+    for s in specs:
+        z = a[-1] @ s["W"].astype(np.float32).T + (s["b"].astype(np.float32) if s["b"] is not None else 0.0)
+        z = z.astype(np.float16).astype(np.float32)
+        zs.append(z)
+        a.append(np.maximum(z, 0) if s["act"] == int(Activation.ReLU) else z)
+    g = (2.0 * (a[-1] - t.astype(np.float32))).astype(np.float16).astype(np.float32)
+    tW, tB = [None] * len(specs), [None] * len(specs)
+    for l in reversed(range(len(specs))):
+        dz = g * (zs[l] > 0) if specs[l]["act"] == int(Activation.ReLU) else g
+        tW[l] = np.abs(dz).T.astype(np.float64) @ np.abs(a[l]).astype(np.float64)
+        tB[l] = np.abs(dz).sum(0).astype(np.float64)
+        g = (dz @ specs[l]["W"].astype(np.float32)).astype(np.float16).astype(np.float32)
+    return tW, tB
+
+
+def test_train_step_gradients_element_by_element():
+    # Per element of every gradient of the training configuration (8 -> 64 x4 -> 1, batch 2^14 here): agreement with
+    # the fp64-accumulating oracle to 2 ulp of fp16 at the element's own magnitude (about 1e-3 relative), or to the
+    # accumulation floor 2^-19 * sum|terms| where that is larger, which is the case only for elements that are
+    # cancellation-dominated (|g| below about 2^-9 * sum|terms|); most elements are held to the first term.
+    rng = np.random.default_rng(2020)
+    dims = [8, 64, 64, 64, 64, 1]
+    B = 1 << 14
+    specs = make_specs(rng, dims)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = np.sin(x.astype(np.float32).sum(1, keepdims=True)).astype(np.float16)
+    layers = build(specs, grad_layout=ML.TrainingOptimal)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    assert cv.lastKernelName().startswith("mlpTrainPairKernel"), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.TrainingOptimal)
+    rW, rB, _ = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
+    tW, tB = gradient_term_sums(specs, x, t)
+    checked = 0
+    for l in range(len(specs)):
+        for got, ref, terms in ((dW[l], rW[l], tW[l]), (dB[l], rB[l], tB[l])):
+            ulp_bar = 2.0 * ob.f16_ulp(ref.astype(np.float32)).astype(np.float64)
+            solid = ulp_bar >= 2.0 ** -19 * terms
+            err = np.abs(got - ref)
+            bar = np.maximum(ulp_bar, 2.0 ** -19 * terms)
+            bad = err > bar
+            assert not bad.any(), "layer %d: %d of %d elements outside the bar (worst %.3g x its bar)" % (
+                l, bad.sum(), bad.size, (err / np.maximum(bar, 1e-300)).max())
+            checked += int(solid.sum())
+    assert checked > 10000      # most elements are not cancellation-dominated
+
+
+@pytest.mark.parametrize("dims,B,flags", [([8, 64, 64, 64, 64, 1], 5000, 0), ([4, 16, 4], 16, 0), ([8, 32, 32, 6], 777, 0),
+                                          ([8, 64, 64, 64, 64, 1], 3000, cv.FLAG_LAYERWISE_TRAINING), ([20, 50, 7], 300, 0)])
+def test_loss_max_is_the_largest_per_sample_loss(dims, B, flags):
+    # lossMax: what learnGradient leaves in its loss buffer (WaveActiveMax + atomic max, kernels.slang:21-26), from the
+    # paired kernel, the one-wave kernel and the layer-by-layer step; gradients and lossSum are what they are without it
+    rng = np.random.default_rng(sum(dims) + B)
+    specs = make_specs(rng, dims)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
+    layers = build(specs)
+    lmax = torch.full((1,), -1.0, dtype=torch.float32, device=DEV)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossMax=lmax, flags=flags)
+    y = cv.mlpForward(gpu_fwd_layers(specs), to_dev(x)).cpu().numpy()
+    diff = (y.astype(np.float32) - t.astype(np.float32)).astype(np.float16).astype(np.float32)
+    per_sample = (diff * diff).sum(1, dtype=np.float64)
+    assert abs(lmax.item() - per_sample.max()) <= 1e-5 * per_sample.max(), (lmax.item(), per_sample.max())
+    assert abs(loss.item() - per_sample.sum()) <= 1e-4 * per_sample.sum()
+    layers2 = build(specs)
+    _, loss2 = cv.mlpTrainStep(layers2, to_dev(x), to_dev(t), flags=flags)
+    assert loss2.item() == loss.item()
+    for a, b in zip(layers, layers2):
+        assert torch.equal(a.weightsGrad, b.weightsGrad) and torch.equal(a.biasesGrad, b.biasesGrad)
+
+
+def gpu_fwd_layers(specs):
+    return [FeedForwardLayer(s["W"].shape[1], s["W"].shape[0], as_bytes(to_dev(s["W"])),
+                             as_bytes(to_dev(s["b"])) if s["b"] is not None else None, ML.RowMajor, s["W"].shape[1] * 2,
+                             s["act"], s.get("slope", 0.0)) for s in specs]
+
+
+def test_nan_loss_voids_the_whole_step():
+    # A workgroup whose loss partial is NaN voids the step: the loss outputs and every gradient sum the step adds
+    # are NaN (this is how a pair meeting that timed out reports itself; a NaN sample takes the same path)
+    rng = np.random.default_rng(4)
+    dims, B = [8, 64, 64, 64, 64, 1], 4096
+    specs = make_specs(rng, dims)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    x[1234, 3] = np.nan
+    layers = build(specs)
+    lmax = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), None, lossMax=lmax)
+    assert cv.lastKernelName().startswith("mlpTrainPairKernel")
+    assert np.isnan(loss.item()) and np.isnan(lmax.item())
+    for L in layers:
+        assert torch.isnan(L.weightsGrad.view(torch.float32)).all() and torch.isnan(L.biasesGrad.view(torch.float32)).all()
+
+
 def test_train_tie_rule_and_leaky_relu():
     # a hidden unit at exactly z = 0 gets half of the gradient (diff.meta.slang:2258-2277)
     specs = [dict(W=np.array([[1.0], [0.5]] + [[0.0]] * 14, np.float16), b=np.array([-1.0, 0.25] + [0.0] * 14, np.float16), act=1),

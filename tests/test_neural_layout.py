@@ -39,6 +39,21 @@ def test_counts_match_the_reference_buffers(mask, dims, logical, physical):
         assert (l.value, p.value) == (logical, physical)
 
 
+def test_oversized_layer_is_refused():
+    # the converter kernels index a layer's elements with 32-bit integers: 2^31 padded elements or more are refused
+    import ctypes
+    from slang_amd import _lib
+    d = _lib.CvNeuralNetworkDesc()
+    d.layerCount = 2
+    d.dims[0], d.dims[1], d.dims[2] = 8, 65536, 32768         # the second layer has 2^31 weights
+    d.biasMask, d.elementType, d.order = 0, 3, 0
+    l, p = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert _lib.load().cvNeuralNetworkSize(ctypes.byref(d), ctypes.byref(l), ctypes.byref(p)) < 0
+    d.dims[2] = 16384                                          # 2^30: fine
+    assert _lib.load().cvNeuralNetworkSize(ctypes.byref(d), ctypes.byref(l), ctypes.byref(p)) == 0
+    assert l.value == 8 * 65536 + 65536 * 16384
+
+
 def host_test_network():
     mask, dims = 0b101, [5, 13, 7, 19]
     portable = np.array([nl.make_portable_value(i) for i in range(321)], np.float32)

@@ -77,6 +77,20 @@ def test_gradients_against_central_differences():
             assert np.allclose(grads[k][~kink], num[~kink], rtol=2e-2, atol=2e-3), (op, k)
 
 
+def test_half_results_are_rounded_once_and_scale():
+    # the oracle rounds its double results to half in one step: a*b + c = (1.5 + 1.5 ulp) - 2^-24 is below the tie
+    a = np.full(4, 1.0009765625, np.float16); b = np.full(4, 1.5, np.float16); c = np.full(4, -2.0 ** -24, np.float16)
+    assert (ob.elementwise(T.FMA, a, b, c, 0.0).view(np.uint16) == 0x3E01).all()
+    c0 = np.zeros(4, np.float16)
+    assert (ob.elementwise(T.FMA, a, b, c0, 0.0).view(np.uint16) == 0x3E02).all()       # the exact tie goes to even
+    x = np.array([1.0, -2.5, 3.0, 0.1], np.float16)
+    assert np.array_equal(ob.elementwise(T.SCALE, x, None, None, 0.3), (x.astype(np.float32) * np.float32(np.float16(0.3))).astype(np.float16))
+    xf = x.astype(np.float32)
+    assert np.array_equal(ob.elementwise(T.SCALE, xf, None, None, 0.3), (xf.astype(np.float64) * np.float64(np.float32(0.3))).astype(np.float32))
+    da, _, _ = ob.elementwise_backward(T.SCALE, np.ones(4, np.float32), xf, None, None, 2.0)
+    assert (da == 2.0).all()
+
+
 def test_tie_rules_and_identities():
     one = np.ones(4, np.float32)
     x = np.array([1.0, 2.0, 3.0, -1.0], np.float32)
