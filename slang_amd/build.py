@@ -54,9 +54,9 @@ PER_FILE_FLAGS = {
 # assembly.  For these the build checks, on the generated code, that
 #   - nothing spills (hipcc's kernel-resource-usage remarks): a spill or reload of such a register would
 #     move stale data;
-#   - between a hand-issued load (`global_load_dwordx4 ... nt` into v[a:b]) and the next `s_waitcnt vmcnt`
-#     no instruction reads or writes v[a:b] (the device assembly, scanned in program order; the loop
-#     bodies of these kernels are straight-line code).
+#   - between a hand-issued load (`global_load_dwordx4 ... nt` into v[a:b]) and the `s_waitcnt vmcnt(n)` that
+#     covers it no instruction reads or writes v[a:b] (the device assembly, scanned in program order and once
+#     around the loop; see _check_inflight_registers).
 HAND_PIPELINED_KERNELS = {"cv_mlp_fp8.hip": "mlpWideKernel"}
 
 
@@ -71,8 +71,19 @@ def _check_no_spills(src: str, needle: str, remarks: str) -> None:
                     raise RuntimeError("%s: %s of %s is not zero (%s)" % (src, key.rstrip(":"), name, line.strip()))
 
 
+_VECTOR_PREFIXES = ("v_", "ds_", "global_", "scratch_", "buffer_", "flat_")
+_VMEM_PREFIXES = ("global_", "scratch_", "buffer_", "flat_")
+
+
 def _check_inflight_registers(src: str, needle: str, asm_text: str) -> int:
-    """Returns the number of hand-issued loads checked; raises if a pending register is touched."""
+    """Returns the number of hand-issued loads checked; raises if a pending register is touched.
+
+    From a hand-issued load (`global_load_dwordx4 v[a:b], ... nt`) every path of the function's control flow is followed
+    (both sides of a conditional branch, around the loop) until the wait that covers the load: an `s_waitcnt vmcnt(n)`
+    with n no larger than the number of vector-memory instructions issued on that path since the load (a larger n can
+    return while the load is still on its way), or until the program ends.  On the way no instruction may name a
+    register of v[a:b].  The scan fails closed: a line it cannot classify, a vector instruction whose register operands
+    it cannot parse, an indirect jump or a path that runs off the end of the function is an error."""
     import re
     lines = asm_text.split("\n")
     checked = 0
@@ -86,23 +97,65 @@ def _check_inflight_registers(src: str, needle: str, asm_text: str) -> int:
         end = i + 1
         while end < len(lines) and not lines[end].startswith(".Lfunc_end"):
             end += 1
-        body = lines[i:end]
-        for j, line in enumerate(body):
-            lm = re.search(r"global_load_dwordx4 v\[(\d+):(\d+)\],.* nt\b", line)
+        # the function as a list of instructions; a label points at the instruction that follows it
+        insts, labels = [], {}
+        for line in lines[i + 1:end]:
+            text = line.split(";")[0].strip()
+            lm = re.match(r"^(\.?\w+):$", text)
+            if lm:
+                labels[lm.group(1)] = len(insts)
+            elif text and not text.startswith("."):
+                insts.append(text)
+        for j, text in enumerate(insts):
+            lm = re.match(r"global_load_dwordx4 v\[(\d+):(\d+)\],.* nt\b", text)
             if not lm:
                 continue
             lo, hi = int(lm.group(1)), int(lm.group(2))
             checked += 1
-            k = j + 1
-            while k < len(body) and "s_waitcnt vmcnt" not in body[k]:
-                text = body[k].split(";")[0]
-                if re.match(r"\s+(v_|ds_|global_|scratch_|buffer_|flat_)", text):
-                    for rm in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", text):
-                        a, b = (int(rm.group(3)),) * 2 if rm.group(3) else (int(rm.group(1)), int(rm.group(2)))
-                        if not (b < lo or a > hi):
-                            raise RuntimeError("%s: %s touches v[%d:%d] while its load is pending: %s"
-                                               % (src, name, lo, hi, body[k].strip()))
-                k += 1
+            fewest = {}                      # instruction index -> fewest younger vector-memory instructions seen there
+            work = [(j + 1, 0)]
+            while work:
+                k, younger = work.pop()
+                while True:
+                    if k >= len(insts):
+                        raise RuntimeError("%s: %s: a path from the load into v[%d:%d] runs off the end of the function" % (src, name, lo, hi))
+                    if k in fewest and fewest[k] <= younger:
+                        break                # been here with no more vector-memory instructions behind the load
+                    fewest[k] = younger
+                    text = insts[k]
+                    op = text.split()[0]
+                    wm = re.match(r"s_waitcnt\b.*vmcnt\((\d+)\)", text)
+                    if wm and int(wm.group(1)) <= younger:
+                        break                # the load has landed
+                    if op == "s_endpgm":
+                        break
+                    if op == "s_branch" or op.startswith("s_cbranch"):
+                        target = text.split()[-1]
+                        if target not in labels:
+                            raise RuntimeError("%s: %s: branch to an unknown label: %s" % (src, name, text))
+                        if op == "s_branch":
+                            k = labels[target]
+                            continue
+                        work.append((labels[target], younger))
+                    elif op.startswith(("s_setpc", "s_swappc", "s_call")):
+                        raise RuntimeError("%s: %s: indirect control flow while a load is pending: %s" % (src, name, text))
+                    elif op.startswith("s_"):
+                        pass                 # scalar instructions cannot name a vector register
+                    elif op.startswith(_VECTOR_PREFIXES):
+                        operands = text[len(op):]
+                        stripped = re.sub(r"\b[vas]\[\d+:\d+\]|\b[vas]\d+\b", "", operands)
+                        if re.search(r"\bv\[|\bv\d", stripped):
+                            raise RuntimeError("%s: %s: cannot parse the vector registers of '%s'" % (src, name, text))
+                        for rm in re.finditer(r"\bv\[(\d+):(\d+)\]|\bv(\d+)\b", operands):
+                            a, b = (int(rm.group(3)),) * 2 if rm.group(3) else (int(rm.group(1)), int(rm.group(2)))
+                            if not (b < lo or a > hi):
+                                raise RuntimeError("%s: %s touches v[%d:%d] while its load is pending: %s" % (src, name, lo, hi, text))
+                        if op.startswith(_VMEM_PREFIXES):
+                            younger += 1
+                    else:
+                        raise RuntimeError("%s: %s: the scan does not know the instruction form '%s' (between a hand-issued "
+                                           "load and its wait)" % (src, name, text))
+                    k += 1
         i = end
     if checked == 0:
         raise RuntimeError("%s: no hand-issued load found in any %s (the check no longer matches the code)" % (src, needle))
