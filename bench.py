@@ -13,7 +13,9 @@ under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (
 bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
 c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
 matrix pipeline bounds), c5 (training step), ex (one whole iteration of the example at its own shape: training step +
-Adam update, three kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate).  With --workload only that one runs and becomes the headline (profiling runs; also
+Adam update, three kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
+(permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), ew (an
+element-wise operator), ad (the Adam update over 2^24 parameters).  With --workload only that one runs and becomes the headline (profiling runs; also
 c5g = c5 on the layer-by-layer step, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
@@ -546,6 +548,119 @@ def workload_ex(torch, cv, steps, warmup):
     return w
 
 
+def workload_pe(torch, cv, steps, warmup, backward=False, decoder=False):
+    """PermutoEncoder.encode (or its reverse mode) over 2^22 positions.  `pe` / `peb`: the configuration of the
+    reference's own test (tests/neural/permuto-encoder-test.slang: 2 dimensions, 2 features per entry, 2^8 entries per
+    level, 4 levels, fp32) scaled to 2^22 positions.  `ped`: a neural-texture shaped encoder in half (3 dimensions, 2
+    features, 2^12 entries, 8 levels: 16 features per position), the input of a 16-wide decoder MLP.  What a position
+    costs in memory: its coordinates in, levels x features out, and (D+1) gathered table entries per level, which
+    these tables serve from the caches."""
+    import numpy as np
+    dev = "cuda"
+    B = 1 << 22
+    if decoder:
+        D, F, log2, levels, dt = 3, 2, 12, 8, torch.float16
+        enc = cv.PermutoEncoder(D, F, log2, levels, baseScale=4.0, log2PerLevelScale=1.0, dtype=dt)
+    else:
+        D, F, log2, levels, dt = 2, 2, 8, 4, torch.float32
+        enc = cv.PermutoEncoder(D, F, log2, levels, baseScale=1.0, log2PerLevelScale=1.0, maxLevelRatio=1.1, seed=1337, dtype=dt)
+    g = torch.Generator(device=dev); g.manual_seed(20260)
+    pos = torch.rand(B, D, device=dev, generator=g).to(dt)
+    table = (torch.randn(enc.featureTableElements, device=dev, generator=g) * 0.5).to(dt)
+    out = torch.empty(B, enc.outputSize, dtype=dt, device=dev)
+    esz = pos.element_size()
+    if backward:
+        dout = torch.randn(B, enc.outputSize, device=dev, generator=g)
+        dtab = torch.zeros_like(table)
+
+        def step():
+            enc.backward(pos, table, dout, dFeatureTable=dtab)
+        alg = B * (D * esz + enc.outputSize * esz + D * esz)
+    else:
+        def step():
+            enc.encode(pos, table, out=out)
+        alg = B * (D * esz + enc.outputSize * esz)
+    gathered = B * (D + 1) * levels * F * esz
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        n = 1 << 15
+        lv = ob.permuto_levels(D, log2, levels, 4.0 if decoder else 1.0, 1.0, 1337)
+        pn = pos[:n].cpu().numpy(); tn = table.cpu().numpy()
+        t0 = time.perf_counter(); ob.permuto_encode(lv, F, 1.1 * levels, pn, tn); t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d positions, one core; C restatement of PermutoEncoder.encode (forward)" % n}
+
+    key = "ped" if decoder else ("peb" if backward else "pe")
+    return dict(step=step, samples=B, alg_bytes=alg, alg_flops=0, bound="hbm", mfma="f32", dtype="f16" if decoder else "f32",
+                cpu_baseline=cpu_baseline, key=key, extra={"gathered_table_bytes_per_step": gathered},
+                config={"workload": "%s: PermutoEncoder %s, %d dimensions, %d features per entry, 2^%d entries per level, %d levels, %s, "
+                                    "2^22 positions" % (key, "reverse mode (atomic adds into the table gradient)" if backward else "encode",
+                                                        D, F, log2, levels, "fp16" if decoder else "fp32"),
+                        "batch": B})
+
+
+def workload_peb(torch, cv, steps, warmup):
+    return workload_pe(torch, cv, steps, warmup, backward=True)
+
+
+def workload_ped(torch, cv, steps, warmup):
+    return workload_pe(torch, cv, steps, warmup, decoder=True)
+
+
+def workload_ew(torch, cv, steps, warmup):
+    """An element-wise operator of CoopVec<half, 64> over 2^22 vectors: tanh (hlsl.meta.slang:32383-32401), 2 bytes in and
+    2 bytes out per element."""
+    import numpy as np
+    from slang_amd.coopvec import ElementwiseOp
+    dev = "cuda"
+    B, N = 1 << 22, 64
+    g = torch.Generator(device=dev); g.manual_seed(20261)
+    x = (torch.rand(B, N, device=dev, generator=g) * 4 - 2).half()
+    out = torch.empty_like(x)
+
+    def step():
+        cv.elementwise(ElementwiseOp.Tanh, x, out=out)
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        n = 1 << 14
+        xn = x[:n].cpu().numpy()
+        t0 = time.perf_counter(); ob.elementwise(int(ElementwiseOp.Tanh), xn); t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d vectors, one core; the oracle's element loop (double tanh, one rounding to half)" % n}
+
+    return dict(step=step, samples=B, alg_bytes=B * N * 4, alg_flops=0, bound="hbm", mfma="f16", dtype="f16", cpu_baseline=cpu_baseline,
+                key="ew", config={"workload": "ew: element-wise tanh of CoopVec<half,64> over 2^22 vectors", "batch": B, "n": N})
+
+
+def workload_ad(torch, cv, steps, warmup):
+    """adjustParameters (AdamOptimizer::step in half) over 2^24 parameters: per parameter 2 + 2 + 8 bytes read and as
+    many written (parameter, gradient, AdamState)."""
+    import numpy as np
+    dev = "cuda"
+    n = 1 << 24
+    g = torch.Generator(device=dev); g.manual_seed(20262)
+    params = (torch.rand(n, device=dev, generator=g) * 2 - 1).half()
+    grads = (torch.randn(n, device=dev, generator=g) * 0.1).half()
+    states = torch.zeros(n * 8, dtype=torch.uint8, device=dev)
+
+    def step():
+        cv.adjustParameters(states, params, grads)     # the gradients read are zero from the second step on: same traffic
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        m = 1 << 18
+        p = params[:m].cpu().numpy(); gr = (np.random.default_rng(0).standard_normal(m) * 0.1).astype(np.float16)
+        st = np.zeros(m, ob.ADAM_STATE_DTYPE)
+        t0 = time.perf_counter(); ob.slang_adam_step(st, p, gr); t1 = time.perf_counter()
+        return {"value": m / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "%d parameters, one core; C restatement of adjustParameters + AdamOptimizer::step (software half)" % m}
+
+    return dict(step=step, samples=n, alg_bytes=n * 24, alg_flops=0, bound="hbm", mfma="f16", dtype="f16", cpu_baseline=cpu_baseline,
+                key="ad", config={"workload": "ad: adjustParameters (Adam step in half) over 2^24 fp16 parameters", "parameters": n})
+
+
 def workload_op(torch, cv, steps, warmup):
     """stand-alone coopVecOuterProductAccumulate 64x64 over 2^20 vector pairs, fp32 TrainingOptimal destination."""
     from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML
@@ -627,9 +742,10 @@ def workload_rs(torch, cv, steps, warmup):
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": workload_c2b, "c3": workload_c3, "c3c": workload_c3c, "c4": workload_c4,
              "c4n": workload_c4n, "c5": workload_c5, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
+             "pe": workload_pe, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "ex", "op", "rs")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "ex", "op", "rs", "pe", "peb", "ped", "ew", "ad")
 HEADLINE = "c2"
 
 

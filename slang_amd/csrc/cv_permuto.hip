@@ -14,6 +14,7 @@
 
 #include "cv_device.h"
 #include "cv_error.h"
+#include "cv_launch.h"
 
 namespace cv {
 namespace {
@@ -211,11 +212,11 @@ __global__ __launch_bounds__(256) void permutoEncodeKernel(const PermutoArgs a)
     }
 }
 
+// Reverse mode for one position: adds bary[k] * dOut to the table gradient `dTable` (global memory, or a workgroup's
+// private copy in LDS) and, if wanted, writes the position gradient.
 template <int D>
-__global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a)
+__device__ __forceinline__ void permutoBackwardOne(const PermutoArgs& a, uint32_t s, float* dTable)
 {
-    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
-    if (s >= a.batch) return;
     const int F = a.desc.featureDimensionPerEntry;
     float pos[D], dpos[D];
 #pragma unroll
@@ -236,7 +237,7 @@ __global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a
         for (int k = 0; k <= D; ++k) {
             const uint32_t idx = vertexIndex<D>(lv, F, rem0, rank, k);
             for (int f = 0; f < F; ++f) {
-                if (a.dTable) atomicAdd(a.dTable + idx + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
+                if (dTable) atomicAdd(dTable + idx + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
                 dbary[k] += table[idx + f] * gl[f];
             }
         }
@@ -268,6 +269,32 @@ __global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a
     }
 }
 
+template <int D>
+__global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a)
+{
+    const uint32_t s = blockIdx.x * 256u + threadIdx.x;
+    if (s >= a.batch) return;
+    permutoBackwardOne<D>(a, s, a.dTable);
+}
+
+// A small feature table (the reference's own test: 2 048 floats) receives every position's atomic adds on a handful of
+// addresses: 2^22 positions took 123 ms that way.  Here a workgroup accumulates into a private copy of the table in
+// LDS and adds that copy to the table gradient once, at its end: the atomic traffic to memory shrinks by the number
+// of positions per workgroup.
+template <int D>
+__global__ __launch_bounds__(256) void permutoBackwardLdsKernel(const PermutoArgs a, uint32_t tableElems)
+{
+    extern __shared__ float ldsTable[];
+    for (uint32_t i = threadIdx.x; i < tableElems; i += 256u) ldsTable[i] = 0.f;
+    __syncthreads();
+    for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < a.batch; s += gridDim.x * 256u) permutoBackwardOne<D>(a, s, ldsTable);
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < tableElems; i += 256u) {
+        const float v = ldsTable[i];
+        if (v != 0.f) atomicAdd(a.dTable + i, v);
+    }
+}
+
 template <typename T>
 hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
 {
@@ -283,6 +310,32 @@ hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
 
 hipError_t launchBackward(hipStream_t stream, const PermutoArgs& a)
 {
+    // the table as the levels lay it out: offsets and sizes in entries, F floats per entry
+    uint64_t tableElems = 0;
+    for (uint32_t l = 0; l < a.desc.maxLevels; ++l) {
+        const uint64_t e = ((uint64_t)a.desc.levelInfo[l].offsetOfFeatureTable + a.desc.levelInfo[l].featureTableSize) * (uint64_t)a.desc.featureDimensionPerEntry;
+        tableElems = e > tableElems ? e : tableElems;
+    }
+    constexpr uint64_t kLdsTableBytes = 64 * 1024;
+    if (a.dTable && tableElems * 4 <= kLdsTableBytes && a.batch >= 4096u) {
+        int dev = 0, cus = 256;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        const uint32_t want = (a.batch + 255u) / 256u, cap = (uint32_t)cus * 2u;
+        const dim3 grid(want < cap ? want : cap), block(256);
+        const size_t lds = (size_t)tableElems * 4;
+        noteKernel(false, "permutoBackwardLdsKernel<D=%d>", a.desc.dimensions);
+        switch (a.desc.dimensions) {
+#define CV_D(N) case N: { \
+            const hipError_t e = allowDynamicLds<permutoBackwardLdsKernel<N>>((int)lds); \
+            if (e != hipSuccess) return e; \
+            hipLaunchKernelGGL(permutoBackwardLdsKernel<N>, grid, block, lds, stream, a, (uint32_t)tableElems); break; }
+        CV_D(1) CV_D(2) CV_D(3) CV_D(4) CV_D(5) CV_D(6) CV_D(7) CV_D(8)
+#undef CV_D
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
+    noteKernel(false, "permutoBackwardKernel<D=%d>", a.desc.dimensions);
     const dim3 grid((a.batch + 255) / 256), block(256);
     switch (a.desc.dimensions) {
 #define CV_D(N) case N: hipLaunchKernelGGL(permutoBackwardKernel<N>, grid, block, 0, stream, a); break;
@@ -404,7 +457,6 @@ CV_API CvResult cvPermutoEncodeBackward(void* stream, const CvPermutoDesc* desc,
     a.pos = (const uint8_t*)positions; a.posStride = positionStride; a.table = (const uint8_t*)featureTable;
     a.dOut = (const uint8_t*)dOut; a.dOutStride = dOutStride;
     a.dPos = (uint8_t*)dPositions; a.dPosStride = dPositionStride; a.dTable = (float*)dFeatureTable; a.batch = batch;
-    noteKernel(false, "permutoBackwardKernel<D=%d>", desc->dimensions);
     const hipError_t e = launchBackward((hipStream_t)stream, a);
     if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvPermutoEncodeBackward launch: %s", hipGetErrorString(e));
     return CV_OK;
