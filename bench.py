@@ -12,7 +12,7 @@ way in the same run (W warm-up steps, K timed steps, HIP events on the launch st
 under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (c2 with RowMajor weights), c2b (c2 in
 bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
 c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
-matrix pipeline bounds), c5 (training step), ex (one whole iteration of the example at its own shape: training step +
+matrix pipeline bounds), c5 (training step), t32 (training step of a 32-wide network), ex (one whole iteration of the example at its own shape: training step +
 Adam update, three kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
 (permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), ew (an
 element-wise operator), ad (the Adam update over 2^24 parameters).  With --workload only that one runs and becomes the headline (profiling runs; also
@@ -426,13 +426,13 @@ def workload_f32(torch, cv, steps, warmup):
                 cpu_baseline=cpu_baseline, key="f32")
 
 
-def workload_c5(torch, cv, steps, warmup, flags=0):
+def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
     """fp16 training step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, fp32 TrainingOptimal grads."""
     import numpy as np
     from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
                                    FeedForwardLayer)
     dev = "cuda"
-    dims = [8, 64, 64, 64, 64, 1]
+    dims = dims or [8, 64, 64, 64, 64, 1]
     B = 1 << 20
     g = torch.Generator(device=dev); g.manual_seed(20255)
     layers, host = [], []
@@ -472,11 +472,17 @@ def workload_c5(torch, cv, steps, warmup, flags=0):
 
     return dict(step=step, samples=B, alg_bytes=B * dims[0] * 2, alg_flops=B * 2 * (2 * macs + macs_dx),
                 bound="mfma", mfma="f16", dtype="f16",
-                config={"workload": "%s: fp16 train step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, "
+                config={"workload": "%s: fp16 train step %s, ReLU, MSE vs sin(sum x), batch 2^20, "
                                     "fp32 TrainingOptimal gradients, deterministic reduction%s"
-                                    % ("c5g" if flags else "c5", ", layer-by-layer step (the one for arbitrary layer sizes)" if flags else ""),
+                                    % (key or ("c5g" if flags else "c5"), "->".join(str(d) for d in dims),
+                                       ", layer-by-layer step (the one for arbitrary layer sizes)" if flags else ""),
                         "batch": B, "layers": dims},
-                cpu_baseline=cpu_baseline, key="c5g" if flags else "c5")
+                cpu_baseline=cpu_baseline, key=key or ("c5g" if flags else "c5"))
+
+
+def workload_t32(torch, cv, steps, warmup):
+    """the training step of a 32-wide decoder-sized network, 8->32->32->32->4 (the one-wave fused kernel)"""
+    return workload_c5(torch, cv, steps, warmup, dims=[8, 32, 32, 32, 4], key="t32")
 
 
 def workload_c5g(torch, cv, steps, warmup):
@@ -741,11 +747,11 @@ def workload_rs(torch, cv, steps, warmup):
 
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": workload_c2b, "c3": workload_c3, "c3c": workload_c3c, "c4": workload_c4,
-             "c4n": workload_c4n, "c5": workload_c5, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
+             "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
              "pe": workload_pe, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "ex", "op", "rs", "pe", "peb", "ped", "ew", "ad")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "t32", "ex", "op", "rs", "pe", "peb", "ped", "ew", "ad")
 HEADLINE = "c2"
 
 

@@ -10,7 +10,8 @@ namespace {
 // (input feature tiles, input k-tiles, hidden tiles, hidden layers, output tiles)
 #define CV_TRAIN_SHAPES(X) \
     X(1, 1, 1, 1, 1) X(1, 1, 1, 2, 1) X(1, 1, 1, 3, 1) \
-    X(1, 1, 2, 2, 1) X(1, 1, 4, 2, 1) X(1, 1, 4, 3, 1) X(1, 1, 4, 4, 1) X(2, 1, 4, 2, 1)
+    X(1, 1, 2, 1, 1) X(1, 1, 2, 2, 1) X(1, 1, 2, 3, 1) X(1, 1, 2, 4, 1) X(2, 1, 2, 2, 1) X(2, 1, 2, 3, 1) \
+    X(1, 1, 4, 1, 1) X(1, 1, 4, 2, 1) X(1, 1, 4, 3, 1) X(1, 1, 4, 4, 1) X(2, 1, 4, 2, 1) X(2, 1, 4, 3, 1)
 
 struct Shape { int it0, kt0, ht, nhid, mtl; bool ok; };
 

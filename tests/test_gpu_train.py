@@ -83,7 +83,9 @@ def test_ffn_closed_form_backward():
 
 
 @pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 4096 + 21), ([4, 16, 4], 1000), ([2, 16, 16, 16, 1], 2048),
-                                    ([8, 32, 32, 4], 777), ([20, 64, 64, 8], 1500), ([8, 64, 64, 64, 5], 900)])
+                                    ([8, 32, 32, 4], 777), ([20, 64, 64, 8], 1500), ([8, 64, 64, 64, 5], 900),
+                                    ([8, 32, 4], 300), ([8, 32, 32, 32, 4], 1500), ([8, 32, 32, 32, 32, 2], 2100), ([24, 32, 32, 32, 8], 1000),
+                                    ([8, 64, 4], 513), ([24, 64, 64, 64, 6], 1200)])
 def test_train_step_against_oracle(dims, B):
     rng = np.random.default_rng(sum(dims) + B)
     specs = make_specs(rng, dims)
@@ -92,12 +94,21 @@ def test_train_step_against_oracle(dims, B):
     t = np.ascontiguousarray(t)
     layers = build(specs)
     _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t))
+    # one launch for the whole step (plus the reduction): hidden layers of 16, 32 or 64 units all have a fused kernel
+    assert cv.lastKernelName().startswith(("mlpTrainPairKernel", "mlpTrainKernel")), cv.lastKernelName()
     dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
     rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
     for l in range(len(specs)):
         assert rel_err(dW[l], rW[l]) <= 1e-3, (l, rel_err(dW[l], rW[l]))
         assert rel_err(dB[l], rB[l]) <= 1e-3, (l, rel_err(dB[l], rB[l]))
     assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # the layer-by-layer step gives the same gradients to its own bar
+    if max(dims) <= 32:
+        general = build(specs)
+        cv.mlpTrainStep(general, to_dev(x), to_dev(t), flags=cv.FLAG_LAYERWISE_TRAINING)
+        gW, gB = read_grads(general, specs, CT.Float32, ML.RowMajor)
+        for l in range(len(specs)):
+            assert rel_err(gW[l], dW[l]) <= 1e-3 and rel_err(gB[l], dB[l]) <= 1e-3
     # bitwise determinism, and "+=" semantics: a second step doubles the (fp32) gradients exactly
     before = [L.weightsGrad.clone() for L in layers]
     layers2 = build(specs)
