@@ -172,7 +172,11 @@ __device__ __forceinline__ uint32_t vertexIndex(const CvPermutoLevelInfo& lv, in
         key[dim] = (uint32_t)(rem0[dim] + k);
         if (rank[dim] > D - k) key[dim] -= (uint32_t)(D + 1);
     }
-    return lv.offsetOfFeatureTable * (uint32_t)F + (baseConvertHash(key, D) % lv.featureTableSize) * (uint32_t)F;
+    // (a table of 2^n entries, which is what prepareLevelInfo makes, is indexed with a mask: the general remainder
+    // is a division by a run-time value, some forty instructions per vertex)
+    const uint32_t hash = baseConvertHash(key, D), size = lv.featureTableSize;
+    const uint32_t slot = (size & (size - 1u)) == 0u ? (hash & (size - 1u)) : hash % size;
+    return lv.offsetOfFeatureTable * (uint32_t)F + slot * (uint32_t)F;
 }
 
 template <typename T, int D>
