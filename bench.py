@@ -606,6 +606,67 @@ def workload_pe(torch, cv, steps, warmup, backward=False, decoder=False):
                         "batch": B})
 
 
+def workload_pef(torch, cv, steps, warmup, fused=True):
+    """The neural-texture pipeline: encoder of `ped` (3 dimensions, 2 features, 2^12 entries, 8 levels, half) and its
+    decoder 16 -> 64 -> 64 -> 3 (ReLU) over 2^22 positions.  `pef`: one kernel (cvPermutoMlpForward), the encoded vectors
+    never reach memory; `peu`: cvPermutoEncode then cvMlpForward, which write and re-read 32 bytes per position."""
+    import numpy as np
+    from slang_amd.coopvec import Activation, CoopVecMatrixLayout as ML, FeedForwardLayer
+    dev = "cuda"
+    B = 1 << 22
+    D, F, log2, levels = 3, 2, 12, 8
+    enc = cv.PermutoEncoder(D, F, log2, levels, baseScale=4.0, log2PerLevelScale=1.0, dtype=torch.float16)
+    g = torch.Generator(device=dev); g.manual_seed(20263)
+    pos = torch.rand(B, D, device=dev, generator=g).half()
+    table = (torch.randn(enc.featureTableElements, device=dev, generator=g) * 0.5).half()
+    dims = [16, 64, 64, 3]
+    layers, host = [], []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = (torch.randn(fo, fi, device=dev, generator=g) * (2.0 / fi) ** 0.5).half()
+        b = (torch.rand(fo, device=dev, generator=g) * 0.2 - 0.1).half()
+        layers.append(FeedForwardLayer(fi, fo, W.view(torch.uint8).flatten(), b.view(torch.uint8), ML.RowMajor, fi * 2,
+                                       Activation.ReLU if i < len(dims) - 2 else Activation.NoActivation, 0.0))
+        host.append((W, b))
+    out = torch.empty(B, dims[-1], dtype=torch.float16, device=dev)
+    feats = torch.empty(B, dims[0], dtype=torch.float16, device=dev)
+    plan = cv.MlpForwardPlan(layers)
+
+    if fused:
+        def step():
+            enc.encodeAndEval(pos, table, layers, out=out)
+    else:
+        def step():
+            enc.encode(pos, table, out=feats)
+            plan(feats, out=out)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+
+    def cpu_baseline():
+        import oracle_binding as ob
+        n = 1 << 14
+        lv = ob.permuto_levels(D, log2, levels, 4.0, 1.0, 1337)
+        pn = pos[:n].cpu().numpy(); tn = table.cpu().numpy()
+        specs = [dict(W=W.cpu().numpy(), b=b.cpu().numpy(), act=1 if i < len(host) - 1 else 0, slope=0.0) for i, (W, b) in enumerate(host)]
+        t0 = time.perf_counter()
+        f = ob.permuto_encode(lv, F, 1.1 * levels, pn, tn)
+        ob.ref_mlp_forward(specs, f, ob.F16)
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d positions, one core; C restatements of PermutoEncoder.encode and of the layer chain" % n}
+
+    key = "pef" if fused else "peu"
+    return dict(step=step, samples=B, alg_bytes=B * (D * 2 + dims[-1] * 2), alg_flops=B * 2 * macs, bound="hbm", mfma="f16", dtype="f16",
+                cpu_baseline=cpu_baseline, key=key,
+                config={"workload": "%s: PermutoEncoder (3 dimensions, 2 features per entry, 2^12 entries per level, 8 levels, fp16) + decoder "
+                                    "16->64->64->3 (ReLU), 2^22 positions, %s" % (key, "one kernel" if fused else "two calls, features through memory"),
+                        "batch": B, "layers": dims})
+
+
+def workload_peu(torch, cv, steps, warmup):
+    return workload_pef(torch, cv, steps, warmup, fused=False)
+
+
 def workload_peb(torch, cv, steps, warmup):
     return workload_pe(torch, cv, steps, warmup, backward=True)
 
@@ -748,10 +809,10 @@ def workload_rs(torch, cv, steps, warmup):
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": workload_c2b, "c3": workload_c3, "c3c": workload_c3c, "c4": workload_c4,
              "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
-             "pe": workload_pe, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
+             "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "t32", "ex", "op", "rs", "pe", "peb", "ped", "ew", "ad")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "t32", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad")
 HEADLINE = "c2"
 
 

@@ -422,6 +422,19 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp,
                              const void* input, size_t inputStride,
                              void* output, size_t outputStride, uint32_t batch);
 
+/* encode + network in one kernel.  A Slang thread hands the result of PermutoEncoder::encode
+ * (source/standard-modules/neural/permuto-encoder.slang:319-337) straight to the first layer of its
+ * network (layers.slang:34-110; network.slang:41-47), so the encoded vector never exists in memory;
+ * this is that composition for a batch: output[s] = mlp(encode(positions[s])), bit for bit what
+ * cvPermutoEncode followed by cvMlpForward returns.  FLOAT16 encoders (1..4 dimensions, 1, 2 or 4
+ * features per entry, level records in level order) in front of FLOAT16 networks of at least two
+ * layers whose first layer takes maxLevels * featureDimensionPerEntry inputs, every dimension <= 128;
+ * CV_E_NOT_AVAILABLE otherwise (call the two entry points instead).  The feature table must be aligned
+ * to one entry. */
+CV_API CvResult cvPermutoMlpForward(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                    const void* featureTable, const CvMlpDesc* mlp, void* output, size_t outputStride,
+                                    uint32_t batch);
+
 /* Forward + reverse pass of loss_s = sum_i (y[s][i] - target[s][i])^2 with seed `lossScale`
  * (the example: bwd_diff(loss)(network, x, y, 1.0h), kernels.slang:20): accumulates
  * sum_s dY (x) X into every layer's weightsGrad and sum_s dY into biasesGrad ("+=").

@@ -146,6 +146,9 @@ SIGNATURES = {
                                                 ctypes.c_uint32]),
     "cvPermutoEncode": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
                                          ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_uint32]),
+    "cvPermutoMlpForward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_void_p, ctypes.POINTER(CvMlpDesc), ctypes.c_void_p, ctypes.c_size_t,
+                                             ctypes.c_uint32]),
     "cvPermutoEncodeBackward": (ctypes.c_int32, [ctypes.c_void_p, ctypes.POINTER(CvPermutoDesc), ctypes.c_void_p, ctypes.c_size_t,
                                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p,
                                                  ctypes.c_size_t, ctypes.c_void_p, ctypes.c_uint32]),

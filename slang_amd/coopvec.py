@@ -534,6 +534,26 @@ class PermutoEncoder:
                                            out.stride(0) * es, positions.shape[0]))
         return out
 
+    def encodeAndEval(self, positions: torch.Tensor, featureTable: torch.Tensor, layers, *,
+                      out: Optional[torch.Tensor] = None, flags: int = 0, stream=None) -> torch.Tensor:
+        """network.eval(encoder.encode(position)) for every row of positions, in one kernel: what a Slang thread does
+        when it hands encode's result (:319-337) to its network; the encoded vectors never reach memory.  Same bits as
+        mlpForward(layers, self.encode(positions, featureTable)); half encoders and networks only."""
+        if positions.dtype != self.dtype or featureTable.dtype != self.dtype or positions.dim() != 2 or positions.stride(1) != 1:
+            raise CoopVecError(SLANG_E_INVALID_ARG, "positions [batch, D] and featureTable must have the encoder's dtype")
+        if featureTable.numel() < self.featureTableElements or not featureTable.is_contiguous():
+            raise CoopVecError(SLANG_E_BUFFER_TOO_SMALL, "featureTable holds fewer than %d elements" % self.featureTableElements)
+        batch = positions.shape[0]
+        if out is None:
+            out = torch.empty((batch, layers[-1].outputSize), dtype=torch.float16, device=positions.device)
+        outCt, outStride = _vector_info(out, CoopVecComponentType.Float16, "out")
+        d, keep = _mlp_desc(layers, CoopVecComponentType.Float16, CoopVecComponentType.Float32, flags, 0)
+        es = positions.element_size()
+        _check(_lib.load().cvPermutoMlpForward(_stream_handle(stream), ctypes.byref(self.desc), positions.data_ptr(),
+                                               positions.stride(0) * es, featureTable.data_ptr(), ctypes.byref(d),
+                                               out.data_ptr(), outStride, batch))
+        return out
+
     def backward(self, positions: torch.Tensor, featureTable: torch.Tensor, dOut: torch.Tensor, *,
                  dFeatureTable: Optional[torch.Tensor] = None, wantPositionGrad: bool = True, stream=None):
         """bwd_diff of encode: returns (dPositions or None, dFeatureTable); the table gradient is added to."""

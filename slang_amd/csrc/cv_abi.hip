@@ -694,6 +694,50 @@ CV_API CvResult cvMlpForward(void* stream, const CvMlpDesc* mlp, const void* inp
     return fromHip(e, "cvMlpForward launch");
 }
 
+CV_API CvResult cvPermutoMlpForward(void* stream, const CvPermutoDesc* desc, const void* positions, size_t positionStride,
+                                    const void* featureTable, const CvMlpDesc* mlp, void* output, size_t outputStride, uint32_t batch)
+{
+    const char* who = "cvPermutoMlpForward";
+    CvResult rc = cv::checkPermutoDesc(who, desc);
+    if (CV_FAILED(rc)) return rc;
+    cv::MlpArgs a;
+    memset(&a, 0, sizeof(a));
+    rc = fillMlpLayers(who, mlp, a.layers);
+    if (CV_FAILED(rc)) return rc;
+    const int F = desc->featureDimensionPerEntry, L = mlp->numLayers;
+    if (desc->elementType != CV_FLOAT16 || mlp->weightType != CV_FLOAT16 || mlp->inputType != CV_FLOAT16 ||
+        mlp->inputEncoding != CV_ENCODE_NONE || L < 2)
+        return fail(CV_E_NOT_AVAILABLE, "%s: a FLOAT16 encoder in front of a FLOAT16 network of at least two layers without another "
+                    "input encoding; otherwise call cvPermutoEncode and cvMlpForward", who);
+    if (desc->dimensions > 4 || (F != 1 && F != 2 && F != 4))
+        return fail(CV_E_NOT_AVAILABLE, "%s: dimensions=%d (1..4), featureDimensionPerEntry=%d (1, 2 or 4); otherwise call "
+                    "cvPermutoEncode and cvMlpForward", who, desc->dimensions, F);
+    if ((uint32_t)mlp->layers[0].inputSize != desc->maxLevels * (uint32_t)F)
+        return fail(CV_E_INVALID_ARG, "%s: the first layer takes %d inputs, the encoder produces %u", who, mlp->layers[0].inputSize,
+                    desc->maxLevels * (uint32_t)F);
+    for (uint32_t l = 0; l < desc->maxLevels; ++l)
+        if (desc->levelInfo[l].currentLevelIndex != l)
+            return fail(CV_E_NOT_AVAILABLE, "%s: level record %u writes level %u (records in level order only)", who, l,
+                        desc->levelInfo[l].currentLevelIndex);
+    if (batch == 0) return CV_OK;
+    if (!positions || !featureTable || !output) return fail(CV_E_INVALID_ARG, "%s: null argument", who);
+    if ((uintptr_t)positions % 2 || positionStride % 2 || (uintptr_t)featureTable % (2u * (uint32_t)F) || (uintptr_t)output % 2 || outputStride % 2)
+        return fail(CV_E_INVALID_ARG, "%s: misaligned argument (positions and output to 2 bytes, the feature table to one entry)", who);
+    if (batch > 1 && (positionStride < (size_t)desc->dimensions * 2 || outputStride < (size_t)mlp->layers[L - 1].outputSize * 2))
+        return fail(CV_E_INVALID_ARG, "%s: vector stride smaller than the vector", who);
+    a.numLayers = L;
+    a.out = (uint8_t*)output; a.outStride = outputStride; a.batch = batch;
+    a.outAlign = alignOf(output, outputStride);
+    a.noWideTiles = (mlp->flags & CV_FLAG_FORWARD_TILE16) ? 1 : 0;
+    const int cus = currentDeviceCUs(&rc);
+    if (CV_FAILED(rc)) return rc;
+    const hipError_t e = cv::launchPermutoMlp((hipStream_t)stream, *desc, positions, positionStride, featureTable, a, cus);
+    if (e == hipErrorInvalidValue)
+        return fail(CV_E_NOT_AVAILABLE, "%s: every dimension of the network must be <= 128, its weights must fit in LDS beside the level "
+                    "records and its activations must be NONE, RELU or LEAKY_RELU; otherwise call cvPermutoEncode and cvMlpForward", who);
+    return fromHip(e, "cvPermutoMlpForward launch");
+}
+
 CV_API CvResult cvMlpTrainStepWorkspaceSize(const CvMlpDesc* mlp, uint32_t batch, size_t* outBytes)
 {
     if (!outBytes) return fail(CV_E_INVALID_ARG, "cvMlpTrainStepWorkspaceSize: outBytes is null");

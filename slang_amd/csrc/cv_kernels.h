@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "coopvec.h"
 #include "cv_layout.h"
 
 namespace cv {
@@ -72,6 +73,12 @@ enum : int { kEncodeNone = 0, kEncodeXYSquares = 1 };
 hipError_t launchMlpForward(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
 // any layer sizes up to 128 (weights read from LDS); hipErrorInvalidValue beyond that
 hipError_t launchMlpGeneric(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);
+// permutohedral encoding of fp16 positions fused in front of an fp16 network (weights in LDS, every dimension <= 128);
+// hipErrorInvalidValue for encoders or networks the kernel does not take
+hipError_t launchPermutoMlp(hipStream_t stream, const CvPermutoDesc& desc, const void* positions, uint64_t positionStride,
+                            const void* featureTable, const MlpArgs& mlp, int numCUs);
+// CV_OK, or the reason why an encoder description is malformed (recorded as the thread's last error)
+CvResult checkPermutoDesc(const char* who, const CvPermutoDesc* desc);
 // networks of one type T = float (MmaKind::F32) or bfloat16 (MmaKind::Bf16): vectors, weights, biases, results;
 // same limits as launchMlpGeneric
 hipError_t launchMlpFloat(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);

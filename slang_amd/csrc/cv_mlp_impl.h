@@ -96,8 +96,9 @@ __device__ __forceinline__ void carrierFromAcc(const floatx4& acc, const Carrier
     h01 = __builtin_convertvector(a01, halfx2);
     h23 = __builtin_convertvector(a23, halfx2);
     if (c.act == kActLeakyRelu || (SMOOTH && c.act >= kActSigmoid)) {   // leaky: max(z, z*slope) in half, fflayer.slang:64-65
-        h01 = halfx2{activateHalf(h01.x, c.act, c.slope), activateHalf(h01.y, c.act, c.slope)};
-        h23 = halfx2{activateHalf(h23.x, c.act, c.slope), activateHalf(h23.y, c.act, c.slope)};
+        const int act = SMOOTH ? c.act : (int)kActLeakyRelu;      // without SMOOTH the transcendental code is not even compiled
+        h01 = halfx2{activateHalf(h01.x, act, c.slope), activateHalf(h01.y, act, c.slope)};
+        h23 = halfx2{activateHalf(h23.x, act, c.slope), activateHalf(h23.y, act, c.slope)};
     }
     h01 = __builtin_elementwise_max(h01, c.floor2);
     h23 = __builtin_elementwise_max(h23, c.floor2);

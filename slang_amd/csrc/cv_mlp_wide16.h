@@ -99,8 +99,66 @@ __device__ __forceinline__ void interleavePhase()
 // rows).  Up to 32 outputs.  Hidden layers are ReLU; the last layer's activation (none or ReLU)
 // is read from the arguments.  Work distribution as in mlpWideKernel: one workgroup per compute unit, whose waves
 // draw pairs of tiles from a counter in LDS.
-template <int H, int NH, int K0, int WAVES, bool HAS_BIAS>
-__global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
+// Where a pair of tiles gets its first-layer operands from.  This one reads fp16 vectors in contiguous rows:
+//   K0 == 8 : 8 bytes per lane: inputs 4h .. 4h+3 of sample n, the lane's operand of the one k-step as they are;
+//   K0 == 16: 16 bytes: inputs 8h .. 8h+7;  K0 == 32: 32 bytes: inputs 16h .. 16h+15.
+// Rows beyond the end of the batch read the last row instead (their results are not stored).
+template <int K0>
+struct Wide16MemoryFront {
+    static constexpr int NDW = K0 / 4;     // dwords per lane and tile
+    struct Input { uint32_t v[2][NDW]; };
+    const uint8_t* in;
+    __device__ __forceinline__ Input load(uint32_t p, int n, int h, uint32_t lastSample) const
+    {
+        Input x;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint32_t s = (2u * p + (uint32_t)j) * 32u + (uint32_t)n;
+            s = s < lastSample ? s : lastSample;
+            const uint8_t* row = in + (uint64_t)s * (2u * K0) + (uint32_t)h * (uint32_t)K0;
+            if constexpr (K0 == 8) {
+                const u32x2 r = *(const u32x2*)row;
+                x.v[j][0] = r.x; x.v[j][1] = r.y;
+            } else {
+#pragma unroll
+                for (int i = 0; i < NDW / 4; ++i) {
+                    const u32x4 r = *(const u32x4*)(row + 16 * i);
+                    x.v[j][4 * i] = r.x; x.v[j][4 * i + 1] = r.y; x.v[j][4 * i + 2] = r.z; x.v[j][4 * i + 3] = r.w;
+                }
+            }
+        }
+        return x;
+    }
+    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
+    template <int NS>
+    __device__ __forceinline__ void operands(const Input& x, uint32_t (&B)[2][NS][4], int, int) const
+    {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if constexpr (K0 == 8) {
+                B[j][0][0] = x.v[j][0]; B[j][0][1] = x.v[j][1]; B[j][0][2] = 0u; B[j][0][3] = 0u;
+            } else if constexpr (K0 == 16) {
+                // lane (n,0) holds inputs 0..7, lane (n,1) inputs 8..15; k-step s wants 8s + 4h .. 8s + 4h + 3
+#pragma unroll
+                for (int d = 0; d < 2; ++d) {
+                    const u32x2 r = __builtin_amdgcn_permlane32_swap(x.v[j][d], x.v[j][2 + d], false, false);
+                    B[j][0][d] = r.x; B[j][1][d] = r.y;
+                    B[j][0][2 + d] = 0u; B[j][1][2 + d] = 0u;
+                }
+            } else {
+                // lane (n,0) holds inputs 0..15, lane (n,1) inputs 16..31; k-step s wants 16s + 8h .. 16s + 8h + 7
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const u32x2 r = __builtin_amdgcn_permlane32_swap(x.v[j][d], x.v[j][4 + d], false, false);
+                    B[j][0][d] = r.x; B[j][1][d] = r.y;
+                }
+            }
+        }
+    }
+};
+
+template <int H, int NH, int K0, int WAVES, bool HAS_BIAS, class Front>
+__device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& front)
 {
     constexpr int KS = 2 * H;                          // k-steps of a hidden vector
     // k-steps of the input vector, and the inputs per lane and k-step.  The result of a matrix instruction depends on
@@ -180,60 +238,8 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     const bool storeQuads = outDim % 4 == 0 && a.outAlign >= 8u;
     const halfx2 zero2 = {(half_t)0.f, (half_t)0.f};
 
-    // A pair's input, per tile and lane.  Rows beyond the end of the batch read the last row instead (their results
-    // are not stored).
-    //   K0 == 8 : 8 bytes: inputs 4h .. 4h+3 of sample n, the lane's operand of the one k-step as they are;
-    //   K0 == 16: 16 bytes: inputs 8h .. 8h+7;  K0 == 32: 32 bytes: inputs 16h .. 16h+15.
-    constexpr int NDW = K0 / 4;     // dwords per lane and tile
-    struct Input { uint32_t v[2][NDW]; };
-    auto loadPair = [&](uint32_t p) -> Input {
-        Input in;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            uint32_t s = (2u * p + (uint32_t)j) * 32u + (uint32_t)n;
-            s = s < lastSample ? s : lastSample;
-            const uint8_t* row = a.in + (uint64_t)s * (2u * K0) + (uint32_t)h * (uint32_t)K0;
-            if constexpr (K0 == 8) {
-                const u32x2 x = *(const u32x2*)row;
-                in.v[j][0] = x.x; in.v[j][1] = x.y;
-            } else {
-#pragma unroll
-                for (int i = 0; i < NDW / 4; ++i) {
-                    const u32x4 x = *(const u32x4*)(row + 16 * i);
-                    in.v[j][4 * i] = x.x; in.v[j][4 * i + 1] = x.y; in.v[j][4 * i + 2] = x.z; in.v[j][4 * i + 3] = x.w;
-                }
-            }
-        }
-        return in;
-    };
-
     uint32_t B[2][KS > S0 ? KS : S0][4];
     floatx16 acc[2][H];
-    // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second
-    auto firstOperands = [&](const Input& in) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            if constexpr (K0 == 8) {
-                B[j][0][0] = in.v[j][0]; B[j][0][1] = in.v[j][1]; B[j][0][2] = 0u; B[j][0][3] = 0u;
-            } else if constexpr (K0 == 16) {
-                // lane (n,0) holds inputs 0..7, lane (n,1) inputs 8..15; k-step s wants 8s + 4h .. 8s + 4h + 3
-#pragma unroll
-                for (int d = 0; d < 2; ++d) {
-                    const u32x2 r = __builtin_amdgcn_permlane32_swap(in.v[j][d], in.v[j][2 + d], false, false);
-                    B[j][0][d] = r.x; B[j][1][d] = r.y;
-                    B[j][0][2 + d] = 0u; B[j][1][2 + d] = 0u;
-                }
-            } else {
-                // lane (n,0) holds inputs 0..15, lane (n,1) inputs 16..31; k-step s wants 16s + 8h .. 16s + 8h + 7
-#pragma unroll
-                for (int d = 0; d < 4; ++d) {
-                    const u32x2 r = __builtin_amdgcn_permlane32_swap(in.v[j][d], in.v[j][4 + d], false, false);
-                    B[j][0][d] = r.x; B[j][1][d] = r.y;
-                }
-            }
-        }
-    };
-
     const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // (the lane's offset passes through an empty asm statement once per round of the loop: the lines are the same for
     // every tile, and the optimiser would otherwise keep all of them in registers, which the weights need)
@@ -321,14 +327,14 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     constexpr int NV = 16 * H;      // vector-ALU instructions of one tile's carrier
     constexpr int NL = HAS_BIAS ? 4 * H : 0;
     auto endPhase = []() { __builtin_amdgcn_sched_barrier(0); };
-    Input in = loadPair(pair);
+    typename Front::Input in = front.load(pair, n, h, lastSample);
     seedLayer(0, 0);
     seedLayer(0, 1);
     while (true) {
         const uint32_t next = claim();
         if constexpr (HAS_BIAS) asm volatile("" : "+v"(seedOff[0]), "+v"(seedOff[1]));
-        firstOperands(in);
-        in = loadPair(next < numPairs ? next : numPairs - 1u);      // beyond the end: loaded again, never used
+        front.operands(in, B, n, h);
+        in = front.load(next < numPairs ? next : numPairs - 1u, n, h, lastSample);      // beyond the end: loaded again, never used
         firstLayer(0);
         endPhase();
         firstLayer(1); carrier(0); seedLayer(1, 0);
@@ -350,16 +356,28 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
     }
 }
 
+template <int H, int NH, int K0, int WAVES, bool HAS_BIAS>
+__global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
+{
+    mlpWide16Body<H, NH, K0, WAVES, HAS_BIAS>(a, Wide16MemoryFront<K0>{a.in});
+}
+
+// waves per workgroup (one workgroup per compute unit): as many as the weights leave registers for
+// (16 waves: 128 registers each, 12: 168, 8: 256); the build fails if an instantiation spills
+template <int H, int NH, int K0>
+constexpr int wide16Waves()
+{
+    constexpr int KS = 2 * H, S0 = K0 == 8 ? 1 : 2;
+    constexpr int WREGS = 4 * (H * S0 + (NH - 1) * H * KS + KS);
+    return (WREGS + 48 * H + 32 <= 128) ? 16 : ((WREGS + 48 * H + 32 <= 168) ? 12 : 8);
+}
+
 // Shapes: fp16 vectors of 8, 16 or 32 elements in contiguous rows at a 16-byte aligned address, ReLU hidden layers of
 // exactly 32 or 64 units (one to four of them), at most 32 outputs (checked by the dispatcher in cv_mlp_f16.hip).
 template <int H, int NH, int K0, bool HAS_BIAS>
 hipError_t launchMlpWide16Shape(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
-    // one workgroup per compute unit, as many waves as the weights leave registers for
-    // (16 waves: 128 registers each, 12: 168, 8: 256); the build fails if an instantiation spills
-    constexpr int KS = 2 * H, S0 = K0 == 8 ? 1 : 2;
-    constexpr int WREGS = 4 * (H * S0 + (NH - 1) * H * KS + KS);
-    constexpr int WAVES = (WREGS + 48 * H + 32 <= 128) ? 16 : ((WREGS + 48 * H + 32 <= 168) ? 12 : 8);
+    constexpr int WAVES = wide16Waves<H, NH, K0>();
     const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
     const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
     noteKernel(false, "mlpWide16Kernel<f16,32x32x16,inputs=%d,hidden=%dx%d,%s,waves=%d>", K0, NH, 32 * H,

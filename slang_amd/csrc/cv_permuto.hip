@@ -14,7 +14,9 @@
 
 #include "cv_device.h"
 #include "cv_error.h"
+#include "cv_kernels.h"
 #include "cv_launch.h"
+#include "cv_permuto_impl.h"
 
 namespace cv {
 namespace {
@@ -106,79 +108,6 @@ struct PermutoArgs {
     uint32_t batch;
 };
 
-// elevated point, closest remainder-0 point and rank of one position on one level (:74-152)
-template <int D>
-__device__ __forceinline__ void latticeGeometry(const float* pos, const CvPermutoLevelInfo& lv, float* elevated, int* rem0, int* rank)
-{
-    float sum = 0.0f;
-#pragma unroll
-    for (int dim = D - 1; dim >= 0; --dim) {
-        const float cf = (pos[dim] + lv.shiftsPerDim[dim]) * lv.scalesPerDim[dim];
-        elevated[dim + 1] = sum - (float)(dim + 1) * cf;
-        sum += cf;
-    }
-    elevated[0] = sum;
-    int isum = 0;
-#pragma unroll
-    for (int dim = 0; dim <= D; ++dim) {
-        rank[dim] = 0;
-        const float v = elevated[dim] * (1.0f / (float)(D + 1));
-        const float up = ceilf(v) * (float)(D + 1), down = floorf(v) * (float)(D + 1);
-        rem0[dim] = (up - elevated[dim] < elevated[dim] - down) ? (int)up : (int)down;
-        isum += rem0[dim];
-    }
-    isum /= (D + 1);
-#pragma unroll
-    for (int dim = 0; dim < D; ++dim) {
-        const float di = elevated[dim] - (float)rem0[dim];
-#pragma unroll
-        for (int other = dim + 1; other <= D; ++other) {
-            if (di < elevated[other] - (float)rem0[other]) rank[dim]++;
-            else rank[other]++;
-        }
-    }
-#pragma unroll
-    for (int dim = 0; dim <= D; ++dim) {
-        rank[dim] += isum;
-        if (rank[dim] < 0) { rank[dim] += D + 1; rem0[dim] += D + 1; }
-        else if (rank[dim] > D) { rank[dim] -= D + 1; rem0[dim] -= D + 1; }
-    }
-}
-
-// barycentric[k] of the remainder-k vertex (:166-179), without indexing registers by a run-time value
-template <int D>
-__device__ __forceinline__ void barycentricWeights(const float* elevated, const int* rem0, const int* rank, float* bary)
-{
-#pragma unroll
-    for (int i = 0; i <= D + 1; ++i) bary[i] = 0.0f;
-#pragma unroll
-    for (int dim = 0; dim <= D; ++dim) {
-        const float delta = (elevated[dim] - (float)rem0[dim]) * (1.0f / (float)(D + 1));
-#pragma unroll
-        for (int i = 0; i <= D + 1; ++i) {
-            if (i == D - rank[dim]) bary[i] += delta;
-            if (i == D + 1 - rank[dim]) bary[i] -= delta;
-        }
-    }
-    bary[0] += 1.0f + bary[D + 1];
-}
-
-template <int D>
-__device__ __forceinline__ uint32_t vertexIndex(const CvPermutoLevelInfo& lv, int F, const int* rem0, const int* rank, int k)
-{
-    uint32_t key[D];
-#pragma unroll
-    for (int dim = 0; dim < D; ++dim) {                                // :296-304
-        key[dim] = (uint32_t)(rem0[dim] + k);
-        if (rank[dim] > D - k) key[dim] -= (uint32_t)(D + 1);
-    }
-    // (a table of 2^n entries, which is what prepareLevelInfo makes, is indexed with a mask: the general remainder
-    // is a division by a run-time value, some forty instructions per vertex)
-    const uint32_t hash = baseConvertHash(key, D), size = lv.featureTableSize;
-    const uint32_t slot = (size & (size - 1u)) == 0u ? (hash & (size - 1u)) : hash % size;
-    return lv.offsetOfFeatureTable * (uint32_t)F + slot * (uint32_t)F;
-}
-
 template <typename T, int D>
 __global__ __launch_bounds__(256) void permutoEncodeKernel(const PermutoArgs a)
 {
@@ -199,20 +128,59 @@ __global__ __launch_bounds__(256) void permutoEncodeKernel(const PermutoArgs a)
         int rem0[D + 1], rank[D + 1];
         latticeGeometry<D>(pos, lv, elevated, rem0, rank);
         barycentricWeights<D>(elevated, rem0, rank, bary);
+        uint32_t idx[D + 1];
+        vertexIndices<D>(lv, F, rem0, rank, idx);
         for (int f0 = 0; f0 < F; f0 += 4) {                            // four features of the entry at a time
             T acc[4] = {(T)0.f, (T)0.f, (T)0.f, (T)0.f};
 #pragma unroll
             for (int k = 0; k <= D; ++k) {
-                const uint32_t idx = vertexIndex<D>(lv, F, rem0, rank, k);
                 const T w = (T)bary[k];
 #pragma unroll
                 for (int f = 0; f < 4; ++f)
-                    if (f0 + f < F) acc[f] = (T)(acc[f] + (T)(w * table[idx + f0 + f]));    // in T, vertex by vertex (:312-316)
+                    if (f0 + f < F) acc[f] = (T)(acc[f] + (T)(w * table[idx[k] + f0 + f]));    // in T, vertex by vertex (:312-316)
             }
 #pragma unroll
             for (int f = 0; f < 4; ++f)
                 if (f0 + f < F) o[f0 + f] = acc[f];
         }
+    }
+}
+
+// The same encoding with one thread per (position, level), the level running fastest: a wave's 64 results are
+// consecutive in memory (one thread per position writes F elements at the pitch of a whole row, which the memory
+// system does not merge: 2.1 bytes written per byte of output), no thread loops over levels, and a feature table that
+// fits is held in LDS, where a gather of 64 scattered entries costs a few cycles instead of one cache line per lane.
+// The arithmetic per (position, level) is that of permutoEncodeKernel, instruction for instruction.
+template <typename T, int D, int F, bool LDS_TABLE>
+__global__ __launch_bounds__(1024) void permutoEncodePairsKernel(const PermutoArgs a, uint32_t tableElems, uint32_t levelShift)
+{
+    typedef typename PermutoEntry<T, F>::type Entry;
+    extern __shared__ __align__(16) uint8_t ldsRaw[];
+    CvPermutoLevelInfo* levels = (CvPermutoLevelInfo*)ldsRaw;
+    const T* ldsTable = (const T*)(ldsRaw + kMaxLevels * sizeof(CvPermutoLevelInfo));
+    const uint32_t L = a.desc.maxLevels;
+    {
+        constexpr uint32_t words = sizeof(CvPermutoLevelInfo) / 4u;
+        const uint32_t* src = (const uint32_t*)a.desc.levelInfo;
+        for (uint32_t i = threadIdx.x; i < L * words; i += blockDim.x) ((uint32_t*)levels)[i] = src[i];
+        if constexpr (LDS_TABLE) {
+            const Entry* t = (const Entry*)a.table;
+            Entry* dst = (Entry*)(ldsRaw + kMaxLevels * sizeof(CvPermutoLevelInfo));
+            for (uint32_t i = threadIdx.x; i < tableElems / (uint32_t)F; i += blockDim.x) dst[i] = t[i];
+        }
+    }
+    __syncthreads();
+    const T* table = LDS_TABLE ? ldsTable : (const T*)a.table;
+    const uint64_t pairs = (uint64_t)a.batch * L;
+    for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += (uint64_t)gridDim.x * blockDim.x) {
+        const uint32_t s = levelShift < 32u ? (uint32_t)(p >> levelShift) : (uint32_t)(p / L);
+        const uint32_t l = (uint32_t)(p - (uint64_t)s * L);
+        const CvPermutoLevelInfo& lv = levels[l];
+        float pos[D];
+#pragma unroll
+        for (int d = 0; d < D; ++d) pos[d] = (float)((const T*)(a.pos + (size_t)s * a.posStride))[d];
+        const Entry acc = permutoEncodeEntry<T, D, F>(pos, lv, table, a.desc.maxLevel);
+        *(Entry*)((T*)(a.out + (size_t)s * a.outStride) + lv.currentLevelIndex * F) = acc;
     }
 }
 
@@ -237,12 +205,13 @@ __device__ __forceinline__ void permutoBackwardOne(const PermutoArgs& a, uint32_
 #pragma unroll
         for (int i = 0; i <= D + 1; ++i) dbary[i] = 0.f;
         const float* gl = g + lv.currentLevelIndex * F;
+        uint32_t idx[D + 1];
+        vertexIndices<D>(lv, F, rem0, rank, idx);
 #pragma unroll
         for (int k = 0; k <= D; ++k) {
-            const uint32_t idx = vertexIndex<D>(lv, F, rem0, rank, k);
             for (int f = 0; f < F; ++f) {
-                if (dTable) atomicAdd(dTable + idx + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
-                dbary[k] += table[idx + f] * gl[f];
+                if (dTable) atomicAdd(dTable + idx[k] + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
+                dbary[k] += table[idx[k] + f] * gl[f];
             }
         }
         if (!a.dPos) continue;
@@ -299,9 +268,67 @@ __global__ __launch_bounds__(256) void permutoBackwardLdsKernel(const PermutoArg
     }
 }
 
+// the table as the levels lay it out: offsets and sizes in entries, F elements per entry
+uint64_t tableElements(const CvPermutoDesc& d)
+{
+    uint64_t n = 0;
+    for (uint32_t l = 0; l < d.maxLevels; ++l) {
+        const uint64_t e = ((uint64_t)d.levelInfo[l].offsetOfFeatureTable + d.levelInfo[l].featureTableSize) * (uint64_t)d.featureDimensionPerEntry;
+        n = e > n ? e : n;
+    }
+    return n;
+}
+
+constexpr size_t kPairsLevelBytes = kMaxLevels * sizeof(CvPermutoLevelInfo);
+constexpr size_t kPairsTableBytes = 144 * 1024;      // with the level records: within the 160 KB of a compute unit
+
+template <typename T, int D, int F>
+hipError_t launchEncodePairs(hipStream_t stream, const PermutoArgs& a)
+{
+    const uint64_t tableElems = tableElements(a.desc);
+    const bool inLds = tableElems * sizeof(T) <= kPairsTableBytes;
+    const size_t lds = kPairsLevelBytes + (inLds ? (size_t)tableElems * sizeof(T) : 0);
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    const uint64_t pairs = (uint64_t)a.batch * a.desc.maxLevels, want = (pairs + 1023u) / 1024u;
+    const uint64_t cap = (uint64_t)cus * (lds <= 80 * 1024 ? 2u : 1u);
+    const dim3 grid((uint32_t)(want < cap ? want : cap)), block(1024);
+    const uint32_t L = a.desc.maxLevels;
+    const uint32_t shift = (L & (L - 1u)) == 0u ? (uint32_t)__builtin_ctz(L) : 0xffffffffu;
+    hipError_t e;
+    if (inLds) {
+        e = allowDynamicLds<permutoEncodePairsKernel<T, D, F, true>>((int)(kPairsLevelBytes + kPairsTableBytes));
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((permutoEncodePairsKernel<T, D, F, true>), grid, block, lds, stream, a, (uint32_t)tableElems, shift);
+    } else {
+        hipLaunchKernelGGL((permutoEncodePairsKernel<T, D, F, false>), grid, block, lds, stream, a, (uint32_t)tableElems, shift);
+    }
+    return hipGetLastError();
+}
+
+// the kernel above takes entries of 4, 8 or 16 bytes at addresses that are multiples of their size
+template <typename T>
+bool pairsEligible(const PermutoArgs& a)
+{
+    const size_t eb = (size_t)a.desc.featureDimensionPerEntry * sizeof(T);
+    const int F = a.desc.featureDimensionPerEntry;
+    if (a.desc.dimensions > 4 || (F != 1 && F != 2 && F != 4 && F != 8) || eb > 16) return false;
+    return (uintptr_t)a.table % eb == 0 && (uintptr_t)a.out % eb == 0 && a.outStride % eb == 0 && tableElements(a.desc) <= 0xffffffffull;
+}
+
 template <typename T>
 hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
 {
+    if (pairsEligible<T>(a)) {
+        noteKernel(false, "permutoEncodePairsKernel<%s,D=%d,F=%d>", sizeof(T) == 4 ? "f32" : "f16", a.desc.dimensions, a.desc.featureDimensionPerEntry);
+        switch (a.desc.dimensions * 16 + a.desc.featureDimensionPerEntry) {
+#define CV_DF(N, G) case N * 16 + G: if constexpr (G * sizeof(T) <= 16) return launchEncodePairs<T, N, G>(stream, a); break;
+        CV_DF(1, 1) CV_DF(1, 2) CV_DF(1, 4) CV_DF(1, 8) CV_DF(2, 1) CV_DF(2, 2) CV_DF(2, 4) CV_DF(2, 8)
+        CV_DF(3, 1) CV_DF(3, 2) CV_DF(3, 4) CV_DF(3, 8) CV_DF(4, 1) CV_DF(4, 2) CV_DF(4, 4) CV_DF(4, 8)
+#undef CV_DF
+        }
+    }
+    noteKernel(false, "permutoEncodeKernel<%s,D=%d>", sizeof(T) == 4 ? "f32" : "f16", a.desc.dimensions);
     const dim3 grid((a.batch + 255) / 256), block(256);
     switch (a.desc.dimensions) {
 #define CV_D(N) case N: hipLaunchKernelGGL((permutoEncodeKernel<T, N>), grid, block, 0, stream, a); break;
@@ -314,12 +341,7 @@ hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
 
 hipError_t launchBackward(hipStream_t stream, const PermutoArgs& a)
 {
-    // the table as the levels lay it out: offsets and sizes in entries, F floats per entry
-    uint64_t tableElems = 0;
-    for (uint32_t l = 0; l < a.desc.maxLevels; ++l) {
-        const uint64_t e = ((uint64_t)a.desc.levelInfo[l].offsetOfFeatureTable + a.desc.levelInfo[l].featureTableSize) * (uint64_t)a.desc.featureDimensionPerEntry;
-        tableElems = e > tableElems ? e : tableElems;
-    }
+    const uint64_t tableElems = tableElements(a.desc);
     constexpr uint64_t kLdsTableBytes = 64 * 1024;
     if (a.dTable && tableElems * 4 <= kLdsTableBytes && a.batch >= 4096u) {
         int dev = 0, cus = 256;
@@ -350,7 +372,9 @@ hipError_t launchBackward(hipStream_t stream, const PermutoArgs& a)
     return hipGetLastError();
 }
 
-CvResult checkDesc(const char* who, const CvPermutoDesc* d)
+} // namespace
+
+CvResult checkPermutoDesc(const char* who, const CvPermutoDesc* d)
 {
     if (!d) return failWith(CV_E_INVALID_ARG, "%s: desc is null", who);
     if (d->dimensions < 1 || d->dimensions > kMaxDims) return failWith(CV_E_INVALID_ARG, "%s: dimensions=%d (1..%d)", who, d->dimensions, kMaxDims);
@@ -365,7 +389,6 @@ CvResult checkDesc(const char* who, const CvPermutoDesc* d)
     return CV_OK;
 }
 
-} // namespace
 } // namespace cv
 
 extern "C" {
@@ -419,7 +442,7 @@ CV_API CvResult cvPermutoEncode(void* stream, const CvPermutoDesc* desc, const v
                                 const void* featureTable, void* out, size_t outStride, uint32_t batch)
 {
     using namespace cv;
-    CvResult rc = checkDesc("cvPermutoEncode", desc);
+    CvResult rc = checkPermutoDesc("cvPermutoEncode", desc);
     if (CV_FAILED(rc)) return rc;
     if (batch == 0) return CV_OK;
     const uint32_t esz = desc->elementType == CV_FLOAT32 ? 4u : 2u;
@@ -433,7 +456,6 @@ CV_API CvResult cvPermutoEncode(void* stream, const CvPermutoDesc* desc, const v
     a.desc = *desc;
     a.pos = (const uint8_t*)positions; a.posStride = positionStride; a.table = (const uint8_t*)featureTable;
     a.out = (uint8_t*)out; a.outStride = outStride; a.batch = batch;
-    noteKernel(false, "permutoEncodeKernel<%s,D=%d>", esz == 4 ? "f32" : "f16", desc->dimensions);
     const hipError_t e = esz == 4 ? launchEncode<float>((hipStream_t)stream, a) : launchEncode<half_t>((hipStream_t)stream, a);
     if (e != hipSuccess) return failWith(CV_E_INTERNAL_FAIL, "cvPermutoEncode launch: %s", hipGetErrorString(e));
     return CV_OK;
@@ -444,7 +466,7 @@ CV_API CvResult cvPermutoEncodeBackward(void* stream, const CvPermutoDesc* desc,
                                         void* dPositions, size_t dPositionStride, void* dFeatureTable, uint32_t batch)
 {
     using namespace cv;
-    CvResult rc = checkDesc("cvPermutoEncodeBackward", desc);
+    CvResult rc = checkPermutoDesc("cvPermutoEncodeBackward", desc);
     if (CV_FAILED(rc)) return rc;
     if (desc->elementType != CV_FLOAT32)
         return failWith(CV_E_NOT_AVAILABLE, "cvPermutoEncodeBackward: FLOAT32 data only (the table gradient is accumulated with fp32 atomic adds)");

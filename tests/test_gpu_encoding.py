@@ -154,6 +154,37 @@ def test_permuto_encoder_against_oracle(D, F, levels_n):
     assert np.array_equal(o16, ob.permuto_encode(levels, F, max_level, p16, t16))
 
 
+@pytest.mark.parametrize("D,F,levels_n,log2", [(2, 2, 5, 8), (3, 8, 3, 6), (4, 1, 7, 12), (2, 4, 16, 4), (3, 2, 8, 14), (5, 4, 2, 9)])
+def test_permuto_encoder_kernel_choices(D, F, levels_n, log2):
+    # one thread per (position, level) with the table in LDS or in memory, level counts that are no power of two,
+    # positions outside the unit cube, output rows at a pitch, and the one-thread-per-position kernel for what the
+    # other does not take (more than four dimensions, entries over 16 bytes, unaligned buffers): all bit for bit the oracle
+    rng = np.random.default_rng(D * 1000 + F * 10 + levels_n)
+    levels = ob.permuto_levels(D, log2, levels_n, 1.5, 0.7, 99)
+    max_level = float(np.float32(1.1) * np.float32(levels_n))
+    B = 3001
+    pos = rng.uniform(-4, 4, (B, D)).astype(np.float32)
+    for dt, npdt in ((torch.float32, np.float32), (torch.float16, np.float16)):
+        enc = cv.PermutoEncoder(D, F, log2, levels_n, baseScale=1.5, log2PerLevelScale=0.7, maxLevelRatio=1.1, seed=99, dtype=dt)
+        p, t = pos.astype(npdt), rng.standard_normal(enc.featureTableElements).astype(npdt)
+        want = ob.permuto_encode(levels, F, max_level, p, t)
+        out = enc.encode(to_dev(p), to_dev(t))
+        name = cv.lastKernelName()
+        pairs = D <= 4 and F * np.dtype(npdt).itemsize <= 16
+        assert name.startswith("permutoEncodePairsKernel" if pairs else "permutoEncodeKernel"), name
+        assert np.array_equal(out.cpu().numpy(), want)
+        # rows at a pitch of one extra entry; then a table that starts one element into its allocation
+        wide = torch.zeros(B, levels_n * F + F, dtype=dt, device=DEV)
+        enc.encode(to_dev(p), to_dev(t), out=wide[:, :levels_n * F])
+        assert np.array_equal(wide[:, :levels_n * F].cpu().numpy(), want) and not wide[:, levels_n * F:].any()
+        shifted = torch.zeros(t.size + 1, dtype=dt, device=DEV)
+        shifted[1:] = to_dev(t)
+        out2 = enc.encode(to_dev(p), shifted[1:])
+        assert np.array_equal(out2.cpu().numpy(), want)
+        if F > 1:
+            assert cv.lastKernelName().startswith("permutoEncodeKernel"), cv.lastKernelName()
+
+
 def test_encoder_feeds_the_mlp():
     # encode positions, run the decoder MLP on the fp16 features: the neural-texture shape
     rng = np.random.default_rng(8)
@@ -167,3 +198,63 @@ def test_encoder_feeds_the_mlp():
     y = cv.mlpForward(layers, feats)
     ref = ob.ref_mlp_forward(specs, feats.cpu().numpy(), ob.F16)
     assert (np.abs(y.cpu().numpy().astype(np.float32) - ref.astype(np.float32)) <= 2e-2 * np.abs(ref.astype(np.float32)) + 2e-2).mean() > 0.999
+
+
+@pytest.mark.parametrize("D,F,levels_n,log2,dims,B,kernel", [
+    (3, 2, 8, 12, [16, 64, 64, 3], 4099, "permutoWide16Kernel"),     # the neural-texture shape; table (128 KB) and network in LDS
+    (2, 2, 16, 8, [32, 32, 4], 777, "permutoWide16Kernel"),
+    (4, 2, 8, 10, [16, 64, 8], 64, "permutoWide16Kernel"),
+    (3, 2, 16, 11, [32, 64, 64, 1], 3000, "permutoWide16Kernel"),
+    (2, 4, 4, 8, [16, 32, 5], 17, "permutoMlpKernel"),               # four features per entry
+    (4, 1, 12, 10, [12, 128, 128, 7], 1000, "permutoMlpKernel"),     # 128-wide layers; a first layer narrower than its 16-column tile
+    (3, 2, 8, 15, [16, 64, 64, 3], 2500, "permutoMlpKernel"),        # a 1 MB table stays in memory
+    (1, 2, 16, 6, [32, 48, 16, 1], 1, "permutoMlpKernel"),
+])
+def test_encoder_and_network_in_one_kernel(D, F, levels_n, log2, dims, B, kernel):
+    # cvPermutoMlpForward == cvPermutoEncode followed by cvMlpForward, bit for bit, on the 32-sample-tile kernel where the
+    # decoder allows it and on the run-time-size kernel otherwise (or when asked for)
+    rng = np.random.default_rng(D * 100 + F * 10 + len(dims))
+    enc = cv.PermutoEncoder(D, F, log2, levels_n, baseScale=2.0, log2PerLevelScale=0.9, maxLevelRatio=0.9, seed=5, dtype=torch.float16)
+    pos = to_dev(rng.uniform(-1, 2, (B, D)).astype(np.float16))
+    table = to_dev((rng.standard_normal(enc.featureTableElements) * 0.5).astype(np.float16))
+    specs = make_specs(rng, dims)
+    if kernel == "permutoMlpKernel":
+        specs[0]["act"], specs[0]["slope"] = 2, float(np.float16(0.01))      # a leaky layer among the ReLU ones
+    layers = build(specs)
+    feats = enc.encode(pos, table)
+    want = cv.mlpForward(layers, feats)
+    got = enc.encodeAndEval(pos, table, layers)
+    name = cv.lastKernelName()
+    assert name.startswith(kernel + "<D=%d,F=%d" % (D, F)), name
+    if kernel == "permutoMlpKernel":
+        assert name.endswith("memory>" if log2 == 15 else "LDS>"), name
+    assert torch.equal(got, want)
+    got16 = enc.encodeAndEval(pos, table, layers, flags=cv.FLAG_FORWARD_TILE16)
+    assert cv.lastKernelName().startswith("permutoMlpKernel"), cv.lastKernelName()
+    assert torch.equal(got16, want)
+    levels = ob.permuto_levels(D, log2, levels_n, 2.0, 0.9, 5)
+    max_level = float(np.float32(0.9) * np.float32(levels_n))
+    f_ref = ob.permuto_encode(levels, F, max_level, pos.cpu().numpy(), table.cpu().numpy())
+    assert np.array_equal(feats.cpu().numpy(), f_ref)
+    # rows of the result at a pitch
+    wide = torch.full((B, dims[-1] + 3), 7.0, dtype=torch.float16, device=DEV)
+    enc.encodeAndEval(pos, table, layers, out=wide[:, :dims[-1]])
+    assert torch.equal(wide[:, :dims[-1]], want) and bool((wide[:, dims[-1]:] == 7.0).all())
+
+
+def test_encoder_and_network_argument_checks():
+    rng = np.random.default_rng(3)
+    enc = cv.PermutoEncoder(3, 2, 8, 4, baseScale=1.0, log2PerLevelScale=1.0, dtype=torch.float16)
+    pos = to_dev(rng.uniform(0, 1, (8, 3)).astype(np.float16))
+    table = to_dev(rng.standard_normal(enc.featureTableElements).astype(np.float16))
+    with pytest.raises(cv.CoopVecError) as e:          # first layer does not match the encoder's output
+        enc.encodeAndEval(pos, table, build(make_specs(rng, [16, 32, 4])))
+    assert e.value.result == cv.SLANG_E_INVALID_ARG
+    with pytest.raises(cv.CoopVecError) as e:          # a single layer is not a network
+        enc.encodeAndEval(pos, table, build(make_specs(rng, [8, 4])))
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+    enc5 = cv.PermutoEncoder(5, 2, 8, 4, baseScale=1.0, log2PerLevelScale=1.0, dtype=torch.float16)
+    with pytest.raises(cv.CoopVecError) as e:          # five dimensions: the two-call form
+        enc5.encodeAndEval(to_dev(rng.uniform(0, 1, (8, 5)).astype(np.float16)),
+                           to_dev(rng.standard_normal(enc5.featureTableElements).astype(np.float16)), build(make_specs(rng, [8, 16, 4])))
+    assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
