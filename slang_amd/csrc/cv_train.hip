@@ -41,7 +41,11 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ta.lossScale = t.lossScale;
     ta.partials = t.workspace;
     ta.wantLossMax = t.lossMax ? 1 : 0;
-    const uint32_t blocks = (uint32_t)numCUs;      // one resident workgroup per compute unit
+    // one resident workgroup per compute unit, fewer when the batch has less work than that: a workgroup takes four
+    // 16-sample tiles (on 64-wide networks four 32-sample rounds) at a time, and every workgroup launched writes a
+    // partial that the second kernel reads (the example's 16 samples: one workgroup instead of 256)
+    const uint32_t units = Net::HT == 4 ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
+    const uint32_t blocks = units < (uint32_t)numCUs ? (units ? units : 1u) : (uint32_t)numCUs;
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
