@@ -46,6 +46,24 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // partial that the second kernel reads (the example's 16 samples: one workgroup instead of 256)
     const uint32_t units = Net::HT == 4 ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
     const uint32_t blocks = units < (uint32_t)numCUs ? (units ? units : 1u) : (uint32_t)numCUs;
+    TrainReduceArgs ra;
+    for (int l = 0; l < Net::L; ++l) {
+        ra.layers[l].wGrad = t.wGrad[l];
+        ra.layers[l].bGrad = t.bGrad[l];
+        ra.layers[l].gradShape = t.gradShape[l];
+        ra.layers[l].in = t.mlp.layers[l].in;
+        ra.layers[l].out = t.mlp.layers[l].out;
+    }
+    ra.numLayers = Net::L;
+    ra.gradCt = t.gradCt;
+    ra.partials = t.workspace;
+    ra.numPartials = blocks;
+    ra.lossSum = t.lossSum;
+    ra.lossMax = t.lossMax;
+    constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
+    // a launch of one workgroup of the one-wave-per-SIMD kernel finishes the step itself
+    ta.finishInKernel = (blocks == 1 && Net::HT != 4) ? 1 : 0;
+    ta.finish = ra;
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
@@ -71,21 +89,7 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     if (variant == 0) hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    TrainReduceArgs ra;
-    for (int l = 0; l < Net::L; ++l) {
-        ra.layers[l].wGrad = t.wGrad[l];
-        ra.layers[l].bGrad = t.bGrad[l];
-        ra.layers[l].gradShape = t.gradShape[l];
-        ra.layers[l].in = t.mlp.layers[l].in;
-        ra.layers[l].out = t.mlp.layers[l].out;
-    }
-    ra.numLayers = Net::L;
-    ra.gradCt = t.gradCt;
-    ra.partials = t.workspace;
-    ra.numPartials = blocks;
-    ra.lossSum = t.lossSum;
-    ra.lossMax = t.lossMax;
-    constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
+    if (ta.finishInKernel) return hipSuccess;
     hipLaunchKernelGGL((mlpTrainReduceKernel<Net>), dim3((total + 63) / 64), dim3(64 * kReduceWaves), 0, stream, ra);
     return hipGetLastError();
 }

@@ -68,15 +68,6 @@ struct TrainNet : UniformNet<KT0_, HT_, NHID_, MTL_> {
     static constexpr int partialFloats = totalGradTiles * 256 + totalDbTiles * 16 + 16;
 };
 
-struct TrainArgs {
-    MlpArgs mlp;                 // layers, input, batch (out/outStride unused)
-    const uint8_t* targets;      // fp16 [batch][lastOut] or nullptr: sin(sum of the inputs)
-    uint64_t targetStride;
-    float lossScale;
-    float* partials;             // [gridDim.x][partialFloats]
-    int32_t wantLossMax;         // also track the largest per-sample loss (slot 1 behind the loss sum of a partial)
-};
-
 struct TrainReduceArgs {
     struct Layer {
         uint8_t* wGrad; uint8_t* bGrad;
@@ -90,6 +81,20 @@ struct TrainReduceArgs {
     float* lossSum;              // optional
     float* lossMax;              // optional
 };
+
+struct TrainArgs {
+    MlpArgs mlp;                 // layers, input, batch (out/outStride unused)
+    const uint8_t* targets;      // fp16 [batch][lastOut] or nullptr: sin(sum of the inputs)
+    uint64_t targetStride;
+    float lossScale;
+    float* partials;             // [gridDim.x][partialFloats]
+    int32_t wantLossMax;         // also track the largest per-sample loss (slot 1 behind the loss sum of a partial)
+    // A launch of a single workgroup (a batch of at most four tiles, such as the example's 16 samples) adds its partial to
+    // the gradients itself: no second kernel.  `finish` then holds what that kernel would have been given.
+    int32_t finishInKernel;
+    TrainReduceArgs finish;
+};
+
 
 // The largest per-sample loss of a workgroup, kept as the bits of a non-negative float (whose order is that of the
 // integers; a NaN compares above everything, so it wins).  A maximum does not depend on the order of its operands: the
@@ -652,6 +657,58 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1] = __builtin_bit_cast(float, ldsLossMax);
         }
     }
+    if (!ta.finishInKernel) return;
+    // ---- the only workgroup of the launch: what mlpTrainReduceKernel would do with this one partial --------------
+    __threadfence_block();
+    __syncthreads();
+    constexpr uint32_t nValues = Net::totalGradTiles * 256 + Net::totalDbTiles * 16;
+    const TrainReduceArgs& ra = ta.finish;
+    const float lossPart = part[nValues];
+    const bool voidStep = lossPart != lossPart;                  // see mlpTrainReduceKernel
+    for (uint32_t p = threadIdx.x; p <= nValues; p += 256u) {
+        float s = 0.f + part[p];                                   // the sum of one partial, as sumPartials forms it
+        if (voidStep) s = __builtin_nanf("");
+        if (p == nValues) {
+            if (ra.lossSum) *ra.lossSum = s;
+        } else {
+            addToGradients<Net>(ra, p, s);
+        }
+    }
+    if (ra.lossMax && threadIdx.x == 0) *ra.lossMax = voidStep ? __builtin_nanf("") : part[nValues + 1];
+}
+
+// Adds value p of a step's summed partial (dW tiles in accumulator order, then db tiles) to the element of the gradient
+// buffers it belongs to ("+=", any layout, fp16 or fp32).
+template <class Net>
+__device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32_t p, float s)
+{
+    constexpr int L = Net::L;
+    constexpr uint32_t nW = Net::totalGradTiles * 256;
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
+        constexpr uint32_t w0 = Net::gradTileBase(l) * 256, w1 = w0 + MTO * NI * 256;
+        constexpr uint32_t b0 = nW + Net::dbTileBase(l) * 16, b1 = b0 + MTO * 16;
+        const TrainReduceArgs::Layer& ly = ra.layers[l];
+        if (p >= w0 && p < w1) {
+            const uint32_t q = p - w0, tile = q >> 8, ln = (q >> 2) & 63u, r = q & 3u;
+            const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
+            const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
+            const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
+            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) {
+                uint8_t* d = ly.wGrad + elemOffset(ly.gradShape, o, i);
+                if (ra.gradCt == kF32) *(float*)d += s;
+                else *(half_t*)d = (half_t)((float)*(half_t*)d + s);
+            }
+        } else if (p >= b0 && p < b1) {
+            const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
+            const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
+            if (ly.bGrad && o < (uint32_t)ly.out) {
+                if (ra.gradCt == kF32) ((float*)ly.bGrad)[o] += s;
+                else ((half_t*)ly.bGrad)[o] = (half_t)((float)((half_t*)ly.bGrad)[o] + s);
+            }
+        }
+    });
 }
 
 // Sums the workgroup partials in a fixed order and adds them to the gradient buffers.
@@ -688,31 +745,7 @@ __global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const 
         if (ra.lossSum) *ra.lossSum = s;
         return;
     }
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
-        constexpr uint32_t w0 = Net::gradTileBase(l) * 256, w1 = w0 + MTO * NI * 256;
-        constexpr uint32_t b0 = nW + Net::dbTileBase(l) * 16, b1 = b0 + MTO * 16;
-        const TrainReduceArgs::Layer& ly = ra.layers[l];
-        if (p >= w0 && p < w1) {
-            const uint32_t q = p - w0, tile = q >> 8, ln = (q >> 2) & 63u, r = q & 3u;
-            const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
-            const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
-            const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
-            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) {
-                uint8_t* d = ly.wGrad + elemOffset(ly.gradShape, o, i);
-                if (ra.gradCt == kF32) *(float*)d += s;
-                else *(half_t*)d = (half_t)((float)*(half_t*)d + s);
-            }
-        } else if (p >= b0 && p < b1) {
-            const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
-            const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
-            if (ly.bGrad && o < (uint32_t)ly.out) {
-                if (ra.gradCt == kF32) ((float*)ly.bGrad)[o] += s;
-                else ((half_t*)ly.bGrad)[o] = (half_t)((float)((half_t*)ly.bGrad)[o] + s);
-            }
-        }
-    });
+    addToGradients<Net>(ra, p, s);
 }
 
 } // namespace
