@@ -98,12 +98,14 @@ hipError_t launchPermutoWide16Shape(hipStream_t stream, const PermutoWideArgs& p
     // is in the matrix pipeline.  The build fails if an instantiation spills.
     constexpr int WAVES = H == 1 ? 16 : (NH == 1 ? 12 : 8);
     auto kernel = permutoWide16Kernel<H, NH, K0, WAVES, D, F>;
-    hipFuncAttributes attr;
-    hipError_t e = hipFuncGetAttributes(&attr, (const void*)kernel);
-    if (e != hipSuccess) return e;
+    // LDS the kernel declares itself (weights in operand order, biases): a property of the instantiation, asked once
+    static const size_t staticLds = [&]() -> size_t {
+        hipFuncAttributes attr;
+        return hipFuncGetAttributes(&attr, (const void*)kernel) == hipSuccess ? attr.sharedSizeBytes : (size_t)160 * 1024;
+    }();
     const size_t dynBytes = kWideLevelBytes + (size_t)pa.tableElems * 2;
-    if (attr.sharedSizeBytes + dynBytes > 160 * 1024) return hipErrorInvalidValue;      // the table does not fit beside the weights
-    e = allowDynamicLds<permutoWide16Kernel<H, NH, K0, WAVES, D, F>>((int)dynBytes);
+    if (staticLds + dynBytes > 160 * 1024) return hipErrorInvalidValue;      // the table does not fit beside the weights
+    hipError_t e = allowDynamicLds<permutoWide16Kernel<H, NH, K0, WAVES, D, F>>((int)dynBytes);
     if (e != hipSuccess) return e;
     const uint32_t numPairs = ((pa.mlp.batch + 31u) / 32u + 1u) / 2u;
     const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
