@@ -25,7 +25,18 @@ struct AdamConstants { float beta1, beta2, eps, lr; };
 
 // AdamOptimizer::step (adam.slang:20-36) behind the guards of adjustParameters (kernels.slang:39-43) for one
 // parameter; returns false when the gradient is NaN (the update is skipped; the caller clears the gradient either way)
-__device__ __forceinline__ bool adamUpdate(AdamState& st, half_t& param, float g, const AdamConstants& k)
+// pow(beta1, t) and pow(beta2, t) as half, for the half-rounded step count t (adam.slang:30-31).  The two powf are
+// two thirds of the update's instructions, and all parameters of a network normally share one step count, so a
+// workgroup evaluates them once for the count `shared` (its first state's) and a lane whose own count differs
+// evaluates them itself: same function, same arguments, same bits.
+struct AdamPowers { float it, p1, p2; };
+
+__device__ __forceinline__ AdamPowers adamPowers(float it, const AdamConstants& k)
+{
+    return AdamPowers{it, (float)H(powf((float)H(k.beta1), it)), (float)H(powf((float)H(k.beta2), it))};
+}
+
+__device__ __forceinline__ bool adamUpdate(AdamState& st, half_t& param, float g, const AdamConstants& k, const AdamPowers& shared)
 {
     if (g != g) return false;
     const float beta1 = (float)H(k.beta1), beta2 = (float)H(k.beta2), eps = (float)H(k.eps), lr = (float)H(k.lr);
@@ -36,8 +47,10 @@ __device__ __forceinline__ bool adamUpdate(AdamState& st, half_t& param, float g
     mean = (float)H((float)H(beta1 * mean) + (float)H(omb1 * g));
     var = (float)H((float)H(beta2 * var) + (float)H((float)H(omb2 * g) * g));
     const float it = (float)H((float)st.iteration);
-    const float meanHat = (float)H(mean / (float)H(1.0f - (float)H(powf(beta1, it))));
-    const float varHat = (float)H(var / (float)H(1.0f - (float)H(powf(beta2, it))));
+    AdamPowers pw = shared;
+    if (it != shared.it) pw = adamPowers(it, k);
+    const float meanHat = (float)H(mean / (float)H(1.0f - pw.p1));
+    const float varHat = (float)H(var / (float)H(1.0f - pw.p2));
     const float denom = (float)H(sqrtf((float)H(fmaxf(0.0f, varHat) + eps)));
     param = H((float)param - (float)H((float)H(lr * meanHat) / denom));
     st.mean = H(mean);
@@ -45,14 +58,30 @@ __device__ __forceinline__ bool adamUpdate(AdamState& st, half_t& param, float g
     return true;
 }
 
-__global__ __launch_bounds__(256) void adamKernel(AdamState* states, half_t* params, half_t* grads, uint32_t count,
-                                                  AdamConstants k)
+// the powers for the step count that follows the one stored in `first`, evaluated by the first wave of the workgroup
+__device__ __forceinline__ AdamPowers sharedAdamPowers(const AdamState* first, const AdamConstants& k, float* lds /* 3 floats */)
 {
-    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
-    if (tid >= count) return;
-    AdamState st = states[tid];
-    half_t p = params[tid];
-    if (adamUpdate(st, p, (float)grads[tid], k)) {
+    if (threadIdx.x < 64u) {
+        const AdamPowers pw = adamPowers((float)H((float)(first->iteration + 1)), k);
+        if (threadIdx.x == 0) { lds[0] = pw.it; lds[1] = pw.p1; lds[2] = pw.p2; }
+    }
+    __syncthreads();
+    return AdamPowers{lds[0], lds[1], lds[2]};
+}
+
+__global__ __launch_bounds__(1024) void adamKernel(AdamState* states, half_t* params, half_t* grads, uint32_t count,
+                                                   AdamConstants k)
+{
+    __shared__ float ldsPowers[3];
+    const uint32_t tid = blockIdx.x * 1024u + threadIdx.x;
+    const bool on = tid < count;
+    const uint32_t i = on ? tid : count - 1u;
+    AdamState st = states[i];                 // requested before the powers are worked out
+    half_t p = params[i];
+    const float g = (float)grads[i];
+    const AdamPowers shared = sharedAdamPowers(states + blockIdx.x * 1024u, k, ldsPowers);
+    if (!on) return;
+    if (adamUpdate(st, p, g, k, shared)) {
         params[tid] = p;
         states[tid] = st;
     }
@@ -81,6 +110,8 @@ struct AdamLayersArgs {
 
 __global__ __launch_bounds__(256) void adamLayersKernel(const AdamLayersArgs a)
 {
+    __shared__ float ldsPowers[3];
+    const AdamPowers shared = sharedAdamPowers(a.layers[0].wStates, a.k, ldsPowers);
     const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
     if (tid >= a.total) return;
     int l = 0;
@@ -105,7 +136,7 @@ __global__ __launch_bounds__(256) void adamLayersKernel(const AdamLayersArgs a)
     const float g = a.gradCt == kF32 ? (float)H(*(const float*)grad) : (float)*(const half_t*)grad;
     AdamState st = *state;
     half_t p = *param;
-    if (adamUpdate(st, p, g, a.k)) {
+    if (adamUpdate(st, p, g, a.k, shared)) {
         *param = p;
         *state = st;
     }
@@ -123,7 +154,7 @@ extern "C" CV_API CvResult cvAdamStep(void* stream, void* states, void* params, 
     if ((uintptr_t)states % 4 || (uintptr_t)params % 2 || (uintptr_t)gradients % 2)
         return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: misaligned argument");
     cv::noteKernel(false, "adamKernel");
-    hipLaunchKernelGGL(cv::adamKernel, dim3((count + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(cv::adamKernel, dim3((count + 1023) / 1024), dim3(1024), 0, (hipStream_t)stream,
                        (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count,
                        cv::AdamConstants{beta1, beta2, epsilon, learningRate});
     const hipError_t e = hipGetLastError();
