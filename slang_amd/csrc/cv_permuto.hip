@@ -186,10 +186,12 @@ __global__ __launch_bounds__(1024) void permutoEncodePairsKernel(const PermutoAr
 
 // Reverse mode for one position: adds bary[k] * dOut to the table gradient `dTable` (global memory, or a workgroup's
 // private copy in LDS) and, if wanted, writes the position gradient.
-template <int D>
+// FT: the features per entry when they are 1, 2 or 4 (the loops over them unrolled, the loads of a level issued together:
+// with a run-time count every element was a load and a wait of its own), else 0.
+template <int D, int FT>
 __device__ __forceinline__ void permutoBackwardOne(const PermutoArgs& a, uint32_t s, float* dTable)
 {
-    const int F = a.desc.featureDimensionPerEntry;
+    const int F = FT ? FT : a.desc.featureDimensionPerEntry;
     float pos[D], dpos[D];
 #pragma unroll
     for (int d = 0; d < D; ++d) { pos[d] = ((const float*)(a.pos + (size_t)s * a.posStride))[d]; dpos[d] = 0.f; }
@@ -207,11 +209,29 @@ __device__ __forceinline__ void permutoBackwardOne(const PermutoArgs& a, uint32_
         const float* gl = g + lv.currentLevelIndex * F;
         uint32_t idx[D + 1];
         vertexIndices<D>(lv, F, rem0, rank, idx);
+        if constexpr (FT > 0) {
+            float gv[FT], tv[D + 1][FT];
 #pragma unroll
-        for (int k = 0; k <= D; ++k) {
-            for (int f = 0; f < F; ++f) {
-                if (dTable) atomicAdd(dTable + idx[k] + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
-                dbary[k] += table[idx[k] + f] * gl[f];
+            for (int f = 0; f < FT; ++f) gv[f] = gl[f];
+#pragma unroll
+            for (int k = 0; k <= D; ++k)
+#pragma unroll
+                for (int f = 0; f < FT; ++f) tv[k][f] = table[idx[k] + f];
+#pragma unroll
+            for (int k = 0; k <= D; ++k) {
+#pragma unroll
+                for (int f = 0; f < FT; ++f) {
+                    if (dTable) atomicAdd(dTable + idx[k] + f, bary[k] * gv[f]);    // readFeatureValueBwd, :222-238
+                    dbary[k] += tv[k][f] * gv[f];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k <= D; ++k) {
+                for (int f = 0; f < F; ++f) {
+                    if (dTable) atomicAdd(dTable + idx[k] + f, bary[k] * gl[f]);    // readFeatureValueBwd, :222-238
+                    dbary[k] += table[idx[k] + f] * gl[f];
+                }
             }
         }
         if (!a.dPos) continue;
@@ -242,28 +262,34 @@ __device__ __forceinline__ void permutoBackwardOne(const PermutoArgs& a, uint32_
     }
 }
 
-template <int D>
+template <int D, int FT>
 __global__ __launch_bounds__(256) void permutoBackwardKernel(const PermutoArgs a)
 {
     const uint32_t s = blockIdx.x * 256u + threadIdx.x;
     if (s >= a.batch) return;
-    permutoBackwardOne<D>(a, s, a.dTable);
+    permutoBackwardOne<D, FT>(a, s, a.dTable);
 }
 
 // A small feature table (the reference's own test: 2 048 floats) receives every position's atomic adds on a handful of
 // addresses: 2^22 positions took 123 ms that way.  Here a workgroup accumulates into a private copy of the table in
 // LDS and adds that copy to the table gradient once, at its end: the atomic traffic to memory shrinks by the number
 // of positions per workgroup.
-template <int D>
-__global__ __launch_bounds__(256) void permutoBackwardLdsKernel(const PermutoArgs a, uint32_t tableElems)
+// As many copies of the table as fit (a power of two, up to 16) share the lanes of a wave among them: lanes of one
+// instruction that add to the same address are served one after the other, and with 64 lanes on a level of a few hundred
+// entries that is the common case (measured: 230 cycles per LDS atomic instruction with one copy).
+template <int D, int FT>
+__global__ __launch_bounds__(1024) void permutoBackwardLdsKernel(const PermutoArgs a, uint32_t tableElems, uint32_t copies)
 {
     extern __shared__ float ldsTable[];
-    for (uint32_t i = threadIdx.x; i < tableElems; i += 256u) ldsTable[i] = 0.f;
+    for (uint32_t i = threadIdx.x; i < tableElems * copies; i += blockDim.x) ldsTable[i] = 0.f;
     __syncthreads();
-    for (uint32_t s = blockIdx.x * 256u + threadIdx.x; s < a.batch; s += gridDim.x * 256u) permutoBackwardOne<D>(a, s, ldsTable);
+    float* mine = ldsTable + (threadIdx.x & (copies - 1u)) * tableElems;
+    for (uint64_t s = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; s < a.batch; s += (uint64_t)gridDim.x * blockDim.x)
+        permutoBackwardOne<D, FT>(a, (uint32_t)s, mine);
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < tableElems; i += 256u) {
-        const float v = ldsTable[i];
+    for (uint32_t i = threadIdx.x; i < tableElems; i += blockDim.x) {
+        float v = ldsTable[i];
+        for (uint32_t c = 1; c < copies; ++c) v += ldsTable[c * tableElems + i];
         if (v != 0.f) atomicAdd(a.dTable + i, v);
     }
 }
@@ -342,31 +368,39 @@ hipError_t launchEncode(hipStream_t stream, const PermutoArgs& a)
 hipError_t launchBackward(hipStream_t stream, const PermutoArgs& a)
 {
     const uint64_t tableElems = tableElements(a.desc);
+    const int fe = a.desc.featureDimensionPerEntry, ft = (fe == 1 || fe == 2 || fe == 4) ? fe : 0;
     constexpr uint64_t kLdsTableBytes = 64 * 1024;
     if (a.dTable && tableElems * 4 <= kLdsTableBytes && a.batch >= 4096u) {
         int dev = 0, cus = 256;
         if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        const uint32_t want = (a.batch + 255u) / 256u, cap = (uint32_t)cus * 2u;
-        const dim3 grid(want < cap ? want : cap), block(256);
-        const size_t lds = (size_t)tableElems * 4;
-        noteKernel(false, "permutoBackwardLdsKernel<D=%d>", a.desc.dimensions);
-        switch (a.desc.dimensions) {
-#define CV_D(N) case N: { \
-            const hipError_t e = allowDynamicLds<permutoBackwardLdsKernel<N>>((int)lds); \
+        uint32_t copies = 1;
+        while (copies < 16u && (size_t)tableElems * 4 * (copies * 2u) <= 2 * kLdsTableBytes) copies *= 2u;
+        const size_t lds = (size_t)tableElems * 4 * copies;
+        // workgroups of 16 waves, one or two to a compute unit as the copies leave room
+        const uint32_t want = (a.batch + 1023u) / 1024u, cap = (uint32_t)cus * (lds <= 80 * 1024 ? 2u : 1u);
+        const dim3 grid(want < cap ? want : cap), block(1024);
+        noteKernel(false, "permutoBackwardLdsKernel<D=%d,%u copies>", a.desc.dimensions, copies);
+        switch (a.desc.dimensions * 8 + ft) {
+#define CV_DF(N, G) case N * 8 + G: { \
+            const hipError_t e = allowDynamicLds<permutoBackwardLdsKernel<N, G>>((int)(2 * kLdsTableBytes)); \
             if (e != hipSuccess) return e; \
-            hipLaunchKernelGGL(permutoBackwardLdsKernel<N>, grid, block, lds, stream, a, (uint32_t)tableElems); break; }
+            hipLaunchKernelGGL((permutoBackwardLdsKernel<N, G>), grid, block, lds, stream, a, (uint32_t)tableElems, copies); break; }
+#define CV_D(N) CV_DF(N, 0) CV_DF(N, 1) CV_DF(N, 2) CV_DF(N, 4)
         CV_D(1) CV_D(2) CV_D(3) CV_D(4) CV_D(5) CV_D(6) CV_D(7) CV_D(8)
 #undef CV_D
+#undef CV_DF
         default: return hipErrorInvalidValue;
         }
         return hipGetLastError();
     }
     noteKernel(false, "permutoBackwardKernel<D=%d>", a.desc.dimensions);
     const dim3 grid((a.batch + 255) / 256), block(256);
-    switch (a.desc.dimensions) {
-#define CV_D(N) case N: hipLaunchKernelGGL(permutoBackwardKernel<N>, grid, block, 0, stream, a); break;
+    switch (a.desc.dimensions * 8 + ft) {
+#define CV_DF(N, G) case N * 8 + G: hipLaunchKernelGGL((permutoBackwardKernel<N, G>), grid, block, 0, stream, a); break;
+#define CV_D(N) CV_DF(N, 0) CV_DF(N, 1) CV_DF(N, 2) CV_DF(N, 4)
     CV_D(1) CV_D(2) CV_D(3) CV_D(4) CV_D(5) CV_D(6) CV_D(7) CV_D(8)
 #undef CV_D
+#undef CV_DF
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
