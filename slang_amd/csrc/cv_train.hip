@@ -31,6 +31,11 @@ Shape classify(const MlpArgs& a)
     return s;
 }
 
+// workgroups of the fused kernels per compute unit (the workspace holds one partial for each).  Two of the paired kernel
+// would fit for 32-wide networks (71 KB of LDS, under 128 registers) and were slower: 80 against 72 us for 8-32-32-32-4.
+template <class Net>
+constexpr int kWorkgroupsPerCU = 1;
+
 template <class Net>
 hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
 {
@@ -44,8 +49,10 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // one resident workgroup per compute unit, fewer when the batch has less work than that: a workgroup takes four
     // 16-sample tiles (on 64-wide networks four 32-sample rounds) at a time, and every workgroup launched writes a
     // partial that the second kernel reads (the example's 16 samples: one workgroup instead of 256)
-    const uint32_t units = Net::HT == 4 ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
-    const uint32_t blocks = units < (uint32_t)numCUs ? (units ? units : 1u) : (uint32_t)numCUs;
+    constexpr bool kPairShape = Net::HT == 4 || Net::HT == 2;
+    const uint32_t units = kPairShape ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
+    const uint32_t resident = (uint32_t)numCUs * (uint32_t)kWorkgroupsPerCU<Net>;
+    const uint32_t blocks = units < resident ? (units ? units : 1u) : resident;
     TrainReduceArgs ra;
     for (int l = 0; l < Net::L; ++l) {
         ra.layers[l].wGrad = t.wGrad[l];
@@ -61,9 +68,6 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     ra.lossSum = t.lossSum;
     ra.lossMax = t.lossMax;
     constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
-    // a launch of one workgroup of the one-wave-per-SIMD kernel finishes the step itself
-    ta.finishInKernel = (blocks == 1 && Net::HT != 4) ? 1 : 0;
-    ta.finish = ra;
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
@@ -71,11 +75,14 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     const bool xy = t.mlp.inEncoding == kEncodeXYSquares;
     const bool dwords = !xy && t.mlp.layers[0].in % 2 == 0 && t.mlp.inAlign >= 4u;
     const int variant = !plain || !(xy || dwords) ? 0 : xy ? 2 : 1;
+    // a launch of one workgroup of the one-wave-per-SIMD kernel finishes the step itself
+    ta.finishInKernel = (blocks == 1 && !(kPairShape && variant != 0)) ? 1 : 0;
+    ta.finish = ra;
     noteKernel(false, "mlpTrainKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s> + mlpTrainReduceKernel", Net::IT0, Net::KT0,
                Net::HT, Net::L - 1, Net::MTL,
                variant == 0 ? "runtime-act,any-input" : variant == 1 ? "relu/none,dword-input" : "relu/none,xy-input");
     // 64-wide networks with the plain activations run on the two-waves-per-SIMD kernel
-    constexpr bool kPair = Net::HT == 4;
+    constexpr bool kPair = kPairShape;
     if constexpr (kPair) {
         if (variant != 0)
             noteKernel(false, "mlpTrainPairKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,relu/none,%s> + mlpTrainReduceKernel", Net::IT0,
@@ -102,7 +109,7 @@ size_t trainWorkspaceBytes(const MlpArgs& a, int numCUs)
     if (!s.ok) return 0;
 #define CV_X(I0, K0, HT, NH, ML) \
     if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \
-        return (size_t)numCUs * TrainNet<I0, K0, HT, NH, ML>::partialFloats * sizeof(float);
+        return (size_t)numCUs * kWorkgroupsPerCU<TrainNet<I0, K0, HT, NH, ML>> * TrainNet<I0, K0, HT, NH, ML>::partialFloats * sizeof(float);
     CV_TRAIN_SHAPES(CV_X)
 #undef CV_X
     return 0;
