@@ -229,24 +229,34 @@ __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
     }
 }
 
-__global__ __launch_bounds__(64) void lossFinalKernel(const float* partials, uint32_t n, float* lossSum, float* lossMax)
+// the sum (fixed order: a thread's strided share, sixteen neighbouring threads per lane of the first wave, then lanes
+// 32 ... 1 places apart) and the maximum of the per-workgroup loss partials
+__global__ __launch_bounds__(1024) void lossFinalKernel(const float* partials, uint32_t n, float* lossSum, float* lossMax)
 {
-    __shared__ float red[64];
+    __shared__ float red[1024];
     __shared__ uint32_t maxBits;
     if (threadIdx.x == 0) maxBits = 0u;
     __syncthreads();
     float c = 0.f;
-    for (uint32_t i = threadIdx.x; i < n; i += 64u) {
+    uint32_t m = 0u;
+    for (uint32_t i = threadIdx.x; i < n; i += 1024u) {
         c += partials[i];
-        atomicMax(&maxBits, __builtin_bit_cast(uint32_t, partials[n + i]));
+        const uint32_t b = __builtin_bit_cast(uint32_t, partials[n + i]);     // non-negative floats or NaN: ordered like their bits
+        m = b > m ? b : m;
     }
     red[threadIdx.x] = c;
+    if (m) atomicMax(&maxBits, m);
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x < 64u) {
         float s = 0.f;
-        for (int i = 0; i < 64; ++i) s += red[i];
-        if (lossSum) *lossSum = s;
-        if (lossMax) *lossMax = __builtin_bit_cast(float, maxBits);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) s += red[threadIdx.x * 16 + k];
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+        if (threadIdx.x == 0) {
+            if (lossSum) *lossSum = s;
+            if (lossMax) *lossMax = __builtin_bit_cast(float, maxBits);
+        }
     }
 }
 
@@ -337,7 +347,7 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
         else hipLaunchKernelGGL(lossGradKernel<half_t>, dim3(p.lossBlocks), dim3(256), 0, stream, la);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         if (t.lossSum || t.lossMax) {
-            hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(64), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum, t.lossMax);
+            hipLaunchKernelGGL(lossFinalKernel, dim3(1), dim3(1024), 0, stream, (const float*)(ws + p.lossPartials), p.lossBlocks, t.lossSum, t.lossMax);
             if ((e = hipGetLastError()) != hipSuccess) return e;
         }
     }
