@@ -13,9 +13,11 @@ under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (
 bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
 c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
 matrix pipeline bounds), c5 (training step), t32 (training step of a 32-wide network), ex (one whole iteration of the example at its own shape: training step +
-Adam update, three kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
-(permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), ew (an
-element-wise operator), ad (the Adam update over 2^24 parameters).  With --workload only that one runs and becomes the headline (profiling runs; also
+Adam update, two kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
+(permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), pef / peu
+(that encoder and its decoder network in one kernel / as two calls), ew (an element-wise operator), ad (the Adam update
+over 2^24 parameters), cm (the example's per-iteration layout conversion), nf (the neural module's FFLayer chain over a
+parameter block).  With --workload only that one runs and becomes the headline (profiling runs; also
 c5g = c5 on the layer-by-layer step, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
@@ -675,6 +677,63 @@ def workload_ped(torch, cv, steps, warmup):
     return workload_pe(torch, cv, steps, warmup, decoder=True)
 
 
+def workload_cm(torch, cv, steps, warmup):
+    """convertCooperativeVectorMatrix as the example calls it once per iteration (mlp-training-coopvec.cpp:203-236): the
+    weight gradients of every layer from TrainingOptimal to RowMajor, fp16, one call; here for config 5's five layers
+    (12.9 K elements).  Launch-bound."""
+    from slang_amd.coopvec import CoopVecComponentType as CT, CoopVecMatrixLayout as ML, CooperativeVectorMatrixDesc as D
+    dev = "cuda"
+    dims = [8, 64, 64, 64, 64, 1]
+    src, dst, so, do = [], [], 0, 0
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        ssz = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float16, ML.TrainingOptimal)
+        dsz = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float16, ML.RowMajor, fi * 2)
+        src.append(D(fo, fi, CT.Float16, ML.TrainingOptimal, ssz, so, 0)); so += (ssz + 63) // 64 * 64
+        dst.append(D(fo, fi, CT.Float16, ML.RowMajor, dsz, do, fi * 2)); do += (dsz + 63) // 64 * 64
+    g = torch.Generator(device=dev); g.manual_seed(20264)
+    sbuf = torch.randint(0, 255, (so,), dtype=torch.uint8, device=dev, generator=g)
+    dbuf = torch.zeros(do, dtype=torch.uint8, device=dev)
+    elems = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+
+    def step():
+        cv.convertCooperativeVectorMatrix(dbuf, dst, sbuf, src)
+
+    w = dict(step=step, samples=elems, alg_bytes=elems * 4, alg_flops=0, bound="hbm", mfma="f16", dtype="f16", cpu_baseline=lambda: None,
+             key="cm", config={"workload": "cm: convertCooperativeVectorMatrix, the five weight-gradient matrices of 8->64x4->1 from "
+                                           "TrainingOptimal to RowMajor (fp16) in one call, as once per iteration of the example",
+                               "elements": elems, "launches_per_step": 1})
+    w["graph"] = True
+    w["launch_floor_us"] = 1.6
+    return w
+
+
+def workload_nf(torch, cv, steps, warmup):
+    """The neural module's front: FFLayer chain 32 -> 64 -> 64 -> 8 (ReLU) of halfs evaluated from one parameter block in
+    the optimal layout (cvNeuralMlpForward after cvNeuralToOptimalLayout; layers.slang:34-110), 2^22 samples."""
+    import numpy as np
+    from slang_amd.coopvec import Activation
+    dev = "cuda"
+    B = 1 << 22
+    dims = [32, 64, 64, 8]
+    conv = cv.NetworkParameterLayoutConverter(torch.float16, 0b111, *dims)
+    g = torch.Generator(device=dev); g.manual_seed(20265)
+    portable = (torch.randn(conv.ElementCountLogical, device=dev, generator=g) * 0.15).half()
+    optimal = conv.toOptimalLayout(portable)
+    x = torch.randn(B, dims[0], device=dev, generator=g).half()
+    out = torch.empty(B, dims[-1], dtype=torch.float16, device=dev)
+    acts = [Activation.ReLU, Activation.ReLU, Activation.NoActivation]
+
+    def step():
+        conv.eval(optimal, x, optimalLayout=True, activations=acts, out=out)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+    return dict(step=step, samples=B, alg_bytes=B * (dims[0] + dims[-1]) * 2, alg_flops=B * 2 * macs, bound="hbm", mfma="f16", dtype="f16",
+                cpu_baseline=lambda: None, key="nf",
+                config={"workload": "nf: cvNeuralMlpForward, FFLayer chain 32->64->64->8 (ReLU) of halfs from one parameter block in the "
+                                    "optimal layout, 2^22 samples", "batch": B, "layers": dims})
+
+
 def workload_ew(torch, cv, steps, warmup):
     """An element-wise operator of CoopVec<half, 64> over 2^22 vectors: tanh (hlsl.meta.slang:32383-32401), 2 bytes in and
     2 bytes out per element."""
@@ -809,10 +868,10 @@ def workload_rs(torch, cv, steps, warmup):
 
 WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": workload_c2b, "c3": workload_c3, "c3c": workload_c3c, "c4": workload_c4,
              "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
-             "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
+             "cm": workload_cm, "nf": workload_nf, "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "t32", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "t32", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf")
 HEADLINE = "c2"
 
 
