@@ -33,7 +33,7 @@ struct PermutoMlpArgs {
 constexpr uint32_t kLevelDwords = CV_PERMUTO_MAX_LEVELS * sizeof(CvPermutoLevelInfo) / 4;
 constexpr uint32_t kLdsLimitDwords = 160 * 1024 / 4;
 
-template <int D, int F, int MAXT, bool LDS_TABLE, bool SMOOTH>
+template <int D, int F, int MAXT, bool LDS_TABLE>
 __global__ __launch_bounds__(1024) void permutoMlpKernel(const PermutoMlpArgs pa)
 {
     using Mma = F16Mma;
@@ -107,14 +107,14 @@ __global__ __launch_bounds__(1024) void permutoMlpKernel(const PermutoMlpArgs pa
             }
         }
 #ifndef PM_NO_MLP
-        genericRunLayers<Mma, MAXT, SMOOTH>(ga, lds, lane, sample, act);
+        genericRunLayers<Mma, MAXT, false>(ga, lds, lane, sample, act);      // plain, ReLU and leaky ReLU layers
 #else
         if (sample < a.batch && g == 0) *(uint16_t*)(a.out + (size_t)sample * a.outStride) = (uint16_t)(act[0][0] ^ act[0][1]);
 #endif
     }
 }
 
-template <int D, int F, int MAXT, bool SMOOTH>
+template <int D, int F, int MAXT>
 hipError_t launchShape(hipStream_t stream, PermutoMlpArgs& pa, uint32_t netDwords, int numCUs)
 {
     pa.levelDword = (netDwords + 3u) & ~3u;
@@ -132,11 +132,11 @@ hipError_t launchShape(hipStream_t stream, PermutoMlpArgs& pa, uint32_t netDword
         return hipGetLastError();
     };
     if (inLds) {
-        const hipError_t e = allowDynamicLds<permutoMlpKernel<D, F, MAXT, true, SMOOTH>>((int)(kLdsLimitDwords * 4));
-        return e != hipSuccess ? e : launch(permutoMlpKernel<D, F, MAXT, true, SMOOTH>);
+        const hipError_t e = allowDynamicLds<permutoMlpKernel<D, F, MAXT, true>>((int)(kLdsLimitDwords * 4));
+        return e != hipSuccess ? e : launch(permutoMlpKernel<D, F, MAXT, true>);
     }
-    const hipError_t e = allowDynamicLds<permutoMlpKernel<D, F, MAXT, false, SMOOTH>>((int)(kLdsLimitDwords * 4));
-    return e != hipSuccess ? e : launch(permutoMlpKernel<D, F, MAXT, false, SMOOTH>);
+    const hipError_t e = allowDynamicLds<permutoMlpKernel<D, F, MAXT, false>>((int)(kLdsLimitDwords * 4));
+    return e != hipSuccess ? e : launch(permutoMlpKernel<D, F, MAXT, false>);
 }
 
 } // namespace
@@ -192,7 +192,7 @@ hipError_t launchPermutoMlp(hipStream_t stream, const CvPermutoDesc& desc, const
     const bool small = widest <= 4;
     if (hasSmoothActivation(mlp)) return hipErrorInvalidValue;      // plain, ReLU and leaky ReLU layers only
     switch (D * 16 + F) {
-#define CV_DF(N, G) case N * 16 + G: return small ? launchShape<N, G, 4, false>(stream, pa, netDwords, numCUs) : launchShape<N, G, 8, false>(stream, pa, netDwords, numCUs);
+#define CV_DF(N, G) case N * 16 + G: return small ? launchShape<N, G, 4>(stream, pa, netDwords, numCUs) : launchShape<N, G, 8>(stream, pa, netDwords, numCUs);
     CV_DF(1, 1) CV_DF(1, 2) CV_DF(1, 4) CV_DF(2, 1) CV_DF(2, 2) CV_DF(2, 4) CV_DF(3, 1) CV_DF(3, 2) CV_DF(3, 4) CV_DF(4, 1) CV_DF(4, 2) CV_DF(4, 4)
 #undef CV_DF
     }
