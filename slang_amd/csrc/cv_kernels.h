@@ -79,6 +79,9 @@ hipError_t launchPermutoMlp(hipStream_t stream, const CvPermutoDesc& desc, const
                             const void* featureTable, const MlpArgs& mlp, int numCUs);
 // CV_OK, or the reason why an encoder description is malformed (recorded as the thread's last error)
 CvResult checkPermutoDesc(const char* who, const CvPermutoDesc* desc);
+// the fp16 run-time-size kernel that also leaves every layer's pre-activations (tapZ[l]) and activations (tapX[l]) in
+// memory as [batch][out_l] halfs, where the pointer is not null; hipErrorInvalidValue beyond its limits
+hipError_t launchMlpGenericTaps(hipStream_t stream, const MlpArgs& args, uint8_t* const* tapZ, uint8_t* const* tapX, int numCUs);
 // networks of one type T = float (MmaKind::F32) or bfloat16 (MmaKind::Bf16): vectors, weights, biases, results;
 // same limits as launchMlpGeneric
 hipError_t launchMlpFloat(hipStream_t stream, MmaKind kind, const MlpArgs& args, int numCUs);

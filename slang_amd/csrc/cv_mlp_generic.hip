@@ -15,7 +15,7 @@ namespace cv {
 
 namespace {
 
-template <class Mma, int MAXT, bool SMOOTH>
+template <class Mma, int MAXT, bool SMOOTH, bool TAPS = false>
 __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
 {
     constexpr int kGenMaxKT = MAXT / 2;
@@ -73,21 +73,22 @@ __global__ __launch_bounds__(256) void mlpGenericKernel(const GenArgs ga)
             }
         }
 
-        genericRunLayers<Mma, MAXT, SMOOTH>(ga, lds, lane, sample, act);
+        genericRunLayers<Mma, MAXT, SMOOTH, TAPS>(ga, lds, lane, sample, act);
     }
 }
 
-template <class Mma, int MAXT, bool SMOOTH>
+template <class Mma, int MAXT, bool SMOOTH, bool TAPS = false>
 hipError_t launchGenericSized(hipStream_t stream, const GenArgs& ga, size_t ldsBytes, int numCUs)
 {
-    const hipError_t ea = allowDynamicLds<mlpGenericKernel<Mma, MAXT, SMOOTH>>((int)(kGenLdsDwords * 4));
+    const hipError_t ea = allowDynamicLds<mlpGenericKernel<Mma, MAXT, SMOOTH, TAPS>>((int)(kGenLdsDwords * 4));
     if (ea != hipSuccess) return ea;
     int perCU = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpGenericKernel<Mma, MAXT, SMOOTH>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCU, mlpGenericKernel<Mma, MAXT, SMOOTH, TAPS>, 256, ldsBytes) != hipSuccess || perCU < 1) perCU = 1;
     const uint32_t numTiles = (ga.mlp.batch + 15) / 16, need = (numTiles + 3) / 4;
     const uint32_t cap = (uint32_t)numCUs * (uint32_t)perCU;
-    noteKernel(false, "mlpGenericKernel<%s,up to %d rows%s>", Mma::kName, 16 * MAXT, SMOOTH ? ",smooth activations" : "");
-    hipLaunchKernelGGL((mlpGenericKernel<Mma, MAXT, SMOOTH>), dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
+    noteKernel(false, "mlpGenericKernel<%s,up to %d rows%s%s>", Mma::kName, 16 * MAXT, SMOOTH ? ",smooth activations" : "",
+               TAPS ? ",every layer's vectors stored" : "");
+    hipLaunchKernelGGL((mlpGenericKernel<Mma, MAXT, SMOOTH, TAPS>), dim3(need < cap ? need : cap), dim3(256), ldsBytes, stream, ga);
     return hipGetLastError();
 }
 
@@ -105,6 +106,23 @@ hipError_t launchGeneric(hipStream_t stream, const MlpArgs& a, int numCUs)
 }
 
 } // namespace
+
+hipError_t launchMlpGenericTaps(hipStream_t stream, const MlpArgs& a, uint8_t* const* tapZ, uint8_t* const* tapX, int numCUs)
+{
+    if (a.batch == 0) return hipSuccess;
+    if (hasSmoothActivation(a)) return hipErrorInvalidValue;
+    GenArgs ga;
+    uint32_t widest = 0;
+    const uint32_t dwords = planGeneric<F16Mma>(a, ga, kGenLdsDwords, &widest);
+    if (!dwords) return hipErrorInvalidValue;
+    for (int l = 0; l < kMaxMlpLayers; ++l) {
+        ga.tapZ[l] = l < a.numLayers ? tapZ[l] : nullptr;
+        ga.tapX[l] = l < a.numLayers ? tapX[l] : nullptr;
+    }
+    const size_t ldsBytes = (size_t)dwords * 4;
+    return widest <= 4 ? launchGenericSized<F16Mma, 4, false, true>(stream, ga, ldsBytes, numCUs)
+                       : launchGenericSized<F16Mma, 8, false, true>(stream, ga, ldsBytes, numCUs);
+}
 
 hipError_t launchMlpGeneric(hipStream_t stream, MmaKind kind, const MlpArgs& a, int numCUs)
 {

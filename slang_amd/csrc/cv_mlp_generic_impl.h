@@ -20,6 +20,10 @@ struct GenArgs {
     MlpArgs mlp;
     GenLayer gl[kMaxMlpLayers];
     uint32_t biasDwordBase;  // biases follow the fragments in LDS
+    // (TAPS instantiations only) where to leave every layer's pre-activation / activation vectors, [batch][out_l] halfs in
+    // contiguous rows, or null: what the backward pass of the layer-by-layer training step reads
+    uint8_t* tapZ[kMaxMlpLayers];
+    uint8_t* tapX[kMaxMlpLayers];
 };
 
 // Tile counts and LDS placement of every layer; the dwords of LDS taken (fragments, then biases), or 0 when a layer is
@@ -79,7 +83,7 @@ __device__ __forceinline__ void genericStage(const GenArgs& ga, uint32_t* lds)
 // registers and run more waves per SIMD; 8 up to 128).  SMOOTH: some layer has one of the neural module's smooth
 // activations (their exp / division code, inlined per element, is four fifths of the kernel: networks of plain, ReLU and
 // leaky ReLU layers run an instantiation without it)
-template <class Mma, int MAXT, bool SMOOTH>
+template <class Mma, int MAXT, bool SMOOTH, bool TAPS = false>
 __device__ __forceinline__ void genericRunLayers(const GenArgs& ga, const uint32_t* lds, int lane, uint32_t sample,
                                                  uint32_t (&act)[MAXT / 2][Mma::kFD])
 {
@@ -112,6 +116,47 @@ __device__ __forceinline__ void genericRunLayers(const GenArgs& ga, const uint32
             }
         }
         CarrierCfg cc = makeCarrierCfg<Mma>(a.layers[l].act, a.layers[l].slope);
+        if constexpr (TAPS) {
+            // rows 4t .. 4t+3 of the lane group, as halfs before and after the activation (the roundings of the carrier)
+            uint8_t* tz = ga.tapZ[l];
+            uint8_t* tx = ga.tapX[l];
+            const int outL = a.layers[l].out, rowsL = 4 * MT;
+            const bool quads = outL % 4 == 0;
+            if ((tz || tx) && sample < a.batch) {
+                const size_t row = (size_t)sample * (size_t)outL * 2u;
+#pragma unroll
+                for (int t = 0; t < kGenMaxTiles; ++t) {
+                    const int r0 = g * rowsL + 4 * t;
+                    if (t < MT && r0 < outL) {
+                        typedef float floatx2 __attribute__((ext_vector_type(2)));
+                        const halfx2 z01 = __builtin_convertvector(floatx2{acc[t][0], acc[t][1]}, halfx2);
+                        const halfx2 z23 = __builtin_convertvector(floatx2{acc[t][2], acc[t][3]}, halfx2);
+                        halfx2 x01, x23;
+                        carrierFromAcc<SMOOTH>(acc[t], cc, x01, x23);
+                        if (l + 1 == L) {       // the last layer's result is not clamped for a carrier
+                            const half_t lo = a.layers[l].act == kActRelu ? (half_t)0.f : (half_t)-__builtin_inff();
+                            CarrierCfg last = cc;
+                            last.floor2 = halfx2{lo, lo};
+                            carrierFromAcc<SMOOTH>(acc[t], last, x01, x23);
+                        }
+                        const uint32_t zb[2] = {__builtin_bit_cast(uint32_t, z01), __builtin_bit_cast(uint32_t, z23)};
+                        const uint32_t xb[2] = {__builtin_bit_cast(uint32_t, x01), __builtin_bit_cast(uint32_t, x23)};
+                        if (quads) {
+                            if (tz) *(u32x2*)(tz + row + 2 * r0) = u32x2{zb[0], zb[1]};
+                            if (tx) *(u32x2*)(tx + row + 2 * r0) = u32x2{xb[0], xb[1]};
+                        } else {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                if (r0 + r < outL) {
+                                    if (tz) *(uint16_t*)(tz + row + 2 * (r0 + r)) = (uint16_t)(zb[r / 2] >> (16 * (r & 1)));
+                                    if (tx) *(uint16_t*)(tx + row + 2 * (r0 + r)) = (uint16_t)(xb[r / 2] >> (16 * (r & 1)));
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
         if (l + 1 < L) {
             // this layer's accumulators become the next layer's B operand
 #pragma unroll

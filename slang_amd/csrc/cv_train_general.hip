@@ -308,9 +308,35 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
     // ---- forward ------------------------------------------------------------------------------
     const uint8_t* xl[kMaxMlpLayers];
     uint64_t xlStride[kMaxMlpLayers];
+    // fp16 networks up to 128 wide: one launch of the run-time-size forward kernel that leaves every layer's
+    // pre-activations and activations where the per-layer launches below would (same arithmetic, same bits); the input
+    // is read once and no vector makes a second trip through memory
+    bool forwardDone = false;
+    if (!f32) {
+        MlpArgs fa = a;
+        fa.in = x; fa.inStride = xStride; fa.inEncoding = kEncodeNone;
+        fa.inAlign = alignOfPtr(fa.in, fa.inStride);
+        fa.out = ws + p.act[L - 1]; fa.outStride = (uint64_t)a.layers[L - 1].out * esz;
+        fa.outAlign = alignOfPtr(fa.out, fa.outStride);
+        fa.inHalfAsE4M3 = 0;
+        uint8_t* tapZ[kMaxMlpLayers] = {};
+        uint8_t* tapX[kMaxMlpLayers] = {};
+        for (int l = 0; l < L; ++l) {
+            const bool last = l + 1 == L;
+            if (!last || p.z[l] != p.act[l]) tapZ[l] = ws + p.z[l];
+            if (!last && p.act[l] != p.z[l]) tapX[l] = ws + p.act[l];
+        }
+        e = launchMlpGenericTaps(stream, fa, tapZ, tapX, numCUs);
+        if (e == hipSuccess) forwardDone = true;
+        else if (e != hipErrorInvalidValue) return e;
+    }
     for (int l = 0; l < L; ++l) {
         const MlpLayerArgs& ly = a.layers[l];
         xl[l] = x; xlStride[l] = xStride;
+        if (forwardDone) {
+            x = ws + p.act[l]; xStride = (uint64_t)ly.out * esz;
+            continue;
+        }
         MatMulArgs m;
         memset(&m, 0, sizeof(m));
         m.in = x; m.inStride = xStride;
