@@ -121,6 +121,41 @@ def test_gpu_adam_matches_oracle():
 
 
 @pytest.mark.gpu
+def test_gpu_adam_with_step_counts_that_differ_between_parameters():
+    # the kernel evaluates pow(beta, t) once per workgroup for the count its first state holds; a parameter with another
+    # count must get its own powers: states with random counts, one step, against the oracle
+    import torch
+    from slang_amd import coopvec as cv
+    rng = np.random.default_rng(11)
+    n = 3000
+    p = rng.uniform(-1, 1, n).astype(np.float16)
+    st = np.zeros(n, ob.ADAM_STATE_DTYPE)
+    st["iteration"] = rng.integers(0, 60, n)
+    st["iteration"][:1200] = 17                      # a whole workgroup with one count, then mixed ones
+    st["mean"] = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    st["variance"] = rng.uniform(0, 0.01, n).astype(np.float16)
+    g = (rng.standard_normal(n) * 0.1).astype(np.float16)
+    pd = torch.from_numpy(p.copy()).cuda()
+    sd = torch.from_numpy(st.copy().view(np.uint8)).cuda()
+    gd = torch.from_numpy(g.copy()).cuda()
+    cv.adjustParameters(sd, pd, gd)
+    got, stg = pd.cpu().numpy(), sd.cpu().numpy().view(ob.ADAM_STATE_DTYPE)
+    variants = []
+    for n1 in range(-2, 3):
+        for n2 in range(-2, 3):
+            pv, sv, gv = p.copy(), st.copy(), g.copy()
+            ob.slang_adam_step(sv, pv, gv, pow_nudge=(n1, n2))
+            variants.append((pv, sv, (n1, n2)))
+    ref_p, ref_s = [(pv, sv) for pv, sv, k in variants if k == (0, 0)][0]
+    assert stg.tobytes() == ref_s.tobytes()
+    differs = got.view(np.uint16) != ref_p.view(np.uint16)
+    explained = np.zeros(n, bool)
+    for pv, _, _ in variants:
+        explained |= got.view(np.uint16) == pv.view(np.uint16)
+    assert explained[differs].all() and differs.sum() <= n // 100
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("grad_type", ["f16", "f32"])
 def test_network_adam_step_equals_convert_plus_adam(grad_type):
     # cvMlpAdamStep reads every layer's gradient where the training step left it (TrainingOptimal here) and updates
