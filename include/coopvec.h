@@ -110,6 +110,12 @@ typedef enum CvActivation {
 #define CV_FLAG_LAYERWISE_TRAINING 2u
 /* cvMlpForward: keep to the kernels that work on 16-sample tiles (cross-checks of the 32-sample-tile kernels) */
 #define CV_FLAG_FORWARD_TILE16 4u
+/* cvMlpTrainStep: where it applies (fp16, up to 16 inputs, one to four RELU hidden layers of 64 units, up to 16 outputs
+ * without activation, Row/ColumnMajor weights, at least 16384 samples) take the fused kernel whose waves share a tile of
+ * samples by kind of work (forward, backward, weight gradients) and keep the weights in registers.  Same rounding points
+ * and the same bar as the default kernels, in which every wave takes whole samples through the step; measured slower
+ * than those on MI355X (8-64-64-64-64-1 at 2^20 samples: 151 against 124 us), hence not the default. */
+#define CV_FLAG_TRAIN_SPLIT_BY_ROLE 8u
 
 /* Mirrors the fields the example fills in rhi::CooperativeVectorMatrixDesc
  * (mlp-training-coopvec.cpp:204-225).  `offset` is in bytes from the buffer handed to

@@ -91,6 +91,7 @@ def componentTypeToRhi(componentType: int) -> RhiCooperativeVectorComponentType:
 FLAG_FP8_MATRIX_PIPELINE = 1   # CV_FLAG_FP8_MATRIX_PIPELINE of include/coopvec.h
 FLAG_LAYERWISE_TRAINING = 2    # CV_FLAG_LAYERWISE_TRAINING
 FLAG_FORWARD_TILE16 = 4         # CV_FLAG_FORWARD_TILE16: keep cvMlpForward to the kernels on 16-sample tiles
+FLAG_TRAIN_SPLIT_BY_ROLE = 8    # CV_FLAG_TRAIN_SPLIT_BY_ROLE: cvMlpTrainStep on the kernel whose waves share a tile by kind of work
 
 
 class Activation(enum.IntEnum):

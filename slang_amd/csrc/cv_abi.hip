@@ -819,6 +819,7 @@ static CvResult trainStep(const char* who, void* stream, const CvMlpDesc* mlp, c
     t.mlp.batch = batch;
     t.mlp.inAlign = alignOf(input, inputStride);
     t.mlp.inEncoding = encoded ? cv::kEncodeXYSquares : cv::kEncodeNone;
+    t.splitByRole = (mlp->flags & CV_FLAG_TRAIN_SPLIT_BY_ROLE) ? 1 : 0;
     t.targets = (const uint8_t*)targets;
     t.targetStride = targetStride;
     t.lossScale = lossScale;

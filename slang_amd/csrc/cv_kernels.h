@@ -101,11 +101,19 @@ struct TrainLaunch {
     float* lossSum;
     float* lossMax;              // optional: max over the samples of the per-sample loss
     float* workspace;            // partials
+    int32_t splitByRole;         // take the kernel of launchMlpTrainTeam where trainTeamTakes() says it applies
 };
 // Bytes of workspace the training step needs for this network on a device with numCUs compute
 // units; 0 when no built-in specialisation covers the layer shapes.
 size_t trainWorkspaceBytes(const MlpArgs& shapes, int numCUs);
 hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCUs);
+// The fused step whose waves share a tile of samples by kind of work (forward, backward, weight gradients) and keep the
+// weights in registers: up to 16 inputs, one to four ReLU hidden layers of 64 units, up to 16 outputs without activation,
+// Row/ColumnMajor weights, batches of at least kTrainTeamMinBatch samples.  Same workspace and partials as launchMlpTrain,
+// which calls it for a step that asks for it (splitByRole) where trainTeamTakes() says it applies.
+constexpr uint32_t kTrainTeamMinBatch = 16384;
+bool trainTeamTakes(const TrainLaunch& args);
+hipError_t launchMlpTrainTeam(hipStream_t stream, const TrainLaunch& args, int numCUs);
 // The same step layer by layer through the batched kernels, for any layer sizes: per-layer vectors
 // of the whole batch are parked in the workspace, whose size therefore grows with mlp.batch.
 size_t trainGeneralWorkspaceBytes(const MlpArgs& shapesAndBatch, int numCUs, int carrierCt);

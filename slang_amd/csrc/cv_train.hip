@@ -53,20 +53,7 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     const uint32_t units = kPairShape ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
     const uint32_t resident = (uint32_t)numCUs * (uint32_t)kWorkgroupsPerCU<Net>;
     const uint32_t blocks = units < resident ? (units ? units : 1u) : resident;
-    TrainReduceArgs ra;
-    for (int l = 0; l < Net::L; ++l) {
-        ra.layers[l].wGrad = t.wGrad[l];
-        ra.layers[l].bGrad = t.bGrad[l];
-        ra.layers[l].gradShape = t.gradShape[l];
-        ra.layers[l].in = t.mlp.layers[l].in;
-        ra.layers[l].out = t.mlp.layers[l].out;
-    }
-    ra.numLayers = Net::L;
-    ra.gradCt = t.gradCt;
-    ra.partials = t.workspace;
-    ra.numPartials = blocks;
-    ra.lossSum = t.lossSum;
-    ra.lossMax = t.lossMax;
+    const TrainReduceArgs ra = makeTrainReduceArgs<Net>(t, blocks);
     constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
@@ -120,6 +107,7 @@ hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& t, int numCUs)
     if (t.mlp.batch == 0) return hipSuccess;
     const Shape s = classify(t.mlp);
     if (!s.ok) return hipErrorInvalidValue;
+    if (trainTeamTakes(t)) return launchMlpTrainTeam(stream, t, numCUs);
 #define CV_X(I0, K0, HT, NH, ML) \
     if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \
         return launchNet<TrainNet<I0, K0, HT, NH, ML>>(stream, t, numCUs);

@@ -96,6 +96,27 @@ struct TrainArgs {
 };
 
 
+// what the second kernel of a step is given: where the sums of `blocks` partials go
+template <class Net>
+TrainReduceArgs makeTrainReduceArgs(const TrainLaunch& t, uint32_t blocks)
+{
+    TrainReduceArgs ra;
+    for (int l = 0; l < Net::L; ++l) {
+        ra.layers[l].wGrad = t.wGrad[l];
+        ra.layers[l].bGrad = t.bGrad[l];
+        ra.layers[l].gradShape = t.gradShape[l];
+        ra.layers[l].in = t.mlp.layers[l].in;
+        ra.layers[l].out = t.mlp.layers[l].out;
+    }
+    ra.numLayers = Net::L;
+    ra.gradCt = t.gradCt;
+    ra.partials = t.workspace;
+    ra.numPartials = blocks;
+    ra.lossSum = t.lossSum;
+    ra.lossMax = t.lossMax;
+    return ra;
+}
+
 // The largest per-sample loss of a workgroup, kept as the bits of a non-negative float (whose order is that of the
 // integers; a NaN compares above everything, so it wins).  A maximum does not depend on the order of its operands: the
 // LDS atomic keeps the result reproducible.
