@@ -13,7 +13,7 @@ under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (
 bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
 c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
 matrix pipeline bounds), c5 (training step), c5r (c5 on the kernel whose waves share a tile by kind of work: opt-in, slower),
-t32 (training step of a 32-wide network), ex (one whole iteration of the example at its own shape: training step +
+t32 / t128 (training steps of a 32-wide and of a 128-wide network), ex (one whole iteration of the example at its own shape: training step +
 Adam update, two kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
 (permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), pef / peu
 (that encoder and its decoder network in one kernel / as two calls), ew (an element-wise operator), ad (the Adam update
@@ -489,6 +489,11 @@ def workload_t32(torch, cv, steps, warmup):
     return workload_c5(torch, cv, steps, warmup, dims=[8, 32, 32, 32, 4], key="t32")
 
 
+def workload_t128(torch, cv, steps, warmup):
+    """the training step of a 128-wide network, 16->128->128->8 (the fused kernel in which four waves share the dW accumulators)"""
+    return workload_c5(torch, cv, steps, warmup, dims=[16, 128, 128, 8], key="t128")
+
+
 def workload_c5g(torch, cv, steps, warmup):
     return workload_c5(torch, cv, steps, warmup, flags=cv.FLAG_LAYERWISE_TRAINING)
 
@@ -877,8 +882,8 @@ WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": w
              "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
              "cm": workload_cm, "nf": workload_nf, "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
-             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf")
+             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf")
 HEADLINE = "c2"
 
 

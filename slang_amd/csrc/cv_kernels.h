@@ -111,6 +111,10 @@ hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& args, int numCU
 // weights in registers: up to 16 inputs, one to four ReLU hidden layers of 64 units, up to 16 outputs without activation,
 // Row/ColumnMajor weights, batches of at least kTrainTeamMinBatch samples.  Same workspace and partials as launchMlpTrain,
 // which calls it for a step that asks for it (splitByRole) where trainTeamTakes() says it applies.
+// The fused step for 128-wide hidden layers (one or two of them, ReLU; up to 32 inputs, up to 16 outputs without
+// activation): bytes of workspace, 0 where it does not apply; launchMlpTrain / trainWorkspaceBytes call these.
+size_t trainQuadWorkspaceBytes(const MlpArgs& shapes, int numCUs);
+hipError_t launchMlpTrainQuad(hipStream_t stream, const TrainLaunch& args, int numCUs);
 constexpr uint32_t kTrainTeamMinBatch = 16384;
 bool trainTeamTakes(const TrainLaunch& args);
 hipError_t launchMlpTrainTeam(hipStream_t stream, const TrainLaunch& args, int numCUs);

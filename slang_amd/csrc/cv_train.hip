@@ -94,6 +94,7 @@ size_t trainWorkspaceBytes(const MlpArgs& a, int numCUs)
 {
     const Shape s = classify(a);
     if (!s.ok) return 0;
+    if (s.ht == 8) return trainQuadWorkspaceBytes(a, numCUs);
 #define CV_X(I0, K0, HT, NH, ML) \
     if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \
         return (size_t)numCUs * kWorkgroupsPerCU<TrainNet<I0, K0, HT, NH, ML>> * TrainNet<I0, K0, HT, NH, ML>::partialFloats * sizeof(float);
@@ -107,6 +108,7 @@ hipError_t launchMlpTrain(hipStream_t stream, const TrainLaunch& t, int numCUs)
     if (t.mlp.batch == 0) return hipSuccess;
     const Shape s = classify(t.mlp);
     if (!s.ok) return hipErrorInvalidValue;
+    if (s.ht == 8) return launchMlpTrainQuad(stream, t, numCUs);
     if (trainTeamTakes(t)) return launchMlpTrainTeam(stream, t, numCUs);
 #define CV_X(I0, K0, HT, NH, ML) \
     if (s.it0 == I0 && s.kt0 == K0 && s.ht == HT && s.nhid == NH && s.mtl == ML) \

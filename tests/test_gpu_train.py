@@ -440,3 +440,78 @@ def test_full_size_training_step_properties():
     for a, s in zip(la, l1):
         fa, fs = a.weightsGrad.view(torch.float32), s.weightsGrad.view(torch.float32)
         assert (fa - fs).norm().item() <= 1e-5 * fa.norm().item()
+
+
+@pytest.mark.parametrize("dims,B,targets,grad_ct,grad_layout", [
+    ([16, 128, 128, 8], 4096 + 37, True, CT.Float32, ML.RowMajor),
+    ([16, 128, 128, 8], 3000, False, CT.Float16, ML.TrainingOptimal),
+    ([7, 128, 3], 1111, True, CT.Float32, ML.TrainingOptimal),            # rows of 14 bytes
+    ([24, 120, 128, 16], 2500, True, CT.Float32, ML.RowMajor),            # two input tiles, a hidden layer of 120
+    ([32, 128, 1], 700, False, CT.Float32, ML.RowMajor),
+])
+def test_train_step_128_wide_hidden_layers(dims, B, targets, grad_ct, grad_layout):
+    # one or two ReLU hidden layers of 113..128 units: the fused kernel in which four waves share the dW accumulators
+    rng = np.random.default_rng(sum(dims) + B)
+    specs = make_specs(rng, dims)
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16) if targets else None
+    layers = build(specs, grad_ct, grad_layout)
+    lmax = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t) if targets else None, gradType=grad_ct, lossMax=lmax)
+    assert cv.lastKernelName().startswith("mlpTrainQuadKernel"), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, grad_ct, grad_layout)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 1.0, tie_rule=True)
+    tol = 1e-3 if grad_ct == CT.Float32 else 2e-3
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= tol, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l], rB[l]) <= tol, (l, rel_err(dB[l], rB[l]))
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # the layer-by-layer step on the same data: same rounding points, other order of the fp32 sums
+    general = build(specs, grad_ct, grad_layout)
+    lmax2 = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _, loss2 = cv.mlpTrainStep(general, to_dev(x), to_dev(t) if targets else None, gradType=grad_ct, flags=cv.FLAG_LAYERWISE_TRAINING,
+                               lossMax=lmax2)
+    assert "layer-by-layer" in cv.lastKernelName()
+    gW, gB = read_grads(general, specs, grad_ct, grad_layout)
+    for l in range(len(specs)):
+        assert rel_err(gW[l], dW[l]) <= tol and rel_err(gB[l], dB[l]) <= tol, l
+    assert abs(loss2.item() - loss.item()) <= 1e-4 * loss.item()
+    assert abs(lmax2.item() - lmax.item()) <= 1e-3 * lmax.item()
+    # bitwise determinism
+    again = build(specs, grad_ct, grad_layout)
+    cv.mlpTrainStep(again, to_dev(x), to_dev(t) if targets else None, gradType=grad_ct)
+    for a, b in zip(layers, again):
+        assert torch.equal(a.weightsGrad, b.weightsGrad) and torch.equal(a.biasesGrad, b.biasesGrad)
+
+
+def test_train_step_128_wide_tie_rule_and_other_activations():
+    # exact small numbers: pre-activations of +0 take half the gradient; the fused kernel and the oracle agree bit for bit
+    rng = np.random.default_rng(17)
+    dims, B = [16, 128, 128, 2], 640
+    specs = []
+    for i in range(len(dims) - 1):
+        fo, fi = dims[i + 1], dims[i]
+        W = np.zeros((fo, fi), np.float16)
+        for r in range(fo):
+            W[r, rng.choice(fi, 2, replace=False)] = rng.choice(np.array([-1, 1], np.float16), 2)
+        b = rng.integers(-1, 2, fo).astype(np.float16)
+        if i + 2 < len(dims):
+            W[::3] = 0; b[::3] = 0
+        specs.append(dict(W=W, b=b, act=int(Activation.NoActivation if i == len(dims) - 2 else Activation.ReLU), slope=0.0))
+    x = rng.integers(-1, 2, (B, dims[0])).astype(np.float16)
+    t = rng.integers(-2, 3, (B, dims[-1])).astype(np.float16)
+    layers = build(specs)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=1.0 / 16)
+    assert cv.lastKernelName().startswith("mlpTrainQuadKernel"), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, _ = ob.ref_mlp_train(specs, x, t, 1.0 / 16, tie_rule=True)
+    nW, nB, _ = ob.ref_mlp_train(specs, x, t, 1.0 / 16, tie_rule=False)
+    for l in range(len(specs)):
+        assert np.array_equal(dW[l], rW[l]) and np.array_equal(dB[l], rB[l]), l
+    assert not np.array_equal(nB[0], rB[0])
+    # leaky ReLU on a 128-wide network: no fused kernel, the layer-by-layer step takes it
+    leaky = make_specs(rng, [16, 128, 8], act=Activation.LeakyReLU, slope=0.125)
+    xs = rng.uniform(-1, 1, (500, 16)).astype(np.float16)
+    L2 = build(leaky)
+    cv.mlpTrainStep(L2, to_dev(xs), None)
+    assert "layer-by-layer" in cv.lastKernelName()
