@@ -749,18 +749,23 @@ __global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const 
     const bool ownsLoss = blockIdx.x == (nW + nB) / 64u;      // the workgroup whose values include the loss
     if (threadIdx.x == 0) maxBits = 0u;
     __syncthreads();
+    // (the loss partials are requested here and looked at behind the sums: one round trip to memory for both)
     bool voidStep = false;
-    for (uint32_t b = threadIdx.x; b < ra.numPartials; b += 64u * kReduceWaves) {
-        const float* lossOf = ra.partials + (size_t)b * Net::partialFloats + nW + nB;
-        const float lp = lossOf[0];
+    float lp0 = 0.f;
+    if (threadIdx.x < ra.numPartials) lp0 = ra.partials[(size_t)threadIdx.x * Net::partialFloats + nW + nB];
+    for (uint32_t b = threadIdx.x + 64u * kReduceWaves; b < ra.numPartials; b += 64u * kReduceWaves) {
+        const float lp = ra.partials[(size_t)b * Net::partialFloats + nW + nB];
         voidStep = voidStep || lp != lp;
-        if (ra.lossMax && ownsLoss) atomicMax(&maxBits, __builtin_bit_cast(uint32_t, lossOf[1]));
     }
-    voidStep = __syncthreads_or(voidStep) != 0;
+    if (ra.lossMax && ownsLoss)
+        for (uint32_t b = threadIdx.x; b < ra.numPartials; b += 64u * kReduceWaves)
+            atomicMax(&maxBits, __builtin_bit_cast(uint32_t, ra.partials[(size_t)b * Net::partialFloats + nW + nB + 1]));
+    float s;
+    const bool mine = sumPartials(ra.partials + p, Net::partialFloats, ra.numPartials, inRange, red, s);
+    voidStep = __syncthreads_or(voidStep || lp0 != lp0) != 0;
     if (ra.lossMax && ownsLoss && threadIdx.x == 0)
         *ra.lossMax = voidStep ? __builtin_nanf("") : __builtin_bit_cast(float, maxBits);
-    float s;
-    if (!sumPartials(ra.partials + p, Net::partialFloats, ra.numPartials, inRange, red, s) || !inRange) return;
+    if (!mine || !inRange) return;
     if (voidStep) s = __builtin_nanf("");
     if (p == nW + nB) {
         if (ra.lossSum) *ra.lossSum = s;
