@@ -58,8 +58,10 @@ struct QuadSplit {
     }
 };
 
-// ReLU on the hidden layers, none on the last one (the launcher sends everything else to the layer-by-layer step).
-template <class Net>
+// ReLU on the hidden layers (LEAKY: each hidden layer ReLU or leaky ReLU, as the arguments say: max(z, z*slope) with the
+// product rounded to fp16, fflayer.slang:64-65), none on the last one (the launcher sends everything else to the
+// layer-by-layer step).
+template <class Net, bool LEAKY>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mlpTrainQuadKernel(const TrainArgs ta)
 {
     typedef F16Mma Mma;
@@ -235,8 +237,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 halfx2 z23 = __builtin_convertvector(floatx2{acc[t][2], acc[t][3]}, halfx2);
                 if constexpr (relu) {
                     zs[l][t][0] = z01; zs[l][t][1] = z23;
-                    z01 = __builtin_elementwise_max(z01, zero2);
-                    z23 = __builtin_elementwise_max(z23, zero2);
+                    halfx2 s01 = zero2, s23 = zero2;
+                    if constexpr (LEAKY) {
+                        if (a.layers[l].act != kActRelu) {
+                            const half_t sl = (half_t)a.layers[l].slope;
+                            s01 = z01 * halfx2{sl, sl}; s23 = z23 * halfx2{sl, sl};
+                        }
+                    }
+                    z01 = __builtin_elementwise_max(z01, s01);
+                    z23 = __builtin_elementwise_max(z23, s23);
                 }
                 car[t][0] = z01; car[t][1] = z23;
             }
@@ -383,8 +392,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     typedef float floatx2 __attribute__((ext_vector_type(2)));
                     const halfx2 g01 = __builtin_convertvector(floatx2{gacc[t][0], gacc[t][1]}, halfx2);
                     const halfx2 g23 = __builtin_convertvector(floatx2{gacc[t][2], gacc[t][3]}, halfx2);
-                    dz[t][0] = g01 * maxGradMultiplier(zs[l - 1][t][0]);
-                    dz[t][1] = g23 * maxGradMultiplier(zs[l - 1][t][1]);
+                    if constexpr (LEAKY) {
+                        const half_t sl = (half_t)a.layers[l - 1].slope;
+                        dz[t][0] = applyActGrad<true>(g01, maxGradMultiplier(zs[l - 1][t][0]), a.layers[l - 1].act, halfx2{sl, sl});
+                        dz[t][1] = applyActGrad<true>(g23, maxGradMultiplier(zs[l - 1][t][1]), a.layers[l - 1].act, halfx2{sl, sl});
+                    } else {
+                        dz[t][0] = g01 * maxGradMultiplier(zs[l - 1][t][0]);
+                        dz[t][1] = g23 * maxGradMultiplier(zs[l - 1][t][1]);
+                    }
                 }
                 packS(dz, MTI, Net::ktOut(l - 1), bS);
             }

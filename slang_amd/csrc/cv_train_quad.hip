@@ -6,7 +6,8 @@ namespace cv {
 
 namespace {
 
-// (16-feature tiles of the input, hidden layers): up to 32 inputs, one or two hidden layers of 113..128 units, up to 16 outputs
+// (16-feature tiles of the input, hidden layers): up to 32 inputs, one or two hidden layers of 113..128 units (ReLU or leaky
+// ReLU), up to 16 outputs without activation
 #define CV_TRAIN_QUAD_SHAPES(X) X(1, 1) X(1, 2) X(2, 1) X(2, 2)
 
 template <int IT0, int NH>
@@ -26,8 +27,11 @@ hipError_t launchQuad(hipStream_t stream, const TrainLaunch& t, int numCUs)
     const uint32_t blocks = rounds < (uint32_t)numCUs ? rounds : (uint32_t)numCUs;
     const TrainReduceArgs ra = makeTrainReduceArgs<Net>(t, blocks);
     ta.finish = ra;
-    noteKernel(false, "mlpTrainQuadKernel<IT0=%d,HT=8,hidden=%d,MTL=1,relu/none> + mlpTrainReduceKernel", IT0, NH);
-    hipLaunchKernelGGL((mlpTrainQuadKernel<Net>), dim3(blocks), dim3(256), 0, stream, ta);
+    bool leaky = false;
+    for (int l = 0; l + 1 < Net::L; ++l) leaky = leaky || t.mlp.layers[l].act == kActLeakyRelu;
+    noteKernel(false, "mlpTrainQuadKernel<IT0=%d,HT=8,hidden=%d,MTL=1,%s> + mlpTrainReduceKernel", IT0, NH, leaky ? "leaky-or-relu/none" : "relu/none");
+    if (leaky) hipLaunchKernelGGL((mlpTrainQuadKernel<Net, true>), dim3(blocks), dim3(256), 0, stream, ta);
+    else       hipLaunchKernelGGL((mlpTrainQuadKernel<Net, false>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     constexpr uint32_t total = Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1;
@@ -43,7 +47,7 @@ void classifyQuad(const MlpArgs& a, int& it0, int& nh)
     if (L < 2 || L > 3 || a.inEncoding != kEncodeNone) return;
     if (a.layers[0].in < 1 || a.layers[0].in > 32 || a.layers[L - 1].out > 16 || a.layers[L - 1].act != kActNone) return;
     for (int l = 0; l + 1 < L; ++l)
-        if (optMT((uint32_t)a.layers[l].out) != 8u || a.layers[l].act != kActRelu) return;
+        if (optMT((uint32_t)a.layers[l].out) != 8u || (a.layers[l].act != kActRelu && a.layers[l].act != kActLeakyRelu)) return;
     it0 = (int)optMT((uint32_t)a.layers[0].in);
     nh = L - 1;
 }

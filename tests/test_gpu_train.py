@@ -509,9 +509,25 @@ def test_train_step_128_wide_tie_rule_and_other_activations():
     for l in range(len(specs)):
         assert np.array_equal(dW[l], rW[l]) and np.array_equal(dB[l], rB[l]), l
     assert not np.array_equal(nB[0], rB[0])
-    # leaky ReLU on a 128-wide network: no fused kernel, the layer-by-layer step takes it
-    leaky = make_specs(rng, [16, 128, 8], act=Activation.LeakyReLU, slope=0.125)
-    xs = rng.uniform(-1, 1, (500, 16)).astype(np.float16)
-    L2 = build(leaky)
-    cv.mlpTrainStep(L2, to_dev(xs), None)
+    # leaky ReLU (on one layer, ReLU on the other): the fused kernel's second instantiation, against the oracle and the
+    # layer-by-layer step
+    leaky = make_specs(rng, [16, 128, 128, 8], act=Activation.LeakyReLU, slope=0.125)
+    leaky[1]["act"] = int(Activation.ReLU)
+    xs = rng.uniform(-1, 1, (1500, 16)).astype(np.float16)
+    ts = rng.uniform(-1, 1, (1500, 8)).astype(np.float16)
+    L2, L3 = build(leaky), build(leaky)
+    _, loss = cv.mlpTrainStep(L2, to_dev(xs), to_dev(ts))
+    assert cv.lastKernelName().startswith("mlpTrainQuadKernel") and "leaky" in cv.lastKernelName(), cv.lastKernelName()
+    cv.mlpTrainStep(L3, to_dev(xs), to_dev(ts), flags=cv.FLAG_LAYERWISE_TRAINING)
+    assert "layer-by-layer" in cv.lastKernelName()
+    aW, aB = read_grads(L2, leaky, CT.Float32, ML.RowMajor)
+    gW, gB = read_grads(L3, leaky, CT.Float32, ML.RowMajor)
+    rW, rB, rloss = ob.ref_mlp_train(leaky, xs, ts, 1.0, tie_rule=True)
+    for l in range(3):
+        assert rel_err(aW[l], rW[l]) <= 1e-3 and rel_err(aB[l], rB[l]) <= 1e-3, l
+        assert rel_err(aW[l], gW[l]) <= 1e-3 and rel_err(aB[l], gB[l]) <= 1e-3, l
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # a last layer with an activation: no fused kernel for these widths
+    leaky[2]["act"] = int(Activation.ReLU)
+    cv.mlpTrainStep(build(leaky), to_dev(xs), to_dev(ts))
     assert "layer-by-layer" in cv.lastKernelName()
