@@ -230,7 +230,8 @@ typedef struct CvMatMulDesc {
     int32_t     biasInterpretation;
     /* extras */
     int32_t     activation;     /* CvActivation */
-    float       leakySlope;
+    float       leakySlope;     /* rounded to half where resultType is FLOAT16 (the example's slope is a vector of the layer's
+                                 * element type, fflayer.slang:64) */
     int32_t     accumulate;
     uint32_t    batch;          /* number of samples */
     uint32_t    flags;          /* CV_FLAG_* */
@@ -390,7 +391,8 @@ typedef struct CvMlpLayer {
     int32_t     gradLayout;     /* layout of `weightsGrad` */
     uint32_t    gradStride;
     int32_t     activation;     /* CvActivation applied to this layer's output */
-    float       leakySlope;
+    float       leakySlope;     /* taken in the vectors' type: rounded to half for a network of half vectors, as the example
+                                 * builds it (fflayer.slang:64, CoopVec<NFloat, OutputSize>(0.001h)) */
 } CvMlpLayer;
 
 /* Encoding applied to a sample in front of layer 0.

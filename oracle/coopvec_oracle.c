@@ -724,6 +724,9 @@ int cvo_ref_matmul_i32(const void* x, size_t xStride, int xType, int k,
     return 0;
 }
 
+/* The slope of a half network is a half value: fflayer.slang:64 builds it as CoopVec<NFloat, OutputSize>(0.001h). */
+static inline float slope_as_half(float slope) { return cvo_f16_to_f32(cvo_f32_to_f16_rne(slope)); }
+
 static inline uint16_t act_f16(uint16_t z, int act, float slope)
 {
     float zf = cvo_f16_to_f32(z);
@@ -731,7 +734,7 @@ static inline uint16_t act_f16(uint16_t z, int act, float slope)
     case CVO_ACT_RELU: return (zf > 0.f) ? z : (uint16_t)((zf != zf) ? z : 0); /* max(z,0); NaN stays */
     case CVO_ACT_LEAKY_RELU: {
         /* max(out, out * slope) evaluated in half, fflayer.slang:64-65 */
-        uint16_t zs = cvo_f32_to_f16_rne(zf * slope);
+        uint16_t zs = cvo_f32_to_f16_rne(zf * slope_as_half(slope));
         return (zf >= cvo_f16_to_f32(zs)) ? z : zs; }
     }
     return z;
@@ -846,13 +849,13 @@ int cvo_ref_mlp_train(const CvoLayer* layers, int numLayers,
                     d = (zi > 0.f) ? gi : ((zi == 0.f && maxTieRule) ? cvo_f16_to_f32(cvo_f32_to_f16_rne(0.5f * gi)) : 0.f);
                     break;
                 case CVO_ACT_LEAKY_RELU: { /* max(z, z*s) */
-                    float zsv = cvo_f16_to_f32(cvo_f32_to_f16_rne(zi * L->leakySlope));
+                    float zsv = cvo_f16_to_f32(cvo_f32_to_f16_rne(zi * slope_as_half(L->leakySlope)));
                     float da, db;
                     if (zi > zsv) { da = gi; db = 0.f; }
                     else if (zi < zsv) { da = 0.f; db = gi; }
                     else if (maxTieRule) { da = db = cvo_f16_to_f32(cvo_f32_to_f16_rne(0.5f * gi)); }
                     else { da = gi; db = 0.f; }
-                    float dbs = cvo_f16_to_f32(cvo_f32_to_f16_rne(db * L->leakySlope));
+                    float dbs = cvo_f16_to_f32(cvo_f32_to_f16_rne(db * slope_as_half(L->leakySlope)));
                     d = cvo_f16_to_f32(cvo_f32_to_f16_rne(da + dbs));
                     break; }
                 default: d = gi;

@@ -425,7 +425,9 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* d)
     a.outCt = d->resultType;
     a.act = d->activation;
     if (d->resultType == CV_UINT32 && a.act == CV_ACT_RELU) a.act = CV_ACT_NONE;   // max(u, 0) == u
-    a.slope = d->leakySlope;
+    // the slope is taken in the result's type where that is half: the example builds it as a vector of the layer's element
+    // type (fflayer.slang:64, CoopVec<NFloat, OutputSize>(0.001h))
+    a.slope = d->resultType == CV_FLOAT16 ? (float)(_Float16)d->leakySlope : d->leakySlope;
     a.accumulate = d->accumulate ? 1 : 0;
     a.batch = d->batch;
     a.inUnsigned = combo.inUnsigned ? 1 : 0;
@@ -636,7 +638,9 @@ static CvResult fillMlpLayers(const char* who, const CvMlpDesc* mlp, cv::MlpLaye
         if ((uintptr_t)o.w % (isOptimal(L.weightLayout) ? 16u : wEsz) || (!isOptimal(L.weightLayout) && L.weightStride % wEsz) ||
             (uintptr_t)o.bias % cv::elemSize(mlp->biasType))
             return fail(CV_E_INVALID_ARG, "%s: layer %d: weights/bias misaligned", who, l);
-        o.in = L.inputSize; o.out = L.outputSize; o.act = L.activation; o.slope = L.leakySlope;
+        // the slope of a network of half vectors is a half value (fflayer.slang:64: CoopVec<NFloat, OutputSize>(0.001h))
+        o.in = L.inputSize; o.out = L.outputSize; o.act = L.activation;
+        o.slope = uniformT ? L.leakySlope : (float)(_Float16)L.leakySlope;
     }
     return CV_OK;
 }

@@ -123,11 +123,12 @@ __device__ __forceinline__ void storeFragmentChunk(uint32_t* d, const uint32_t (
 }
 
 template <int ESZ, int EPL>
-__device__ __forceinline__ bool fragmentSourceIsDirect(const MatrixShape& shape, bool transposed, int MT, int KT, uint32_t rows,
-                                                       uint32_t cols, uint32_t rowOff, uint32_t xorByte)
+__device__ __forceinline__ bool fragmentSourceIsDirect(const MatrixShape& shape, bool transposed, int MT, int KT, uint32_t gs,
+                                                       uint32_t rows, uint32_t cols, uint32_t rowOff, uint32_t xorByte)
 {
     return shape.layout == kInferencingOptimal && !transposed && rowOff == 0 && xorByte == 0 &&
-           optMT(shape.rows) == (uint32_t)MT && optKT(shape.cols, EPL) == (uint32_t)KT && shape.rows == rows && shape.cols == cols;
+           optMT(shape.rows) == (uint32_t)MT && optKT(shape.cols, EPL) == (uint32_t)KT && optGS(shape.cols) == gs &&
+           shape.rows == rows && shape.cols == cols;
 }
 
 // firstThread: the thread that takes chunk 0.  A kernel that stages several small matrices gives each its own
@@ -140,7 +141,7 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
 {
     constexpr int DW = ESZ * EPL / 4;
     const int chunks = MT * KT * 64;
-    const bool direct = fragmentSourceIsDirect<ESZ, EPL>(shape, transposed, MT, KT, rows, cols, rowOff, xorByte);
+    const bool direct = fragmentSourceIsDirect<ESZ, EPL>(shape, transposed, MT, KT, gs, rows, cols, rowOff, xorByte);
     const uint32_t vt = threadIdx.x >= firstThread ? threadIdx.x - firstThread : threadIdx.x + blockDim.x - firstThread;
     for (int c = (int)vt; c < chunks; c += blockDim.x) {
         uint32_t v[DW];
@@ -161,7 +162,7 @@ struct FragmentStage {
                                          uint32_t rows, uint32_t cols)
     {
         const int chunks = MT * KT * 64;
-        const bool direct = fragmentSourceIsDirect<ESZ, EPL>(shape, transposed, MT, KT, rows, cols, 0, 0);
+        const bool direct = fragmentSourceIsDirect<ESZ, EPL>(shape, transposed, MT, KT, gs, rows, cols, 0, 0);
 #pragma unroll
         for (int it = 0; it < ITERS; ++it) {
             const int c = (int)threadIdx.x + it * BLOCK;

@@ -2,6 +2,7 @@
 #include "cv_train_impl.h"
 #include "cv_train_pair.h"
 #include "cv_error.h"
+#include <algorithm>
 
 namespace cv {
 
@@ -22,9 +23,11 @@ Shape classify(const MlpArgs& a)
     if (L < 2) return s;
     s.it0 = (int)optMT((uint32_t)a.layers[0].in);
     s.kt0 = (int)optKT((uint32_t)a.layers[0].in, 8);
-    s.ht = (int)optMT((uint32_t)a.layers[0].out);
-    for (int l = 1; l + 1 < L; ++l)
-        if ((int)optMT((uint32_t)a.layers[l].out) != s.ht) return s;
+    // the widest hidden layer decides the tiling: 1, 2, 4 or 8 tiles of 16 units; narrower hidden layers are padded to it
+    // (rows and columns of zeros in the staged weights)
+    int widest = 0;
+    for (int l = 0; l + 1 < L; ++l) widest = std::max(widest, (int)optMT((uint32_t)a.layers[l].out));
+    s.ht = widest <= 2 ? widest : widest <= 4 ? 4 : widest <= 8 ? 8 : widest;
     s.nhid = L - 1;
     s.mtl = (int)optMT((uint32_t)a.layers[L - 1].out);
     s.ok = true;

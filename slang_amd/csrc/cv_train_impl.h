@@ -218,7 +218,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int l = decltype(lc)::value;
         constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
         const MlpLayerArgs& ly = a.layers[l];
-        const uint32_t gs = optGS((uint32_t)ly.in);
+        // k-slots per lane group: those of the kernel's tiling (a hidden layer narrower than the widest one is padded to it)
+        const uint32_t gs = l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0);
         stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, gs,
                                (uint32_t)ly.out, (uint32_t)ly.in);
         if constexpr (l > 0) {

@@ -170,7 +170,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
         static_assert(MT * 16 <= 512, "one bias value per thread and layer");
         const MlpLayerArgs& ly = a.layers[l];
-        stW[l].load(ly.w, ly.shape, false, MT, KT, optGS((uint32_t)ly.in), (uint32_t)ly.out, (uint32_t)ly.in);
+        // (k-slots per lane group: those of the kernel's tiling; a hidden layer narrower than the widest one is padded to it)
+        stW[l].load(ly.w, ly.shape, false, MT, KT, l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0), (uint32_t)ly.out, (uint32_t)ly.in);
         const int e = threadIdx.x, t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
         const int row = gg * ROWS + 4 * t + r;
         stB[l] = (e < MT * 16 && ly.bias && row < ly.out) ? (float)((const half_t*)ly.bias)[row] : 0.f;

@@ -94,7 +94,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
         static_assert(Split::divides(l), "the tiles of a layer divide among the four waves");
         const MlpLayerArgs& ly = a.layers[l];
-        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, optGS((uint32_t)ly.in),
+        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT,
+                               l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0),
                                (uint32_t)ly.out, (uint32_t)ly.in);
         for (int e = threadIdx.x; e < MT * 16; e += 256) {
             const int t = e >> 4, gg = (e >> 2) & 3, r = e & 3, row = gg * ROWS + 4 * t + r;

@@ -6,7 +6,7 @@ namespace cv {
 
 namespace {
 
-// (16-feature tiles of the input, hidden layers): up to 32 inputs, one or two hidden layers of 113..128 units (ReLU or leaky
+// (16-feature tiles of the input, hidden layers): up to 32 inputs, one or two hidden layers, the wider of 65..128 units (ReLU or leaky
 // ReLU), up to 16 outputs without activation
 #define CV_TRAIN_QUAD_SHAPES(X) X(1, 1) X(1, 2) X(2, 1) X(2, 2)
 
@@ -46,8 +46,9 @@ void classifyQuad(const MlpArgs& a, int& it0, int& nh)
     const int L = a.numLayers;
     if (L < 2 || L > 3 || a.inEncoding != kEncodeNone) return;
     if (a.layers[0].in < 1 || a.layers[0].in > 32 || a.layers[L - 1].out > 16 || a.layers[L - 1].act != kActNone) return;
+    // (the caller sends networks here whose widest hidden layer has 65 to 128 units; a narrower one is padded)
     for (int l = 0; l + 1 < L; ++l)
-        if (optMT((uint32_t)a.layers[l].out) != 8u || (a.layers[l].act != kActRelu && a.layers[l].act != kActLeakyRelu)) return;
+        if (optMT((uint32_t)a.layers[l].out) > 8u || (a.layers[l].act != kActRelu && a.layers[l].act != kActLeakyRelu)) return;
     it0 = (int)optMT((uint32_t)a.layers[0].in);
     nh = L - 1;
 }

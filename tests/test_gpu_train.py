@@ -85,7 +85,10 @@ def test_ffn_closed_form_backward():
 @pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 4096 + 21), ([4, 16, 4], 1000), ([2, 16, 16, 16, 1], 2048),
                                     ([8, 32, 32, 4], 777), ([20, 64, 64, 8], 1500), ([8, 64, 64, 64, 5], 900),
                                     ([8, 32, 4], 300), ([8, 32, 32, 32, 4], 1500), ([8, 32, 32, 32, 32, 2], 2100), ([24, 32, 32, 32, 8], 1000),
-                                    ([8, 64, 4], 513), ([24, 64, 64, 64, 6], 1200)])
+                                    ([8, 64, 4], 513), ([24, 64, 64, 64, 6], 1200),
+                                    # hidden layers of different widths, and widths between the tile counts the kernels are built
+                                    # for: the widest one decides, the others are padded to it
+                                    ([8, 16, 64, 4], 1500), ([20, 48, 24, 5], 700), ([8, 48, 48, 48, 3], 900), ([5, 40, 2], 333)])
 def test_train_step_against_oracle(dims, B):
     rng = np.random.default_rng(sum(dims) + B)
     specs = make_specs(rng, dims)
@@ -330,6 +333,7 @@ def test_train_fp16_training_optimal_gradients_and_convert():
     ([12, 100, 100, 9], 1000, Activation.LeakyReLU, 0.1),
     ([64, 160, 96, 32], 900, Activation.ReLU, 0.0),         # wider than 128
     ([8, 64, 64, 64, 64, 1], 2000, Activation.ReLU, 0.0),   # a fused shape, forced through the general step below
+    ([16, 128, 128, 128, 4], 600, Activation.ReLU, 0.0),    # three 128-wide hidden layers: no fused kernel
 ])
 @pytest.mark.parametrize("grad_ct,grad_layout", [(CT.Float32, ML.RowMajor), (CT.Float16, ML.TrainingOptimal)])
 def test_general_training_step_against_oracle(dims, B, act, slope, grad_ct, grad_layout):
@@ -338,7 +342,7 @@ def test_general_training_step_against_oracle(dims, B, act, slope, grad_ct, grad
     x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
     t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
     layers = build(specs, grad_ct, grad_layout)
-    fused_shape = dims == [8, 64, 64, 64, 64, 1]
+    fused_shape = max(dims[1:-1]) <= 128      # these also have a fused kernel: the general step is asked for
     flags = cv.FLAG_LAYERWISE_TRAINING if fused_shape else 0
     _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), gradType=grad_ct, flags=flags)
     assert "layer-by-layer" in cv.lastKernelName()
@@ -358,7 +362,7 @@ def test_general_training_step_against_oracle(dims, B, act, slope, grad_ct, grad
         # the fused kernel on the same step: same rounding points, only the order of the fp32 sums differs
         layers3 = build(specs, grad_ct, grad_layout)
         _, loss3 = cv.mlpTrainStep(layers3, to_dev(x), to_dev(t), gradType=grad_ct)
-        assert "mlpTrain" in cv.lastKernelName() and "layer-by-layer" not in cv.lastKernelName()
+        assert ("mlpTrain" in cv.lastKernelName() and "layer-by-layer" not in cv.lastKernelName()) == (len(dims) <= 4 or max(dims[1:-1]) <= 64)
         fW, fB = read_grads(layers3, specs, grad_ct, grad_layout)
         for l in range(len(specs)):
             assert rel_err(fW[l], dW[l]) <= (1e-4 if grad_ct == CT.Float32 else 1e-3)
@@ -376,7 +380,7 @@ def test_general_training_step_tie_rule_and_sin_target():
     specs[0]["W"][:4] = 0                                   # four hidden units of layer 0 are always exactly 0
     x = rng.uniform(-1, 1, (B, 8)).astype(np.float16)
     layers = build(specs)
-    _, loss = cv.mlpTrainStep(layers, to_dev(x), None)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), None, flags=cv.FLAG_LAYERWISE_TRAINING)
     assert "layer-by-layer" in cv.lastKernelName()
     dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
     rW, rB, rloss = ob.ref_mlp_train(specs, x, None, 1.0, tie_rule=True)
@@ -398,7 +402,7 @@ def test_train_argument_validation():
         cv.mlpTrainStep(layers, x, None, workspace=torch.zeros(need - 16, dtype=torch.uint8, device=DEV))
     assert e.value.result == cv.SLANG_E_BUFFER_TOO_SMALL
     # layer sizes outside the fused shapes take the layer-by-layer step, whose workspace grows with the batch
-    specs = make_specs(rng, [8, 16, 64, 4])
+    specs = make_specs(rng, [8, 16, 160, 4])
     assert cv.mlpTrainStepWorkspaceSize(build(specs), 4096) > cv.mlpTrainStepWorkspaceSize(build(specs), 16) > 0
     with pytest.raises(cv.CoopVecError) as e:      # one layer has nothing to chain
         cv.mlpTrainStepWorkspaceSize(build(make_specs(rng, [8, 4])), 10)
@@ -448,9 +452,11 @@ def test_full_size_training_step_properties():
     ([7, 128, 3], 1111, True, CT.Float32, ML.TrainingOptimal),            # rows of 14 bytes
     ([24, 120, 128, 16], 2500, True, CT.Float32, ML.RowMajor),            # two input tiles, a hidden layer of 120
     ([32, 128, 1], 700, False, CT.Float32, ML.RowMajor),
+    ([16, 80, 100, 8], 1300, True, CT.Float32, ML.RowMajor),              # padded to 128
+    ([12, 100, 30, 9], 1000, True, CT.Float32, ML.TrainingOptimal),
 ])
 def test_train_step_128_wide_hidden_layers(dims, B, targets, grad_ct, grad_layout):
-    # one or two ReLU hidden layers of 113..128 units: the fused kernel in which four waves share the dW accumulators
+    # one or two ReLU hidden layers, the wider of 65..128 units: the fused kernel in which four waves share the dW accumulators
     rng = np.random.default_rng(sum(dims) + B)
     specs = make_specs(rng, dims)
     x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)

@@ -41,7 +41,7 @@ def test_no_alloc_on_the_layer_by_layer_step_and_its_limit():
     # layer sizes without a fused kernel take the layer-by-layer step, whose scratch grows with the batch:
     # a small batch fits the built-in array (same result as cvMlpTrainStep, bit for bit), a large one does not
     rng = np.random.default_rng(1)
-    specs = make_specs(rng, [8, 16, 64, 4])
+    specs = make_specs(rng, [8, 16, 160, 4])
     x = to_dev(rng.uniform(-1, 1, (300, 8)).astype(np.float16))
     ref_layers, layers = build(specs), build(specs)
     _, ref_loss = cv.mlpTrainStep(ref_layers, x, None)
