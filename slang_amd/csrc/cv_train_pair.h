@@ -564,7 +564,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             constexpr int W = kTilesPerPhase * 256;      // floats from one wave's tiles to the next wave's
             const float sum = ((r[(0 + rpar) * W] + r[(2 + rpar) * W]) + r[(4 + rpar) * W]) + r[(6 + rpar) * W];
             const int eo = (Split::byOut(l) ? rpar * OO : 0) + j / OI, ei = (Split::byIn(l) ? rpar * OI : 0) + j % OI;
-            if (!Split::single(l) || rpar == 0) part[(Net::gradTileBase(l) + eo * NI + ei) * 256 + ridx] = sum;
+            // (a streaming store: nobody on this die reads the partial, and it need not wait in the die's L2 for the write-back at
+            // the kernel's end; 2.2 us of the step)
+            if (!Split::single(l) || rpar == 0) __builtin_nontemporal_store(sum, &part[(Net::gradTileBase(l) + eo * NI + ei) * 256 + ridx]);
         });
         if constexpr (q0 == 0) {
             // bias gradients: 16 values per output row (four waves of a parity x four lane groups), summed by one thread

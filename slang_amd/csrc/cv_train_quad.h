@@ -423,7 +423,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         }
     }
 
-    // ---- the workgroup's partial: every dW tile lies in one wave ------------------------------------------------------
+    // ---- the workgroup's partial: every dW tile lies in one wave (streaming stores: nobody on this die reads them, and they
+    // need not wait in its L2 for the write-back at the kernel's end) -----------------------------------------------------
     if (timeouts && lane == 0) atomicOr(ldsFlag + 5, 1u);
     if (ta.wantLossMax) noteLossMax(ldsFlag + 4, lossMaxAcc);
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
@@ -436,7 +437,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             for (int eo = 0; eo < OO; ++eo) {
 #pragma unroll
                 for (int ei = 0; ei < OI; ++ei)
-                    *(floatx4*)&part[(Net::gradTileBase(l) + (eo0 + eo) * NI + ei0 + ei) * 256 + lane * 4] = accW[Split::locBase(l) + eo * OI + ei];
+                    __builtin_nontemporal_store(accW[Split::locBase(l) + eo * OI + ei],
+                                                (floatx4*)&part[(Net::gradTileBase(l) + (eo0 + eo) * NI + ei0 + ei) * 256 + lane * 4]);
                 if (Split::byOut(l) || p == 0) {
                     // a row's bias gradient lies in the four lane groups (eight samples of the round's 32 + 32 each)
                     float s = accB[Split::locDbBase(l) + eo];

@@ -612,7 +612,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();
     if (role >= 2 && team == 0) forEach([&](float x, uint32_t p, bool mine) { if (mine) ldsPart[p] = x + ldsPart[p]; });
     __syncthreads();
-    for (uint32_t i = threadIdx.x; i < (nW + nB) / 4u; i += 512u) ((floatx4*)part)[i] = ((const floatx4*)ldsPart)[i];
+    for (uint32_t i = threadIdx.x; i < (nW + nB) / 4u; i += 512u) __builtin_nontemporal_store(((const floatx4*)ldsPart)[i], (floatx4*)part + i);
     if (wave == 0) {
         float s = ldsLoss[lane] + ldsLoss[64 + lane];
 #pragma unroll
