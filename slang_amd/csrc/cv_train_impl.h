@@ -699,13 +699,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     if (ra.lossMax && threadIdx.x == 0) *ra.lossMax = voidStep ? __builtin_nanf("") : part[nValues + 1];
 }
 
-// Adds value p of a step's summed partial (dW tiles in accumulator order, then db tiles) to the element of the gradient
-// buffers it belongs to ("+=", any layout, fp16 or fp32).
+// Where value p of a step's summed partial (dW tiles in accumulator order, then db tiles) belongs in the gradient buffers
+// ("+=", any layout, fp16 or fp32): the element's address, or null for a value of the tiling's padding.
 template <class Net>
-__device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32_t p, float s)
+__device__ __forceinline__ uint8_t* gradientSlot(const TrainReduceArgs& ra, uint32_t p)
 {
     constexpr int L = Net::L;
     constexpr uint32_t nW = Net::totalGradTiles * 256;
+    const uint32_t esz = ra.gradCt == kF32 ? 4u : 2u;
+    uint8_t* slot = nullptr;
     staticFor<0, L>([&](auto lc) {
         constexpr int l = decltype(lc)::value;
         constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
@@ -717,20 +719,29 @@ __device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32
             const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
             const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
             const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
-            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) {
-                uint8_t* d = ly.wGrad + elemOffset(ly.gradShape, o, i);
-                if (ra.gradCt == kF32) *(float*)d += s;
-                else *(half_t*)d = (half_t)((float)*(half_t*)d + s);
-            }
+            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) slot = ly.wGrad + elemOffset(ly.gradShape, o, i);
         } else if (p >= b0 && p < b1) {
             const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
             const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
-            if (ly.bGrad && o < (uint32_t)ly.out) {
-                if (ra.gradCt == kF32) ((float*)ly.bGrad)[o] += s;
-                else ((half_t*)ly.bGrad)[o] = (half_t)((float)((half_t*)ly.bGrad)[o] + s);
-            }
+            if (ly.bGrad && o < (uint32_t)ly.out) slot = ly.bGrad + (size_t)o * esz;
         }
     });
+    return slot;
+}
+__device__ __forceinline__ float loadGradient(const uint8_t* slot, int gradCt)
+{
+    return gradCt == kF32 ? *(const float*)slot : (float)*(const half_t*)slot;
+}
+__device__ __forceinline__ void storeGradient(uint8_t* slot, int gradCt, float v)
+{
+    if (gradCt == kF32) *(float*)slot = v;
+    else *(half_t*)slot = (half_t)v;
+}
+template <class Net>
+__device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32_t p, float s)
+{
+    uint8_t* slot = gradientSlot<Net>(ra, p);
+    if (slot) storeGradient(slot, ra.gradCt, loadGradient(slot, ra.gradCt) + s);
 }
 
 // Sums the workgroup partials in a fixed order and adds them to the gradient buffers.
@@ -761,6 +772,13 @@ __global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const 
     if (ra.lossMax && ownsLoss)
         for (uint32_t b = threadIdx.x; b < ra.numPartials; b += 64u * kReduceWaves)
             atomicMax(&maxBits, __builtin_bit_cast(uint32_t, ra.partials[(size_t)b * Net::partialFloats + nW + nB + 1]));
+    // (so is the gradient element the sum is added to: wave 0, which stores the sums, asks for it before they are formed)
+    uint8_t* slot = nullptr;
+    float old = 0.f;
+    if (threadIdx.x < 64u && inRange && p < nW + nB) {
+        slot = gradientSlot<Net>(ra, p);
+        if (slot) old = loadGradient(slot, ra.gradCt);
+    }
     float s;
     const bool mine = sumPartials(ra.partials + p, Net::partialFloats, ra.numPartials, inRange, red, s);
     voidStep = __syncthreads_or(voidStep || lp0 != lp0) != 0;
@@ -772,7 +790,7 @@ __global__ __launch_bounds__(64 * kReduceWaves) void mlpTrainReduceKernel(const 
         if (ra.lossSum) *ra.lossSum = s;
         return;
     }
-    addToGradients<Net>(ra, p, s);
+    if (slot) storeGradient(slot, ra.gradCt, old + s);
 }
 
 } // namespace
