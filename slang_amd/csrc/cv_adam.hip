@@ -88,6 +88,46 @@ __global__ __launch_bounds__(1024) void adamKernel(AdamState* states, half_t* pa
     grads[tid] = (half_t)0;
 }
 
+// The same with four consecutive parameters per thread: 8-byte accesses to the parameters and gradients, two of 16 bytes to
+// the states, all of them streaming (every byte is touched once); for counts that are a multiple of four at addresses
+// aligned to those accesses.
+__global__ __launch_bounds__(256) void adamKernel4(AdamState* states, half_t* params, half_t* grads, uint32_t quads, AdamConstants k)
+{
+    __shared__ float ldsPowers[3];
+    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
+    const bool on = tid < quads;
+    const uint32_t q = on ? tid : quads - 1u;
+    const u32x4 s01 = __builtin_nontemporal_load((const u32x4*)(states + 4u * q));
+    const u32x4 s23 = __builtin_nontemporal_load((const u32x4*)(states + 4u * q) + 1);
+    const u32x2 pw = __builtin_nontemporal_load((const u32x2*)(params + 4u * q));
+    const u32x2 gw = __builtin_nontemporal_load((const u32x2*)(grads + 4u * q));
+    const AdamPowers shared = sharedAdamPowers(states + blockIdx.x * 1024u, k, ldsPowers);
+    if (!on) return;
+    const uint32_t sIn[8] = {s01.x, s01.y, s01.z, s01.w, s23.x, s23.y, s23.z, s23.w};
+    uint32_t sOut[8];
+    half_t p[4], g[4];
+    *(u32x2*)p = pw;
+    *(u32x2*)g = gw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        AdamState st;
+        const halfx2 mv = __builtin_bit_cast(halfx2, sIn[2 * i]);
+        st.mean = mv.x; st.variance = mv.y; st.iteration = (int32_t)sIn[2 * i + 1];
+        half_t pi = p[i];
+        if (adamUpdate(st, pi, (float)g[i], k, shared)) {
+            p[i] = pi;
+            sOut[2 * i] = __builtin_bit_cast(uint32_t, halfx2{st.mean, st.variance});
+            sOut[2 * i + 1] = (uint32_t)st.iteration;
+        } else {
+            sOut[2 * i] = sIn[2 * i]; sOut[2 * i + 1] = sIn[2 * i + 1];
+        }
+    }
+    __builtin_nontemporal_store(*(const u32x2*)p, (u32x2*)(params + 4u * tid));
+    __builtin_nontemporal_store(u32x4{sOut[0], sOut[1], sOut[2], sOut[3]}, (u32x4*)(states + 4u * tid));
+    __builtin_nontemporal_store(u32x4{sOut[4], sOut[5], sOut[6], sOut[7]}, (u32x4*)(states + 4u * tid) + 1);
+    __builtin_nontemporal_store(u32x2{0u, 0u}, (u32x2*)(grads + 4u * tid));
+}
+
 // The same update for a whole network, read straight from the gradient buffers the training step fills: the example
 // first copies every weight gradient from its TrainingOptimal buffer to a row-major one
 // (mlp-training-coopvec.cpp:203-236) and clears the TrainingOptimal segment at the top of the next iteration
@@ -153,10 +193,17 @@ extern "C" CV_API CvResult cvAdamStep(void* stream, void* states, void* params, 
     if (!states || !params || !gradients) return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: null argument");
     if ((uintptr_t)states % 4 || (uintptr_t)params % 2 || (uintptr_t)gradients % 2)
         return cv::failWith(CV_E_INVALID_ARG, "cvAdamStep: misaligned argument");
-    cv::noteKernel(false, "adamKernel");
-    hipLaunchKernelGGL(cv::adamKernel, dim3((count + 1023) / 1024), dim3(1024), 0, (hipStream_t)stream,
-                       (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count,
-                       cv::AdamConstants{beta1, beta2, epsilon, learningRate});
+    if (count % 4u == 0 && (uintptr_t)states % 16 == 0 && (uintptr_t)params % 8 == 0 && (uintptr_t)gradients % 8 == 0) {
+        cv::noteKernel(false, "adamKernel4");
+        hipLaunchKernelGGL(cv::adamKernel4, dim3((count / 4u + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                           (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count / 4u,
+                           cv::AdamConstants{beta1, beta2, epsilon, learningRate});
+    } else {
+        cv::noteKernel(false, "adamKernel");
+        hipLaunchKernelGGL(cv::adamKernel, dim3((count + 1023) / 1024), dim3(1024), 0, (hipStream_t)stream,
+                           (cv::AdamState*)states, (cv::half_t*)params, (cv::half_t*)gradients, count,
+                           cv::AdamConstants{beta1, beta2, epsilon, learningRate});
+    }
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return cv::failWith(CV_E_INTERNAL_FAIL, "cvAdamStep launch: %s", hipGetErrorString(e));
     return CV_OK;

@@ -32,7 +32,7 @@ enum : int {
     kOpLog2, kOpExp2, kOpTanh, kOpAtan, kOpFma, kOpRelu, kOpLeakyRelu, kOpSigmoid, kOpSilu, kOpQuickGelu, kOpScale, kOpCount
 };
 
-__host__ __device__ inline int operandCount(int op)
+__host__ __device__ constexpr int operandCount(int op)
 {
     switch (op) {
     case kOpAdd: case kOpSub: case kOpMul: case kOpDiv: case kOpMin: case kOpMax: case kOpStep: return 2;
@@ -89,11 +89,25 @@ __device__ __forceinline__ float evalOp(int op, float a, float b, float c, float
 // rounded half result for + - * / (a float holds more than twice the bits of a half plus two); fma is not of that kind
 // (a float result can land on a half tie that the exact value misses), so it is summed exactly in double (exact for
 // half operands whenever the result is finite) and rounded to half once.
+// tanh for a result that is rounded to half: 1 - 2 / (1 + exp(2|x|)) from the hardware's exp2 and reciprocal (1 ulp of a
+// float each; an overflowing exponential ends at exactly 1), and below |x| = 1/16, where that difference cancels, x - x^3/3
+// (the next term is 2 x^5/15, under 2 * 10^-6 of x there): errors of 10^-7 absolute above and 2 * 10^-6 relative below, far
+// inside a half's spacing of 5 * 10^-4.  Half the instructions of the float routine.
+__device__ __forceinline__ float tanhForHalf(float x)
+{
+    const float ax = __builtin_fabsf(x);
+    const float t = __builtin_amdgcn_exp2f(ax * 2.885390082f);             // exp(2|x|), 2 / ln 2 = 2.88539...
+    const float big = __builtin_fmaf(-2.f, __builtin_amdgcn_rcpf(1.f + t), 1.f);
+    const float small = ax * __builtin_fmaf(x * x, -1.f / 3.f, 1.f);
+    return __builtin_copysignf(ax < 0.0625f ? small : big, x);
+}
+
 template <typename T>
 __device__ __forceinline__ T evalOpAs(int op, float a, float b, float c, float param)
 {
     if constexpr (std::is_same<T, half_t>::value) {
         if (op == kOpFma) return halfOfDouble((double)a * (double)b + (double)c);
+        if (op == kOpTanh) return (half_t)tanhForHalf(a);
     }
     return (T)evalOp(op, a, b, c, param);
 }
@@ -177,21 +191,38 @@ __global__ __launch_bounds__(256) void elementwiseKernel(const EwArgs e)
 
 // dense rows (stride = n elements) of a unary / binary operator on 16-byte pieces: the whole batch is
 // one flat array
+// (the operator is a template parameter of the loop: chosen once per thread, not once per element)
+template <typename T, int OP>
+__device__ __forceinline__ void elementwiseDenseLoop(const EwArgs& e, uint64_t pieces)
+{
+    constexpr int PER = 16 / sizeof(T);
+    constexpr int nOps = operandCount(OP);
+    for (uint64_t p = (uint64_t)blockIdx.x * 256u + threadIdx.x; p < pieces; p += (uint64_t)gridDim.x * 256u) {
+        T va[PER], vb[PER], vc[PER], vo[PER];
+        // (streaming accesses: every byte is touched once)
+        *(u32x4*)va = __builtin_nontemporal_load((const u32x4*)(e.a + p * 16u));
+        if constexpr (nOps >= 2) *(u32x4*)vb = __builtin_nontemporal_load((const u32x4*)(e.b + p * 16u));
+        if constexpr (nOps >= 3) *(u32x4*)vc = __builtin_nontemporal_load((const u32x4*)(e.c + p * 16u));
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            vo[i] = evalOpAs<T>(OP, (float)va[i], nOps >= 2 ? (float)vb[i] : 0.f, nOps >= 3 ? (float)vc[i] : 0.f, e.param);
+        __builtin_nontemporal_store(*(const u32x4*)vo, (u32x4*)(e.out + p * 16u));
+    }
+}
+
+template <typename T, int OP = 0>
+__device__ __forceinline__ void elementwiseDenseDispatch(const EwArgs& e, uint64_t pieces)
+{
+    if constexpr (OP < kOpCount) {
+        if (e.op == OP) elementwiseDenseLoop<T, OP>(e, pieces);
+        else elementwiseDenseDispatch<T, OP + 1>(e, pieces);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void elementwiseDenseKernel(const EwArgs e, uint64_t pieces)
 {
-    constexpr int PER = 16 / sizeof(T);
-    const int nOps = operandCount(e.op);
-    for (uint64_t p = (uint64_t)blockIdx.x * 256u + threadIdx.x; p < pieces; p += (uint64_t)gridDim.x * 256u) {
-        T va[PER], vb[PER], vc[PER], vo[PER];
-        *(u32x4*)va = *(const u32x4*)(e.a + p * 16u);
-        if (nOps >= 2) *(u32x4*)vb = *(const u32x4*)(e.b + p * 16u);
-        if (nOps >= 3) *(u32x4*)vc = *(const u32x4*)(e.c + p * 16u);
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-            vo[i] = evalOpAs<T>(e.op, (float)va[i], nOps >= 2 ? (float)vb[i] : 0.f, nOps >= 3 ? (float)vc[i] : 0.f, e.param);
-        *(u32x4*)(e.out + p * 16u) = *(const u32x4*)vo;
-    }
+    elementwiseDenseDispatch<T>(e, pieces);
 }
 
 // The operators Slang declares on integer vectors (arithmetic, min / max / clamp: hlsl.meta.slang:32115-32229) and,

@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CV_MLP_STRE
                                 halfx2 p0, p1;
                                 carrierNoLeaky(acc[j][t], cc[l], p0, p1);
                                 const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
-                                o[t] = v;
+                                storeStream8(&o[t], v);      // (written once, read by nobody here)
                             }
                         }
                     }

@@ -79,11 +79,11 @@ def test_nan_skips_and_infinities_clip():
 
 
 @pytest.mark.gpu
-def test_gpu_adam_matches_oracle():
+@pytest.mark.parametrize("n", [5000, 5003])      # four parameters per thread, and the kernel for any count
+def test_gpu_adam_matches_oracle(n):
     import torch
     from slang_amd import coopvec as cv
     rng = np.random.default_rng(7)
-    n = 5000
     p = rng.uniform(-1, 1, n).astype(np.float16)
     st = np.zeros(n, ob.ADAM_STATE_DTYPE)
     pd = torch.from_numpy(p.copy()).cuda()
