@@ -300,7 +300,7 @@ __global__ __launch_bounds__(64 * WAVES) void mlpWideKernel(const MlpArgs a)
                     p1 = __builtin_elementwise_max(p1, zero2);
                 }
                 const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
-                *(u32x2*)(obase + (outLane + 16u * q)) = v;
+                storeStream8(obase + (outLane + 16u * q), v);      // (written once, read by nobody here)
             }
         }
     };

@@ -307,13 +307,13 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
             }
             if (storeQuads) {
                 const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};
-                *(u32x2*)(orow + 2 * row0) = v;
+                storeStream8(orow + 2 * row0, v);      // (written once, read by nobody here)
             } else {
                 half_t* o16 = (half_t*)(orow + 2 * row0);
-                o16[0] = p0.x;
-                if (row0 + 1 < outDim) o16[1] = p0.y;
-                if (row0 + 2 < outDim) o16[2] = p1.x;
-                if (row0 + 3 < outDim) o16[3] = p1.y;
+                __builtin_nontemporal_store(p0.x, o16);
+                if (row0 + 1 < outDim) __builtin_nontemporal_store(p0.y, o16 + 1);
+                if (row0 + 2 < outDim) __builtin_nontemporal_store(p1.x, o16 + 2);
+                if (row0 + 3 < outDim) __builtin_nontemporal_store(p1.y, o16 + 3);
             }
         }
     };
