@@ -180,7 +180,8 @@ __global__ __launch_bounds__(1024) void permutoEncodePairsKernel(const PermutoAr
 #pragma unroll
         for (int d = 0; d < D; ++d) pos[d] = (float)((const T*)(a.pos + (size_t)s * a.posStride))[d];
         const Entry acc = permutoEncodeEntry<T, D, F>(pos, lv, table, a.desc.maxLevel);
-        *(Entry*)((T*)(a.out + (size_t)s * a.outStride) + lv.currentLevelIndex * F) = acc;
+        // (a streaming store: the encoded vectors are written once and read by the next kernel)
+        __builtin_nontemporal_store(acc, (Entry*)((T*)(a.out + (size_t)s * a.outStride) + lv.currentLevelIndex * F));
     }
 }
 
