@@ -85,17 +85,6 @@ __device__ __forceinline__ void teamAwait(const volatile TeamLdsWord* flag, uint
     timeouts |= spins >= kTeamSpinLimit ? 1u : 0u;
 }
 
-// maxGradMultiplier (cv_train_impl.h) in two instructions: z * 65504, then * 65504 + 0.5 with the result clamped to [0, 1]
-// by the instruction's own modifier: {1, 0.5, 0} for z > 0, z == 0, z < 0 (and 0 for a NaN, as max and min give there)
-__device__ __forceinline__ halfx2 teamMaxGradMultiplier(halfx2 z)
-{
-    const halfx2 big = {(half_t)65504.f, (half_t)65504.f}, hlf = {(half_t)0.5f, (half_t)0.5f};
-    const halfx2 t = z * big;
-    halfx2 m;
-    asm("v_pk_fma_f16 %0, %1, %2, %3 clamp" : "=v"(m) : "v"(t), "v"(big), "v"(hlf));
-    return m;
-}
-
 __device__ __forceinline__ u32x2 teamReadTr(const uint32_t* p)
 {
     typedef short shortx4 __attribute__((ext_vector_type(4)));
@@ -419,7 +408,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             const halfx2 gg = __builtin_convertvector(floatx2{g[cs][T][r0 + 2 * i], g[cs][T][r0 + 2 * i + 1]}, halfx2);
-                            const halfx2 dz = gg * teamMaxGradMultiplier(__builtin_bit_cast(halfx2, z[cs][s][i]));
+                            const halfx2 dz = gg * maxGradMultiplier(__builtin_bit_cast(halfx2, z[cs][s][i]));
                             B[s][i] = __builtin_bit_cast(uint32_t, dz);
                         }
                     }
