@@ -11,8 +11,8 @@ namespace {
 // (input feature tiles, input k-tiles, hidden tiles, hidden layers, output tiles)
 #define CV_TRAIN_SHAPES(X) \
     X(1, 1, 1, 1, 1) X(1, 1, 1, 2, 1) X(1, 1, 1, 3, 1) \
-    X(1, 1, 2, 1, 1) X(1, 1, 2, 2, 1) X(1, 1, 2, 3, 1) X(1, 1, 2, 4, 1) X(2, 1, 2, 2, 1) X(2, 1, 2, 3, 1) \
-    X(1, 1, 4, 1, 1) X(1, 1, 4, 2, 1) X(1, 1, 4, 3, 1) X(1, 1, 4, 4, 1) X(2, 1, 4, 2, 1) X(2, 1, 4, 3, 1)
+    X(1, 1, 2, 1, 1) X(1, 1, 2, 2, 1) X(1, 1, 2, 3, 1) X(1, 1, 2, 4, 1) X(2, 1, 2, 1, 1) X(2, 1, 2, 2, 1) X(2, 1, 2, 3, 1) X(2, 1, 2, 4, 1) \
+    X(1, 1, 4, 1, 1) X(1, 1, 4, 2, 1) X(1, 1, 4, 3, 1) X(1, 1, 4, 4, 1) X(2, 1, 4, 1, 1) X(2, 1, 4, 2, 1) X(2, 1, 4, 3, 1) X(2, 1, 4, 4, 1)
 
 struct Shape { int it0, kt0, ht, nhid, mtl; bool ok; };
 
@@ -29,6 +29,8 @@ Shape classify(const MlpArgs& a)
     for (int l = 0; l + 1 < L; ++l) widest = std::max(widest, (int)optMT((uint32_t)a.layers[l].out));
     s.ht = widest <= 2 ? widest : widest <= 4 ? 4 : widest <= 8 ? 8 : widest;
     s.nhid = L - 1;
+    // (16-wide networks with four hidden layers or more than 16 inputs have no instantiation of their own)
+    if (s.ht == 1 && (s.nhid > 3 || s.it0 > 1)) s.ht = 2;
     s.mtl = (int)optMT((uint32_t)a.layers[L - 1].out);
     s.ok = true;
     return s;
@@ -52,7 +54,11 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // one resident workgroup per compute unit, fewer when the batch has less work than that: a workgroup takes four
     // 16-sample tiles (on 64-wide networks four 32-sample rounds) at a time, and every workgroup launched writes a
     // partial that the second kernel reads (the example's 16 samples: one workgroup instead of 256)
-    constexpr bool kPairShape = Net::HT == 4 || Net::HT == 2;
+    // the paired kernel's LDS: weights, transposes, biases, four pairs' tiles of a round (64-wide networks with four hidden
+    // layers and more than 16 inputs exceed it and run on the one-wave kernel)
+    constexpr int kPairLdsBytes = 4 * ((Net::totalFrags + (Net::totalTFrags > 0 ? Net::totalTFrags : 1)) * 256 + Net::totalBiasTiles * 16 +
+                                       4 * Net::totalXTiles * 256 + 8 * Net::MTMAX * 256 + 12);
+    constexpr bool kPairShape = (Net::HT == 4 || Net::HT == 2) && kPairLdsBytes <= 160 * 1024;
     const uint32_t units = kPairShape ? (t.mlp.batch + 31u) / 32u : ((t.mlp.batch + 15u) / 16u + 3u) / 4u;
     const uint32_t resident = (uint32_t)numCUs * (uint32_t)kWorkgroupsPerCU<Net>;
     const uint32_t blocks = units < resident ? (units ? units : 1u) : resident;

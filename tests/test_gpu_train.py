@@ -537,3 +537,35 @@ def test_train_step_128_wide_tie_rule_and_other_activations():
     leaky[2]["act"] = int(Activation.ReLU)
     cv.mlpTrainStep(build(leaky), to_dev(xs), to_dev(ts))
     assert "layer-by-layer" in cv.lastKernelName()
+
+
+def test_fused_and_layer_by_layer_steps_agree_on_random_shapes():
+    # networks drawn at random within what the fused kernels take (up to 32 inputs, 16 outputs, four hidden layers of up to 64
+    # units or two of up to 128, ReLU or leaky ReLU, hidden layers of different widths): the step the library picks and the
+    # layer-by-layer step have the same rounding points and differ in the order of their fp32 sums only
+    rng = np.random.default_rng(20260)
+    fused = 0
+    for case in range(40):
+        wide = case % 4 == 3
+        nhid = int(rng.integers(1, 3 if wide else 5))
+        top = 128 if wide else 64
+        dims = [int(rng.integers(1, 33))] + [int(rng.integers(top // 2 + 1 if h == 0 else 3, top + 1)) for h in range(nhid)] + [int(rng.integers(1, 17))]
+        leaky = case % 3 == 1
+        B = int(rng.integers(1, 700))
+        specs = make_specs(rng, dims, act=Activation.LeakyReLU if leaky else Activation.ReLU, slope=0.125 if leaky else 0.0,
+                           bias=case % 5 != 0)
+        x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+        t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16) if case % 2 else None
+        a, b = build(specs), build(specs)
+        _, la = cv.mlpTrainStep(a, to_dev(x), to_dev(t) if t is not None else None)
+        name = cv.lastKernelName()
+        fused += "layer-by-layer" not in name
+        _, lb = cv.mlpTrainStep(b, to_dev(x), to_dev(t) if t is not None else None, flags=cv.FLAG_LAYERWISE_TRAINING)
+        aW, aB = read_grads(a, specs, CT.Float32, ML.RowMajor)
+        bW, bB = read_grads(b, specs, CT.Float32, ML.RowMajor)
+        for l in range(len(specs)):
+            scaleW, scaleB = max(np.linalg.norm(bW[l]), 1e-6), max(np.linalg.norm(bB[l]), 1e-6)
+            assert np.linalg.norm(aW[l] - bW[l]) <= 1e-3 * scaleW, (case, dims, B, name, l)
+            assert np.linalg.norm(aB[l] - bB[l]) <= 1e-3 * scaleB, (case, dims, B, name, l)
+        assert abs(la.item() - lb.item()) <= 1e-4 * max(abs(lb.item()), 1e-6), (case, dims, B, name)
+    assert fused == 40
