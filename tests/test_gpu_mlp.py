@@ -569,3 +569,34 @@ def test_full_size_e4m3_decoder():
     assert torch.equal(ys.view(torch.int16), y1[idx].view(torch.int16))
     frac, _ = end_to_end_ok(y1[idx].cpu().numpy(), specs, xs, ob.E4M3, hid)
     assert frac >= 0.999, frac
+
+
+def test_fused_forward_equals_the_chain_of_single_layers_on_random_shapes():
+    # Networks drawn at random (every layer up to 128 wide, one to five layers, ReLU or leaky ReLU, with and without
+    # biases, fp16 and e4m3 weights, RowMajor and InferencingOptimal, batches that end inside a tile): whichever kernel
+    # cvMlpForward picks, its result equals the chain of coopVecMatMulAdd launches bit for bit.
+    rng = np.random.default_rng(20261)
+    kernels = set()
+    for case in range(48):
+        wtype = CT.FloatE4M3 if case % 3 == 2 else CT.Float16
+        nl = int(rng.integers(2, 6))
+        shape_kind = case % 4
+        if shape_kind == 0:      # the shapes of the specialised kernels
+            width = int(rng.choice([16, 32, 64]))
+            dims = [int(rng.choice([8, 16, 32]))] + [width] * (nl - 1) + [int(rng.integers(1, 17))]
+        else:
+            dims = [int(rng.integers(1, 129)) for _ in range(nl + 1)]
+        leaky = wtype == CT.Float16 and case % 5 == 1
+        specs = make_net(rng, dims, wtype, act=Activation.LeakyReLU if leaky else Activation.ReLU, slope=0.0625 if leaky else 0.0,
+                         bias=("rand", "none", "zero")[case % 3], init="he" if wtype == CT.Float16 else "half")
+        B = int(rng.integers(1, 3000))
+        if wtype == CT.Float16:
+            xd = to_dev(rng.uniform(-1, 1, (B, dims[0])).astype(np.float16))
+        else:
+            xd = to_dev(ob.encode_e4m3(rng.standard_normal((B, dims[0])) * 0.5))
+        layout = ML.InferencingOptimal if case % 2 else ML.RowMajor
+        y = cv.mlpForward(gpu_layers(specs, wtype, layout), xd, weightType=wtype)
+        kernels.add(cv.lastKernelName().split("<")[0])
+        yc = chain_of_single_layers(specs, xd, wtype)
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), (case, dims, B, cv.lastKernelName())
+    assert len(kernels) >= 3, kernels
