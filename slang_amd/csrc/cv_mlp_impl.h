@@ -137,7 +137,13 @@ __device__ __forceinline__ void fragFromCarrier(halfx2 lo01, halfx2 lo23, halfx2
     }
 }
 
-template <class Mma, class Net, int NT, int S>
+// LEAN (kChunkRowDwords or kChunkDirect, the kind of all weight matrices; kChunkNone: the general instantiation): for
+// calls bound by launch latency.  Every lane's slice of an input vector is whole, 4-byte aligned dwords and every weight
+// matrix is one that ChunkInFlight takes.  Input loads then are straight-line code (a
+// dword outside the slice is fetched from the start of the row, which always exists, and masked when the tile is used)
+// and the weights are requested before anything waits: no wait for one load stands between two others, and a batch of
+// one super-tile per wave costs one round trip to memory for inputs, weights and biases together.
+template <class Mma, class Net, int NT, int S, int LEAN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void mlpForwardKernel(const MlpArgs a)
 {
     constexpr int EPL = Mma::kEpl, FD = Mma::kFD, ESZ = Mma::kEsz, RAW = Mma::kRawDW;
@@ -148,45 +154,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     __shared__ __attribute__((aligned(16))) uint32_t ldsW[Net::totalFrags * 64 * RAW];
     __shared__ __attribute__((aligned(16))) uint16_t ldsB[Net::totalBiasTiles * 16];
 
-    // ---- stage weights (fragment order) and biases (fp16, kernel row order) into LDS -------
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
-        const MlpLayerArgs& ly = a.layers[l];
-        const uint32_t gs = optGS((uint32_t)ly.in);
-        uint32_t* base = ldsW + Net::fragBase(l) * 64 * RAW;
-        stageFragments<ESZ, EPL>(base, ly.w, ly.shape, false, MT, KT, gs, (uint32_t)ly.out, (uint32_t)ly.in, 0, 0,
-                                 (uint32_t)(Net::fragBase(l) * 64) % 256u);
-        // bias of tile t, lane group g, r: row g*ROWS + 4t + r  ->  ldsB[(biasBase + t)*16 + 4g + r]
-        // (each layer from another wave of the workgroup, like its weights: the loads of the layers overlap)
-        for (int e = (int)((threadIdx.x + 256u - 64u * (l % 4)) % 256u); e < MT * 16; e += 256) {
-            const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
-            const int row = g * ROWS + 4 * t + r;
-            uint16_t v = 0;
-            if (ly.bias && row < ly.out) v = ((const uint16_t*)ly.bias)[row];
-            ldsB[(Net::biasBase(l) + t) * 16 + 4 * g + r] = v;
-        }
-    });
-    __syncthreads();
-
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, n = lane & 15;
-
-    // ---- weights and biases to registers ---------------------------------------------------
-    uint32_t W[L][Net::MTMAX][Net::KTMAX][FD];
-    uint32_t Bs[L][Net::MTMAX][2];          // 4 fp16 biases per tile, packed
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-#pragma unroll
-        for (int t = 0; t < Net::mt(l); ++t) {
-#pragma unroll
-            for (int kt = 0; kt < Net::kt(l); ++kt)
-                Mma::decode(&ldsW[((Net::fragBase(l) + t * Net::kt(l) + kt) * 64 + lane) * RAW], W[l][t][kt]);
-            const uint16_t* bp = &ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
-            Bs[l][t][0] = (uint32_t)bp[0] | ((uint32_t)bp[1] << 16);
-            Bs[l][t][1] = (uint32_t)bp[2] | ((uint32_t)bp[3] << 16);
-        }
-    });
 
     // ---- per-lane constants ----------------------------------------------------------------
     const uint32_t gs0 = optGS((uint32_t)a.layers[0].in);
@@ -208,27 +177,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const uint32_t numTiles = (a.batch + TILE - 1) / TILE;
     const uint32_t tileStride = gridDim.x * 4;
     uint32_t tile = blockIdx.x * 4 + wave;
-    if (tile >= numTiles) return;
     const uint8_t* inLane = a.in + (size_t)colBase * (a.inHalfAsE4M3 ? 2 : ESZ);
     uint8_t* outLane = a.out + (size_t)rowBase * 2;
     const uint32_t lastSample = a.batch - 1;
-
-    CarrierCfg cc[L];
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        cc[l] = makeCarrierCfg<Mma>(a.layers[l].act, a.layers[l].slope);
-        if constexpr (l + 1 == L) {   // the last layer's output is not re-quantised: plain ReLU floor
-            const half_t lo = a.layers[l].act == kActRelu ? (half_t)0.f : (half_t)-__builtin_inff();
-            cc[l].floor2 = halfx2{lo, lo};
-        }
-    });
 
     auto loadTile = [&](uint32_t (&buf)[S][IN_DW], uint32_t t) {
 #pragma unroll
         for (int j = 0; j < S; ++j) {
             const uint32_t s = min(t * TILE + 16 * j + n, lastSample);
             const uint8_t* p = inLane + (size_t)s * a.inStride;
-            if (loadMode == 3) {
+            if constexpr (LEAN != kChunkNone) {
+                const uint8_t* row = a.in + (size_t)s * a.inStride;
+#pragma unroll
+                for (int i = 0; i < IN_DW; ++i) buf[j][i] = *(const uint32_t*)(4 * i < validBytes ? p + 4 * i : row);
+            } else if (loadMode == 3) {
                 // a float2 sample; lane group 0 owns all four encoded inputs
 #pragma unroll
                 for (int i = 0; i < IN_DW; ++i) buf[j][i] = 0u;
@@ -290,6 +252,118 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         }
     };
 
+    // the first super-tile's inputs are requested with the weights: the round trips to memory overlap (a wave without a
+    // tile loads the batch's last sample and leaves after the barrier)
+    uint32_t bufA[S][IN_DW], bufB[S][IN_DW];
+    if constexpr (LEAN == kChunkNone) loadTile(bufA, tile);
+    // (the wave's number as the scalar it is: the lean instantiation branches around the layers of other waves)
+    const int waveS = __builtin_amdgcn_readfirstlane(wave);
+
+    // ---- stage weights (fragment order) and biases (fp16, kernel row order) into LDS -------
+    // (each layer from another wave of the workgroup: the loads of the layers overlap.  The lean instantiations request
+    // weights, biases and the first inputs and then wait once; the general one requests a thread's bias element, from an
+    // address that always exists, before its weights, so that the first wait of the staging covers it)
+    uint32_t chunk[L][RAW];     // (lean instantiations) a thread's chunk of every layer while its loads are in flight
+    int chunkValid[L];
+    if constexpr (LEAN != kChunkNone) {
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int MT = Net::mt(l), KT = Net::kt(l), CHUNKS = MT * KT * 64;
+            static_assert(CHUNKS <= 256, "one chunk per thread and layer");
+            const MlpLayerArgs& ly = a.layers[l];
+            const int c = (int)((threadIdx.x + 256u - (uint32_t)(Net::fragBase(l) * 64) % 256u) % 256u);
+#pragma unroll
+            for (int d = 0; d < RAW; ++d) chunk[l][d] = 0u;
+            chunkValid[l] = 0;
+            if (((waveS + 4 - Net::fragBase(l) % 4) & 3) * 64 < CHUNKS)        // (a wave skips the layers that are other waves')
+                ChunkInFlight<ESZ, EPL, LEAN>::request(chunk[l], chunkValid[l], ly.w, ly.shape, MT, KT, optGS((uint32_t)ly.in),
+                                                        (uint32_t)ly.out, (uint32_t)ly.in, c);
+        });
+    }
+    uint16_t biasElem[L];
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), ROWS = 4 * MT;
+        static_assert(MT * 16 <= 256, "one bias element per thread");
+        const MlpLayerArgs& ly = a.layers[l];
+        const int e = (int)((threadIdx.x + 256u - 64u * (l % 4)) % 256u);
+        const int row = ((e >> 2) & 3) * ROWS + 4 * (e >> 4) + (e & 3);
+        const bool have = e < MT * 16 && ly.bias && row < ly.out;
+        if constexpr (LEAN != kChunkNone) {
+            // (at its start the kernel waits once, for everything: a thread without an element skips the request)
+            biasElem[l] = 0;
+            if (((waveS + 4 - l % 4) & 3) * 64 < MT * 16) {
+                if (have) biasElem[l] = ((const uint16_t*)ly.bias)[row];
+            }
+        } else {
+            biasElem[l] = *(have ? (const uint16_t*)ly.bias + row : (const uint16_t*)a.out);   // (the output holds a half at least)
+        }
+    });
+    if constexpr (LEAN != kChunkNone) {
+        loadTile(bufA, tile);
+        // (every request stands before this point and every use after it: left alone, the compiler moves a layer's
+        // packing up into its request, and with it the wait for its loads)
+#pragma unroll
+        for (int l = 0; l < L; ++l)
+#pragma unroll
+            for (int d = 0; d < RAW; ++d) asm volatile("" : "+v"(chunk[l][d]) : : "memory");
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int CHUNKS = Net::mt(l) * Net::kt(l) * 64;
+            const int c = (int)((threadIdx.x + 256u - (uint32_t)(Net::fragBase(l) * 64) % 256u) % 256u);
+            if (c < CHUNKS) ChunkInFlight<ESZ, EPL, LEAN>::finish(chunk[l], chunkValid[l], ldsW + (Net::fragBase(l) * 64 + c) * RAW);
+        });
+    } else {
+        staticFor<0, L>([&](auto lc) {
+            constexpr int l = decltype(lc)::value;
+            constexpr int MT = Net::mt(l), KT = Net::kt(l);
+            const MlpLayerArgs& ly = a.layers[l];
+            const uint32_t gs = optGS((uint32_t)ly.in);
+            uint32_t* base = ldsW + Net::fragBase(l) * 64 * RAW;
+            stageFragments<ESZ, EPL>(base, ly.w, ly.shape, false, MT, KT, gs, (uint32_t)ly.out, (uint32_t)ly.in, 0, 0,
+                                     (uint32_t)(Net::fragBase(l) * 64) % 256u);
+        });
+    }
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), ROWS = 4 * MT;
+        const MlpLayerArgs& ly = a.layers[l];
+        // bias of tile t, lane group g, r: row g*ROWS + 4t + r  ->  ldsB[(biasBase + t)*16 + 4g + r]
+        const int e = (int)((threadIdx.x + 256u - 64u * (l % 4)) % 256u);
+        const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
+        const int row = g * ROWS + 4 * t + r;
+        if (e < MT * 16) ldsB[(Net::biasBase(l) + t) * 16 + 4 * g + r] = (ly.bias && row < ly.out) ? biasElem[l] : (uint16_t)0;
+    });
+    __syncthreads();
+
+    if (tile >= numTiles) return;
+
+    // ---- weights and biases to registers ---------------------------------------------------
+    uint32_t W[L][Net::MTMAX][Net::KTMAX][FD];
+    uint32_t Bs[L][Net::MTMAX][2];          // 4 fp16 biases per tile, packed
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+#pragma unroll
+        for (int t = 0; t < Net::mt(l); ++t) {
+#pragma unroll
+            for (int kt = 0; kt < Net::kt(l); ++kt)
+                Mma::decode(&ldsW[((Net::fragBase(l) + t * Net::kt(l) + kt) * 64 + lane) * RAW], W[l][t][kt]);
+            const uint16_t* bp = &ldsB[(Net::biasBase(l) + t) * 16 + 4 * g];
+            Bs[l][t][0] = (uint32_t)bp[0] | ((uint32_t)bp[1] << 16);
+            Bs[l][t][1] = (uint32_t)bp[2] | ((uint32_t)bp[3] << 16);
+        }
+    });
+
+    CarrierCfg cc[L];
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        cc[l] = makeCarrierCfg<Mma>(a.layers[l].act, a.layers[l].slope);
+        if constexpr (l + 1 == L) {   // the last layer's output is not re-quantised: plain ReLU floor
+            const half_t lo = a.layers[l].act == kActRelu ? (half_t)0.f : (half_t)-__builtin_inff();
+            cc[l].floor2 = halfx2{lo, lo};
+        }
+    });
+
     auto computeStore = [&](const uint32_t (&buf)[S][IN_DW], uint32_t t0) {
 #pragma unroll
         for (int r0 = 0; r0 < S; r0 += NT) {
@@ -297,7 +371,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 #pragma unroll
             for (int j = 0; j < NT; ++j)
 #pragma unroll
-                for (int kt = 0; kt < Net::KT0; ++kt) Mma::decode(&buf[r0 + j][kt * RAW], act[j][kt]);
+                for (int kt = 0; kt < Net::KT0; ++kt) {
+                    if constexpr (LEAN != kChunkNone) {
+                        uint32_t own[RAW];
+#pragma unroll
+                        for (int d = 0; d < RAW; ++d) own[d] = 4 * (kt * RAW + d) < validBytes ? buf[r0 + j][kt * RAW + d] : 0u;
+                        Mma::decode(own, act[j][kt]);
+                    } else {
+                        Mma::decode(&buf[r0 + j][kt * RAW], act[j][kt]);
+                    }
+                }
 
             staticFor<0, L>([&](auto lc) {
                 constexpr int l = decltype(lc)::value;
@@ -364,8 +447,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         }
     };
 
-    uint32_t bufA[S][IN_DW], bufB[S][IN_DW];
-    loadTile(bufA, tile);
+    if constexpr (LEAN != kChunkNone) {
+        // a wave with one super-tile, the launch-latency case, requests nothing more
+        if (tile + tileStride >= numTiles) {
+            computeStore(bufA, tile);
+            return;
+        }
+    }
     while (true) {
         const uint32_t t1 = tile + tileStride;
         loadTile(bufB, t1 < numTiles ? t1 : tile);
@@ -383,6 +471,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 #define CV_MLP_PREFETCH_DW 8      // input dwords per lane held in flight per buffer
 #endif
 
+// true when no layer of the network has more lane-chunks than a workgroup has threads (what the lean instantiations of
+// mlpForwardKernel assume)
+template <class Net>
+constexpr bool oneChunkPerThread()
+{
+    for (int l = 0; l < Net::L; ++l)
+        if (Net::mt(l) * Net::kt(l) * 64 > 256) return false;
+    return true;
+}
+
 template <class Mma, class Net>
 hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
@@ -393,15 +491,37 @@ hipError_t launchMlpNet(hipStream_t stream, const MlpArgs& a, int numCUs)
     constexpr int IN_DW = Mma::kRawDW * Net::KT0;
     constexpr int S0 = CV_MLP_PREFETCH_DW / IN_DW;
     constexpr int S = S0 < NT ? NT : (S0 > 16 ? 16 : S0 / NT * NT);
-    const int blocksPerCU = residentBlocksPerCU<mlpForwardKernel<Mma, Net, NT, S>>(256);
+    // the small networks, whose calls are the ones bound by launch latency, have the lean instantiations
+    int lean = kChunkNone;
+    constexpr bool kLean = NT == 4 && oneChunkPerThread<Net>();
+    if (kLean && a.inEncoding == kEncodeNone && !a.inHalfAsE4M3 && a.inAlign >= 4u && (a.layers[0].in * Mma::kEsz) % 4 == 0) {
+        for (int l = 0; l < Net::L; ++l) {
+            const MlpLayerArgs& ly = a.layers[l];
+            const int kind = chunkInFlightKind<Mma::kEsz, Mma::kEpl>(ly.w, ly.shape, Net::mt(l), Net::kt(l), optGS((uint32_t)ly.in),
+                                                                      (uint32_t)ly.out, (uint32_t)ly.in);
+            lean = l == 0 || kind == lean ? kind : kChunkNone;
+            if (lean == kChunkNone) break;
+        }
+    }
+    const int blocksPerCU = residentBlocksPerCU<mlpForwardKernel<Mma, Net, NT, S, kChunkNone>>(256);
     const uint32_t tile = 16 * S;
     const uint32_t numTiles = (a.batch + tile - 1) / tile;
     const uint32_t blocksNeeded = (numTiles + 3) / 4;
     const uint32_t blocksMax = (uint32_t)numCUs * (uint32_t)blocksPerCU;
     const uint32_t blocks = blocksNeeded < blocksMax ? blocksNeeded : blocksMax;
-    noteKernel(false, "mlpForwardKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d>", Mma::kName, Net::KT0, Net::HT,
-               Net::L - 1, Net::MTL, NT, S);
-    hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S>), dim3(blocks), dim3(256), 0, stream, a);
+    noteKernel(false, "mlpForwardKernel<%s,KT0=%d,HT=%d,hidden=%d,MTL=%d,NT=%d,S=%d%s>", Mma::kName, Net::KT0, Net::HT,
+               Net::L - 1, Net::MTL, NT, S, lean == kChunkRowDwords ? ",lean,RowMajor" : lean == kChunkDirect ? ",lean,InferencingOptimal" : "");
+    if constexpr (kLean) {
+        if (lean == kChunkRowDwords) {
+            hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S, kChunkRowDwords>), dim3(blocks), dim3(256), 0, stream, a);
+            return hipGetLastError();
+        }
+        if (lean == kChunkDirect) {
+            hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S, kChunkDirect>), dim3(blocks), dim3(256), 0, stream, a);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((mlpForwardKernel<Mma, Net, NT, S, kChunkNone>), dim3(blocks), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -123,7 +123,7 @@ __device__ __forceinline__ void storeFragmentChunk(uint32_t* d, const uint32_t (
 }
 
 template <int ESZ, int EPL>
-__device__ __forceinline__ bool fragmentSourceIsDirect(const MatrixShape& shape, bool transposed, int MT, int KT, uint32_t gs,
+__host__ __device__ __forceinline__ bool fragmentSourceIsDirect(const MatrixShape& shape, bool transposed, int MT, int KT, uint32_t gs,
                                                        uint32_t rows, uint32_t cols, uint32_t rowOff, uint32_t xorByte)
 {
     return shape.layout == kInferencingOptimal && !transposed && rowOff == 0 && xorByte == 0 &&
@@ -149,6 +149,68 @@ __device__ __forceinline__ void stageFragments(uint32_t* ldsDst, const uint8_t* 
         storeFragmentChunk<DW>(ldsDst + (size_t)c * DW, v);
     }
 }
+
+// One lane-chunk per thread in two passes, for kernels whose cost is launch latency: request() only issues loads, all
+// from addresses that exist, and finish() masks and stores.  Between the two a kernel requests its other chunks and
+// whatever else it needs at its start, so that all of it costs one round trip to memory.  Takes a matrix already in this
+// fragment order (kChunkDirect), or a RowMajor one whose rows are whole aligned dwords (kChunkRowDwords: a chunk then is
+// up to CHUNK / 4 neighbouring dwords of a row).  The kind is a template parameter, so that a request is straight-line
+// code; chunkInFlightKind names it on the host (kChunkNone: the source goes through stageFragments).
+enum : int { kChunkNone = 0, kChunkRowDwords = 1, kChunkDirect = 2 };
+template <int ESZ, int EPL>
+__host__ __device__ __forceinline__ int chunkInFlightKind(const uint8_t* w, const MatrixShape& shape, int MT, int KT, uint32_t gs,
+                                                          uint32_t rows, uint32_t cols)
+{
+    if (shape.layout == kRowMajor)
+        return ((uintptr_t)w & 3u) == 0 && (shape.stride & 3u) == 0 && ((size_t)shape.cols * ESZ & 3u) == 0 ? kChunkRowDwords : kChunkNone;
+    return fragmentSourceIsDirect<ESZ, EPL>(shape, false, MT, KT, gs, rows, cols, 0, 0) ? kChunkDirect : kChunkNone;
+}
+
+// v: the chunk's dwords as they lie in memory; validBytes: how many of its bytes exist
+template <int ESZ, int EPL, int KIND>
+struct ChunkInFlight {
+    static constexpr int CHUNK = ESZ * EPL, DW = CHUNK / 4;
+    static_assert(ESZ <= 2 && (CHUNK == 8 || CHUNK == 16), "one or two 8-byte words per lane-chunk");
+    static_assert(KIND == kChunkRowDwords || KIND == kChunkDirect, "kind of source");
+    static __device__ __forceinline__ void request(uint32_t (&v)[DW], int& validBytes, const uint8_t* w, const MatrixShape& shape,
+                                                   int MT, int KT, uint32_t gs, uint32_t rows, uint32_t cols, int c)
+    {
+        if constexpr (KIND == kChunkDirect) {
+            validBytes = CHUNK;
+            if constexpr (DW == 4) {
+                const u32x4 x = *(const u32x4*)(w + (size_t)c * CHUNK);
+                v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+            } else {
+                const u32x2 x = *(const u32x2*)(w + (size_t)c * CHUNK);
+                v[0] = x.x; v[1] = x.y;
+            }
+            return;
+        }
+        // (the geometry of fetchFragmentChunk)
+        const int lane = c & 63, f = c >> 6;
+        const int kt = f % KT, t = f / KT, g = lane >> 4, i = lane & 15;
+        const uint32_t row = (uint32_t)((i >> 2) * 4 * MT + 4 * t + (i & 3));
+        const uint32_t q0 = (uint32_t)(kt * EPL), col0 = g * gs + q0;
+        int nvalid = 0;
+        if (row < rows && q0 < gs && col0 < cols) {
+            const uint32_t a = gs - q0, b = cols - col0;
+            nvalid = (int)(a < b ? a : b);
+            if (nvalid > EPL) nvalid = EPL;
+        }
+        validBytes = nvalid * ESZ;
+        const size_t line = shape.stride ? shape.stride : (size_t)shape.cols * ESZ;
+        const size_t first = nvalid > 0 ? (size_t)row * line + (size_t)col0 * ESZ : 0;
+#pragma unroll
+        for (int d = 0; d < DW; ++d) v[d] = *(const uint32_t*)(w + (4 * d < validBytes ? first + 4 * d : 0));
+    }
+    static __device__ __forceinline__ void finish(const uint32_t (&v)[DW], int validBytes, uint32_t* ldsDst)
+    {
+        uint32_t out[DW];
+#pragma unroll
+        for (int d = 0; d < DW; ++d) out[d] = 4 * d < validBytes ? v[d] : 0u;
+        storeFragmentChunk<DW>(ldsDst, out);
+    }
+};
 
 // The same in two passes, for kernels that stage several matrices: load() of every matrix first, then store() of
 // every matrix, so that all of a thread's loads are in flight together and the whole staging costs one round trip to
