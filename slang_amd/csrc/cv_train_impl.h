@@ -183,6 +183,111 @@ __device__ __forceinline__ halfx2 applyActGrad(halfx2 gv, halfx2 m, int act, hal
     return da + db * slope2;
 }
 
+// Where value p of a step's summed partial (dW tiles in accumulator order, then db tiles) belongs in the gradient buffers
+// ("+=", any layout, fp16 or fp32): the element's address, or null for a value of the tiling's padding.
+template <class Net>
+__device__ __forceinline__ uint8_t* gradientSlot(const TrainReduceArgs& ra, uint32_t p)
+{
+    constexpr int L = Net::L;
+    constexpr uint32_t nW = Net::totalGradTiles * 256;
+    const uint32_t esz = ra.gradCt == kF32 ? 4u : 2u;
+    uint8_t* slot = nullptr;
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
+        constexpr uint32_t w0 = Net::gradTileBase(l) * 256, w1 = w0 + MTO * NI * 256;
+        constexpr uint32_t b0 = nW + Net::dbTileBase(l) * 16, b1 = b0 + MTO * 16;
+        const TrainReduceArgs::Layer& ly = ra.layers[l];
+        if (p >= w0 && p < w1) {
+            const uint32_t q = p - w0, tile = q >> 8, ln = (q >> 2) & 63u, r = q & 3u;
+            const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
+            const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
+            const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
+            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) slot = ly.wGrad + elemOffset(ly.gradShape, o, i);
+        } else if (p >= b0 && p < b1) {
+            const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
+            const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
+            if (ly.bGrad && o < (uint32_t)ly.out) slot = ly.bGrad + (size_t)o * esz;
+        }
+    });
+    return slot;
+}
+__device__ __forceinline__ float loadGradient(const uint8_t* slot, int gradCt)
+{
+    return gradCt == kF32 ? *(const float*)slot : (float)*(const half_t*)slot;
+}
+__device__ __forceinline__ void storeGradient(uint8_t* slot, int gradCt, float v)
+{
+    if (gradCt == kF32) *(float*)slot = v;
+    else *(half_t*)slot = (half_t)v;
+}
+template <class Net>
+__device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32_t p, float s)
+{
+    uint8_t* slot = gradientSlot<Net>(ra, p);
+    if (slot) storeGradient(slot, ra.gradCt, loadGradient(slot, ra.gradCt) + s);
+}
+
+// Stages the weights of every layer as A fragments of the forward pass (ldsW), their transposes as A fragments of the dX
+// pass (ldsWT, layers 1 and up) and the biases as fp32 (ldsB); BLOCK threads, ends behind a barrier.
+template <class Net, int BLOCK>
+__device__ __forceinline__ void stageTrainingWeights(const MlpArgs& a, uint32_t* ldsW, uint32_t* ldsWT, float* ldsB)
+{
+    constexpr int L = Net::L, EPL = 8, RAW = 4;
+    // All loads of all layers first, then all stores: one round trip to memory for the whole staging (layer after
+    // layer, each matrix and each bias vector waiting for its own loads, it took 14 us of the paired kernel's 131 us).  W^T is not
+    // fetched from memory: used as its transpose, a row-major matrix hands a lane eight elements from eight rows, one
+    // 2-byte load each that touches 64 cache lines per instruction (7 us per workgroup, more when all of them do it at
+    // once); its fragments are gathered from the W fragments once those lie in LDS.
+    constexpr int kStageIters = (Net::MTMAX * Net::KTMAX * 64 + BLOCK - 1) / BLOCK;
+    FragmentStage<2, EPL, kStageIters, BLOCK> stW[L];
+    float stB[L];
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
+        static_assert(MT * 16 <= BLOCK, "one bias value per thread and layer");
+        const MlpLayerArgs& ly = a.layers[l];
+        // (k-slots per lane group: those of the kernel's tiling; a hidden layer narrower than the widest one is padded to it)
+        stW[l].load(ly.w, ly.shape, false, MT, KT, l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0), (uint32_t)ly.out, (uint32_t)ly.in);
+        const int e = threadIdx.x, t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
+        const int row = gg * ROWS + 4 * t + r;
+        stB[l] = (e < MT * 16 && ly.bias && row < ly.out) ? (float)((const half_t*)ly.bias)[row] : 0.f;
+    });
+    staticFor<0, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l);
+        stW[l].store(ldsW + Net::fragBase(l) * 64 * RAW, MT, KT);
+        if ((int)threadIdx.x < MT * 16) ldsB[Net::biasBase(l) * 16 + threadIdx.x] = stB[l];
+    });
+    __syncthreads();
+    // Lane 16*g + i of W^T fragment (t, kt) of layer l holds W[g*gsOut + kt*8 + s][(i/4)*4*MTI + 4*t + i%4], s < 8 (output
+    // unit on the k axis, input unit as the row); element W[o][c] lies in W fragment ((o % (4*MT)) / 4, (c % gsIn) / 8) at
+    // lane 16*(c / gsIn) + 4*(o / (4*MT)) + o%4, slot c % 8 (cv_layout.h).  Rows and columns past the matrix are zero there.
+    staticFor<1, L>([&](auto lc) {
+        constexpr int l = decltype(lc)::value;
+        constexpr int MT = Net::mt(l), KT = Net::kt(l), MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
+        constexpr int gsOut = 4 * MT, gsIn = 4 * MTI, chunks = MTI * KTO * 64;
+        const uint16_t* src = (const uint16_t*)(ldsW + Net::fragBase(l) * 64 * RAW);
+        for (int c = threadIdx.x; c < chunks; c += BLOCK) {
+            const int ln = c & 63, f = c >> 6, kt = f % KTO, t = f / KTO, g = ln >> 4, i = ln & 15;
+            const int col = (i >> 2) * 4 * MTI + 4 * t + (i & 3);         // the input unit
+            const int gW = col / gsIn, ktW = (col % gsIn) / EPL, sW = (col % gsIn) % EPL;
+            uint32_t v[EPL];
+#pragma unroll
+            for (int s2 = 0; s2 < EPL; ++s2) {
+                const int q = kt * EPL + s2, o = g * gsOut + q;          // the output unit
+                const int tW = (o % (4 * MT)) / 4, iW = 4 * (o / (4 * MT)) + o % 4;
+                const int idx = (((q < gsOut ? tW : 0) * KT + ktW) * 64 + 16 * gW + (q < gsOut ? iW : 0)) * EPL + sW;
+                const uint32_t x = src[idx];
+                v[s2] = q < gsOut ? x : 0u;
+            }
+            *(u32x4*)&ldsWT[(Net::tFragBase(l) * 64 + c) * RAW] = u32x4{v[0] | v[1] << 16, v[2] | v[3] << 16, v[4] | v[5] << 16, v[6] | v[7] << 16};
+        }
+    });
+    __syncthreads();
+
+}
+
 // LOADS selects how the network input is fetched.  kLoadDwords (every lane's slice is whole, 4-byte
 // aligned dwords) and kLoadXY (float2 samples of the example's encoding) are straight-line code: every
 // lane loads from an address that is always valid and masks afterwards, so the requests of the next
@@ -217,30 +322,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __shared__ __attribute__((aligned(16))) uint32_t ldsXF[4 * Net::totalXTiles * 256];
 
     // ---- stage W (A operand of the forward pass), W^T (A operand of dX) and biases ----------
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
-        const MlpLayerArgs& ly = a.layers[l];
-        // k-slots per lane group: those of the kernel's tiling (a hidden layer narrower than the widest one is padded to it)
-        const uint32_t gs = l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0);
-        stageFragments<2, EPL>(ldsW + Net::fragBase(l) * 64 * RAW, ly.w, ly.shape, false, MT, KT, gs,
-                               (uint32_t)ly.out, (uint32_t)ly.in);
-        if constexpr (l > 0) {
-            // rows of W^T are this layer's inputs (tiled like the previous layer's outputs),
-            // its k axis are this layer's outputs
-            constexpr int MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
-            stageFragments<2, EPL>(ldsWT + Net::tFragBase(l) * 64 * RAW, ly.w, ly.shape, true, MTI, KTO, 4u * MT,
-                                   (uint32_t)ly.in, (uint32_t)ly.out);
-        }
-        for (int e = threadIdx.x; e < MT * 16; e += 256) {
-            const int t = e >> 4, g = (e >> 2) & 3, r = e & 3;
-            const int row = g * ROWS + 4 * t + r;
-            float v = 0.f;
-            if (ly.bias && row < ly.out) v = (float)((const half_t*)ly.bias)[row];
-            ldsB[(Net::biasBase(l) + t) * 16 + 4 * g + r] = v;
-        }
-    });
-    __syncthreads();
+    stageTrainingWeights<Net, 256>(a, ldsW, ldsWT, ldsB);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, n = lane & 15;
@@ -645,28 +727,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
     // ---- workgroup partial: sum the four waves in a fixed order, one tile at a time ----------
+    // The only workgroup of a launch (ta.finishInKernel) does with its sums what mlpTrainReduceKernel would do with this one
+    // partial: they go from its registers to the gradients.  The gradient elements they are added to are requested ahead,
+    // eight tiles at a time, so that a group of tiles costs one round trip to memory, and the loss is summed first: a NaN
+    // there makes every sum of the step NaN (see mlpTrainReduceKernel).
     float* part = ta.partials + (size_t)blockIdx.x * Net::partialFloats;
-#pragma unroll
-    for (int i = 0; i < Net::totalGradTiles; ++i) {
-        *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[i];
-        __syncthreads();
-        const float s = ((ldsRed[threadIdx.x] + ldsRed[256 + threadIdx.x]) + ldsRed[512 + threadIdx.x]) + ldsRed[768 + threadIdx.x];
-        part[i * 256 + threadIdx.x] = s;
-        __syncthreads();
-    }
-    // bias gradients: lane (g,q) holds the sum over its samples; sum the 4 lane groups and 4 waves
-#pragma unroll
-    for (int i = 0; i < Net::totalDbTiles; ++i) {
-        ldsRed[wave * 64 + lane] = accB[i];
-        __syncthreads();
-        if (threadIdx.x < 16) {
-            float s = 0.f;
-            for (int w = 0; w < 4; ++w)
-                for (int gg = 0; gg < 4; ++gg) s += ldsRed[w * 64 + gg * 16 + threadIdx.x];
-            part[Net::totalGradTiles * 256 + i * 16 + threadIdx.x] = s;
-        }
-        __syncthreads();
-    }
+    constexpr uint32_t nValues = Net::totalGradTiles * 256 + Net::totalDbTiles * 16;
+    const bool finish = ta.finishInKernel != 0;
+    const TrainReduceArgs& ra = ta.finish;
+    __shared__ float ldsLossSum;
     ldsRed[threadIdx.x] = lossAcc;
     if (ta.wantLossMax) noteLossMax(&ldsLossMax, lossMaxAcc);
     __syncthreads();
@@ -678,73 +747,77 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
         if (lane == 0) {
-            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16] = s;
-            part[Net::totalGradTiles * 256 + Net::totalDbTiles * 16 + 1] = __builtin_bit_cast(float, ldsLossMax);
+            ldsLossSum = s;
+            if (!finish) {
+                part[nValues] = s;
+                part[nValues + 1] = __builtin_bit_cast(float, ldsLossMax);
+            }
         }
     }
-    if (!ta.finishInKernel) return;
-    // ---- the only workgroup of the launch: what mlpTrainReduceKernel would do with this one partial --------------
-    __threadfence_block();
+    // bias gradients' destinations (threads 0 .. 15 hold one element of every tile)
+    float oldB[Net::totalDbTiles];
+#pragma unroll
+    for (int i = 0; i < Net::totalDbTiles; ++i) {
+        oldB[i] = 0.f;
+        if (finish && threadIdx.x < 16) {
+            const uint8_t* slot = gradientSlot<Net>(ra, Net::totalGradTiles * 256 + i * 16 + threadIdx.x);
+            if (slot) oldB[i] = loadGradient(slot, ra.gradCt);
+        }
+    }
     __syncthreads();
-    constexpr uint32_t nValues = Net::totalGradTiles * 256 + Net::totalDbTiles * 16;
-    const TrainReduceArgs& ra = ta.finish;
-    const float lossPart = part[nValues];
-    const bool voidStep = lossPart != lossPart;                  // see mlpTrainReduceKernel
-    for (uint32_t p = threadIdx.x; p <= nValues; p += 256u) {
-        float s = 0.f + part[p];                                   // the sum of one partial, as sumPartials forms it
-        if (voidStep) s = __builtin_nanf("");
-        if (p == nValues) {
-            if (ra.lossSum) *ra.lossSum = s;
-        } else {
-            addToGradients<Net>(ra, p, s);
+    const bool voidStep = finish && ldsLossSum != ldsLossSum;
+    constexpr int kAhead = 8;
+#pragma unroll
+    for (int i0 = 0; i0 < Net::totalGradTiles; i0 += kAhead) {
+        float old[kAhead];
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            old[k] = 0.f;
+            if (finish && i0 + k < Net::totalGradTiles) {
+                const uint8_t* slot = gradientSlot<Net>(ra, (i0 + k) * 256 + threadIdx.x);
+                if (slot) old[k] = loadGradient(slot, ra.gradCt);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < kAhead; ++k) {
+            const int i = i0 + k;
+            if (i >= Net::totalGradTiles) break;
+            *(floatx4*)&ldsRed[wave * 256 + lane * 4] = accW[i];
+            __syncthreads();
+            float s = ((ldsRed[threadIdx.x] + ldsRed[256 + threadIdx.x]) + ldsRed[512 + threadIdx.x]) + ldsRed[768 + threadIdx.x];
+            if (!finish) {
+                part[i * 256 + threadIdx.x] = s;
+            } else {
+                s = voidStep ? __builtin_nanf("") : 0.f + s;         // (the sum of one partial, as sumPartials forms it)
+                uint8_t* slot = gradientSlot<Net>(ra, i * 256 + threadIdx.x);
+                if (slot) storeGradient(slot, ra.gradCt, old[k] + s);
+            }
+            __syncthreads();
         }
     }
-    if (ra.lossMax && threadIdx.x == 0) *ra.lossMax = voidStep ? __builtin_nanf("") : part[nValues + 1];
-}
-
-// Where value p of a step's summed partial (dW tiles in accumulator order, then db tiles) belongs in the gradient buffers
-// ("+=", any layout, fp16 or fp32): the element's address, or null for a value of the tiling's padding.
-template <class Net>
-__device__ __forceinline__ uint8_t* gradientSlot(const TrainReduceArgs& ra, uint32_t p)
-{
-    constexpr int L = Net::L;
-    constexpr uint32_t nW = Net::totalGradTiles * 256;
-    const uint32_t esz = ra.gradCt == kF32 ? 4u : 2u;
-    uint8_t* slot = nullptr;
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MTO = Net::nOt(l), NI = Net::nIt(l);
-        constexpr uint32_t w0 = Net::gradTileBase(l) * 256, w1 = w0 + MTO * NI * 256;
-        constexpr uint32_t b0 = nW + Net::dbTileBase(l) * 16, b1 = b0 + MTO * 16;
-        const TrainReduceArgs::Layer& ly = ra.layers[l];
-        if (p >= w0 && p < w1) {
-            const uint32_t q = p - w0, tile = q >> 8, ln = (q >> 2) & 63u, r = q & 3u;
-            const uint32_t eo = tile / NI, ei = tile % NI, gq = ln >> 4, qi = ln & 15u;
-            const uint32_t o = gq * (4u * MTO) + 4u * eo + r;
-            const uint32_t i = (qi >> 2) * (4u * NI) + 4u * ei + (qi & 3u);
-            if (ly.wGrad && o < (uint32_t)ly.out && i < (uint32_t)ly.in) slot = ly.wGrad + elemOffset(ly.gradShape, o, i);
-        } else if (p >= b0 && p < b1) {
-            const uint32_t q = p - b0, eo = q >> 4, qo = q & 15u;
-            const uint32_t o = (qo >> 2) * (4u * MTO) + 4u * eo + (qo & 3u);
-            if (ly.bGrad && o < (uint32_t)ly.out) slot = ly.bGrad + (size_t)o * esz;
+    // bias gradients: lane (g,q) holds the sum over its samples; sum the 4 lane groups and 4 waves
+#pragma unroll
+    for (int i = 0; i < Net::totalDbTiles; ++i) {
+        ldsRed[wave * 64 + lane] = accB[i];
+        __syncthreads();
+        if (threadIdx.x < 16) {
+            float s = 0.f;
+            for (int w = 0; w < 4; ++w)
+                for (int gg = 0; gg < 4; ++gg) s += ldsRed[w * 64 + gg * 16 + threadIdx.x];
+            if (!finish) {
+                part[Net::totalGradTiles * 256 + i * 16 + threadIdx.x] = s;
+            } else {
+                s = voidStep ? __builtin_nanf("") : 0.f + s;
+                uint8_t* slot = gradientSlot<Net>(ra, Net::totalGradTiles * 256 + i * 16 + threadIdx.x);
+                if (slot) storeGradient(slot, ra.gradCt, oldB[i] + s);
+            }
         }
-    });
-    return slot;
-}
-__device__ __forceinline__ float loadGradient(const uint8_t* slot, int gradCt)
-{
-    return gradCt == kF32 ? *(const float*)slot : (float)*(const half_t*)slot;
-}
-__device__ __forceinline__ void storeGradient(uint8_t* slot, int gradCt, float v)
-{
-    if (gradCt == kF32) *(float*)slot = v;
-    else *(half_t*)slot = (half_t)v;
-}
-template <class Net>
-__device__ __forceinline__ void addToGradients(const TrainReduceArgs& ra, uint32_t p, float s)
-{
-    uint8_t* slot = gradientSlot<Net>(ra, p);
-    if (slot) storeGradient(slot, ra.gradCt, loadGradient(slot, ra.gradCt) + s);
+        __syncthreads();
+    }
+    if (finish && threadIdx.x == 0) {
+        if (ra.lossSum) *ra.lossSum = voidStep ? __builtin_nanf("") : 0.f + ldsLossSum;
+        if (ra.lossMax) *ra.lossMax = voidStep ? __builtin_nanf("") : __builtin_bit_cast(float, ldsLossMax);
+    }
 }
 
 // Sums the workgroup partials in a fixed order and adds them to the gradient buffers.

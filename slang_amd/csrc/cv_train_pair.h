@@ -156,58 +156,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     uint32_t* const ldsLossMax = ldsFlag + FLAG_DW;
     if (threadIdx.x < FLAG_DW + MAX_DW) ldsFlag[threadIdx.x] = 0u;
 
-    // ---- stage W, W^T and biases ----------------------------------------------------------------
-    // All loads of all layers first, then all stores: one round trip to memory for the whole staging (layer after
-    // layer, each matrix and each bias vector waiting for its own loads, it took 14 us of a 131 us kernel).  W^T is not
-    // fetched from memory: used as its transpose, a row-major matrix hands a lane eight elements from eight rows, one
-    // 2-byte load each that touches 64 cache lines per instruction (7 us per workgroup, more when all of them do it at
-    // once); its fragments are gathered from the W fragments once those lie in LDS.
-    constexpr int kStageIters = (Net::MTMAX * Net::KTMAX * 64 + 511) / 512;
-    FragmentStage<2, EPL, kStageIters, 512> stW[L];
-    float stB[L];
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MT = Net::mt(l), KT = Net::kt(l), ROWS = 4 * MT;
-        static_assert(MT * 16 <= 512, "one bias value per thread and layer");
-        const MlpLayerArgs& ly = a.layers[l];
-        // (k-slots per lane group: those of the kernel's tiling; a hidden layer narrower than the widest one is padded to it)
-        stW[l].load(ly.w, ly.shape, false, MT, KT, l == 0 ? optGS((uint32_t)ly.in) : 4u * (uint32_t)Net::mt(l > 0 ? l - 1 : 0), (uint32_t)ly.out, (uint32_t)ly.in);
-        const int e = threadIdx.x, t = e >> 4, gg = (e >> 2) & 3, r = e & 3;
-        const int row = gg * ROWS + 4 * t + r;
-        stB[l] = (e < MT * 16 && ly.bias && row < ly.out) ? (float)((const half_t*)ly.bias)[row] : 0.f;
-    });
-    staticFor<0, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MT = Net::mt(l), KT = Net::kt(l);
-        stW[l].store(ldsW + Net::fragBase(l) * 64 * RAW, MT, KT);
-        if ((int)threadIdx.x < MT * 16) ldsB[Net::biasBase(l) * 16 + threadIdx.x] = stB[l];
-    });
-    __syncthreads();
-    // Lane 16*g + i of W^T fragment (t, kt) of layer l holds W[g*gsOut + kt*8 + s][(i/4)*4*MTI + 4*t + i%4], s < 8 (output
-    // unit on the k axis, input unit as the row); element W[o][c] lies in W fragment ((o % (4*MT)) / 4, (c % gsIn) / 8) at
-    // lane 16*(c / gsIn) + 4*(o / (4*MT)) + o%4, slot c % 8 (cv_layout.h).  Rows and columns past the matrix are zero there.
-    staticFor<1, L>([&](auto lc) {
-        constexpr int l = decltype(lc)::value;
-        constexpr int MT = Net::mt(l), KT = Net::kt(l), MTI = Net::mt(l - 1), KTO = Net::ktOut(l);
-        constexpr int gsOut = 4 * MT, gsIn = 4 * MTI, chunks = MTI * KTO * 64;
-        const uint16_t* src = (const uint16_t*)(ldsW + Net::fragBase(l) * 64 * RAW);
-        for (int c = threadIdx.x; c < chunks; c += 512) {
-            const int ln = c & 63, f = c >> 6, kt = f % KTO, t = f / KTO, g = ln >> 4, i = ln & 15;
-            const int col = (i >> 2) * 4 * MTI + 4 * t + (i & 3);         // the input unit
-            const int gW = col / gsIn, ktW = (col % gsIn) / EPL, sW = (col % gsIn) % EPL;
-            uint32_t v[EPL];
-#pragma unroll
-            for (int s2 = 0; s2 < EPL; ++s2) {
-                const int q = kt * EPL + s2, o = g * gsOut + q;          // the output unit
-                const int tW = (o % (4 * MT)) / 4, iW = 4 * (o / (4 * MT)) + o % 4;
-                const int idx = (((q < gsOut ? tW : 0) * KT + ktW) * 64 + 16 * gW + (q < gsOut ? iW : 0)) * EPL + sW;
-                const uint32_t x = src[idx];
-                v[s2] = q < gsOut ? x : 0u;
-            }
-            *(u32x4*)&ldsWT[(Net::tFragBase(l) * 64 + c) * RAW] = u32x4{v[0] | v[1] << 16, v[2] | v[3] << 16, v[4] | v[5] << 16, v[6] | v[7] << 16};
-        }
-    });
-    __syncthreads();
+    stageTrainingWeights<Net, 512>(a, ldsW, ldsWT, ldsB);
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pair = wave >> 1, par = wave & 1;      // partners sit on neighbouring SIMDs
