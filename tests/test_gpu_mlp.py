@@ -600,3 +600,54 @@ def test_fused_forward_equals_the_chain_of_single_layers_on_random_shapes():
         yc = chain_of_single_layers(specs, xd, wtype)
         assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), (case, dims, B, cv.lastKernelName())
     assert len(kernels) >= 3, kernels
+
+
+@pytest.mark.parametrize("layout", [ML.RowMajor, ML.InferencingOptimal, ML.ColumnMajor])
+def test_small_networks_on_the_lean_instantiations(layout):
+    # Networks of 16-wide layers run on mlpForwardKernel's lean instantiations when their matrices are RowMajor with
+    # rows of whole dwords or already in fragment order and the input vectors are whole aligned dwords; everything else
+    # (ColumnMajor, rows or vectors of an odd number of halfs, a 6-byte pitch) stays on the general one.  Either way the
+    # result equals the chain of single layers bit for bit, for batches of one sample, of one super-tile per wave, and
+    # of several.
+    rng = np.random.default_rng(411)
+    lean_seen = 0
+    for dims in ([2, 16, 16, 16, 1], [4, 16, 4], [16, 16, 16, 16, 16], [6, 10, 12, 3], [8, 16, 1], [3, 16, 16, 2], [2, 16, 5, 4]):
+        for bias in ("rand", "none"):
+            specs = make_net(rng, dims, CT.Float16, act=Activation.ReLU, bias=bias, init="he")
+            layers = gpu_layers(specs, CT.Float16, layout)
+            for B, pitch in ((1, 0), (15, 0), (64, 0), (65, 2), (1000, 0), (1000, 1), (70001, 0), (300000, 2)):
+                full = to_dev(rng.uniform(-1, 1, (B, dims[0] + pitch)).astype(np.float16))
+                xd = full[:, :dims[0]]
+                y = cv.mlpForward(layers, xd, weightType=CT.Float16)
+                name = cv.lastKernelName()
+                whole = (dims[0] * 2) % 4 == 0 and ((dims[0] + pitch) * 2) % 4 == 0
+                rows = all((d * 2) % 4 == 0 for d in dims[:-1])
+                expect_lean = whole and (layout == ML.InferencingOptimal or (layout == ML.RowMajor and rows))
+                if name.startswith("mlpForwardKernel"):      # (some of these shapes belong to the run-time-size kernel)
+                    assert ("lean" in name) == expect_lean, (dims, B, pitch, name)
+                    lean_seen += expect_lean
+                yc = chain_of_single_layers(specs, xd.contiguous(), CT.Float16)
+                assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), (dims, bias, B, pitch, name)
+    assert lean_seen > 0 or layout == ML.ColumnMajor
+
+
+def test_lean_instantiation_with_padded_weight_rows():
+    # RowMajor rows with a pitch beyond their length (whole dwords: lean; an odd number of halfs: general)
+    rng = np.random.default_rng(412)
+    dims = [4, 16, 12, 16, 2]
+    specs = make_net(rng, dims, CT.Float16, act=Activation.ReLU, bias="rand", init="he")
+    xd = to_dev(rng.uniform(-1, 1, (777, dims[0])).astype(np.float16))
+    yc = chain_of_single_layers(specs, xd, CT.Float16)
+    for pad, lean in ((2, True), (6, True), (1, False)):
+        layers = []
+        for s in specs:
+            out, fan_in = s["W"].shape
+            padded = np.zeros((out, fan_in + pad), np.float16)
+            padded[:, :fan_in] = s["W"]
+            padded[:, fan_in:] = 7.0            # (never read)
+            layers.append(FeedForwardLayer(fan_in, out, as_bytes(to_dev(padded)), as_bytes(to_dev(s["b"])), ML.RowMajor,
+                                           (fan_in + pad) * 2, s["act"], s["slope"]))
+        y = cv.mlpForward(layers, xd, weightType=CT.Float16)
+        if cv.lastKernelName().startswith("mlpForwardKernel"):
+            assert ("lean" in cv.lastKernelName()) == lean, (pad, cv.lastKernelName())
+        assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), pad
