@@ -24,7 +24,7 @@ ORACLE_DIR = os.path.join(REPO_DIR, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "libcoopvec_oracle.so")
 
 HIP_SOURCES = ["cv_abi.hip", "cv_convert.hip", "cv_matmul_f16.hip", "cv_matmul_fp8.hip",
-               "cv_matmul_i8.hip", "cv_matmul_fp8b.hip", "cv_matmul_bf16.hip", "cv_matmul_f32.hip", "cv_matmul_scalar.hip", "cv_mlp_f16.hip", "cv_mlp_f16w8.hip", "cv_mlp_f16w16.hip", "cv_mlp_f16w32.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip", "cv_mlp_generic.hip", "cv_mlp_float.hip", "cv_train.hip", "cv_train_team.hip", "cv_train_quad.hip", "cv_train_general.hip", "cv_accum.hip", "cv_accum_scalar.hip", "cv_adam.hip", "cv_elementwise.hip", "cv_permuto.hip", "cv_permuto_mlp.hip", "cv_permuto_w16.hip", "cv_permuto_w32.hip", "cv_neural.hip"]
+               "cv_matmul_i8.hip", "cv_matmul_fp8b.hip", "cv_matmul_bf16.hip", "cv_matmul_f32.hip", "cv_matmul_scalar.hip", "cv_mlp_f16.hip", "cv_mlp_f16w8.hip", "cv_mlp_f16w16.hip", "cv_mlp_f16w32.hip", "cv_mlp_fp8.hip", "cv_mlp_fp8n.hip", "cv_mlp_generic.hip", "cv_mlp_float.hip", "cv_train.hip", "cv_train_team.hip", "cv_train_quad.hip", "cv_train_general.hip", "cv_accum.hip", "cv_accum_f32.hip", "cv_accum_scalar.hip", "cv_adam.hip", "cv_elementwise.hip", "cv_permuto.hip", "cv_permuto_mlp.hip", "cv_permuto_w16.hip", "cv_permuto_w32.hip", "cv_neural.hip"]
 
 # packed-fp32 instructions are switched off on purpose (see the flag below): hipcc would
 # otherwise form v_pk_*_f32 from ordinary float code.  -ffp-contract=off: the kernels state every

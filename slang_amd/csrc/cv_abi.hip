@@ -467,7 +467,8 @@ CV_API CvResult cvOuterProductAccumulateWorkspaceSize(int32_t m, int32_t n, uint
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     const size_t fast = cv::outerWorkspaceBytes(m, n, batch ? batch : 1, cus), scalar = cv::accumScalarWorkspaceBytes(m, n, batch ? batch : 1);
-    *outBytes = fast > scalar ? fast : scalar;      // whichever kernel the element types select
+    const size_t f32 = cv::outerF32WorkspaceBytes(m, n, batch ? batch : 1, cus);
+    *outBytes = std::max(fast, std::max(scalar, f32));      // whichever kernel the element types select
     return CV_OK;
 }
 
@@ -500,6 +501,15 @@ CV_API CvResult cvOuterProductAccumulate(void* stream, const void* a, size_t aSt
         if (cv::matrixSize(shape) == 0) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrixStride %u smaller than a row/column", matrixStride);
         uint8_t* dst = (uint8_t*)matrix + matrixOffset;
         if ((uintptr_t)dst % msz || (!isOptimal(layout) && matrixStride % msz)) return fail(CV_E_INVALID_ARG, "cvOuterProductAccumulate: matrix misaligned");
+        if (elementType == CV_FLOAT32 && matrixInterpretation == CV_FLOAT32) {      // the matrix pipeline's fp32 instruction
+            CvResult rc;
+            const int cus = currentDeviceCUs(&rc);
+            if (CV_FAILED(rc)) return rc;
+            const size_t need = cv::outerF32WorkspaceBytes(m, n, batch, cus);
+            if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvOuterProductAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+            return fromHip(cv::launchOuterProductF32((hipStream_t)stream, (const uint8_t*)a, aStride, m, (const uint8_t*)b, bStride, n, batch, dst,
+                                                     shape, workspace, cus), "cvOuterProductAccumulate launch");
+        }
         const size_t need = cv::accumScalarWorkspaceBytes(m, n, batch);
         if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvOuterProductAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
         return fromHip(cv::launchAccumScalar((hipStream_t)stream, (const uint8_t*)a, aStride, m, (const uint8_t*)b, bStride, n, elementType, batch,
@@ -539,7 +549,8 @@ CV_API CvResult cvReduceSumAccumulateWorkspaceSize(int32_t n, uint32_t batch, si
     const int cus = currentDeviceCUs(&rc);
     if (CV_FAILED(rc)) return rc;
     const size_t fast = cv::reduceSumWorkspaceBytes(batch ? batch : 1, cus), scalar = cv::accumScalarWorkspaceBytes(n, 1, batch ? batch : 1);
-    *outBytes = fast > scalar ? fast : scalar;
+    const size_t f32 = cv::outerF32WorkspaceBytes(n, 1, batch ? batch : 1, cus);
+    *outBytes = std::max(fast, std::max(scalar, f32));
     return CV_OK;
 }
 
@@ -559,9 +570,18 @@ CV_API CvResult cvReduceSumAccumulate(void* stream, const void* v, size_t vStrid
         if ((uintptr_t)v % tsz || vStride % tsz || ((uintptr_t)buffer + offset) % tsz || (uintptr_t)workspace % 8)
             return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: misaligned argument");
         if (batch > 1 && vStride < (size_t)n * tsz) return fail(CV_E_INVALID_ARG, "cvReduceSumAccumulate: vector stride smaller than the vector");
+        const cv::MatrixShape shape{(uint32_t)n, 1u, elementType, CV_LAYOUT_ROW_MAJOR, (size_t)tsz};
+        if (elementType == CV_FLOAT32) {      // the matrix pipeline's fp32 instruction
+            CvResult rc;
+            const int cus = currentDeviceCUs(&rc);
+            if (CV_FAILED(rc)) return rc;
+            const size_t need = cv::outerF32WorkspaceBytes(n, 1, batch, cus);
+            if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvReduceSumAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
+            return fromHip(cv::launchOuterProductF32((hipStream_t)stream, (const uint8_t*)v, vStride, n, nullptr, 0, 1, batch,
+                                                     (uint8_t*)buffer + offset, shape, workspace, cus), "cvReduceSumAccumulate launch");
+        }
         const size_t need = cv::accumScalarWorkspaceBytes(n, 1, batch);
         if (workspaceBytes < need) return fail(CV_E_BUFFER_TOO_SMALL, "cvReduceSumAccumulate: workspace of %zu bytes, %zu needed", workspaceBytes, need);
-        const cv::MatrixShape shape{(uint32_t)n, 1u, elementType, CV_LAYOUT_ROW_MAJOR, (size_t)tsz};
         return fromHip(cv::launchAccumScalar((hipStream_t)stream, (const uint8_t*)v, vStride, n, nullptr, 0, 1, elementType, batch,
                                              (uint8_t*)buffer + offset, shape, workspace), "cvReduceSumAccumulate launch");
     }

@@ -137,6 +137,11 @@ struct OuterArgs {
 size_t outerWorkspaceBytes(int m, int n, uint32_t batch, int numCUs);
 hipError_t launchOuterProduct(hipStream_t stream, const OuterArgs& args, int numCUs);
 
+// fp32 vectors into an fp32 matrix on the matrix pipeline (cv_accum_f32.hip); b == nullptr with n == 1 is the reduce-sum form
+size_t outerF32WorkspaceBytes(int m, int n, uint32_t batch, int numCUs);
+hipError_t launchOuterProductF32(hipStream_t stream, const uint8_t* a, uint64_t aStride, int m, const uint8_t* b, uint64_t bStride,
+                                 int n, uint32_t batch, uint8_t* mat, const MatrixShape& shape, void* workspace, int numCUs);
+
 // The scalar definition of both accumulate operators for every plain element type (cv_accum_scalar.hip):
 // matrix[i][j] += cast<MatT>(a[i] * b[j]) summed over the batch; b == nullptr with n == 1 is the reduce-sum form.
 bool isPlainComponent(int ct);

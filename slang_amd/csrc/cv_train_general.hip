@@ -77,6 +77,8 @@ GeneralPlan makePlan(const MlpArgs& a, int numCUs, int carrierCt)
         if (carrierCt != kF16) {
             const size_t sc = accumScalarWorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch);
             if (sc > part) part = sc;
+            const size_t mp = outerF32WorkspaceBytes(a.layers[l].out, a.layers[l].in, (uint32_t)batch, numCUs);
+            if (mp > part) part = mp;
         }
     }
     p.partials = off; off += alignUp(part);
@@ -385,14 +387,21 @@ hipError_t launchMlpTrainGeneral(hipStream_t stream, const TrainLaunch& t, int n
         const uint8_t* dz = ws + dzOff;
         const uint64_t dzStride = (uint64_t)ly.out * esz;
         if (f32) {
-            // fp32 vectors: the scalar accumulate kernels (db: the reduce-sum form, b == 1)
+            // fp32 vectors: into fp32 gradients on the matrix pipeline's fp32 instruction, into half ones through the
+            // scalar accumulate kernels (db: the reduce-sum form, b == 1)
+            const bool pipe = t.gradCt == kF32;
             if (t.bGrad[l]) {
                 const MatrixShape bs{(uint32_t)ly.out, 1u, t.gradCt, kRowMajor, (size_t)elemSize(t.gradCt)};
-                if ((e = launchAccumScalar(stream, dz, dzStride, ly.out, nullptr, 0, 1, ct, batch, t.bGrad[l], bs, ws + p.partials)) != hipSuccess) return e;
+                e = pipe ? launchOuterProductF32(stream, dz, dzStride, ly.out, nullptr, 0, 1, batch, t.bGrad[l], bs, ws + p.partials, numCUs)
+                         : launchAccumScalar(stream, dz, dzStride, ly.out, nullptr, 0, 1, ct, batch, t.bGrad[l], bs, ws + p.partials);
+                if (e != hipSuccess) return e;
             }
             if (t.wGrad[l]) {
-                if ((e = launchAccumScalar(stream, dz, dzStride, ly.out, xl[l], xlStride[l], ly.in, ct, batch, t.wGrad[l], t.gradShape[l],
-                                           ws + p.partials)) != hipSuccess) return e;
+                e = pipe ? launchOuterProductF32(stream, dz, dzStride, ly.out, xl[l], xlStride[l], ly.in, batch, t.wGrad[l], t.gradShape[l],
+                                                 ws + p.partials, numCUs)
+                         : launchAccumScalar(stream, dz, dzStride, ly.out, xl[l], xlStride[l], ly.in, ct, batch, t.wGrad[l], t.gradShape[l],
+                                             ws + p.partials);
+                if (e != hipSuccess) return e;
             }
         }
         if (!f32 && t.bGrad[l]) {

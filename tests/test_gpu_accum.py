@@ -202,7 +202,9 @@ def test_outer_product_float_destinations(t_ct, m_ct):
     mag = np.abs(before.astype(np.float64)) + np.abs(prod).sum(axis=0)
     d = as_bytes(to_dev(before))
     cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, N * before.itemsize, ML.RowMajor, m_ct)
-    assert cv.lastKernelName().startswith("outerScalarKernel"), cv.lastKernelName()
+    # (fp32 vectors into an fp32 matrix have a kernel on the matrix pipeline; every other pair is the scalar definition)
+    kernel = "outerProductF32Kernel" if (t_ct, m_ct) == (CT.Float32, CT.Float32) else "outerScalarKernel"
+    assert cv.lastKernelName().startswith(kernel), cv.lastKernelName()
     got = d.cpu().numpy().view(mt).reshape(M, N).astype(np.float64)
     eps = {np.float16: 2.0 ** -10, np.float32: 2.0 ** -20, np.float64: 2.0 ** -48}[mt]
     assert (np.abs(got - want) <= eps * mag).all()
@@ -283,3 +285,84 @@ def test_reduce_sum_every_plain_type(t_ct):
     with pytest.raises(cv.CoopVecError) as e:                              # the buffer has the vectors' type
         cv.coopVecReduceSumAccumulate(typed(v), d, 0, bufferType=CT.Float16 if t_ct != CT.Float16 else CT.Float32)
     assert e.value.result == cv.SLANG_E_NOT_AVAILABLE
+
+
+# ---------------------------------------------------------------------------------------------
+# fp32 vectors into fp32 destinations: the kernel on v_mfma_f32_16x16x4_f32
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("M,N,B", [(9, 6, 1), (9, 6, 5), (64, 64, 4096), (70, 33, 1500), (128, 16, 70001), (1, 1, 333), (16, 17, 19),
+                                   (17, 16, 64), (130, 129, 300)])
+@pytest.mark.parametrize("layout", [ML.RowMajor, ML.ColumnMajor, ML.TrainingOptimal])
+def test_fp32_outer_product_against_fp64(M, N, B, layout):
+    rng = np.random.default_rng(M * 1000 + N * 10 + B)
+    a = (rng.standard_normal((B, M)) * 2).astype(np.float32); b = (rng.standard_normal((B, N)) * 2).astype(np.float32)
+    before = rng.standard_normal((M, N)).astype(np.float32)
+    prod = a.astype(np.float64)[:, :, None] * b.astype(np.float64)[:, None, :]
+    want = before.astype(np.float64) + prod.sum(axis=0)
+    mag = np.abs(before.astype(np.float64)) + np.abs(prod).sum(axis=0)
+    D = cv.CooperativeVectorMatrixDesc
+    stride = {ML.RowMajor: N * 4, ML.ColumnMajor: M * 4, ML.TrainingOptimal: 0}[layout]
+    size = cv.getCooperativeVectorMatrixSize(M, N, CT.Float32, layout, stride)
+    row_desc = D(M, N, CT.Float32, ML.RowMajor, M * N * 4, 0, N * 4)
+    results = []
+    for _ in range(2):
+        d = torch.zeros(size, dtype=torch.uint8, device=DEV)
+        cv.convertCooperativeVectorMatrix(d, [D(M, N, CT.Float32, layout, size, 0, stride)], as_bytes(to_dev(before)), [row_desc])
+        # strided vectors: rows of a wider array
+        wide_a = torch.zeros((B, M + 3), dtype=torch.float32, device=DEV); wide_a[:, :M] = to_dev(a)
+        cv.coopVecOuterProductAccumulate(wide_a[:, :M], to_dev(b), d, 0, stride, layout, CT.Float32)
+        assert cv.lastKernelName().startswith("outerProductF32Kernel"), cv.lastKernelName()
+        row = torch.zeros(M * N * 4, dtype=torch.uint8, device=DEV)
+        cv.convertCooperativeVectorMatrix(row, [row_desc], d, [D(M, N, CT.Float32, layout, size, 0, stride)])
+        results.append(row.view(torch.float32).cpu().numpy().reshape(M, N).copy())
+    assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32))          # no atomics: the same bits every time
+    assert (np.abs(results[0].astype(np.float64) - want) <= 2.0 ** -20 * mag).all()
+
+
+def test_fp32_outer_product_one_sample_is_the_operator_itself():
+    # one sample: matrix[i][j] += a[i] * b[j] with the product rounded to float, the bits of the Slang fallback
+    rng = np.random.default_rng(77)
+    M, N = 37, 21
+    a = draw(rng, CT.Float32, (1, M)); b = draw(rng, CT.Float32, (1, N)); mat = draw(rng, CT.Float32, (M, N))
+    ref = mat.copy()
+    assert ob.lib().cvo_slang_outer_product_accumulate(ob.ptr(a[0]), M, ob.ptr(b[0]), N, ob.F32, ob.ptr(ref), 0, N * 4, ob.ROW, ob.F32, ob.HALF_RNE) == 0
+    d = as_bytes(to_dev(mat))
+    cv.coopVecOuterProductAccumulate(typed(a), typed(b), d, 0, N * 4, ML.RowMajor, CT.Float32)
+    assert np.array_equal(d.cpu().numpy().view(np.uint32), ref.view(np.uint32).reshape(-1))
+
+
+def test_fp32_outer_product_infinite_element_stays_in_its_row_and_column():
+    # an infinity in the last sample of a ragged batch: the samples past the end that the kernel's loads repeat contribute
+    # nothing, and rows and columns without the infinite element stay finite
+    rng = np.random.default_rng(78)
+    B, M, N = 21, 20, 18
+    a = (rng.standard_normal((B, M))).astype(np.float32); b = (rng.standard_normal((B, N))).astype(np.float32)
+    a[B - 1, 3] = np.inf
+    b[B - 1, 5] = 0.0
+    d = torch.zeros(M * N, dtype=torch.float32, device=DEV)
+    cv.coopVecOuterProductAccumulate(to_dev(a), to_dev(b), d.view(torch.uint8), 0, N * 4, ML.RowMajor, CT.Float32)
+    got = d.cpu().numpy().reshape(M, N)
+    with np.errstate(invalid="ignore"):
+        want = (a.astype(np.float64)[:, :, None] * b.astype(np.float64)[:, None, :]).sum(axis=0)
+    fin = np.isfinite(want)
+    assert np.array_equal(np.isfinite(got), fin) and np.array_equal(np.isnan(got), np.isnan(want))
+    assert not fin[3].any() and fin[np.arange(M) != 3].all()
+    assert np.allclose(got[fin], want[fin], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("N,B", [(1, 7), (9, 5000), (64, 100000), (200, 333), (16, 16)])
+def test_fp32_reduce_sum_against_fp64(N, B):
+    rng = np.random.default_rng(N * 31 + B)
+    v = (rng.standard_normal((B, N)) * 3).astype(np.float32)
+    buf = rng.standard_normal(N).astype(np.float32)
+    want = buf.astype(np.float64) + v.astype(np.float64).sum(axis=0)
+    mag = np.abs(buf.astype(np.float64)) + np.abs(v.astype(np.float64)).sum(axis=0)
+    out = []
+    for _ in range(2):
+        d = as_bytes(to_dev(buf))
+        cv.coopVecReduceSumAccumulate(to_dev(v), d, 0)
+        assert cv.lastKernelName().startswith("outerProductF32Kernel"), cv.lastKernelName()
+        out.append(d.cpu().numpy().view(np.float32).copy())
+    assert np.array_equal(out[0].view(np.uint32), out[1].view(np.uint32))
+    assert (np.abs(out[0].astype(np.float64) - want) <= 2.0 ** -20 * mag).all()
