@@ -19,7 +19,7 @@ Adam update, two kernels in a HIP graph), op / rs (stand-alone outer-product / r
 (that encoder and its decoder network in one kernel / as two calls), ew (an element-wise operator), ad (the Adam update
 over 2^24 parameters), cm (the example's per-iteration layout conversion), nf (the neural module's FFLayer chain over a
 parameter block).  With --workload only that one runs and becomes the headline (profiling runs; also
-c5g = c5 on the layer-by-layer step, copy = a plain device copy of
+c5g = c5 on the layer-by-layer step, f32 / f32t = forward pass / training step of an fp32 network, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
 Before the W warm-up steps of a workload its step runs untimed for --clock-ramp-ms (default 100 ms,
@@ -484,6 +484,72 @@ def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
                 cpu_baseline=cpu_baseline, key=key or ("c5g" if flags else "c5"))
 
 
+def workload_f32t(torch, cv, steps, warmup):
+    """fp32 training step 32->64->64->8 (FFLayer<float> chain), ReLU, MSE against given targets, batch 2^20, fp32 TrainingOptimal
+    gradients: the layer-by-layer step on the fp32 matMul, element-wise and outer-product kernels."""
+    import numpy as np
+    from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
+                                   FeedForwardLayer)
+    dev = "cuda"
+    dims = [32, 64, 64, 8]
+    B = 1 << 20
+    g = torch.Generator(device=dev); g.manual_seed(20256)
+    layers, host = [], []
+    for i in range(len(dims) - 1):
+        fi, fo = dims[i], dims[i + 1]
+        W = torch.randn(fo, fi, device=dev, generator=g) * (2.0 / fi) ** 0.5
+        bias = torch.randn(fo, device=dev, generator=g) * 0.1
+        gsize = cv.getCooperativeVectorMatrixSize(fo, fi, CT.Float32, ML.TrainingOptimal)
+        wg = torch.zeros(gsize, dtype=torch.uint8, device=dev)
+        bg = torch.zeros(fo, dtype=torch.float32, device=dev)
+        last = i == len(dims) - 2
+        layers.append(FeedForwardLayer(fi, fo, W.contiguous().view(torch.uint8).flatten(), bias.view(torch.uint8),
+                                       ML.RowMajor, fi * 4, Activation.NoActivation if last else Activation.ReLU, 0.0,
+                                       wg, bg.view(torch.uint8), ML.TrainingOptimal, 0))
+        host.append((W, bias))
+    x = torch.rand(B, dims[0], device=dev, generator=g) * 2 - 1
+    t = torch.rand(B, dims[-1], device=dev, generator=g) * 2 - 1
+    ws = torch.empty(cv.mlpTrainStepWorkspaceSize(layers, B, weightType=CT.Float32), dtype=torch.uint8, device=dev)
+    loss = torch.zeros(1, dtype=torch.float32, device=dev)
+
+    def step():
+        cv.mlpTrainStep(layers, x, t, workspace=ws, lossSum=loss, lossScale=1.0 / B, weightType=CT.Float32)
+
+    macs = sum(dims[i] * dims[i + 1] for i in range(len(dims) - 1))
+    macs_dx = sum(dims[i] * dims[i + 1] for i in range(1, len(dims) - 1))
+
+    def cpu_baseline():
+        n = 1 << 15
+        xs, ts = x[:n].cpu().numpy(), t[:n].cpu().numpy()
+        Ws = [(W.cpu().numpy(), b.cpu().numpy()) for W, b in host]
+        t0 = time.perf_counter()
+        acts, zs, h = [xs], [], xs
+        for i, (W, b) in enumerate(Ws):
+            z = h @ W.T + b
+            zs.append(z)
+            h = np.maximum(z, 0) if i < len(Ws) - 1 else z
+            acts.append(h)
+        gz = (h - ts) * (2.0 / B)
+        for i in range(len(Ws) - 1, -1, -1):
+            dW = gz.T @ acts[i]; db = gz.sum(axis=0)
+            if i:
+                gz = (gz @ Ws[i][0]) * (zs[i - 1] > 0)
+        t1 = time.perf_counter()
+        return {"value": n / (t1 - t0), "unit": "samples/s", "cores": 1, "kind": "port",
+                "sample": "first %d samples; numpy fp32 backpropagation (for T = float the fallback's arithmetic is plain fp32 "
+                          "products and sums)" % n}
+
+    # (the bytes a layer-by-layer step moves: every per-layer vector of the batch is written once and read by its consumers)
+    widths = dims[1:]
+    moved = B * 4 * (dims[0] * 2 + dims[-1] + sum(w * (2 + 3) for w in widths[:-1]) + widths[-1] * 4 + sum(w * 4 for w in widths[:-1]))
+    return dict(step=step, samples=B, alg_bytes=moved, alg_flops=B * 2 * (2 * macs + macs_dx),
+                bound="hbm", mfma="f32", dtype="f32",
+                config={"workload": "f32t: fp32 train step 32->64->64->8, ReLU, MSE against targets, batch 2^20, fp32 "
+                                    "TrainingOptimal gradients, layer-by-layer step (fp32 networks have no fused one)",
+                        "batch": B, "layers": dims},
+                cpu_baseline=cpu_baseline, key="f32t")
+
+
 def workload_t32(torch, cv, steps, warmup):
     """the training step of a 32-wide decoder-sized network, 8->32->32->32->4 (the one-wave fused kernel)"""
     return workload_c5(torch, cv, steps, warmup, dims=[8, 32, 32, 32, 4], key="t32")
@@ -882,7 +948,7 @@ WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": w
              "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
              "cm": workload_cm, "nf": workload_nf, "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
-             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5f16": workload_c5f16, "f32": workload_f32, "copy": workload_copy}
+             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5f16": workload_c5f16, "f32": workload_f32, "f32t": workload_f32t, "copy": workload_copy}
 DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf")
 HEADLINE = "c2"
 

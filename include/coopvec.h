@@ -244,7 +244,9 @@ CV_API CvResult cvMatMul(void* stream, const CvMatMulDesc* desc);
  * The per-sample atomics of the reference are replaced by an MFMA contraction over the batch,
  * per-workgroup fp32 partials in `workspace` and one fixed-order reduction, so the result is
  * bitwise reproducible.  That kernel takes FLOAT16 vectors and a FLOAT16 or FLOAT32 matrix in any of the four
- * layouts.  Every other pair of the fallback's types (FLOAT16/32/64 and the 8/16/32/64-bit integers for the
+ * layouts; FLOAT32 vectors into a FLOAT32 matrix have one of the same kind on the fp32 matrix instruction (each
+ * product enters its sum through a fused multiply-add; a batch of one sample gives the bits of the reference).
+ * Every other pair of the fallback's types (FLOAT16/32/64 and the 8/16/32/64-bit integers for the
  * vectors and for the matrix, :33261-33315) runs as the scalar definition: the product in the vectors' type,
  * cast to the matrix type, summed over the batch (integers modulo 2^width: bit-exact with the reference;
  * floats in fp32, fp64 for a FLOAT64 matrix, in a fixed order), RowMajor / ColumnMajor (fp32 also the Optimal

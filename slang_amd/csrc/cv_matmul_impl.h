@@ -46,9 +46,9 @@ struct VecAsMatrix : Mma {
     // kStreaming: the flavour also gets the branch-free streaming instantiations (the less common
     // ones run every shape on the general kernel)
     static constexpr bool kStreaming = !std::is_same<Mma, Bf8AsF16Mma>::value;
-    // kAlwaysLarge: every shape runs on matmulLargeKernel (fp32 fragments are too wide to keep a
-    // block of the matrix in registers)
-    static constexpr bool kAlwaysLarge = std::is_same<Mma, F32Mma>::value;
+    // kWideFragments: fp32 fragments are twice as wide; a block of the matrix stays in registers up to 64 rows and two
+    // k-tiles (64 columns), everything larger runs on matmulLargeKernel
+    static constexpr bool kWideFragments = std::is_same<Mma, F32Mma>::value;
     static __device__ __forceinline__ void decodeIn(const uint32_t* raw, uint32_t* frag) { Mma::decode(raw, frag); }
 };
 
@@ -58,7 +58,7 @@ struct VecAsMatrix : Mma {
 struct F16VecAsE4M3 : Fp8AsF16Mma {
     static constexpr const char* kName = "f16-as-e4m3-f16pipe";
     static constexpr int kInEsz = 2, kInRawDW = 4;
-    static constexpr bool kAnySign = false, kStreaming = false, kAlwaysLarge = false;
+    static constexpr bool kAnySign = false, kStreaming = false, kWideFragments = false;
     static __device__ __forceinline__ uint32_t roundTrip(uint32_t h2)
     {
         typedef short shortx2 __attribute__((ext_vector_type(2)));
@@ -84,7 +84,7 @@ struct F16VecAsE4M3 : Fp8AsF16Mma {
 struct I8AnySign : I8Mma {
     static constexpr const char* kName = "i8-any-sign";
     static constexpr int kInEsz = 1, kInRawDW = 4;
-    static constexpr bool kAnySign = true, kStreaming = true, kAlwaysLarge = false;
+    static constexpr bool kAnySign = true, kStreaming = true, kWideFragments = false;
     static __device__ __forceinline__ void decodeIn(const uint32_t* raw, uint32_t* frag) { I8Mma::decode(raw, frag); }
 };
 
@@ -651,7 +651,7 @@ hipError_t launchShape(hipStream_t stream, const MatMulArgs& a, int numCUs, bool
             MatMulArgs b = a;
             b.batch = whole;
             // rows of whole 128-byte lines on both sides (and an output row that leaves through the LDS transpose)
-            constexpr bool kLinesShape = 16 * MT * sizeof(OutT) >= 128;
+            constexpr bool kLinesShape = 16 * MT * sizeof(OutT) >= 128 && !Fl::kWideFragments;
             const bool lines = kLinesShape && (((uintptr_t)a.in | a.inStride | (uintptr_t)a.out | a.outStride) & 127u) == 0;
             hipError_t e;
             if constexpr (kLinesShape) {
@@ -702,17 +702,18 @@ hipError_t dispatchBlock(hipStream_t stream, const MatMulArgs& a, int numCUs, bo
         default: return launchLarge<Fl, 8, OutT>(stream, a, largeKT, numCUs, append);
         }
     }
-    if constexpr (!Fl::kAlwaysLarge) {
-        const int KTs = kt <= 1 ? 1 : kt <= 2 ? 2 : kt <= 4 ? 4 : 0;
-        if (!KTs) return hipErrorInvalidValue;
+    const int KTs = kt <= 1 ? 1 : kt <= 2 ? 2 : kt <= 4 ? 4 : 0;
+    if (!KTs) return hipErrorInvalidValue;
 #define CV_CASE(M_, K_) \
-        if (MTs == M_ && KTs == K_) return launchShape<Fl, M_, K_, OutT>(stream, a, numCUs, append);
-        CV_CASE(1, 1) CV_CASE(1, 2) CV_CASE(1, 4)
-        CV_CASE(2, 1) CV_CASE(2, 2) CV_CASE(2, 4)
-        CV_CASE(4, 1) CV_CASE(4, 2) CV_CASE(4, 4)
+    if (MTs == M_ && KTs == K_) return launchShape<Fl, M_, K_, OutT>(stream, a, numCUs, append);
+    CV_CASE(1, 1) CV_CASE(1, 2)
+    CV_CASE(2, 1) CV_CASE(2, 2)
+    CV_CASE(4, 1) CV_CASE(4, 2)
+    if constexpr (!Fl::kWideFragments) {
+        CV_CASE(1, 4) CV_CASE(2, 4) CV_CASE(4, 4)
         CV_CASE(8, 1) CV_CASE(8, 2) CV_CASE(8, 4)
-#undef CV_CASE
     }
+#undef CV_CASE
     return hipErrorInvalidValue;
 }
 
@@ -724,7 +725,9 @@ hipError_t dispatchShape(hipStream_t stream, const MatMulArgs& a, int numCUs)
 {
     const uint32_t kt = optKT((uint32_t)a.k, Fl::kEpl);
     int blockTiles = 8, largeKT = 0;
-    if (kt > 4 || Fl::kAlwaysLarge) {
+    const bool inRegisters = Fl::kWideFragments ? (kt <= 2 && a.m <= 64) : kt <= 4;
+    if (Fl::kWideFragments && inRegisters) blockTiles = 4;
+    if (!inRegisters) {
         largeKT = (int)((kt + kLargeKC - 1) / kLargeKC * kLargeKC);
         const size_t tileBytes = (size_t)largeKT * 64 * Fl::kRawDW * 4;
         while (blockTiles > 1 && blockTiles * tileBytes > (size_t)kLargeLdsBytes) blockTiles /= 2;
