@@ -151,9 +151,10 @@ struct AdamLayersArgs {
 __global__ __launch_bounds__(256) void adamLayersKernel(const AdamLayersArgs a)
 {
     __shared__ float ldsPowers[3];
-    const AdamPowers shared = sharedAdamPowers(a.layers[0].wStates, a.k, ldsPowers);
-    const uint32_t tid = blockIdx.x * 256u + threadIdx.x;
-    if (tid >= a.total) return;
+    // (a thread past the last element works on the last one and leaves before it stores: no branch around the requests)
+    const uint32_t own = blockIdx.x * 256u + threadIdx.x;
+    const bool on = own < a.total;
+    const uint32_t tid = on ? own : a.total - 1u;
     int l = 0;
 #pragma unroll
     for (int i = 1; i < kMaxAdamLayers; ++i)
@@ -172,15 +173,22 @@ __global__ __launch_bounds__(256) void adamLayersKernel(const AdamLayersArgs a)
         grad = ly.bGrad + (size_t)o * (a.gradCt == kF32 ? 4u : 2u);
         state = ly.bStates + o;
     }
-    // an fp32 gradient buffer holds the sum the half buffer of the example would have held unrounded: rounded here
-    const float g = a.gradCt == kF32 ? (float)H(*(const float*)grad) : (float)*(const half_t*)grad;
+    // Requested before the powers are worked out, and nothing is done with them until then: one trip to memory for the
+    // step count, the state, the parameter and the gradient together.  (A half gradient is read as the two bytes it is;
+    // an fp32 one as four, from an address that holds four either way.)
     AdamState st = *state;
     half_t p = *param;
+    const bool wide = a.gradCt == kF32;
+    const uint32_t gbits = wide ? *(const uint32_t*)grad : (uint32_t)*(const uint16_t*)grad;
+    const AdamPowers shared = sharedAdamPowers(a.layers[0].wStates, a.k, ldsPowers);
+    if (!on) return;
+    // an fp32 gradient buffer holds the sum the half buffer of the example would have held unrounded: rounded here
+    const float g = wide ? (float)H(__builtin_bit_cast(float, gbits)) : (float)__builtin_bit_cast(half_t, (uint16_t)gbits);
     if (adamUpdate(st, p, g, a.k, shared)) {
         *param = p;
         *state = st;
     }
-    if (a.gradCt == kF32) *(float*)grad = 0.f; else *(half_t*)grad = (half_t)0;
+    if (wide) *(float*)grad = 0.f; else *(half_t*)grad = (half_t)0;
 }
 
 } // namespace
