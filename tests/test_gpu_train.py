@@ -569,3 +569,42 @@ def test_fused_and_layer_by_layer_steps_agree_on_random_shapes():
             assert np.linalg.norm(aB[l] - bB[l]) <= 1e-3 * scaleB, (case, dims, B, name, l)
         assert abs(la.item() - lb.item()) <= 1e-4 * max(abs(lb.item()), 1e-6), (case, dims, B, name)
     assert fused == 40
+
+
+@pytest.mark.parametrize("grad_ct,grad_layout", [(CT.Float32, ML.TrainingOptimal), (CT.Float32, ML.RowMajor), (CT.Float16, ML.ColumnMajor)])
+@pytest.mark.parametrize("dims,B", [([4, 16, 4], 16), ([8, 16, 16, 3], 50), ([12, 16, 16, 16, 1], 64), ([4, 16, 4], 1)])
+def test_step_of_a_single_workgroup(dims, B, grad_ct, grad_layout):
+    # A batch of at most four tiles (the example's 16 samples) is one workgroup of the one-wave kernel, which adds its sums
+    # to the gradients itself: "+=" onto what the buffers hold, lossSum and lossMax, the same step twice gives the same
+    # bits, and a sample that is not finite voids every sum of the step.
+    rng = np.random.default_rng(sum(dims) * 7 + B)
+    specs = make_specs(rng, dims, act=Activation.LeakyReLU, slope=float(np.float16(0.01)))
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
+    rW, rB, rLoss = ob.ref_mlp_train(specs, x, t, 0.5, True)
+    runs = []
+    for _ in range(2):
+        layers = build(specs, grad_ct, grad_layout, preset=1.0)
+        lmax = torch.full((1,), -1.0, dtype=torch.float32, device=DEV)
+        _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=0.5, gradType=grad_ct, lossMax=lmax)
+        assert cv.lastKernelName().startswith("mlpTrainKernel") and "Reduce" not in cv.lastKernelName().split("+")[0]
+        dW, dB = read_grads(layers, specs, grad_ct, grad_layout)
+        runs.append((loss.item(), lmax.item(), dW, dB))
+    tol = 2e-3 if grad_ct == CT.Float32 else 1e-2
+    loss0, lmax0, dW, dB = runs[0]
+    assert loss0 == runs[1][0] and lmax0 == runs[1][1]
+    for l in range(len(specs)):
+        assert np.array_equal(dW[l], runs[1][2][l]) and np.array_equal(dB[l], runs[1][3][l])
+        assert rel_err(dW[l], rW[l]) < tol, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l] - 1.0, rB[l]) < tol + (0 if grad_ct == CT.Float32 else 2e-2), (l, rel_err(dB[l] - 1.0, rB[l]))     # the preset stayed
+    assert abs(loss0 - rLoss) <= 2e-3 * abs(rLoss) and 0 < lmax0 <= loss0 + 1e-6
+    # not finite: everything the step adds is NaN
+    x[B // 2, 1] = np.inf
+    layers = build(specs, grad_ct, grad_layout, preset=1.0)
+    lmax = torch.zeros(1, dtype=torch.float32, device=DEV)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=0.5, gradType=grad_ct, lossMax=lmax)
+    assert np.isnan(loss.item()) and np.isnan(lmax.item())
+    dW, dB = read_grads(layers, specs, grad_ct, grad_layout)
+    for l in range(len(specs)):
+        valid = np.ones_like(dW[l], bool)
+        assert np.isnan(dW[l]).all() and np.isnan(dB[l]).all()
