@@ -18,8 +18,8 @@ Adam update, two kernels in a HIP graph), op / rs (stand-alone outer-product / r
 (permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), pef / peu
 (that encoder and its decoder network in one kernel / as two calls), ew (an element-wise operator), ad (the Adam update
 over 2^24 parameters), cm (the example's per-iteration layout conversion), nf (the neural module's FFLayer chain over a
-parameter block).  With --workload only that one runs and becomes the headline (profiling runs; also
-c5g = c5 on the layer-by-layer step, f32 / f32t = forward pass / training step of an fp32 network, copy = a plain device copy of
+parameter block), f32 / f32t (forward pass / training step of an fp32 network).  With --workload only that one runs and becomes the headline (profiling runs; also
+c5g = c5 on the layer-by-layer step, copy = a plain device copy of
 known size for scaling the traffic counters).  Prints ONE JSON line.
 
 Before the W warm-up steps of a workload its step runs untimed for --clock-ramp-ms (default 100 ms,
@@ -949,7 +949,7 @@ WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": w
              "cm": workload_cm, "nf": workload_nf, "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
              "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5f16": workload_c5f16, "f32": workload_f32, "f32t": workload_f32t, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf")
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf", "f32", "f32t")
 HEADLINE = "c2"
 
 
