@@ -89,8 +89,9 @@ struct TrainArgs {
     float lossScale;
     float* partials;             // [gridDim.x][partialFloats]
     int32_t wantLossMax;         // also track the largest per-sample loss (slot 1 behind the loss sum of a partial)
-    // A launch of a single workgroup (a batch of at most four tiles, such as the example's 16 samples) adds its partial to
-    // the gradients itself: no second kernel.  `finish` then holds what that kernel would have been given.
+    // A launch of a single workgroup (a batch of at most four tiles, such as the example's 16 samples) adds its sums to
+    // the gradients itself, from its registers: no partial in memory, no second kernel.  `finish` then holds what that
+    // kernel would have been given.
     int32_t finishInKernel;
     TrainReduceArgs finish;
 };
