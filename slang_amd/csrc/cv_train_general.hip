@@ -206,15 +206,39 @@ __global__ __launch_bounds__(256) void lossGradKernel(const LossArgs a)
             tgtAll = (float)(T)sinf((part[0] + part[1]) + (part[2] + part[3]));
         }
         float sampleLoss = 0.f;
-        for (int i = 0; i < a.outDim; ++i) {
-            const size_t e = (size_t)s * a.outDim + i;
-            const float tv = a.targets ? (float)*(const T*)(a.targets + (size_t)s * a.targetStride + sizeof(T) * i)
-                                       : (exampleLoss ? (float)gt[i & 3] : tgtAll);
-            const T diff = (T)((float)y[e] - tv);
+        // one element: the same arithmetic in the same order, whichever way its operands were fetched
+        auto element = [&](int i, T yv, T zv, float tv) -> T {
+            const T diff = (T)((float)yv - tv);
             loss += (float)diff * (float)diff;
             sampleLoss += (float)diff * (float)diff;
             const T g = (T)(2.0f * (float)diff * a.lossScale);
-            dzOut[e] = activationGrad<T>(g, z[e], a.act, a.slope);
+            (void)i;
+            return activationGrad<T>(g, zv, a.act, a.slope);
+        };
+        constexpr int EPC = 16 / (int)sizeof(T);                   // elements of a 16-byte piece
+        const size_t e0 = (size_t)s * a.outDim;
+        const bool pieces = a.outDim % EPC == 0 && (((uintptr_t)a.y | (uintptr_t)a.z | (uintptr_t)a.dz) & 15u) == 0 &&
+                            (!a.targets || (((uintptr_t)a.targets | a.targetStride) & 15u) == 0);
+        if (pieces) {
+            // rows of whole aligned 16-byte pieces: three loads and one store per piece instead of per element
+            for (int i0 = 0; i0 < a.outDim; i0 += EPC) {
+                T yv[EPC], zv[EPC], tvv[EPC], gv[EPC];
+                *(u32x4*)yv = *(const u32x4*)(y + e0 + i0);
+                *(u32x4*)zv = *(const u32x4*)(z + e0 + i0);
+                if (a.targets) *(u32x4*)tvv = *(const u32x4*)(a.targets + (size_t)s * a.targetStride + sizeof(T) * i0);
+#pragma unroll
+                for (int k = 0; k < EPC; ++k) {
+                    const float tv = a.targets ? (float)tvv[k] : (exampleLoss ? (float)gt[(i0 + k) & 3] : tgtAll);
+                    gv[k] = element(i0 + k, yv[k], zv[k], tv);
+                }
+                *(u32x4*)(dzOut + e0 + i0) = *(const u32x4*)gv;
+            }
+        } else {
+            for (int i = 0; i < a.outDim; ++i) {
+                const float tv = a.targets ? (float)*(const T*)(a.targets + (size_t)s * a.targetStride + sizeof(T) * i)
+                                           : (exampleLoss ? (float)gt[i & 3] : tgtAll);
+                dzOut[e0 + i] = element(i, y[e0 + i], z[e0 + i], tv);
+            }
         }
         lossMax = (sampleLoss > lossMax || sampleLoss != sampleLoss) ? sampleLoss : lossMax;
     }
