@@ -339,3 +339,32 @@ def test_query_lists_what_matmul_accepts():
                  (CT.BFloat16, CT.BFloat16, CT.BFloat16, CT.BFloat16),
                  (CT.Float32, CT.Float32, CT.Float32, CT.Float32)]:
         assert tuple(int(v) for v in want) in keys
+
+
+def test_float32_blocks_in_registers_and_in_lds():
+    # Up to 64 rows and 64 columns an fp32 block stays in registers (the kernels of the 16-bit types, their streaming form
+    # for whole aligned vectors); anything larger is staged in LDS.  Large and ragged batches, padded vector rows, `+=`.
+    rng = np.random.default_rng(4242)
+    for M, K, B, pad in ((64, 64, 70001, 0), (64, 32, 4096, 0), (8, 64, 1000, 4), (33, 17, 999, 0), (64, 64, 513, 3), (128, 64, 2000, 0),
+                         (64, 128, 2000, 0)):
+        x = rng.standard_normal((B, K)).astype(np.float32)
+        W = (rng.standard_normal((M, K)) / np.sqrt(K)).astype(np.float32)
+        b = rng.uniform(-0.5, 0.5, M).astype(np.float32)
+        ref64 = x.astype(np.float64) @ W.astype(np.float64).T + b
+        mag = np.abs(x.astype(np.float64)) @ np.abs(W.astype(np.float64)).T + np.abs(b)
+        bound = (K + 1) * 2.0 ** -23 * mag
+        wide = torch.zeros((B, K + pad), dtype=torch.float32, device=DEV); wide[:, :K] = to_dev(x)
+        y = cv.coopVecMatMulAdd(wide[:, :K], CT.Float32, as_bytes(to_dev(W)), 0, CT.Float32, as_bytes(to_dev(b)), 0, CT.Float32,
+                                ML.RowMajor, False, 4 * K, M=M, resultType=CT.Float32)
+        name = cv.lastKernelName()
+        assert name.startswith("matmulKernel<f32" if M <= 64 and K <= 64 else "matmulLargeKernel<f32"), (M, K, name)
+        if (M, K, pad) == (64, 64, 0):
+            assert "streaming" in name, name
+        assert (np.abs(y.cpu().numpy() - ref64) <= bound).all(), (M, K, B)
+        # the member form: this += W x (no bias)
+        acc0 = rng.standard_normal((B, M)).astype(np.float32)
+        out = to_dev(acc0)
+        cv.coopVecMatMul(wide[:, :K], CT.Float32, as_bytes(to_dev(W)), 0, CT.Float32, ML.RowMajor, False, 4 * K, M=M,
+                         resultType=CT.Float32, out=out, accumulate=True)
+        want = acc0.astype(np.float64) + (ref64 - b)
+        assert (np.abs(out.cpu().numpy() - want) <= bound + 2.0 ** -23 * np.abs(want)).all(), (M, K, B, "accumulate")
