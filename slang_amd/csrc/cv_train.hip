@@ -67,29 +67,35 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     // ReLU on every hidden layer and none on the last one gets the straight-line instantiation
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
+    // (the paired kernel also takes hidden layers with leaky ReLU, the example's activation)
+    bool leaky = t.mlp.layers[Net::L - 1].act == kActNone && !plain;
+    for (int l = 0; l + 1 < Net::L; ++l) leaky = leaky && (t.mlp.layers[l].act == kActRelu || t.mlp.layers[l].act == kActLeakyRelu);
     // straight-line input loads: float2 samples of the example's encoding, or slices of whole aligned dwords
     const bool xy = t.mlp.inEncoding == kEncodeXYSquares;
     const bool dwords = !xy && t.mlp.layers[0].in % 2 == 0 && t.mlp.inAlign >= 4u;
     const int variant = !plain || !(xy || dwords) ? 0 : xy ? 2 : 1;
+    const bool pairLeaky = kPairShape && leaky && dwords;
     // a launch of one workgroup of the one-wave-per-SIMD kernel finishes the step itself
-    ta.finishInKernel = (blocks == 1 && !(kPairShape && variant != 0)) ? 1 : 0;
+    ta.finishInKernel = (blocks == 1 && !(kPairShape && (variant != 0 || pairLeaky))) ? 1 : 0;
     ta.finish = ra;
     noteKernel(false, "mlpTrainKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s> + mlpTrainReduceKernel", Net::IT0, Net::KT0,
                Net::HT, Net::L - 1, Net::MTL,
                variant == 0 ? "runtime-act,any-input" : variant == 1 ? "relu/none,dword-input" : "relu/none,xy-input");
-    // 64-wide networks with the plain activations run on the two-waves-per-SIMD kernel
+    // 64- and 32-wide networks with these activations run on the two-waves-per-SIMD kernel
     constexpr bool kPair = kPairShape;
     if constexpr (kPair) {
-        if (variant != 0)
-            noteKernel(false, "mlpTrainPairKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,relu/none,%s> + mlpTrainReduceKernel", Net::IT0,
-                       Net::KT0, Net::HT, Net::L - 1, Net::MTL, variant == 1 ? "dword-input" : "xy-input");
-        if (variant == 1)      hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords>), dim3(blocks), dim3(512), 0, stream, ta);
+        if (variant != 0 || pairLeaky)
+            noteKernel(false, "mlpTrainPairKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s,%s> + mlpTrainReduceKernel", Net::IT0,
+                       Net::KT0, Net::HT, Net::L - 1, Net::MTL, pairLeaky ? "leaky-or-relu/none" : "relu/none",
+                       variant == 2 ? "xy-input" : "dword-input");
+        if (pairLeaky)         hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords, true>), dim3(blocks), dim3(512), 0, stream, ta);
+        else if (variant == 1) hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords>), dim3(blocks), dim3(512), 0, stream, ta);
         else if (variant == 2) hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadXY>), dim3(blocks), dim3(512), 0, stream, ta);
     } else {
         if (variant == 1)      hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadDwords>), dim3(blocks), dim3(256), 0, stream, ta);
         else if (variant == 2) hipLaunchKernelGGL((mlpTrainKernel<Net, kActRelu, kActNone, kLoadXY>), dim3(blocks), dim3(256), 0, stream, ta);
     }
-    if (variant == 0) hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
+    if (variant == 0 && !pairLeaky) hipLaunchKernelGGL((mlpTrainKernel<Net, -1, -1, kLoadAny>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (ta.finishInKernel) return hipSuccess;

@@ -125,7 +125,9 @@ __device__ __forceinline__ uint32_t pairAwait(const volatile LdsWord* theirs, ui
 
 // ReLU on the hidden layers, none on the last one (the launcher sends everything else to the
 // one-wave kernel); LOADS as in mlpTrainKernel.
-template <class Net, int LOADS>
+// LEAKY: each hidden layer ReLU or leaky ReLU, as the arguments say (max(z, z * slope) with the slope as a half, the
+// multiplier of applyActGrad on the way back: fflayer.slang:60-66); without it every hidden layer is ReLU.
+template <class Net, int LOADS, bool LEAKY = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlpTrainPairKernel(const TrainArgs ta)
 {
     typedef F16Mma Mma;
@@ -301,8 +303,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 halfx2 z23 = __builtin_convertvector(floatx2{acc[t][2], acc[t][3]}, halfx2);
                 if constexpr (relu) {
                     zs[l][t][0] = z01; zs[l][t][1] = z23;
-                    z01 = __builtin_elementwise_max(z01, zero2);
-                    z23 = __builtin_elementwise_max(z23, zero2);
+                    halfx2 s01 = zero2, s23 = zero2;
+                    if constexpr (LEAKY) {
+                        if (a.layers[l].act != kActRelu) {
+                            const half_t sl = (half_t)a.layers[l].slope;
+                            s01 = z01 * halfx2{sl, sl}; s23 = z23 * halfx2{sl, sl};
+                        }
+                    }
+                    z01 = __builtin_elementwise_max(z01, s01);
+                    z23 = __builtin_elementwise_max(z23, s23);
                 }
                 car[t][0] = z01; car[t][1] = z23;
             }
@@ -448,8 +457,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     typedef float floatx2 __attribute__((ext_vector_type(2)));
                     const halfx2 g01 = __builtin_convertvector(floatx2{gacc[t][0], gacc[t][1]}, halfx2);
                     const halfx2 g23 = __builtin_convertvector(floatx2{gacc[t][2], gacc[t][3]}, halfx2);
-                    dz[t][0] = g01 * maxGradMultiplier(zs[l - 1][t][0]);
-                    dz[t][1] = g23 * maxGradMultiplier(zs[l - 1][t][1]);
+                    if constexpr (LEAKY) {
+                        const half_t sl = (half_t)a.layers[l - 1].slope;
+                        dz[t][0] = applyActGrad<true>(g01, maxGradMultiplier(zs[l - 1][t][0]), a.layers[l - 1].act, halfx2{sl, sl});
+                        dz[t][1] = applyActGrad<true>(g23, maxGradMultiplier(zs[l - 1][t][1]), a.layers[l - 1].act, halfx2{sl, sl});
+                    } else {
+                        dz[t][0] = g01 * maxGradMultiplier(zs[l - 1][t][0]);
+                        dz[t][1] = g23 * maxGradMultiplier(zs[l - 1][t][1]);
+                    }
                 }
                 packS(dz, MTI, Net::ktOut(l - 1), bS);
             }

@@ -608,3 +608,63 @@ def test_step_of_a_single_workgroup(dims, B, grad_ct, grad_layout):
     for l in range(len(specs)):
         valid = np.ones_like(dW[l], bool)
         assert np.isnan(dW[l]).all() and np.isnan(dB[l]).all()
+
+
+@pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 4099), ([8, 32, 32, 32, 4], 1500), ([20, 64, 64, 8], 777), ([8, 48, 24, 3], 640)])
+def test_leaky_relu_networks_on_the_paired_kernel(dims, B):
+    # hidden layers with leaky ReLU (the example's activation, fflayer.slang:60-66), also mixed with ReLU layers: the paired
+    # kernel, held against the oracle, against the one-wave kernel (taken by vectors at a 2-byte pitch), and to the tie rule
+    rng = np.random.default_rng(sum(dims) * 3 + B)
+    slope = float(np.float16(0.01))
+    specs = make_specs(rng, dims, act=Activation.LeakyReLU, slope=slope)
+    if len(specs) > 2:
+        specs[1]["act"] = int(Activation.ReLU); specs[1]["slope"] = 0.0        # a ReLU layer among the leaky ones
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    x[5] = 0                                                                     # (pre-activations equal to the biases)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
+    layers = build(specs)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=0.25)
+    assert cv.lastKernelName().startswith("mlpTrainPairKernel") and "leaky-or-relu" in cv.lastKernelName(), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 0.25, tie_rule=True)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3, (l, rel_err(dW[l], rW[l]))
+        assert rel_err(dB[l], rB[l]) <= 1e-3, (l, rel_err(dB[l], rB[l]))
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # the same step on the one-wave kernel
+    wide = torch.zeros((B, dims[0] + 1), dtype=torch.float16, device=DEV); wide[:, :dims[0]] = to_dev(x)
+    other = build(specs)
+    _, loss1 = cv.mlpTrainStep(other, wide[:, :dims[0]], to_dev(t), lossScale=0.25)
+    assert cv.lastKernelName().startswith("mlpTrainKernel"), cv.lastKernelName()
+    oW, oB = read_grads(other, specs, CT.Float32, ML.RowMajor)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], oW[l]) <= 2e-6 and rel_err(dB[l], oB[l]) <= 2e-6, (l, rel_err(dW[l], oW[l]), rel_err(dB[l], oB[l]))
+    assert abs(loss.item() - loss1.item()) <= 1e-6 * abs(loss1.item())
+    # bitwise determinism
+    again = build(specs)
+    cv.mlpTrainStep(again, to_dev(x), to_dev(t), lossScale=0.25)
+    for a, b in zip(layers, again):
+        assert torch.equal(a.weightsGrad, b.weightsGrad) and torch.equal(a.biasesGrad, b.biasesGrad)
+
+
+def test_leaky_tie_rule_on_the_paired_kernel():
+    # a hidden unit at exactly z = 0 of a leaky layer passes (1 + slope) / 2 of the gradient (diff.meta.slang:2258-2277 on
+    # max(z, z * slope)); the oracle with the tie rule switched off disagrees
+    slope = 0.25
+    W0 = np.zeros((32, 8), np.float16); W0[0, 0] = 1.0; W0[1, 0] = 0.5; W0[2, 0] = -1.0
+    b0 = np.zeros(32, np.float16); b0[0] = -1.0; b0[1] = 0.25; b0[2] = 0.5
+    W1 = np.zeros((1, 32), np.float16); W1[0, 0] = 2.0; W1[0, 1] = 1.0; W1[0, 2] = 4.0
+    specs = [dict(W=W0, b=b0, act=int(Activation.LeakyReLU), slope=slope), dict(W=W1, b=None, act=0, slope=0.0)]
+    B = 64
+    x = np.zeros((B, 8), np.float16); x[:, 0] = 1.0             # z = [0, 0.75, -0.5, 0 ...]
+    t = np.zeros((B, 1), np.float16)
+    layers = build(specs)
+    cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=1.0 / B)
+    assert cv.lastKernelName().startswith("mlpTrainPairKernel") and "leaky" in cv.lastKernelName(), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, _ = ob.ref_mlp_train(specs, x, t, 1.0 / B, True)
+    nW, nB, _ = ob.ref_mlp_train(specs, x, t, 1.0 / B, False)
+    assert np.allclose(dB[0], rB[0], rtol=1e-3, atol=1e-6) and not np.allclose(rB[0][:1], nB[0][:1], rtol=1e-3)
+    y = 0.75 + 4.0 * (-0.5 * slope)                             # the network's output
+    assert abs(dB[0][0] - 2 * y * 2.0 * (1 + slope) / 2) <= 1e-2 * abs(dB[0][0])
+    assert abs(dB[0][2] - 2 * y * 4.0 * slope) <= 1e-2 * abs(dB[0][2])
