@@ -19,8 +19,11 @@ static bool wide16Shape(const MlpArgs& a, int& H, int& NH, int& K0)
     if (a.inStride != 2u * (uint64_t)K0 || ((uintptr_t)a.in & 15u) != 0 || a.batch == 0 || a.batch > (1u << 31)) return false;
     const int width = a.layers[0].out;
     if (width != 32 && width != 64) return false;
+    // (hidden layers all ReLU or all leaky ReLU)
+    const int hiddenAct = a.layers[0].act;
+    if (hiddenAct != kActRelu && hiddenAct != kActLeakyRelu) return false;
     for (int l = 0; l < L; ++l) {
-        if (l + 1 < L && (a.layers[l].out != width || a.layers[l].act != kActRelu)) return false;
+        if (l + 1 < L && (a.layers[l].out != width || a.layers[l].act != hiddenAct)) return false;
         if (l > 0 && a.layers[l].in != width) return false;
     }
     if (a.layers[L - 1].act != kActNone && a.layers[L - 1].act != kActRelu) return false;
@@ -28,7 +31,8 @@ static bool wide16Shape(const MlpArgs& a, int& H, int& NH, int& K0)
     H = width / 32; NH = L - 1;
     // 64-byte rows with one or two hidden layers are bound by their memory traffic, which the streaming kernel
     // moves faster (whole rows through LDS): 71 against 82 us for 32-64-64-8 over 2^22 samples
-    if (K0 == 32 && NH < 3) return false;
+    // (a leaky network has no streaming instantiation and stays here: 32-64-64-8 over 2^22 samples 191 us on the 16-sample kernel)
+    if (K0 == 32 && NH < 3 && hiddenAct == kActRelu) return false;
     return true;
 }
 

@@ -157,7 +157,10 @@ struct Wide16MemoryFront {
     }
 };
 
-template <int H, int NH, int K0, int WAVES, bool HAS_BIAS, class Front>
+// LEAKY: every hidden layer is leaky ReLU, max(z, z * slope) on the rounded halfs with the slope as a half (what the
+// single-layer operator evaluates, fflayer.slang:60-66): one more packed multiply per pair of values; else every hidden
+// layer is ReLU.
+template <int H, int NH, int K0, int WAVES, bool HAS_BIAS, bool LEAKY = false, class Front = void>
 __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& front)
 {
     constexpr int KS = 2 * H;                          // k-steps of a hidden vector
@@ -266,15 +269,19 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
 #pragma unroll
             for (int T = 0; T < H; ++T) acc[j][T] = mfma32(W0[T][s], B[j][s], acc[j][T]);
     };
-    // accumulators -> fp16 -> ReLU = operands of the next layer, in place
-    auto carrier = [&](int j) {
+    // accumulators -> fp16 -> activation of layer l = operands of the next layer, in place
+    halfx2 slope2[NH];
+#pragma unroll
+    for (int l = 0; l < NH; ++l) { const half_t sl = (half_t)a.layers[l].slope; slope2[l] = halfx2{sl, sl}; }
+    auto carrier = [&](int j, int l) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
             const int T = s / 2, r0 = 8 * (s % 2);
             typedef float floatx2 __attribute__((ext_vector_type(2)));
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const halfx2 p = __builtin_elementwise_max(__builtin_convertvector(floatx2{acc[j][T][r0 + 2 * i], acc[j][T][r0 + 2 * i + 1]}, halfx2), zero2);
+                const halfx2 z = __builtin_convertvector(floatx2{acc[j][T][r0 + 2 * i], acc[j][T][r0 + 2 * i + 1]}, halfx2);
+                const halfx2 p = __builtin_elementwise_max(z, LEAKY ? z * slope2[l] : zero2);
                 B[j][s][i] = __builtin_bit_cast(uint32_t, p);
             }
         }
@@ -324,7 +331,7 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
     // accumulators just freed, a whole phase before the matrix instruction that takes them as C operand.  The order
     // within a phase is given to the scheduler explicitly (left alone it requests the biases right in front of their
     // use and the wave sits out the LDS latency once per layer and tile); nothing moves across a phase boundary.
-    constexpr int NV = 16 * H;      // vector-ALU instructions of one tile's carrier
+    constexpr int NV = (LEAKY ? 24 : 16) * H;      // vector-ALU instructions of one tile's carrier
     constexpr int NL = HAS_BIAS ? 4 * H : 0;
     auto endPhase = []() { __builtin_amdgcn_sched_barrier(0); };
     typename Front::Input in = front.load(pair, n, h, lastSample);
@@ -337,16 +344,16 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
         in = front.load(next < numPairs ? next : numPairs - 1u, n, h, lastSample);      // beyond the end: loaded again, never used
         firstLayer(0);
         endPhase();
-        firstLayer(1); carrier(0); seedLayer(1, 0);
+        firstLayer(1); carrier(0, 0); seedLayer(1, 0);
         interleavePhase<H * S0, NV, NL>(); endPhase();
 #pragma unroll
         for (int l = 1; l < NH; ++l) {
-            hiddenLayer(l, 0); carrier(1); seedLayer(l, 1);
+            hiddenLayer(l, 0); carrier(1, l - 1); seedLayer(l, 1);
             interleavePhase<H * KS, NV, NL>(); endPhase();
-            hiddenLayer(l, 1); carrier(0); seedLayer(l + 1, 0);
+            hiddenLayer(l, 1); carrier(0, l); seedLayer(l + 1, 0);
             interleavePhase<H * KS, NV, NL>(); endPhase();
         }
-        lastLayer(0); carrier(1); seedLayer(NH, 1);
+        lastLayer(0); carrier(1, NH - 1); seedLayer(NH, 1);
         interleavePhase<KS, NV, HAS_BIAS ? 4 : 0>(); endPhase();
         lastLayer(1); storeTile(0, 2u * pair); seedLayer(0, 0);
         endPhase();
@@ -356,10 +363,10 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
     }
 }
 
-template <int H, int NH, int K0, int WAVES, bool HAS_BIAS>
+template <int H, int NH, int K0, int WAVES, bool HAS_BIAS, bool LEAKY = false>
 __global__ __launch_bounds__(64 * WAVES) void mlpWide16Kernel(const MlpArgs a)
 {
-    mlpWide16Body<H, NH, K0, WAVES, HAS_BIAS>(a, Wide16MemoryFront<K0>{a.in});
+    mlpWide16Body<H, NH, K0, WAVES, HAS_BIAS, LEAKY>(a, Wide16MemoryFront<K0>{a.in});
 }
 
 // waves per workgroup (one workgroup per compute unit): as many as the weights leave registers for
@@ -374,15 +381,15 @@ constexpr int wide16Waves()
 
 // Shapes: fp16 vectors of 8, 16 or 32 elements in contiguous rows at a 16-byte aligned address, ReLU hidden layers of
 // exactly 32 or 64 units (one to four of them), at most 32 outputs (checked by the dispatcher in cv_mlp_f16.hip).
-template <int H, int NH, int K0, bool HAS_BIAS>
+template <int H, int NH, int K0, bool HAS_BIAS, bool LEAKY = false>
 hipError_t launchMlpWide16Shape(hipStream_t stream, const MlpArgs& a, int numCUs)
 {
     constexpr int WAVES = wide16Waves<H, NH, K0>();
     const uint32_t numPairs = ((a.batch + 31u) / 32u + 1u) / 2u;
     const uint32_t blocks = numPairs < (uint32_t)numCUs ? numPairs : (uint32_t)numCUs;
-    noteKernel(false, "mlpWide16Kernel<f16,32x32x16,inputs=%d,hidden=%dx%d,%s,waves=%d>", K0, NH, 32 * H,
+    noteKernel(false, "mlpWide16Kernel<f16,32x32x16,inputs=%d,hidden=%dx%d%s,%s,waves=%d>", K0, NH, 32 * H, LEAKY ? ",leaky" : "",
                HAS_BIAS ? "bias" : "nobias", WAVES);
-    hipLaunchKernelGGL((mlpWide16Kernel<H, NH, K0, WAVES, HAS_BIAS>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
+    hipLaunchKernelGGL((mlpWide16Kernel<H, NH, K0, WAVES, HAS_BIAS, LEAKY>), dim3(blocks), dim3(64 * WAVES), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -392,8 +399,12 @@ hipError_t launchMlpWide16K(hipStream_t stream, const MlpArgs& a, int numCUs, in
 {
     bool hasBias = false;
     for (int l = 0; l < a.numLayers; ++l) hasBias = hasBias || a.layers[l].bias != nullptr;
+    // (the dispatcher lets in hidden layers that are all ReLU or all leaky ReLU; the leaky instantiation is the one with
+    // biases, which an absent bias vector enters as zeros)
+    const bool leaky = a.layers[0].act == kActLeakyRelu;
 #define CV_W16(h_, nh_) if (H == h_ && NH == nh_) \
-        return hasBias ? launchMlpWide16Shape<h_, nh_, K0, true>(stream, a, numCUs) : launchMlpWide16Shape<h_, nh_, K0, false>(stream, a, numCUs);
+        return leaky ? launchMlpWide16Shape<h_, nh_, K0, true, true>(stream, a, numCUs) \
+             : hasBias ? launchMlpWide16Shape<h_, nh_, K0, true>(stream, a, numCUs) : launchMlpWide16Shape<h_, nh_, K0, false>(stream, a, numCUs);
     CV_W16(1, 1) CV_W16(1, 2) CV_W16(1, 3) CV_W16(1, 4) CV_W16(2, 1) CV_W16(2, 2) CV_W16(2, 3) CV_W16(2, 4)
 #undef CV_W16
     return hipErrorInvalidValue;

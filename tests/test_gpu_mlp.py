@@ -369,11 +369,12 @@ def test_fp16_networks_on_32_sample_tiles(dims, B, bias):
 
 
 def test_fp16_32_sample_tiles_fall_back():
-    # leaky ReLU, rows at a stride and other widths stay on the 16-sample kernels (same results either way)
+    # a ReLU layer among leaky ones, rows at a stride and other widths stay on the 16-sample kernels (same results either way)
     rng = np.random.default_rng(99)
     dims, B = [8, 64, 64, 1], 500
     x = rng.uniform(-1, 1, (B, 8)).astype(np.float16)
     specs = make_net(rng, dims, CT.Float16, act=Activation.LeakyReLU, slope=0.01, bias="rand", init="he")
+    specs[0]["act"] = Activation.ReLU
     y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), to_dev(x))
     assert not cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
     assert torch.equal(y.view(torch.int16), chain_of_single_layers(specs, to_dev(x), CT.Float16).view(torch.int16))
@@ -651,3 +652,32 @@ def test_lean_instantiation_with_padded_weight_rows():
         if cv.lastKernelName().startswith("mlpForwardKernel"):
             assert ("lean" in cv.lastKernelName()) == lean, (pad, cv.lastKernelName())
         assert torch.equal(y.view(torch.int16), yc.view(torch.int16)), pad
+
+
+@pytest.mark.parametrize("dims,B", [([8, 64, 64, 64, 64, 1], 100003), ([16, 32, 32, 32, 4], 4097), ([32, 64, 64, 64, 8], 5000), ([8, 32, 3], 129),
+                                    ([16, 64, 64, 16], 70001)])
+@pytest.mark.parametrize("bias", ["rand", "none"])
+def test_leaky_fp16_networks_on_32_sample_tiles(dims, B, bias):
+    # hidden layers that are all leaky ReLU (the example's activation) run on the 32-sample-tile kernel too: equal to the
+    # chain of single layers bit for bit, and inside the oracle bar; one ReLU layer among them sends the call elsewhere
+    rng = np.random.default_rng(sum(dims) + B)
+    slope = 0.01
+    specs = make_net(rng, dims, CT.Float16, act=Activation.LeakyReLU, slope=slope, bias=bias, init="he")
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    xd = to_dev(x)
+    y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), xd, weightType=CT.Float16)
+    assert cv.lastKernelName().startswith("mlpWide16Kernel") and "leaky" in cv.lastKernelName(), cv.lastKernelName()
+    yc = chain_of_single_layers(specs, xd, CT.Float16)
+    assert torch.equal(y.view(torch.int16), yc.view(torch.int16))
+    # End to end against the oracle: the bar on the outputs.  (What lies outside stems from hidden sums at a rounding
+    # boundary, which the two sides round differently; behind a leaky unit such a flip is scaled by the slope, so the
+    # neighbour test that end_to_end_ok applies to ReLU networks does not fit here.)
+    ref, acts = ob.ref_mlp_forward(specs, x, ob.F16, want_acts=True)
+    ab = np.abs(acts[-2].astype(np.float32)) @ np.abs(specs[-1]["W"].astype(np.float32)).T
+    bad = ob.float_parity_violations(y.cpu().numpy(), ref.astype(np.float32), ab, 2.0 ** -18)
+    assert 1.0 - bad.mean() >= 0.99, 1.0 - bad.mean()
+    if len(specs) > 2:
+        specs[1]["act"] = Activation.ReLU
+        y = cv.mlpForward(gpu_layers(specs, CT.Float16, ML.RowMajor), xd, weightType=CT.Float16)
+        assert not cv.lastKernelName().startswith("mlpWide16Kernel"), cv.lastKernelName()
+        assert torch.equal(y.view(torch.int16), chain_of_single_layers(specs, xd, CT.Float16).view(torch.int16))
