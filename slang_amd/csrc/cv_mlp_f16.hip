@@ -26,7 +26,9 @@ static bool wide16Shape(const MlpArgs& a, int& H, int& NH, int& K0)
         if (l + 1 < L && (a.layers[l].out != width || a.layers[l].act != hiddenAct)) return false;
         if (l > 0 && a.layers[l].in != width) return false;
     }
-    if (a.layers[L - 1].act != kActNone && a.layers[L - 1].act != kActRelu) return false;
+    // (the last layer: none or ReLU; a leaky network's may be leaky ReLU as well)
+    if (a.layers[L - 1].act != kActNone && a.layers[L - 1].act != kActRelu &&
+        !(a.layers[L - 1].act == kActLeakyRelu && a.layers[0].act == kActLeakyRelu)) return false;
     if (a.layers[L - 1].out > 32) return false;
     H = width / 32; NH = L - 1;
     // 64-byte rows with one or two hidden layers are bound by their memory traffic, which the streaming kernel

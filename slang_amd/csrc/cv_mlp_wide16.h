@@ -237,6 +237,9 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
     if (pair >= numPairs) return;
     const uint32_t lastSample = a.batch - 1u;
     const bool lastRelu = a.layers[NH].act == kActRelu;
+    const bool lastLeaky = LEAKY && a.layers[NH].act == kActLeakyRelu;
+    const half_t lastSlope = (half_t)a.layers[NH].slope;
+    const halfx2 lastSlope2 = {lastSlope, lastSlope};
     const int outDim = a.layers[NH].out;
     const bool storeQuads = outDim % 4 == 0 && a.outAlign >= 8u;
     const halfx2 zero2 = {(half_t)0.f, (half_t)0.f};
@@ -311,6 +314,12 @@ __device__ __forceinline__ void mlpWide16Body(const MlpArgs& a, const Front& fro
             if (lastRelu) {
                 p0 = __builtin_elementwise_max(p0, zero2);
                 p1 = __builtin_elementwise_max(p1, zero2);
+            }
+            if constexpr (LEAKY) {      // (the example's layers all have the activation, the last one too)
+                if (lastLeaky) {
+                    p0 = __builtin_elementwise_max(p0, p0 * lastSlope2);
+                    p1 = __builtin_elementwise_max(p1, p1 * lastSlope2);
+                }
             }
             if (storeQuads) {
                 const u32x2 v = {__builtin_bit_cast(uint32_t, p0), __builtin_bit_cast(uint32_t, p1)};

@@ -68,13 +68,14 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     bool plain = t.mlp.layers[Net::L - 1].act == kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) plain = plain && t.mlp.layers[l].act == kActRelu;
     // (the paired kernel also takes hidden layers with leaky ReLU, the example's activation)
-    bool leaky = t.mlp.layers[Net::L - 1].act == kActNone && !plain;
-    for (int l = 0; l + 1 < Net::L; ++l) leaky = leaky && (t.mlp.layers[l].act == kActRelu || t.mlp.layers[l].act == kActLeakyRelu);
+    bool leaky = !plain;
+    for (int l = 0; l < Net::L; ++l)
+        leaky = leaky && (t.mlp.layers[l].act == kActRelu || t.mlp.layers[l].act == kActLeakyRelu || (l + 1 == Net::L && t.mlp.layers[l].act == kActNone));
     // straight-line input loads: float2 samples of the example's encoding, or slices of whole aligned dwords
     const bool xy = t.mlp.inEncoding == kEncodeXYSquares;
     const bool dwords = !xy && t.mlp.layers[0].in % 2 == 0 && t.mlp.inAlign >= 4u;
     const int variant = !plain || !(xy || dwords) ? 0 : xy ? 2 : 1;
-    const bool pairLeaky = kPairShape && leaky && dwords;
+    const bool pairLeaky = kPairShape && leaky && (dwords || xy);
     // a launch of one workgroup of the one-wave-per-SIMD kernel finishes the step itself
     ta.finishInKernel = (blocks == 1 && !(kPairShape && (variant != 0 || pairLeaky))) ? 1 : 0;
     ta.finish = ra;
@@ -86,9 +87,9 @@ hipError_t launchNet(hipStream_t stream, const TrainLaunch& t, int numCUs)
     if constexpr (kPair) {
         if (variant != 0 || pairLeaky)
             noteKernel(false, "mlpTrainPairKernel<IT0=%d,KT0=%d,HT=%d,hidden=%d,MTL=%d,%s,%s> + mlpTrainReduceKernel", Net::IT0,
-                       Net::KT0, Net::HT, Net::L - 1, Net::MTL, pairLeaky ? "leaky-or-relu/none" : "relu/none",
-                       variant == 2 ? "xy-input" : "dword-input");
-        if (pairLeaky)         hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords, true>), dim3(blocks), dim3(512), 0, stream, ta);
+                       Net::KT0, Net::HT, Net::L - 1, Net::MTL, pairLeaky ? "leaky-or-relu" : "relu/none", xy ? "xy-input" : "dword-input");
+        if (pairLeaky && xy)   hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadXY, true>), dim3(blocks), dim3(512), 0, stream, ta);
+        else if (pairLeaky)    hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords, true>), dim3(blocks), dim3(512), 0, stream, ta);
         else if (variant == 1) hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadDwords>), dim3(blocks), dim3(512), 0, stream, ta);
         else if (variant == 2) hipLaunchKernelGGL((mlpTrainPairKernel<Net, kLoadXY>), dim3(blocks), dim3(512), 0, stream, ta);
     } else {

@@ -125,8 +125,9 @@ __device__ __forceinline__ uint32_t pairAwait(const volatile LdsWord* theirs, ui
 
 // ReLU on the hidden layers, none on the last one (the launcher sends everything else to the
 // one-wave kernel); LOADS as in mlpTrainKernel.
-// LEAKY: each hidden layer ReLU or leaky ReLU, as the arguments say (max(z, z * slope) with the slope as a half, the
-// multiplier of applyActGrad on the way back: fflayer.slang:60-66); without it every hidden layer is ReLU.
+// LEAKY: each hidden layer ReLU or leaky ReLU and the last layer none, ReLU or leaky ReLU, as the arguments say
+// (max(z, z * slope) with the slope as a half, the multiplier of applyActGrad on the way back: fflayer.slang:60-66);
+// without it every hidden layer is ReLU and the last layer has no activation.
 template <class Net, int LOADS, bool LEAKY = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void mlpTrainPairKernel(const TrainArgs ta)
 {
@@ -312,6 +313,18 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     }
                     z01 = __builtin_elementwise_max(z01, s01);
                     z23 = __builtin_elementwise_max(z23, s23);
+                } else if constexpr (LEAKY) {
+                    // the last layer's own activation (the example's layers all have one, fflayer.slang:60-66)
+                    zs[l][t][0] = z01; zs[l][t][1] = z23;
+                    if (a.layers[l].act != kActNone) {
+                        halfx2 s01 = zero2, s23 = zero2;
+                        if (a.layers[l].act != kActRelu) {
+                            const half_t sl = (half_t)a.layers[l].slope;
+                            s01 = z01 * halfx2{sl, sl}; s23 = z23 * halfx2{sl, sl};
+                        }
+                        z01 = __builtin_elementwise_max(z01, s01);
+                        z23 = __builtin_elementwise_max(z23, s23);
+                    }
                 }
                 car[t][0] = z01; car[t][1] = z23;
             }
@@ -367,8 +380,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     sampleLoss += on ? (float)diff * (float)diff : 0.f;
                     gv[rr] = on ? (half_t)(2.0f * (float)diff * ta.lossScale) : (half_t)0;
                 }
-                dz[t][0] = halfx2{gv[0], gv[1]};       // the last layer has no activation
+                dz[t][0] = halfx2{gv[0], gv[1]};       // (without LEAKY the last layer has no activation)
                 dz[t][1] = halfx2{gv[2], gv[3]};
+                if constexpr (LEAKY) {
+                    const half_t sl = (half_t)a.layers[L - 1].slope;
+                    dz[t][0] = applyActGrad<true>(dz[t][0], maxGradMultiplier(zs[L - 1][t][0]), a.layers[L - 1].act, halfx2{sl, sl});
+                    dz[t][1] = applyActGrad<true>(dz[t][1], maxGradMultiplier(zs[L - 1][t][1]), a.layers[L - 1].act, halfx2{sl, sl});
+                }
             }
             if (ta.wantLossMax) {       // the sample's rows lie in the four lane groups
                 const float whole = sumOverGroups(sampleLoss);

@@ -619,6 +619,8 @@ def test_leaky_relu_networks_on_the_paired_kernel(dims, B):
     specs = make_specs(rng, dims, act=Activation.LeakyReLU, slope=slope)
     if len(specs) > 2:
         specs[1]["act"] = int(Activation.ReLU); specs[1]["slope"] = 0.0        # a ReLU layer among the leaky ones
+    if B % 2:      # the example's layers all carry the activation, the last one too (fflayer.slang:60-66); or a ReLU there
+        specs[-1]["act"] = int(Activation.LeakyReLU if B % 3 else Activation.ReLU); specs[-1]["slope"] = slope if B % 3 else 0.0
     x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
     x[5] = 0                                                                     # (pre-activations equal to the biases)
     t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
