@@ -12,7 +12,7 @@ way in the same run (W warm-up steps, K timed steps, HIP events on the launch st
 under "workloads": c1 (RowMajor weights, as the configuration names them), c2r (c2 with RowMajor weights), c2b (c2 in
 bfloat16), c3, c3c (c3 with ColumnMajor weights), c4 (e4m3 decoded to the fp16 matrix pipeline), c4n (fp8 matrix pipeline),
 c4h (c4 fed with fp16 vectors), c5f (forward pass of config 5's network at batch 2^22: the fp16 inference workload that the
-matrix pipeline bounds), c5 (training step), c5r (c5 on the kernel whose waves share a tile by kind of work: opt-in, slower),
+matrix pipeline bounds), c5 (training step), c5l (c5 with the example's leaky ReLU behind every layer), c5r (c5 on the kernel whose waves share a tile by kind of work: opt-in, slower),
 t32 / t128 (training steps of a 32-wide and of a 128-wide network), ex (one whole iteration of the example at its own shape: training step +
 Adam update, two kernels in a HIP graph), op / rs (stand-alone outer-product / reduce-sum accumulate), pe / peb / ped
 (permutohedral encoder: the reference test's configuration forward and reverse, and a decoder-shaped one in half), pef / peu
@@ -429,7 +429,7 @@ def workload_f32(torch, cv, steps, warmup):
                 cpu_baseline=cpu_baseline, key="f32")
 
 
-def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
+def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None, leaky=False):
     """fp16 training step 8->64->64->64->64->1, ReLU, MSE vs sin(sum x), batch 2^20, fp32 TrainingOptimal grads."""
     import numpy as np
     from slang_amd.coopvec import (Activation, CoopVecComponentType as CT, CoopVecMatrixLayout as ML,
@@ -447,8 +447,10 @@ def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
         wg = torch.zeros(gsize, dtype=torch.uint8, device=dev)
         bg = torch.zeros(fo, dtype=torch.float32, device=dev)
         last = i == len(dims) - 2
+        # (leaky: the example's FeedForwardLayer, max(z, 0.001 z) behind every layer, the last one too: fflayer.slang:60-66)
+        act = Activation.LeakyReLU if leaky else (Activation.NoActivation if last else Activation.ReLU)
         layers.append(FeedForwardLayer(fi, fo, W.contiguous().view(torch.uint8).flatten(), bias.view(torch.uint8),
-                                       ML.RowMajor, fi * 2, Activation.NoActivation if last else Activation.ReLU, 0.0,
+                                       ML.RowMajor, fi * 2, act, 0.001 if leaky else 0.0,
                                        wg, bg.view(torch.uint8), ML.TrainingOptimal, 0))
         host.append((W, bias))
     x = (torch.rand(B, dims[0], device=dev, generator=g) * 2 - 1).half()
@@ -464,7 +466,8 @@ def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
     def cpu_baseline():
         import oracle_binding as ob
         n = 1 << 11
-        specs = [dict(W=W.cpu().numpy(), b=b.cpu().numpy(), act=1 if i < len(host) - 1 else 0)
+        specs = [dict(W=W.cpu().numpy(), b=b.cpu().numpy(), act=(2 if leaky else 1) if (leaky or i < len(host) - 1) else 0,
+                      slope=float(np.float16(0.001)) if leaky else 0.0)
                  for i, (W, b) in enumerate(host)]
         xs = x[:n].cpu().numpy()
         t0 = time.perf_counter(); ob.ref_mlp_train(specs, xs, None, 1.0, True); t1 = time.perf_counter()
@@ -475,9 +478,10 @@ def workload_c5(torch, cv, steps, warmup, flags=0, dims=None, key=None):
 
     return dict(step=step, samples=B, alg_bytes=B * dims[0] * 2, alg_flops=B * 2 * (2 * macs + macs_dx),
                 bound="mfma", mfma="f16", dtype="f16",
-                config={"workload": "%s: fp16 train step %s, ReLU, MSE vs sin(sum x), batch 2^20, "
+                config={"workload": "%s: fp16 train step %s, %s, MSE vs sin(sum x), batch 2^20, "
                                     "fp32 TrainingOptimal gradients, deterministic reduction%s"
                                     % (key or ("c5g" if flags else "c5"), "->".join(str(d) for d in dims),
+                                       "leaky ReLU (slope 0.001) behind every layer, as the example's layers have it" if leaky else "ReLU",
                                        ", layer-by-layer step (the one for arbitrary layer sizes)" if flags == cv.FLAG_LAYERWISE_TRAINING
                                        else ", waves split by kind of work (CV_FLAG_TRAIN_SPLIT_BY_ROLE)" if flags else ""),
                         "batch": B, "layers": dims},
@@ -548,6 +552,11 @@ def workload_f32t(torch, cv, steps, warmup):
                                     "TrainingOptimal gradients, layer-by-layer step (fp32 networks have no fused one)",
                         "batch": B, "layers": dims},
                 cpu_baseline=cpu_baseline, key="f32t")
+
+
+def workload_c5l(torch, cv, steps, warmup):
+    """config 5's network built from the example's layer: leaky ReLU behind every layer (the paired kernel's leaky instantiation)"""
+    return workload_c5(torch, cv, steps, warmup, key="c5l", leaky=True)
 
 
 def workload_t32(torch, cv, steps, warmup):
@@ -948,8 +957,8 @@ WORKLOADS = {"c1": workload_c1, "c2": workload_c2, "c2r": workload_c2r, "c2b": w
              "c4n": workload_c4n, "c5": workload_c5, "t32": workload_t32, "c5f": workload_c5f, "ex": workload_ex, "op": workload_op, "rs": workload_rs,
              "cm": workload_cm, "nf": workload_nf, "pe": workload_pe, "pef": workload_pef, "peu": workload_peu, "peb": workload_peb, "ped": workload_ped, "ew": workload_ew, "ad": workload_ad,
              # only with --workload: variants and the counter-calibration copy
-             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5f16": workload_c5f16, "f32": workload_f32, "f32t": workload_f32t, "copy": workload_copy}
-DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf", "f32", "f32t")
+             "c4h": workload_c4h, "c5g": workload_c5g, "c5r": workload_c5r, "t128": workload_t128, "c5l": workload_c5l, "c5f16": workload_c5f16, "f32": workload_f32, "f32t": workload_f32t, "copy": workload_copy}
+DEFAULT_RUN = ("c1", "c2r", "c2b", "c3", "c3c", "c4", "c4h", "c4n", "c5f", "c5", "c5l", "c5r", "t32", "t128", "ex", "op", "rs", "pe", "peb", "ped", "pef", "peu", "ew", "ad", "cm", "nf", "f32", "f32t")
 HEADLINE = "c2"
 
 
