@@ -247,6 +247,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     }
                     z01 = __builtin_elementwise_max(z01, s01);
                     z23 = __builtin_elementwise_max(z23, s23);
+                } else if constexpr (LEAKY) {
+                    // the last layer's own activation (the example's layers all have one, fflayer.slang:60-66)
+                    zs[l][t][0] = z01; zs[l][t][1] = z23;
+                    if (a.layers[l].act != kActNone) {
+                        halfx2 s01 = zero2, s23 = zero2;
+                        if (a.layers[l].act != kActRelu) {
+                            const half_t sl = (half_t)a.layers[l].slope;
+                            s01 = z01 * halfx2{sl, sl}; s23 = z23 * halfx2{sl, sl};
+                        }
+                        z01 = __builtin_elementwise_max(z01, s01);
+                        z23 = __builtin_elementwise_max(z23, s23);
+                    }
                 }
                 car[t][0] = z01; car[t][1] = z23;
             }
@@ -301,6 +313,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                 }
                 dz[t][0] = halfx2{gv[0], gv[1]};
                 dz[t][1] = halfx2{gv[2], gv[3]};
+                if constexpr (LEAKY) {      // (without LEAKY the last layer has no activation)
+                    const half_t sl = (half_t)a.layers[L - 1].slope;
+                    dz[t][0] = applyActGrad<true>(dz[t][0], maxGradMultiplier(zs[L - 1][t][0]), a.layers[L - 1].act, halfx2{sl, sl});
+                    dz[t][1] = applyActGrad<true>(dz[t][1], maxGradMultiplier(zs[L - 1][t][1]), a.layers[L - 1].act, halfx2{sl, sl});
+                }
             }
             if (ta.wantLossMax) {
                 const float whole = sumOverGroups(sampleLoss);

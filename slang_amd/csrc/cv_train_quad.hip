@@ -27,9 +27,10 @@ hipError_t launchQuad(hipStream_t stream, const TrainLaunch& t, int numCUs)
     const uint32_t blocks = rounds < (uint32_t)numCUs ? rounds : (uint32_t)numCUs;
     const TrainReduceArgs ra = makeTrainReduceArgs<Net>(t, blocks);
     ta.finish = ra;
-    bool leaky = false;
+    // (the leaky instantiation also takes an activation behind the last layer)
+    bool leaky = t.mlp.layers[Net::L - 1].act != kActNone;
     for (int l = 0; l + 1 < Net::L; ++l) leaky = leaky || t.mlp.layers[l].act == kActLeakyRelu;
-    noteKernel(false, "mlpTrainQuadKernel<IT0=%d,HT=8,hidden=%d,MTL=1,%s> + mlpTrainReduceKernel", IT0, NH, leaky ? "leaky-or-relu/none" : "relu/none");
+    noteKernel(false, "mlpTrainQuadKernel<IT0=%d,HT=8,hidden=%d,MTL=1,%s> + mlpTrainReduceKernel", IT0, NH, leaky ? "leaky-or-relu" : "relu/none");
     if (leaky) hipLaunchKernelGGL((mlpTrainQuadKernel<Net, true>), dim3(blocks), dim3(256), 0, stream, ta);
     else       hipLaunchKernelGGL((mlpTrainQuadKernel<Net, false>), dim3(blocks), dim3(256), 0, stream, ta);
     hipError_t e = hipGetLastError();
@@ -45,7 +46,8 @@ void classifyQuad(const MlpArgs& a, int& it0, int& nh)
     it0 = nh = 0;
     const int L = a.numLayers;
     if (L < 2 || L > 3 || a.inEncoding != kEncodeNone) return;
-    if (a.layers[0].in < 1 || a.layers[0].in > 32 || a.layers[L - 1].out > 16 || a.layers[L - 1].act != kActNone) return;
+    if (a.layers[0].in < 1 || a.layers[0].in > 32 || a.layers[L - 1].out > 16 ||
+        (a.layers[L - 1].act != kActNone && a.layers[L - 1].act != kActRelu && a.layers[L - 1].act != kActLeakyRelu)) return;
     // (the caller sends networks here whose widest hidden layer has 65 to 128 units; a narrower one is padded)
     for (int l = 0; l + 1 < L; ++l)
         if (optMT((uint32_t)a.layers[l].out) > 8u || (a.layers[l].act != kActRelu && a.layers[l].act != kActLeakyRelu)) return;

@@ -533,10 +533,11 @@ def test_train_step_128_wide_tie_rule_and_other_activations():
         assert rel_err(aW[l], rW[l]) <= 1e-3 and rel_err(aB[l], rB[l]) <= 1e-3, l
         assert rel_err(aW[l], gW[l]) <= 1e-3 and rel_err(aB[l], gB[l]) <= 1e-3, l
     assert abs(loss.item() - rloss) <= 1e-3 * rloss
-    # a last layer with an activation: no fused kernel for these widths
+    # a last layer with ReLU or leaky ReLU stays on that instantiation (test_activation_behind_the_last_layer_...); any
+    # other activation there has no fused kernel for these widths
     leaky[2]["act"] = int(Activation.ReLU)
     cv.mlpTrainStep(build(leaky), to_dev(xs), to_dev(ts))
-    assert "layer-by-layer" in cv.lastKernelName()
+    assert cv.lastKernelName().startswith("mlpTrainQuadKernel") and "leaky" in cv.lastKernelName(), cv.lastKernelName()
 
 
 def test_fused_and_layer_by_layer_steps_agree_on_random_shapes():
@@ -670,3 +671,29 @@ def test_leaky_tie_rule_on_the_paired_kernel():
     y = 0.75 + 4.0 * (-0.5 * slope)                             # the network's output
     assert abs(dB[0][0] - 2 * y * 2.0 * (1 + slope) / 2) <= 1e-2 * abs(dB[0][0])
     assert abs(dB[0][2] - 2 * y * 4.0 * slope) <= 1e-2 * abs(dB[0][2])
+
+
+@pytest.mark.parametrize("last", [Activation.LeakyReLU, Activation.ReLU])
+def test_activation_behind_the_last_layer_on_the_four_wave_kernel(last):
+    # a 128-wide network of the example's layers (the activation behind every layer, fflayer.slang:60-66) stays fused
+    rng = np.random.default_rng(130 + int(last))
+    dims, B = [16, 128, 100, 8], 1500
+    slope = float(np.float16(0.01))
+    specs = make_specs(rng, dims, act=Activation.LeakyReLU, slope=slope)
+    specs[-1]["act"] = int(last); specs[-1]["slope"] = slope if last == Activation.LeakyReLU else 0.0
+    x = rng.uniform(-1, 1, (B, dims[0])).astype(np.float16)
+    t = rng.uniform(-1, 1, (B, dims[-1])).astype(np.float16)
+    layers = build(specs)
+    _, loss = cv.mlpTrainStep(layers, to_dev(x), to_dev(t), lossScale=0.25)
+    assert cv.lastKernelName().startswith("mlpTrainQuadKernel"), cv.lastKernelName()
+    dW, dB = read_grads(layers, specs, CT.Float32, ML.RowMajor)
+    rW, rB, rloss = ob.ref_mlp_train(specs, x, t, 0.25, tie_rule=True)
+    for l in range(len(specs)):
+        assert rel_err(dW[l], rW[l]) <= 1e-3 and rel_err(dB[l], rB[l]) <= 1e-3, (l, rel_err(dW[l], rW[l]), rel_err(dB[l], rB[l]))
+    assert abs(loss.item() - rloss) <= 1e-3 * rloss
+    # the layer-by-layer step agrees to its own bar
+    general = build(specs)
+    cv.mlpTrainStep(general, to_dev(x), to_dev(t), lossScale=0.25, flags=cv.FLAG_LAYERWISE_TRAINING)
+    gW, gB = read_grads(general, specs, CT.Float32, ML.RowMajor)
+    for l in range(len(specs)):
+        assert rel_err(gW[l], dW[l]) <= 1e-3 and rel_err(gB[l], dB[l]) <= 1e-3
